@@ -1,0 +1,453 @@
+"""Pins the CPU oracle before anything is compared against it.
+
+Sources of truth used here, none of which is the oracle's own formula retyped:
+  * golden vectors produced by the reference's own header-only containers
+    compiled in place (tests/golden/ref_containers.json);
+  * the known-answer vectors held by the reference's unit tests
+    (kraken/test/t/math_test.cc:323-382, kraken/test/worker/emitter_test.cc);
+  * library optimizers (torch.optim on CPU, fp32) that the reference's headers
+    cite as their definition (ps/optim/sgd.h:10, adagrad.h:11-12, adam.h:11-12,
+    rmsprop.h:10-11);
+  * brute force and invariants on small inputs.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+# --------------------------------------------------------------------------- #
+# hash + container vs the compiled reference
+# --------------------------------------------------------------------------- #
+
+def test_hash64_matches_reference_vectors(oracle):
+    g = json.load(open(os.path.join(GOLDEN, "ref_containers.json")))
+    L = oracle.lib()
+    for k, h in g["hash64"]:
+        assert L.kro_hash64(int(k)) == int(h)
+    for a, b, h in g["hash64_pair"]:
+        assert L.kro_hash64_pair(int(a), int(b)) == int(h)
+
+
+def test_container_matches_reference_vectors(oracle):
+    g = json.load(open(os.path.join(GOLDEN, "ref_containers.json")))["container"]
+    ins = np.array([int(x) for x in g["inserted"]], dtype=np.uint64)
+    vals = np.arange(ins.size * 2, dtype=np.float32).reshape(ins.size, 2)
+    t = oracle.SparseTable(2, oracle.init(oracle.INIT_CONSTANT, 0.0))
+    t.load(ins, vals)
+    assert len(t) == g["fresh"]
+    for k, s in zip(ins[:40], g["slots"]):
+        assert oracle.lib().kro_hit_slot(int(k)) == s
+    ids, v, _, _ = t.export()
+    assert [str(int(x)) for x in ids] == g["export_order"]
+    # duplicate inserts are rejected: the first value wins, as in SkipList::Insert
+    first = {}
+    for k, row in zip(ins, vals):
+        first.setdefault(int(k), row[0])
+    for k, row in zip(ids, v):
+        assert row[0] == first[int(k)]
+    for k, hit, col in zip(g["probe"], g["hit"], g["first_col"]):
+        assert t.contains(int(k)) == bool(hit)
+        if hit:
+            assert first[int(k)] == col
+
+
+def test_container_matches_reference_live(oracle):
+    """Same comparison against the compiled reference itself, when it is built."""
+    import ctypes as C
+    L = oracle.ref_lib()
+    if L is None:
+        pytest.skip("oracle/_ref not built (reference tree absent)")
+    rng = np.random.default_rng(5)
+    ids = rng.integers(0, 2**64, size=20000, dtype=np.uint64)
+    ids[::7] = ids[::-7][: ids[::7].size]  # some duplicates
+    vals = rng.standard_normal((ids.size, 3)).astype(np.float32)
+    m = L.ref_map_create()
+    fresh = L.ref_map_insert(m, ids.ctypes.data_as(C.POINTER(C.c_uint64)), ids.size,
+                             vals.ctypes.data_as(C.POINTER(C.c_float)), 3)
+    t = oracle.SparseTable(3, oracle.init(oracle.INIT_CONSTANT, 0.0))
+    t.load(ids, vals)
+    assert len(t) == fresh
+    order = np.empty(ids.size, np.uint64)
+    n = L.ref_map_keys(m, order.ctypes.data_as(C.POINTER(C.c_uint64)))
+    eid, ev, _, _ = t.export()
+    assert n == eid.size and np.array_equal(order[:n], eid)
+    probe = np.concatenate([ids[:500], rng.integers(0, 2**64, size=500, dtype=np.uint64)])
+    hit = np.empty(probe.size, np.uint8)
+    got = np.zeros((probe.size, 3), np.float32)
+    L.ref_map_find(m, probe.ctypes.data_as(C.POINTER(C.c_uint64)), probe.size,
+                   hit.ctypes.data_as(C.POINTER(C.c_uint8)),
+                   got.ctypes.data_as(C.POINTER(C.c_float)), 3)
+    rc, rows = t.pull(probe[hit == 1])
+    assert rc == 0 and np.array_equal(rows, got[hit == 1])
+    for k, h in zip(probe[500:520], hit[500:520]):
+        assert t.contains(int(k)) == bool(h)
+    L.ref_map_destroy(m)
+
+
+# --------------------------------------------------------------------------- #
+# codec known-answer vectors held by the reference's math_test.cc
+# --------------------------------------------------------------------------- #
+
+KAT6 = np.array([-1.0, 1.0, 2.0, 3.0, -4.0, -0.1], np.float32)
+KAT10 = np.array([-1.0, 1.0, 2.0, 3.0, -4.0, -0.1, 0.001, 0.00001, 0.000001, 128], np.float32)
+
+
+def test_kat_abs(oracle):            # math_test.cc:323-331
+    assert np.array_equal(oracle.absf(KAT6), np.array([1, 1, 2, 3, 4, 0.1], np.float32))
+
+
+def test_kat_topk(oracle):           # math_test.cc:333-341 : signed values, descending
+    for hw in (1, 2, 8):
+        got = oracle.topk(KAT6, 4, hw_threads=hw)
+        assert np.array_equal(got, np.array([3.0, 2.0, 1.0, -0.1], np.float32))
+
+
+def test_kat_take(oracle):           # math_test.cc:343-354
+    got = oracle.take(KAT6, [0, 1, 3, 5])
+    assert np.array_equal(got, np.array([-1.0, 1.0, 3.0, -0.1], np.float32))
+
+
+def test_kat_tocoo_todense(oracle):  # math_test.cc:356-370
+    idx, val = oracle.to_coo(KAT10, 0.01)
+    assert np.array_equal(idx, [0, 1, 2, 3, 4, 5, 9])
+    dense = oracle.coo_to_dense(idx, val, 10)
+    expect = np.array([-1.0, 1.0, 2.0, 3.0, -4.0, -0.1, 0.0, 0.0, 0.0, 128], np.float32)
+    assert np.array_equal(dense, expect)
+
+
+def test_kat_ltkeep(oracle):         # math_test.cc:372-382
+    got = oracle.lt_keep(KAT10, 0.01)
+    expect = np.array([0, 0, 0, 0, 0, 0, 0.001, 0.00001, 0.000001, 0], np.float32)
+    assert np.array_equal(got, expect)
+
+
+def test_topk_against_sort_and_chunk_quirk(oracle):
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal(4096).astype(np.float32)
+    k = 1024
+    # t_num divides n: chunked selection equals a full sort
+    got = oracle.topk(x, k, hw_threads=4)
+    assert np.array_equal(got, np.sort(x)[::-1][:k])
+    # t_num = 3 does not divide 4096: the last 4096 % 3 = 1 element is never examined
+    # (t/math.cc:573-586); make that element the maximum and watch it go missing.
+    y = x.copy()
+    y[-1] = 100.0
+    got = oracle.topk(y, k, t_num=3)
+    assert 100.0 not in got
+    assert np.array_equal(got, np.sort(y[:-1])[::-1][:k])
+    assert oracle.kth_largest_abs(y, 1) == 100.0
+
+
+def test_codec_error_feedback_invariants(oracle):
+    rng = np.random.default_rng(1)
+    n = 4096
+    s = oracle.DctState(n)
+    assert oracle.DctState(100).compress(np.ones(100, np.float32)) == (None, None)  # n < 256
+    e_prev = np.zeros(n, np.float32)
+    for step in range(5):
+        g = rng.standard_normal(n).astype(np.float32)
+        idx, val = s.compress(g, life_span=2, eta=0.75)
+        f = g + e_prev
+        k = int(n * (1.0 - 0.75))
+        if step % 2 == 0:
+            tau = np.sort(np.abs(f))[::-1][k - 1]
+            assert s.tau == tau
+            assert idx.size >= k
+        assert np.all(np.diff(idx) > 0)
+        assert np.array_equal(val, f[idx])
+        assert np.all(np.abs(val) >= s.tau)
+        # decode + residual reproduces the corrected gradient exactly
+        dense = oracle.coo_to_dense(idx, val, n)
+        assert np.array_equal(dense + s.residual, f)
+        assert np.all(np.abs(s.residual) < s.tau)
+        e_prev = s.residual
+    assert s.step == 5
+
+
+# --------------------------------------------------------------------------- #
+# optimizers vs the library definitions the reference's headers cite
+# --------------------------------------------------------------------------- #
+
+def _torch_run(make_opt, w0, grads, lr):
+    torch = pytest.importorskip("torch")
+    p = torch.nn.Parameter(torch.tensor(w0.copy()))
+    opt = make_opt(torch, [p], lr)
+    for g in grads:
+        p.grad = torch.tensor(g.copy())
+        opt.step()
+    return p.detach().numpy().copy(), opt.state[p]
+
+
+def _oracle_run(oracle, o, w0, grads, lr):
+    v = oracle.Value(w0)
+    for g in grads:
+        assert v.update(o, g, lr) == 0
+    return v
+
+
+def _inputs(n=37, steps=6, seed=0):
+    rng = np.random.default_rng(seed)
+    w0 = rng.standard_normal(n).astype(np.float32)
+    grads = [(rng.standard_normal(n) * 0.5).astype(np.float32) for _ in range(steps)]
+    return w0, grads
+
+
+RTOL = 2e-6   # a handful of fp32 roundings in a different association order
+ATOL = 2e-7
+
+
+@pytest.mark.parametrize("conf", [
+    {}, {"weight_decay": 0.01}, {"momentum": 0.9}, {"momentum": 0.9, "nesterov": True},
+    {"momentum": 0.8, "dampening": 0.3}, {"momentum": 0.9, "weight_decay": 0.1, "nesterov": True},
+])
+def test_sgd_vs_torch(oracle, conf):
+    w0, grads = _inputs()
+    lr = 0.05
+    v = _oracle_run(oracle, oracle.optim(oracle.SGD, **conf), w0, grads, lr)
+    w, st = _torch_run(lambda t, ps, lr: t.optim.SGD(
+        ps, lr=lr, momentum=conf.get("momentum", 0.0), dampening=conf.get("dampening", 0.0),
+        weight_decay=conf.get("weight_decay", 0.0), nesterov=conf.get("nesterov", False)),
+        w0, grads, lr)
+    np.testing.assert_allclose(v.val, w, rtol=RTOL, atol=ATOL)
+    if "momentum" in conf:
+        np.testing.assert_allclose(v.state(oracle.ST_MOMENTUM_BUFFER),
+                                   st["momentum_buffer"].numpy(), rtol=RTOL, atol=ATOL)
+    else:
+        assert v.state(oracle.ST_MOMENTUM_BUFFER) is None
+
+
+def test_sgd_plain_is_the_references_own_known_answer(oracle):
+    """emitter_test.cc:51-63, 89-110: after == before - lr * g, to 4 ULP."""
+    w0, grads = _inputs(100, 1, seed=3)
+    lr = np.float32(0.37)
+    v = _oracle_run(oracle, oracle.optim(oracle.SGD), w0, grads, float(lr))
+    expect = w0 - lr * grads[0]
+    assert np.array_equal(v.val, expect)
+
+
+@pytest.mark.parametrize("conf", [{}, {"weight_decay": 0.05}, {"eps": 1e-6}])
+def test_adagrad_vs_torch(oracle, conf):
+    w0, grads = _inputs(seed=1)
+    lr = 0.05
+    o = oracle.optim(oracle.ADAGRAD, **conf)
+    v = _oracle_run(oracle, o, w0, grads, lr)
+    w, st = _torch_run(lambda t, ps, lr: t.optim.Adagrad(
+        ps, lr=lr, initial_accumulator_value=0.0, eps=conf.get("eps", 1e-10),
+        weight_decay=conf.get("weight_decay", 0.0)), w0, grads, lr)
+    np.testing.assert_allclose(v.val, w, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(v.state(oracle.ST_STATE_SUM), st["sum"].numpy(), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("conf", [{}, {"weight_decay": 0.02}, {"beta1": 0.8, "beta2": 0.9, "eps": 1e-6}])
+def test_adam_vs_torch(oracle, conf):
+    w0, grads = _inputs(seed=2, steps=8)
+    lr = 1e-2
+    o = oracle.optim(oracle.ADAM, **conf)
+    v = _oracle_run(oracle, o, w0, grads, lr)
+    w, st = _torch_run(lambda t, ps, lr: t.optim.Adam(
+        ps, lr=lr, betas=(conf.get("beta1", 0.9), conf.get("beta2", 0.999)),
+        eps=conf.get("eps", 1e-8), weight_decay=conf.get("weight_decay", 0.0)), w0, grads, lr)
+    np.testing.assert_allclose(v.val, w, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(v.state(oracle.ST_FIRST_MOMENT), st["exp_avg"].numpy(), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(v.state(oracle.ST_SECOND_MOMENT), st["exp_avg_sq"].numpy(), rtol=RTOL, atol=ATOL)
+    assert v.steps == 8 and int(st["step"]) == 8
+
+
+def test_adam_amsgrad_special_cases(oracle):
+    """The reference takes max over the bias-corrected second moment
+    (ps/optim/adam.cc:63,72-75), which torch does not. Two cases still reduce to
+    torch: one step, and a constant gradient (corrected v is then constant and
+    equals torch's max(v)/bc2). The general case is evaluated in float64 below
+    from the order of operations in adam.cc:57-75."""
+    w0, _ = _inputs(seed=4)
+    lr = 1e-2
+    g = np.full_like(w0, 0.3)
+    o = oracle.optim(oracle.ADAM, amsgrad=True)
+    v = _oracle_run(oracle, o, w0, [g] * 5, lr)
+    w, _ = _torch_run(lambda t, ps, lr: t.optim.Adam(ps, lr=lr, amsgrad=True), w0, [g] * 5, lr)
+    np.testing.assert_allclose(v.val, w, rtol=1e-5, atol=1e-6)
+    # shrinking gradients: corrected max stays at the early, larger value
+    grads = [np.full_like(w0, s) for s in (1.0, 0.5, 0.1, 0.01)]
+    v = _oracle_run(oracle, o, w0, grads, lr)
+    w = w0.astype(np.float64)
+    m = np.zeros_like(w)
+    vv = np.zeros_like(w)
+    vmax = np.zeros_like(w)
+    for t, gg in enumerate(grads, 1):
+        gg = gg.astype(np.float64)
+        m = 0.9 * m + (1 - 0.9) * gg
+        vv = 0.999 * vv + (1 - 0.999) * gg * gg
+        vhat = vv / (1 - 0.999 ** t)
+        vmax = np.maximum(vmax, vhat)
+        w = w - (lr * (m / (1 - 0.9 ** t))) / (np.sqrt(vmax) + 1e-8)
+    np.testing.assert_allclose(v.val, w, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(v.state(oracle.ST_SECOND_MOMENT_MAX), vmax, rtol=1e-5)
+
+
+@pytest.mark.parametrize("conf", [
+    {}, {"alpha": 0.9}, {"centered": True}, {"momentum": 0.7}, {"momentum": 0.7, "centered": True},
+    {"weight_decay": 0.03, "alpha": 0.9, "eps": 1e-6},
+])
+def test_rmsprop_vs_torch(oracle, conf):
+    w0, grads = _inputs(seed=5)
+    lr = 1e-2
+    o = oracle.optim(oracle.RMSPROP, **conf)
+    v = _oracle_run(oracle, o, w0, grads, lr)
+    w, st = _torch_run(lambda t, ps, lr: t.optim.RMSprop(
+        ps, lr=lr, alpha=conf.get("alpha", 0.99), eps=conf.get("eps", 1e-8),
+        weight_decay=conf.get("weight_decay", 0.0), momentum=conf.get("momentum", 0.0),
+        centered=conf.get("centered", False)), w0, grads, lr)
+    np.testing.assert_allclose(v.val, w, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(v.state(oracle.ST_SQUARE_AVERAGE), st["square_avg"].numpy(),
+                               rtol=RTOL, atol=ATOL)
+    if conf.get("centered"):
+        np.testing.assert_allclose(v.state(oracle.ST_G_AVE), st["grad_avg"].numpy(), rtol=RTOL, atol=ATOL)
+    if "momentum" in conf:
+        np.testing.assert_allclose(v.state(oracle.ST_MOMENTUM_BUFFER),
+                                   st["momentum_buffer"].numpy(), rtol=1e-5, atol=1e-6)
+
+
+def test_optimizer_defaults_and_lazy_state(oracle):
+    """ps/optim/optim.cc:23-101 defaults; state tensors appear on first use only."""
+    a = oracle.optim(oracle.ADAGRAD)
+    assert a.eps == np.float32(1e-10) and not a.has_weight_decay
+    r = oracle.optim(oracle.RMSPROP)
+    assert r.alpha == np.float32(0.99) and r.eps == np.float32(1e-8)
+    ad = oracle.optim(oracle.ADAM)
+    assert (ad.beta1, ad.beta2, ad.eps) == (np.float32(0.9), np.float32(0.999), np.float32(1e-8))
+    v = oracle.Value(np.ones(4, np.float32))
+    assert v.state(oracle.ST_STATE_SUM) is None and v.steps == 0
+    assert v.update(a, np.ones(5, np.float32), 0.1) == 11      # size mismatch
+    assert v.state(oracle.ST_STATE_SUM) is None
+    assert v.update(a, np.ones(4, np.float32), 0.1) == 0
+    assert v.state(oracle.ST_STATE_SUM) is not None
+
+
+# --------------------------------------------------------------------------- #
+# sparse table semantics, initialisers, dedup
+# --------------------------------------------------------------------------- #
+
+def test_sparse_table_semantics(oracle):
+    """emitter_test.cc:65-110 shape: Constant init insert-on-pull, then SGD push."""
+    v0 = 3.25
+    t = oracle.SparseTable(100, oracle.init(oracle.INIT_CONSTANT, v0))
+    rc, rows = t.pull([0, 1])
+    assert rc == 0 and np.array_equal(rows, np.full((2, 100), v0, np.float32))
+    assert len(t) == 2
+    rng = np.random.default_rng(0)
+    g = rng.standard_normal((2, 100)).astype(np.float32)
+    lr = np.float32(0.6)
+    assert t.push(oracle.optim(oracle.SGD), [0, 1], g, float(lr)) == 0
+    rc, after = t.pull([0, 1])
+    assert np.array_equal(after, np.float32(v0) - lr * g)
+    # pull twice gives identical rows and inserts nothing new
+    rc, again = t.pull([1, 0, 1])
+    assert np.array_equal(again, after[[1, 0, 1]]) and len(t) == 2
+    # unseen id on push -> 12, wrong gradient width -> 11, empty request -> 0
+    assert t.push(oracle.optim(oracle.SGD), [0, 99], g, 0.1) == 12
+    assert t.push(oracle.optim(oracle.SGD), [0, 1], g[:, :50], 0.1) == 11
+    assert t.push(oracle.optim(oracle.SGD), [], np.zeros((0, 100), np.float32), 0.1) == 0
+    rc, none = t.pull([])
+    assert rc == 0 and none.shape == (0, 100)
+
+
+def test_initialisers(oracle):
+    d = 64
+    # Xavier on a 1-D [d] tensor: fan_out = d, fan_in = 1 (t/math.cc:24-50)
+    std = oracle.lib().kro_xavier_std(1.5, d)
+    assert abs(std - 1.5 * np.sqrt(2.0 / (1 + d))) < 1e-7
+    n = 4000
+    ids = np.arange(n, dtype=np.uint64) * np.uint64(2654435761)
+    def rows(init):
+        return np.stack([oracle.init_row(init, int(i), d) for i in ids])
+    x = rows(oracle.init(oracle.INIT_NORMAL, 0.5, 0.01, seed=7))
+    assert abs(x.mean() - 0.5) < 1e-4 and abs(x.std() - 0.01) < 1e-4
+    assert abs(((x - 0.5) / 0.01) ** 4).mean() - 3.0 < 0.1          # kurtosis of a normal
+    # rows and elements are decorrelated
+    assert abs(np.corrcoef(x[:, 0], x[:, 1])[0, 1]) < 0.06
+    assert abs(np.corrcoef(x[0::2, 0], x[1::2, 0])[0, 1]) < 0.08
+    u = rows(oracle.init(oracle.INIT_UNIFORM, -2.0, 3.0, seed=7))
+    assert u.min() >= -2.0 and u.max() <= 3.0
+    assert abs(u.mean() - 0.5) < 0.02 and abs(u.var() - 25.0 / 12.0) < 0.03
+    xu = rows(oracle.init(oracle.INIT_XAVIER_UNIFORM, 1.0, seed=1))
+    bound = np.sqrt(3.0) * np.sqrt(2.0 / (1 + d))
+    assert np.abs(xu).max() <= bound * (1 + 1e-6) and abs(xu.std() - bound / np.sqrt(3)) < 2e-3
+    xn = rows(oracle.init(oracle.INIT_XAVIER_NORMAL, 2.0, seed=1))
+    assert abs(xn.std() - 2.0 * np.sqrt(2.0 / (1 + d))) < 2e-3
+    # a different seed gives different rows, the same seed the same rows
+    a = oracle.init_row(oracle.init(oracle.INIT_NORMAL, 0, 1, seed=1), 42, d)
+    b = oracle.init_row(oracle.init(oracle.INIT_NORMAL, 0, 1, seed=2), 42, d)
+    c = oracle.init_row(oracle.init(oracle.INIT_NORMAL, 0, 1, seed=1), 42, d)
+    assert not np.array_equal(a, b) and np.array_equal(a, c)
+
+
+def _brute_dedup(ids, grads=None):
+    seen = {}
+    uids = []
+    inv = []
+    acc = []
+    for p, i in enumerate(ids):
+        i = int(i)
+        if i not in seen:
+            seen[i] = len(uids)
+            uids.append(i)
+            if grads is not None:
+                acc.append(grads[p].copy())
+        elif grads is not None:
+            acc[seen[i]] = acc[seen[i]] + grads[p]     # fp32 +=, position order
+        inv.append(seen[i])
+    return uids, inv, acc
+
+
+@pytest.mark.parametrize("ids", [
+    [], [5], [5, 5, 5, 5], [1, 2, 3, 4], [9, 1, 9, 2, 1, 9, 2**64 - 1, 0, 2**64 - 1],
+])
+def test_dedup_small(oracle, ids):
+    ids = np.array(ids, dtype=np.uint64)
+    uids, inv = oracle.dedup(ids)
+    bu, bi, _ = _brute_dedup(ids)
+    assert [int(x) for x in uids] == bu and list(inv) == bi
+
+
+def test_dedup_sum_random(oracle):
+    rng = np.random.default_rng(11)
+    ids = rng.zipf(1.3, size=3000).astype(np.uint64)
+    g = rng.standard_normal((ids.size, 8)).astype(np.float32)
+    uids, out = oracle.dedup_sum(ids, g)
+    bu, bi, acc = _brute_dedup(ids, g)
+    assert [int(x) for x in uids] == bu
+    assert np.array_equal(out, np.stack(acc))          # same order => bit-exact
+    u2, inv = oracle.dedup(ids)
+    assert np.array_equal(u2, uids) and np.array_equal(uids[inv], ids)
+    # first-occurrence positions are increasing in unique order
+    first = [int(np.argmax(ids == u)) for u in uids[:50]]
+    assert first == sorted(first)
+
+
+def test_dense_table_and_coo(oracle):
+    rng = np.random.default_rng(3)
+    n = 1000
+    w0 = rng.standard_normal(n).astype(np.float32)
+    g = rng.standard_normal(n).astype(np.float32)
+    t = oracle.DenseTable(w0)
+    assert np.array_equal(t.pull(), w0)                          # emitter_test.cc:36-49
+    lr = np.float32(0.4)
+    assert t.push(oracle.optim(oracle.SGD), g, float(lr)) == 0
+    assert np.array_equal(t.pull(), w0 - lr * g)                 # emitter_test.cc:51-63
+    assert t.push(oracle.optim(oracle.SGD), g[:10], 0.1) == 11
+    # COO gradient == densified gradient; empty COO leaves Adam's step counter alone
+    a = oracle.DenseTable(w0)
+    b = oracle.DenseTable(w0)
+    idx, val = oracle.to_coo(g, 1.0)
+    o = oracle.optim(oracle.ADAM)
+    assert a.push_coo(o, idx, val, 0.01) == 0
+    assert b.push(o, oracle.coo_to_dense(idx, val, n), 0.01) == 0
+    assert np.array_equal(a.pull(), b.pull()) and a.steps == 1
+    assert a.push_coo(o, [], [], 0.01) == 0 and a.steps == 1
+    # repeated COO indices accumulate (t/math.cc:1043 "Should add the r maybe same")
+    d = oracle.coo_to_dense([3, 3, 5], [1.0, 2.0, 4.0], 8)
+    assert np.array_equal(d, np.array([0, 0, 0, 3, 0, 4, 0, 0], np.float32))
