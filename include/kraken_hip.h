@@ -1,0 +1,243 @@
+/*
+ * kraken_hip.h -- C ABI of the MI355X table engine behind Kraken's parameter-server tables.
+ *
+ * Every entry point returns one of Kraken's ErrorCode values
+ * (kraken/common/error_code.h:7-33; 0 = success) or a negative KRK_E_* for
+ * conditions the reference cannot have (device failures). Nothing throws
+ * across this boundary; krk_last_error_string() describes the last failure on
+ * the calling thread. Reference citations are relative to the reference
+ * tree's kraken/ directory.
+ *
+ * Pointer arguments are host pointers unless KRK_DEVICE_PTRS is set in
+ * `flags`, in which case every data pointer of that call (ids, rows,
+ * gradients, outputs) is a device pointer on the table's GPU. Calls are
+ * blocking unless KRK_ASYNC is also set (device pointers only): the work is
+ * then only enqueued on the table's stream and a failure is reported by the
+ * next blocking call or by the object's *_sync() function.
+ *
+ * Threading: any number of host threads may call into one table; calls on one
+ * table are serialised (the reference takes a unique lock per slot for Pull
+ * and Push alike, ps/sparse_table.cc:48,88, and a unique lock for a dense
+ * Push, ps/dense_table.cc:40).
+ */
+#ifndef KRAKEN_HIP_H_
+#define KRAKEN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KRK_VERSION 1
+
+/* flags */
+#define KRK_DEVICE_PTRS 0x1u
+#define KRK_ASYNC 0x2u
+
+/* kraken/common/error_code.h:7-33 */
+#define KRK_SUCCESS 0
+#define KRK_UNSUPPORTED_OPTIM 6
+#define KRK_INTERFACE_UNIMPLEMENTED 10
+#define KRK_GRADIENT_UNCOMPATIBLE 11
+#define KRK_SPARSE_ID_NOT_EXIST 12
+#define KRK_UNSUPPORTED_INITIALIZER 13
+/* no reference counterpart */
+#define KRK_E_DEVICE (-2)       /* a HIP call failed, or no usable GPU            */
+#define KRK_E_ARGUMENT (-3)     /* null handle, negative size, bad flag           */
+#define KRK_E_CAPACITY (-4)     /* output buffer too small / table cannot grow    */
+
+/* kraken/common/info.h:46-72 */
+enum { KRK_ADAGRAD = 0, KRK_ADAM = 1, KRK_RMSPROP = 2, KRK_SGD = 3 };
+enum {
+  KRK_INIT_CONSTANT = 0,
+  KRK_INIT_UNIFORM = 1,
+  KRK_INIT_NORMAL = 2,
+  KRK_INIT_XAVIER_UNIFORM = 3,
+  KRK_INIT_XAVIER_NORMAL = 4
+};
+enum {
+  KRK_ST_STEPS = 0,
+  KRK_ST_MOMENTUM_BUFFER = 1,
+  KRK_ST_STATE_SUM = 2,
+  KRK_ST_FIRST_MOMENT = 3,
+  KRK_ST_SECOND_MOMENT = 4,
+  KRK_ST_SECOND_MOMENT_MAX = 5,
+  KRK_ST_SQUARE_AVERAGE = 6,
+  KRK_ST_G_AVE = 7,
+  KRK_ST_COUNT = 8
+};
+
+/* Flattened Optim::Create (ps/optim/optim.cc:18-105): the has_* flags are what
+ * the presence of a conf key sets there. initial_accumulator has no reference
+ * counterpart (Adagrad's state_sum always starts at zero, ps/optim/adagrad.cc:34-36);
+ * it is added to the stored sum when the denominator is formed and must be 0
+ * for reference behaviour. */
+typedef struct krk_optim {
+  int32_t type;
+  int32_t has_weight_decay;
+  float weight_decay;
+  int32_t has_momentum;
+  float momentum;
+  int32_t has_dampening;
+  float dampening;
+  int32_t nesterov;
+  float beta1;
+  float beta2;
+  float eps;
+  int32_t amsgrad;
+  float alpha;
+  int32_t centered;
+  float initial_accumulator;
+} krk_optim;
+
+/* Fills the defaults of ps/optim/optim.cc:23-101 for `type`. */
+int32_t krk_optim_defaults(int32_t type, krk_optim* o);
+/* Applies one "key=value" conf entry the way Optim::Create + utils::ParseConf
+ * (common/utils.h:50-92) do; unknown keys are ignored, unparsable floats leave
+ * the default, as in the reference. */
+int32_t krk_optim_set(krk_optim* o, const char* key, const char* value);
+
+/* Flattened Initializer::Create (ps/initializer/initializer.cc:22-61).
+ * a,b = value,- | lower,upper | mean,stddev | gain,- | gain,- .
+ * Random initialisers are counter based: a row's values depend only on
+ * (seed, id, element), never on arrival order. The reference seeds from
+ * std::random_device per call (t/math.cc:455-464), so only the distribution
+ * can match. */
+typedef struct krk_init {
+  int32_t type;
+  float a;
+  float b;
+  uint64_t seed;
+} krk_init;
+int32_t krk_init_defaults(int32_t type, krk_init* i);
+int32_t krk_init_set(krk_init* i, const char* key, const char* value);
+
+/* ---- runtime ------------------------------------------------------------- */
+/* Selects the GPU used by objects created afterwards on this thread's process
+ * (default 0). Fails with KRK_E_DEVICE when no gfx950 device is usable. */
+int32_t krk_runtime_init(int32_t device);
+const char* krk_last_error_string(void);
+const char* krk_error_message(int32_t code);   /* ErrorCode::Msg, common/error_code.h:35-93 */
+/* Harness helpers: device buffers and timing without any other GPU library. */
+int32_t krk_malloc(void** dptr, size_t bytes);
+int32_t krk_free(void* dptr);
+int32_t krk_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int32_t krk_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int32_t krk_memset(void* dptr, int value, size_t bytes);
+int32_t krk_device_synchronize(void);
+int32_t krk_mem_info(size_t* free_bytes, size_t* total_bytes);
+
+/* ---- sparse table --------------------------------------------------------- */
+typedef struct krk_sparse krk_sparse;
+
+/* SparseTable ctor (ps/sparse_table.cc:7-16) + Initializer::Create.
+ * capacity_hint = expected number of rows (0 = small default); the table grows
+ * on demand. Element type is fp32 (t/element_type.h code 11). */
+int32_t krk_sparse_create(int64_t dim, const krk_init* init, int64_t capacity_hint,
+                          krk_sparse** out);
+int32_t krk_sparse_destroy(krk_sparse* t);
+int32_t krk_sparse_dim(krk_sparse* t, int64_t* dim);
+int32_t krk_sparse_size(krk_sparse* t, int64_t* rows);
+/* Makes room for `rows` rows up front so that later pulls never reallocate. */
+int32_t krk_sparse_reserve(krk_sparse* t, int64_t rows);
+/* Waits for enqueued work and returns the first deferred error (then clears it). */
+int32_t krk_sparse_sync(krk_sparse* t);
+
+/* SparseTable::Pull (ps/sparse_table.cc:33-75): out[i,:] = row of ids[i];
+ * a missing id is inserted with the table's initializer and returned. ids may
+ * repeat. out is [n, dim] contiguous. */
+int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* out,
+                        uint32_t flags);
+/* SparseTable::Push (ps/sparse_table.cc:77-108) + Optim::Update on each row.
+ * ids must be unique (the worker guarantees it, worker/emitter.cc:516-531).
+ * grad_dim != dim returns 11 and changes nothing. A missing id returns 12;
+ * rows whose ids exist are still updated (the reference stops at the first
+ * missing id in an unspecified visiting order). */
+int32_t krk_sparse_push(krk_sparse* t, const krk_optim* o, const uint64_t* ids, int64_t n,
+                        const float* grads, int64_t grad_dim, float lr, uint32_t flags);
+/* The worker-side half fused in front of Push: Emitter::PushSparseTable's
+ * dedup + duplicate-gradient sum (worker/emitter.cc:510-531) followed by
+ * SparseTable::Push, without materialising the unique list. ids may repeat;
+ * grads is [n, grad_dim]. */
+int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* ids, int64_t n,
+                            const float* grads, int64_t grad_dim, float lr, uint32_t flags);
+/* id -> row lookup alone (ParallelSkipList::HitSlot + SkipList::Find,
+ * common/parallel_skip_list.h:100-102, common/skip_list.h:315-324):
+ * rows[i] = dense row index of ids[i], or -1 when absent. Row indices are
+ * assigned in insertion order and have no reference analogue; hit/miss does. */
+int32_t krk_sparse_lookup(krk_sparse* t, const uint64_t* ids, int64_t n, int32_t* rows,
+                          uint32_t flags);
+/* Bulk insert of explicit rows (SkipList::Insert semantics: an id that is
+ * already present keeps its row, common/skip_list.h:237-243). vals is [n, dim]. */
+int32_t krk_sparse_import(krk_sparse* t, const uint64_t* ids, int64_t n, const float* vals,
+                          uint32_t flags);
+/* Dump for the users of SparseTable::mutable_vals() (checkpoint/checkpoint.cc:465-509):
+ * rows in insertion order. Any of ids/vals/state/steps may be NULL. state_type
+ * selects which optimizer state fills `state` (zeros when it was never
+ * created); steps is Adam's per-row counter. capacity = rows the buffers hold. */
+int32_t krk_sparse_export(krk_sparse* t, uint64_t* ids, float* vals, int32_t state_type,
+                          float* state, int64_t* steps, int64_t capacity, int64_t* rows,
+                          uint32_t flags);
+
+/* Emitter::PullSparseTableImpl's dedup (worker/emitter.cc:131-149): unique ids
+ * in first-occurrence order, inv[p] = index of ids[p] in uids. uids and inv
+ * hold n entries; *n_unique receives U. */
+int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv,
+                  int64_t* n_unique, uint32_t flags);
+
+/* ---- dense table ---------------------------------------------------------- */
+typedef struct krk_dense krk_dense;
+/* DenseTable ctor (ps/dense_table.cc:10-13): the table starts as a copy of val[n]. */
+int32_t krk_dense_create(const float* val, int64_t n, uint32_t flags, krk_dense** out);
+int32_t krk_dense_destroy(krk_dense* t);
+int32_t krk_dense_sync(krk_dense* t);
+int32_t krk_dense_pull(krk_dense* t, float* out, uint32_t flags);      /* ps/dense_table.cc:31-37 */
+/* DenseTable::Push (ps/dense_table.cc:39-43); n != table size returns 11. */
+int32_t krk_dense_push(krk_dense* t, const krk_optim* o, const float* grad, int64_t n, float lr,
+                       uint32_t flags);
+/* COO gradient (values + int64 flat indices, as ToCoo emits them): densified
+ * like CooTensorImpl::ToDense (t/coo_tensor_impl.cc:250-260, repeated indices
+ * add up) and applied; nnz == 0 returns success without touching any state
+ * (ps/optim/adam.cc:25-29). */
+int32_t krk_dense_push_coo(krk_dense* t, const krk_optim* o, const int64_t* idx, const float* val,
+                           int64_t nnz, float lr, uint32_t flags);
+/* Optimizer state for parity dumps; zeros when never created. */
+int32_t krk_dense_state(krk_dense* t, int32_t state_type, float* out, uint32_t flags);
+int32_t krk_dense_steps(krk_dense* t, int64_t* steps);
+
+/* ---- threshold ("DCT") gradient codec -------------------------------------- */
+typedef struct krk_dct krk_dct;
+/* DCTEmitter::DenseBag (worker/dct_emitter.cc:12-14): zero residual, tau 0, step 0. */
+int32_t krk_dct_create(int64_t n, krk_dct** out);
+int32_t krk_dct_destroy(krk_dct* s);
+/* DenseBag::MaybeToCoo (worker/dct_emitter.cc:16-43). idx/val hold `capacity`
+ * entries; *nnz receives the count, or -1 when n < 256 (the gradient is to be
+ * sent dense and no state changes). tau is the true k-th largest |grad + e|;
+ * the reference's chunked TopK can skip the last n mod t_num elements
+ * (t/math.cc:573-586). Returns KRK_E_CAPACITY (state unchanged) when
+ * capacity < nnz. */
+int32_t krk_dct_compress(krk_dct* s, const float* grad, uint64_t life_span, float eta,
+                         int64_t* idx, float* val, int64_t capacity, int64_t* nnz,
+                         uint32_t flags);
+int32_t krk_dct_tau(krk_dct* s, float* tau);
+int32_t krk_dct_step(krk_dct* s, uint64_t* step);
+int32_t krk_dct_residual(krk_dct* s, float* out, uint32_t flags);
+/* CooTensorImpl::ToDense for a 1-D shape (t/math.cc:1006-1046): dense[n] is
+ * zeroed, then dense[idx[j]] += val[j]. */
+int32_t krk_coo_to_dense(const int64_t* idx, const float* val, int64_t nnz, float* dense,
+                         int64_t n, uint32_t flags);
+
+/* ---- timing (HIP events on an object's own stream) ------------------------ */
+typedef struct krk_event krk_event;
+int32_t krk_event_create(krk_event** e);
+int32_t krk_event_destroy(krk_event* e);
+/* Exactly one of sparse/dense/dct is non-NULL: the event is recorded on that object's stream. */
+int32_t krk_event_record(krk_event* e, krk_sparse* sparse, krk_dense* dense, krk_dct* dct);
+int32_t krk_event_elapsed_ms(krk_event* start, krk_event* stop, float* ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KRAKEN_HIP_H_ */

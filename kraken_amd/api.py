@@ -1,0 +1,512 @@
+"""ctypes binding of libkraken_hip.so (include/kraken_hip.h) with the reference's names.
+
+`SparseTable`, `DenseTable`, `Optim.create`, `Initializer.create` and `DenseBag` follow
+kraken/ps/{sparse_table,dense_table}.h, ps/optim/optim.h, ps/initializer/initializer.h and
+worker/dct_emitter.h: same arguments, same integer error codes. There is no CPU path: when the
+library or a GPU is missing every call raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libkraken_hip.so")
+
+DEVICE_PTRS = 0x1
+ASYNC = 0x2
+
+SUCCESS = 0
+UNSUPPORTED_OPTIM = 6
+INTERFACE_UNIMPLEMENTED = 10
+GRADIENT_UNCOMPATIBLE = 11
+SPARSE_ID_NOT_EXIST = 12
+UNSUPPORTED_INITIALIZER = 13
+E_DEVICE, E_ARGUMENT, E_CAPACITY = -2, -3, -4
+
+
+class OptimType:          # common/info.h:46-51
+    kAdagrad, kAdam, kRMSprop, kSGD = 0, 1, 2, 3
+
+
+class InitializerType:    # common/info.h:54-60
+    kConstant, kUniform, kNormal, kXavierUniform, kXavierNormal = range(5)
+
+
+class StateType:          # common/info.h:63-72
+    (kSteps, kMomentumBuffer, kStateSum, kFirstMoment, kSecondMoment, kSecondMomentMax,
+     kSquareAverage, kGAve) = range(8)
+
+
+class krk_optim(C.Structure):
+    _fields_ = [
+        ("type", C.c_int32), ("has_weight_decay", C.c_int32), ("weight_decay", C.c_float),
+        ("has_momentum", C.c_int32), ("momentum", C.c_float), ("has_dampening", C.c_int32),
+        ("dampening", C.c_float), ("nesterov", C.c_int32), ("beta1", C.c_float),
+        ("beta2", C.c_float), ("eps", C.c_float), ("amsgrad", C.c_int32),
+        ("alpha", C.c_float), ("centered", C.c_int32), ("initial_accumulator", C.c_float),
+    ]
+
+
+class krk_init(C.Structure):
+    _fields_ = [("type", C.c_int32), ("a", C.c_float), ("b", C.c_float), ("seed", C.c_uint64)]
+
+
+EXPORTS = {
+    # name: (restype, argtypes)
+    "krk_optim_defaults": (C.c_int32, [C.c_int32, C.POINTER(krk_optim)]),
+    "krk_optim_set": (C.c_int32, [C.POINTER(krk_optim), C.c_char_p, C.c_char_p]),
+    "krk_init_defaults": (C.c_int32, [C.c_int32, C.POINTER(krk_init)]),
+    "krk_init_set": (C.c_int32, [C.POINTER(krk_init), C.c_char_p, C.c_char_p]),
+    "krk_runtime_init": (C.c_int32, [C.c_int32]),
+    "krk_last_error_string": (C.c_char_p, []),
+    "krk_error_message": (C.c_char_p, [C.c_int32]),
+    "krk_malloc": (C.c_int32, [C.POINTER(C.c_void_p), C.c_size_t]),
+    "krk_free": (C.c_int32, [C.c_void_p]),
+    "krk_memcpy_h2d": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "krk_memcpy_d2h": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "krk_memset": (C.c_int32, [C.c_void_p, C.c_int, C.c_size_t]),
+    "krk_device_synchronize": (C.c_int32, []),
+    "krk_mem_info": (C.c_int32, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "krk_sparse_create": (C.c_int32, [C.c_int64, C.POINTER(krk_init), C.c_int64, C.POINTER(C.c_void_p)]),
+    "krk_sparse_destroy": (C.c_int32, [C.c_void_p]),
+    "krk_sparse_dim": (C.c_int32, [C.c_void_p, C.POINTER(C.c_int64)]),
+    "krk_sparse_size": (C.c_int32, [C.c_void_p, C.POINTER(C.c_int64)]),
+    "krk_sparse_reserve": (C.c_int32, [C.c_void_p, C.c_int64]),
+    "krk_sparse_sync": (C.c_int32, [C.c_void_p]),
+    "krk_sparse_pull": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_uint32]),
+    "krk_sparse_push": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_int64, C.c_void_p,
+                                    C.c_int64, C.c_float, C.c_uint32]),
+    "krk_sparse_push_raw": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_int64,
+                                        C.c_void_p, C.c_int64, C.c_float, C.c_uint32]),
+    "krk_sparse_lookup": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_uint32]),
+    "krk_sparse_import": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_uint32]),
+    "krk_sparse_export": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p,
+                                      C.c_void_p, C.c_int64, C.POINTER(C.c_int64), C.c_uint32]),
+    "krk_dedup": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64),
+                              C.c_uint32]),
+    "krk_dense_create": (C.c_int32, [C.c_void_p, C.c_int64, C.c_uint32, C.POINTER(C.c_void_p)]),
+    "krk_dense_destroy": (C.c_int32, [C.c_void_p]),
+    "krk_dense_sync": (C.c_int32, [C.c_void_p]),
+    "krk_dense_pull": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_uint32]),
+    "krk_dense_push": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_int64, C.c_float,
+                                   C.c_uint32]),
+    "krk_dense_push_coo": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_void_p,
+                                       C.c_int64, C.c_float, C.c_uint32]),
+    "krk_dense_state": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_uint32]),
+    "krk_dense_steps": (C.c_int32, [C.c_void_p, C.POINTER(C.c_int64)]),
+    "krk_dct_create": (C.c_int32, [C.c_int64, C.POINTER(C.c_void_p)]),
+    "krk_dct_destroy": (C.c_int32, [C.c_void_p]),
+    "krk_dct_compress": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_float, C.c_void_p,
+                                     C.c_void_p, C.c_int64, C.POINTER(C.c_int64), C.c_uint32]),
+    "krk_dct_tau": (C.c_int32, [C.c_void_p, C.POINTER(C.c_float)]),
+    "krk_dct_step": (C.c_int32, [C.c_void_p, C.POINTER(C.c_uint64)]),
+    "krk_dct_residual": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_uint32]),
+    "krk_coo_to_dense": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64,
+                                     C.c_uint32]),
+    "krk_event_create": (C.c_int32, [C.POINTER(C.c_void_p)]),
+    "krk_event_destroy": (C.c_int32, [C.c_void_p]),
+    "krk_event_record": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "krk_event_elapsed_ms": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
+    "krk_dct2_forward": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_uint32]),
+    "krk_dct2_inverse": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_uint32]),
+}
+
+_lib = None
+
+
+class KrakenHipError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        msg = lib().krk_last_error_string().decode() if _lib is not None else ""
+        super().__init__("%s failed with code %d (%s) %s" % (
+            what, code, lib().krk_error_message(code).decode(), msg))
+
+
+def lib():
+    """Loads the shared library; raises when it has not been built (no fallback exists)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("%s is missing: build it with `python -m kraken_amd.build`; "
+                           "there is no CPU implementation to fall back to" % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    for name, (res, args) in EXPORTS.items():
+        if not hasattr(L, name):
+            continue
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = L
+    return L
+
+
+def _check(rc, what):
+    if rc != SUCCESS:
+        raise KrakenHipError(rc, what)
+
+
+def _ptr(a):
+    if a is None:
+        return None
+    if isinstance(a, DeviceArray):
+        return C.c_void_p(a.ptr)
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class DeviceArray:
+    """A typed device buffer owned by the harness (krk_malloc); not part of the table engine."""
+
+    def __init__(self, shape, dtype):
+        self.shape = tuple(shape) if isinstance(shape, (tuple, list)) else (int(shape),)
+        self.dtype = np.dtype(dtype)
+        self.size = int(np.prod(self.shape)) if self.shape else 1
+        self.nbytes = self.size * self.dtype.itemsize
+        p = C.c_void_p()
+        _check(lib().krk_malloc(C.byref(p), max(self.nbytes, 16)), "krk_malloc")
+        self.ptr = p.value
+
+    @classmethod
+    def from_host(cls, a):
+        a = np.ascontiguousarray(a)
+        d = cls(a.shape, a.dtype)
+        _check(lib().krk_memcpy_h2d(C.c_void_p(d.ptr), a.ctypes.data_as(C.c_void_p), a.nbytes), "h2d")
+        return d
+
+    def to_host(self):
+        out = np.empty(self.shape, self.dtype)
+        _check(lib().krk_memcpy_d2h(out.ctypes.data_as(C.c_void_p), C.c_void_p(self.ptr), self.nbytes),
+               "d2h")
+        return out
+
+    def free(self):
+        if self.ptr:
+            lib().krk_free(C.c_void_p(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def synchronize():
+    _check(lib().krk_device_synchronize(), "krk_device_synchronize")
+
+
+class Optim:
+    """ps/optim/optim.h: built from (OptimType, string conf) like Optim::Create."""
+
+    def __init__(self, raw):
+        self.raw = raw
+
+    @staticmethod
+    def create(optim_type, conf=None):
+        o = krk_optim()
+        rc = lib().krk_optim_defaults(int(optim_type), C.byref(o))
+        if rc != SUCCESS:
+            return None          # Optim::Create returns an empty pointer for an unknown type
+        for k, v in (conf or {}).items():
+            if isinstance(v, bool):
+                v = "true" if v else "false"
+            lib().krk_optim_set(C.byref(o), str(k).encode(), str(v).encode())
+        return Optim(o)
+
+    @property
+    def optim_type(self):
+        return self.raw.type
+
+
+class Initializer:
+    """ps/initializer/initializer.h: built from (InitializerType, string conf)."""
+
+    def __init__(self, raw):
+        self.raw = raw
+
+    @staticmethod
+    def create(init_type, conf=None):
+        i = krk_init()
+        rc = lib().krk_init_defaults(int(init_type), C.byref(i))
+        if rc != SUCCESS:
+            return None
+        for k, v in (conf or {}).items():
+            lib().krk_init_set(C.byref(i), str(k).encode(), str(v).encode())
+        return Initializer(i)
+
+    @property
+    def type(self):
+        return self.raw.type
+
+
+def _flags(*arrays, extra=0):
+    dev = [isinstance(a, DeviceArray) for a in arrays if a is not None]
+    if dev and all(dev):
+        return DEVICE_PTRS | extra
+    if any(dev):
+        raise ValueError("mix of host and device arrays in one call")
+    return extra
+
+
+class SparseTable:
+    """ps/sparse_table.h. Pull/Push return the reference's int32 error code."""
+
+    def __init__(self, dimension, initializer, capacity_hint=0):
+        self.dimension = int(dimension)
+        h = C.c_void_p()
+        _check(lib().krk_sparse_create(self.dimension, C.byref(initializer.raw), capacity_hint,
+                                       C.byref(h)), "krk_sparse_create")
+        self.h = h
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().krk_sparse_destroy(self.h)
+            self.h = None
+
+    __del__ = close
+
+    def __len__(self):
+        n = C.c_int64()
+        _check(lib().krk_sparse_size(self.h, C.byref(n)), "krk_sparse_size")
+        return n.value
+
+    def reserve(self, rows):
+        _check(lib().krk_sparse_reserve(self.h, rows), "krk_sparse_reserve")
+
+    def sync(self):
+        return lib().krk_sparse_sync(self.h)
+
+    def Pull(self, sparse_ids, out=None, async_=False):
+        """-> (code, vals[n, dimension])"""
+        if isinstance(sparse_ids, DeviceArray):
+            n = sparse_ids.size
+            if out is None:
+                out = DeviceArray((n, self.dimension), np.float32)
+        else:
+            sparse_ids = np.ascontiguousarray(sparse_ids, dtype=np.uint64)
+            n = sparse_ids.size
+            if out is None:
+                out = np.empty((n, self.dimension), np.float32)
+        rc = lib().krk_sparse_pull(self.h, _ptr(sparse_ids), n, _ptr(out),
+                                   _flags(sparse_ids, out, extra=ASYNC if async_ else 0))
+        return rc, out
+
+    def Push(self, optim, sparse_ids, grads, lr, async_=False, raw=False):
+        if isinstance(sparse_ids, DeviceArray):
+            n = sparse_ids.size
+            gd = grads.shape[-1]
+        else:
+            sparse_ids = np.ascontiguousarray(sparse_ids, dtype=np.uint64)
+            grads = np.ascontiguousarray(grads, dtype=np.float32)
+            n = sparse_ids.size
+            gd = grads.shape[-1] if grads.ndim > 1 else (grads.size // max(n, 1))
+        fn = lib().krk_sparse_push_raw if raw else lib().krk_sparse_push
+        return fn(self.h, C.byref(optim.raw), _ptr(sparse_ids), n, _ptr(grads), gd, lr,
+                  _flags(sparse_ids, grads, extra=ASYNC if async_ else 0))
+
+    def PushRaw(self, optim, ids, grads, lr, async_=False):
+        """Emitter::PushSparseTable's dedup + sum fused with Push: ids may repeat."""
+        return self.Push(optim, ids, grads, lr, async_=async_, raw=True)
+
+    def lookup(self, ids):
+        if isinstance(ids, DeviceArray):
+            rows = DeviceArray(ids.size, np.int32)
+            n = ids.size
+        else:
+            ids = np.ascontiguousarray(ids, dtype=np.uint64)
+            rows = np.empty(ids.size, np.int32)
+            n = ids.size
+        _check(lib().krk_sparse_lookup(self.h, _ptr(ids), n, _ptr(rows), _flags(ids, rows)),
+               "krk_sparse_lookup")
+        return rows
+
+    def load(self, ids, vals):
+        if not isinstance(ids, DeviceArray):
+            ids = np.ascontiguousarray(ids, dtype=np.uint64)
+            vals = np.ascontiguousarray(vals, dtype=np.float32)
+        _check(lib().krk_sparse_import(self.h, _ptr(ids), ids.size, _ptr(vals), _flags(ids, vals)),
+               "krk_sparse_import")
+
+    def export(self, state_type=None):
+        """-> ids[rows], vals[rows, dim], state[rows, dim] or None, steps[rows] (insertion order)"""
+        n = len(self)
+        ids = np.empty(n, np.uint64)
+        vals = np.empty((n, self.dimension), np.float32)
+        steps = np.empty(n, np.int64)
+        st = np.empty((n, self.dimension), np.float32) if state_type is not None else None
+        rows = C.c_int64()
+        _check(lib().krk_sparse_export(self.h, _ptr(ids), _ptr(vals),
+                                       state_type if state_type is not None else 1, _ptr(st),
+                                       _ptr(steps), n, C.byref(rows), 0), "krk_sparse_export")
+        assert rows.value == n
+        return ids, vals, st, steps
+
+
+class DenseTable:
+    """ps/dense_table.h"""
+
+    def __init__(self, val):
+        if isinstance(val, DeviceArray):
+            self.n = val.size
+            flags = DEVICE_PTRS
+        else:
+            val = np.ascontiguousarray(val, dtype=np.float32).ravel()
+            self.n = val.size
+            flags = 0
+        h = C.c_void_p()
+        _check(lib().krk_dense_create(_ptr(val), self.n, flags, C.byref(h)), "krk_dense_create")
+        self.h = h
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().krk_dense_destroy(self.h)
+            self.h = None
+
+    __del__ = close
+
+    def sync(self):
+        return lib().krk_dense_sync(self.h)
+
+    def Pull(self, out=None):
+        if out is None:
+            out = np.empty(self.n, np.float32)
+        rc = lib().krk_dense_pull(self.h, _ptr(out), _flags(out))
+        return rc, out
+
+    def Push(self, optim, grad, lr, async_=False):
+        if not isinstance(grad, DeviceArray):
+            grad = np.ascontiguousarray(grad, dtype=np.float32).ravel()
+        return lib().krk_dense_push(self.h, C.byref(optim.raw), _ptr(grad), grad.size, lr,
+                                    _flags(grad, extra=ASYNC if async_ else 0))
+
+    def PushCoo(self, optim, indices, values, lr):
+        if not isinstance(indices, DeviceArray):
+            indices = np.ascontiguousarray(indices, dtype=np.int64)
+            values = np.ascontiguousarray(values, dtype=np.float32)
+        return lib().krk_dense_push_coo(self.h, C.byref(optim.raw), _ptr(indices), _ptr(values),
+                                        indices.size, lr, _flags(indices, values))
+
+    def state(self, state_type):
+        out = np.empty(self.n, np.float32)
+        _check(lib().krk_dense_state(self.h, state_type, _ptr(out), 0), "krk_dense_state")
+        return out
+
+    @property
+    def steps(self):
+        s = C.c_int64()
+        _check(lib().krk_dense_steps(self.h, C.byref(s)), "krk_dense_steps")
+        return s.value
+
+
+def dedup(ids):
+    """Emitter::PullSparseTableImpl's dedup -> (uids, inv)"""
+    if isinstance(ids, DeviceArray):
+        n = ids.size
+        uids = DeviceArray(n, np.uint64)
+        inv = DeviceArray(n, np.int64)
+    else:
+        ids = np.ascontiguousarray(ids, dtype=np.uint64)
+        n = ids.size
+        uids = np.empty(n, np.uint64)
+        inv = np.empty(n, np.int64)
+    u = C.c_int64()
+    _check(lib().krk_dedup(_ptr(ids), n, _ptr(uids), _ptr(inv), C.byref(u), _flags(ids, uids, inv)),
+           "krk_dedup")
+    if isinstance(ids, DeviceArray):
+        return uids, inv, u.value
+    return uids[:u.value].copy(), inv
+
+
+class DenseBag:
+    """worker/dct_emitter.h DCTEmitter::DenseBag: error-feedback threshold codec state."""
+
+    def __init__(self, n):
+        self.n = int(n)
+        h = C.c_void_p()
+        _check(lib().krk_dct_create(self.n, C.byref(h)), "krk_dct_create")
+        self.h = h
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().krk_dct_destroy(self.h)
+            self.h = None
+
+    __del__ = close
+
+    def MaybeToCoo(self, life_span, eta, grad, idx=None, val=None):
+        """-> (indices, values) or (None, None) when the gradient is to be sent dense."""
+        dev = isinstance(grad, DeviceArray)
+        if not dev:
+            grad = np.ascontiguousarray(grad, dtype=np.float32).ravel()
+        if idx is None:
+            idx = DeviceArray(self.n, np.int64) if dev else np.empty(self.n, np.int64)
+            val = DeviceArray(self.n, np.float32) if dev else np.empty(self.n, np.float32)
+        nnz = C.c_int64()
+        _check(lib().krk_dct_compress(self.h, _ptr(grad), life_span, eta, _ptr(idx), _ptr(val),
+                                      idx.size, C.byref(nnz), _flags(grad, idx, val)),
+               "krk_dct_compress")
+        if nnz.value < 0:
+            return None, None
+        if dev:
+            return idx, val, nnz.value
+        return idx[:nnz.value].copy(), val[:nnz.value].copy()
+
+    @property
+    def tau(self):
+        t = C.c_float()
+        _check(lib().krk_dct_tau(self.h, C.byref(t)), "krk_dct_tau")
+        return t.value
+
+    @property
+    def step(self):
+        s = C.c_uint64()
+        _check(lib().krk_dct_step(self.h, C.byref(s)), "krk_dct_step")
+        return s.value
+
+    @property
+    def residual(self):
+        out = np.empty(self.n, np.float32)
+        _check(lib().krk_dct_residual(self.h, _ptr(out), 0), "krk_dct_residual")
+        return out
+
+
+def coo_to_dense(indices, values, n):
+    """CooTensorImpl::ToDense for a 1-D shape."""
+    if isinstance(indices, DeviceArray):
+        out = DeviceArray(n, np.float32)
+        nnz = indices.size
+    else:
+        indices = np.ascontiguousarray(indices, dtype=np.int64)
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        out = np.empty(n, np.float32)
+        nnz = indices.size
+    _check(lib().krk_coo_to_dense(_ptr(indices), _ptr(values), nnz, _ptr(out), n,
+                                  _flags(indices, values, out)), "krk_coo_to_dense")
+    return out
+
+
+class Event:
+    def __init__(self):
+        h = C.c_void_p()
+        _check(lib().krk_event_create(C.byref(h)), "krk_event_create")
+        self.h = h
+
+    def record(self, obj):
+        s = obj.h if isinstance(obj, SparseTable) else None
+        d = obj.h if isinstance(obj, DenseTable) else None
+        c = obj.h if isinstance(obj, DenseBag) else None
+        _check(lib().krk_event_record(self.h, s, d, c), "krk_event_record")
+
+    def elapsed_ms(self, stop):
+        ms = C.c_float()
+        _check(lib().krk_event_elapsed_ms(self.h, stop.h, C.byref(ms)), "krk_event_elapsed_ms")
+        return ms.value
+
+    def __del__(self):
+        try:
+            if getattr(self, "h", None):
+                lib().krk_event_destroy(self.h)
+                self.h = None
+        except Exception:
+            pass

@@ -1,0 +1,386 @@
+// Threshold gradient codec ("DCT" = dynamic communication thresholding in the reference):
+// DCTEmitter::DenseBag::MaybeToCoo (worker/dct_emitter.cc:16-43) and its decode,
+// CooTensorImpl::ToDense (t/coo_tensor_impl.cc:250-260).
+//
+//   f = grad + e                                   error feedback
+//   every life_span steps: tau = k-th largest |f|, k = (int64)(n * (1.0 - eta))
+//   emit (idx, f[idx]) for |f| >= tau, idx ascending; e = |f| < tau ? f : 0
+//
+// tau comes from a three-pass radix select over the bit patterns of |f| (non-negative floats
+// order like their bit patterns): 11 + 11 + 10 bits, each pass one LDS histogram per workgroup.
+// The emit step is a count pass, a scan of the per-tile counts and a write pass that recomputes
+// f, so the output order is the input order.
+#include <new>
+
+#include "krk_internal.h"
+
+struct krk_dct : krk::ObjBase {
+  int64_t n = 0;
+  float* e = nullptr;            // residual
+  float* e_next = nullptr;       // written by the emit pass, swapped in on success
+  uint32_t* sel = nullptr;       // device: [0] prefix bits, [1] k remaining (lo), [2] tau bits, [3] nnz
+  uint32_t* hist = nullptr;      // 2048 bins
+  int32_t* tile_counts = nullptr;
+  int32_t* tile_offsets = nullptr;
+  void* scan_tmp = nullptr;
+  uint32_t* host_sel = nullptr;  // pinned
+  float tau = 0.0f;
+  uint64_t step = 0;
+  int64_t tiles = 0;
+};
+
+namespace krk {
+
+constexpr int kCodecBlock = 256;
+constexpr int kCodecItems = 8;
+constexpr int kCodecTile = kCodecBlock * kCodecItems;
+constexpr int kBins = 2048;
+
+__device__ __forceinline__ uint32_t abs_bits(float f) { return __float_as_uint(f) & 0x7FFFFFFFu; }
+
+// Histogram of `bits` bits of |g+e| at `shift`, over the elements whose higher bits equal the
+// prefix chosen by the earlier passes. sel[0] = prefix (already shifted down to those bits).
+__global__ __launch_bounds__(kCodecBlock) void select_hist_kernel(const float* __restrict__ g,
+                                                                  const float* __restrict__ e, int64_t n,
+                                                                  int shift, int bits, int prefix_shift,
+                                                                  const uint32_t* __restrict__ sel,
+                                                                  uint32_t* __restrict__ hist) {
+  __shared__ uint32_t lh[kBins];
+  for (int i = threadIdx.x; i < kBins; i += kCodecBlock) lh[i] = 0;
+  __syncthreads();
+  const uint32_t prefix = sel[0];
+  const uint32_t mask = (1u << bits) - 1u;
+  const int64_t stride = (int64_t)gridDim.x * kCodecBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x; i < n; i += stride) {
+    const uint32_t u = abs_bits(g[i] + e[i]);
+    if (prefix_shift >= 32 || (u >> prefix_shift) == prefix) atomicAdd(&lh[(u >> shift) & mask], 1u);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < kBins; i += kCodecBlock) {
+    const uint32_t c = lh[i];
+    if (c) atomicAdd(&hist[i], c);
+  }
+}
+
+// Walks the histogram from the top bin down until k elements are covered; extends the prefix by
+// that bin and leaves the rank still to be found inside it. One workgroup; clears the histogram.
+__global__ __launch_bounds__(kCodecBlock) void select_pick_kernel(uint32_t* __restrict__ hist, int bits,
+                                                                  uint32_t* __restrict__ sel, int last) {
+  __shared__ uint32_t lh[kBins];
+  const int nb = 1 << bits;
+  for (int i = threadIdx.x; i < kBins; i += kCodecBlock) {
+    lh[i] = i < nb ? hist[i] : 0;
+    hist[i] = 0;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t k = sel[1];
+    int b = nb - 1;
+    for (; b > 0; --b) {
+      const uint32_t c = lh[b];
+      if (c >= k) break;
+      k -= c;
+    }
+    const uint32_t prefix = (sel[0] << bits) | (uint32_t)b;
+    sel[0] = prefix;
+    sel[1] = k;
+    if (last) sel[2] = prefix;   // the full bit pattern of tau
+  }
+}
+
+__global__ void select_begin_kernel(uint32_t* sel, uint32_t k) {
+  sel[0] = 0;
+  sel[1] = k;
+}
+
+// Per tile of kCodecTile consecutive elements: how many have |g+e| >= tau.
+__global__ __launch_bounds__(kCodecBlock) void emit_count_kernel(const float* __restrict__ g,
+                                                                 const float* __restrict__ e, int64_t n,
+                                                                 const uint32_t* __restrict__ sel,
+                                                                 int32_t* __restrict__ tile_counts) {
+  __shared__ int wave_sum[kCodecBlock / 64];
+  const uint32_t tau_bits = sel[2];
+  const int64_t base = (int64_t)blockIdx.x * kCodecTile + (int64_t)threadIdx.x * kCodecItems;
+  int c = 0;
+#pragma unroll
+  for (int i = 0; i < kCodecItems; ++i) {
+    const int64_t j = base + i;
+    if (j < n) c += abs_bits(g[j] + e[j]) >= tau_bits ? 1 : 0;
+  }
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) c += __shfl_down(c, d, 64);
+  if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int s = 0;
+#pragma unroll
+    for (int w = 0; w < kCodecBlock / 64; ++w) s += wave_sum[w];
+    tile_counts[blockIdx.x] = s;
+  }
+}
+
+// Writes the kept (index, value) pairs in input order and the new residual.
+__global__ __launch_bounds__(kCodecBlock) void emit_write_kernel(
+    const float* __restrict__ g, const float* __restrict__ e, int64_t n,
+    const uint32_t* __restrict__ sel, const int32_t* __restrict__ tile_offsets,
+    long long* __restrict__ idx, float* __restrict__ val, float* __restrict__ e_next) {
+  __shared__ int wave_sum[kCodecBlock / 64];
+  const uint32_t tau_bits = sel[2];
+  const int64_t base = (int64_t)blockIdx.x * kCodecTile + (int64_t)threadIdx.x * kCodecItems;
+  float f[kCodecItems];
+  bool keep[kCodecItems];
+  int c = 0;
+#pragma unroll
+  for (int i = 0; i < kCodecItems; ++i) {
+    const int64_t j = base + i;
+    f[i] = j < n ? g[j] + e[j] : 0.0f;
+    keep[i] = j < n && abs_bits(f[i]) >= tau_bits;
+    c += keep[i] ? 1 : 0;
+  }
+  // exclusive scan of the per-thread counts across the workgroup
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  int x = c;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int y = __shfl_up(x, d, 64);
+    if (lane >= d) x += y;
+  }
+  if (lane == 63) wave_sum[wave] = x;
+  __syncthreads();
+  int off = tile_offsets[blockIdx.x] + x - c;
+#pragma unroll
+  for (int w = 0; w < kCodecBlock / 64; ++w)
+    if (w < wave) off += wave_sum[w];
+#pragma unroll
+  for (int i = 0; i < kCodecItems; ++i) {
+    const int64_t j = base + i;
+    if (j < n) {
+      if (keep[i]) {
+        idx[off] = j;
+        val[off] = f[i];
+        ++off;
+      }
+      e_next[j] = keep[i] ? 0.0f : f[i];   // t/math.cc:1098-1123 : |x| < th keeps x
+    }
+  }
+}
+
+__global__ __launch_bounds__(kCodecBlock) void coo_add_kernel(const long long* __restrict__ idx,
+                                                              const float* __restrict__ val, int64_t nnz,
+                                                              float* __restrict__ dense, int64_t n) {
+  const int64_t j = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x;
+  if (j >= nnz) return;
+  const long long i = idx[j];
+  if (i >= 0 && i < n) atomicAdd(&dense[i], val[j]);
+}
+
+static unsigned stream_grid(int64_t n) {
+  int64_t blocks = (n + kCodecBlock - 1) / kCodecBlock;
+  if (blocks > 256 * 8) blocks = 256 * 8;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
+}  // namespace krk
+
+using namespace krk;
+
+extern "C" {
+
+int32_t krk_dct_create(int64_t n, krk_dct** out) {
+  if (!out || n < 0 || n >= (int64_t)0x7FFFFFFF) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  krk_dct* s = new (std::nothrow) krk_dct();
+  if (!s) return KRK_E_DEVICE;
+  s->n = n;
+  s->tiles = (n + kCodecTile - 1) / kCodecTile;
+  if (s->tiles < 1) s->tiles = 1;
+  int32_t rc = s->open_stream();
+  if (rc == KRK_SUCCESS) {
+    const size_t nb = (size_t)(n ? n : 1) * sizeof(float);
+    hipError_t e = hipMalloc((void**)&s->e, nb);
+    if (e == hipSuccess) e = hipMalloc((void**)&s->e_next, nb);
+    if (e == hipSuccess) e = hipMalloc((void**)&s->sel, 64);
+    if (e == hipSuccess) e = hipMalloc((void**)&s->hist, kBins * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMalloc((void**)&s->tile_counts, (size_t)s->tiles * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void**)&s->tile_offsets, (size_t)s->tiles * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc(&s->scan_tmp, scan_scratch_bytes(s->tiles));
+    if (e == hipSuccess) e = hipHostMalloc((void**)&s->host_sel, 64, hipHostMallocDefault);
+    if (e == hipSuccess) e = hipMemsetAsync(s->e, 0, nb, s->stream);   // dct_emitter.cc:54 : val.Clone().Zero()
+    if (e == hipSuccess) e = hipMemsetAsync(s->sel, 0, 64, s->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(s->hist, 0, kBins * sizeof(uint32_t), s->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(s->stream);
+    if (e != hipSuccess) rc = hip_fail(e, "krk_dct_create", __FILE__, __LINE__);
+  }
+  if (rc != KRK_SUCCESS) {
+    krk_dct_destroy(s);
+    return rc;
+  }
+  *out = s;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dct_destroy(krk_dct* s) {
+  if (!s) return KRK_SUCCESS;
+  if (s->stream) (void)hipStreamSynchronize(s->stream);
+  if (s->e) (void)hipFree(s->e);
+  if (s->e_next) (void)hipFree(s->e_next);
+  if (s->sel) (void)hipFree(s->sel);
+  if (s->hist) (void)hipFree(s->hist);
+  if (s->tile_counts) (void)hipFree(s->tile_counts);
+  if (s->tile_offsets) (void)hipFree(s->tile_offsets);
+  if (s->scan_tmp) (void)hipFree(s->scan_tmp);
+  if (s->host_sel) (void)hipHostFree(s->host_sel);
+  s->close_stream();
+  delete s;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dct_compress(krk_dct* s, const float* grad, uint64_t life_span, float eta, int64_t* idx,
+                         float* val, int64_t capacity, int64_t* nnz, uint32_t flags) {
+  if (!s || !nnz) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  KRK_TRY(check_flags(flags));
+  if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;   // the count comes back by value
+  if (life_span == 0 || capacity < 0) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(s->mu);
+  const int64_t n = s->n;
+  if (n < 256) {   // worker/dct_emitter.cc:18-20
+    *nnz = -1;
+    return KRK_SUCCESS;
+  }
+  if (!grad || (capacity > 0 && (!idx || !val))) return KRK_E_ARGUMENT;
+  const float* d_g;
+  KRK_TRY(s->input(grad, (size_t)n, flags, 0, &d_g));
+  const bool reselect = s->step % life_span == 0;   // :25
+  if (reselect) {
+    const int64_t k = (int64_t)((double)n * (1.0 - (double)eta));   // :27
+    if (k < 1 || k > n) {
+      set_error("eta %g keeps %lld of %lld elements; TopK needs 1..n", (double)eta, (long long)k,
+                (long long)n);
+      return KRK_E_ARGUMENT;   // t/math.cc:628-633 rejects k == 0
+    }
+    hipLaunchKernelGGL(select_begin_kernel, dim3(1), dim3(1), 0, s->stream, s->sel, (uint32_t)k);
+    const int pass_bits[3] = {11, 11, 10};
+    int shift = 32;
+    for (int p = 0; p < 3; ++p) {
+      const int prefix_shift = shift;        // bits above this pass are already fixed
+      shift -= pass_bits[p];
+      hipLaunchKernelGGL(select_hist_kernel, dim3(stream_grid(n)), dim3(kCodecBlock), 0, s->stream, d_g,
+                         s->e, n, shift, pass_bits[p], prefix_shift, s->sel, s->hist);
+      hipLaunchKernelGGL(select_pick_kernel, dim3(1), dim3(kCodecBlock), 0, s->stream, s->hist,
+                         pass_bits[p], s->sel, p == 2 ? 1 : 0);
+    }
+    KRK_HIP(hipGetLastError());
+  }
+  hipLaunchKernelGGL(emit_count_kernel, dim3((unsigned)s->tiles), dim3(kCodecBlock), 0, s->stream, d_g,
+                     s->e, n, s->sel, s->tile_counts);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(exclusive_scan_i32(s->tile_counts, s->tile_offsets, s->tiles,
+                             reinterpret_cast<int32_t*>(s->sel + 3), s->scan_tmp, s->stream));
+  KRK_HIP(hipMemcpyAsync(s->host_sel, s->sel, 16, hipMemcpyDeviceToHost, s->stream));
+  KRK_HIP(hipStreamSynchronize(s->stream));
+  const int64_t count = (int64_t)s->host_sel[3];
+  const float new_tau = __builtin_bit_cast(float, s->host_sel[2]);
+  *nnz = count;
+  if (count > capacity) {
+    // nothing was committed: restore the threshold the next call will see
+    if (reselect) {
+      const uint32_t old_bits = __builtin_bit_cast(uint32_t, s->tau);
+      KRK_HIP(hipMemcpyAsync(s->sel + 2, &old_bits, 4, hipMemcpyHostToDevice, s->stream));
+      KRK_HIP(hipStreamSynchronize(s->stream));
+    }
+    set_error("compress needs room for %lld entries, caller offered %lld", (long long)count,
+              (long long)capacity);
+    return KRK_E_CAPACITY;
+  }
+  long long* d_idx;
+  float* d_val;
+  KRK_TRY(s->output(reinterpret_cast<long long*>(idx), (size_t)count, flags, 1, &d_idx));
+  KRK_TRY(s->output(val, (size_t)count, flags, 2, &d_val));
+  hipLaunchKernelGGL(emit_write_kernel, dim3((unsigned)s->tiles), dim3(kCodecBlock), 0, s->stream, d_g,
+                     s->e, n, s->sel, s->tile_offsets, d_idx, d_val, s->e_next);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(s->output_back(reinterpret_cast<long long*>(idx), (size_t)count, flags, 1));
+  KRK_TRY(s->output_back(val, (size_t)count, flags, 2));
+  KRK_HIP(hipStreamSynchronize(s->stream));
+  float* tmp = s->e;
+  s->e = s->e_next;
+  s->e_next = tmp;
+  s->tau = new_tau;
+  s->step += 1;   // :40
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dct_tau(krk_dct* s, float* tau) {
+  if (!s || !tau) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(s->mu);
+  *tau = s->tau;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dct_step(krk_dct* s, uint64_t* step) {
+  if (!s || !step) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(s->mu);
+  *step = s->step;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dct_residual(krk_dct* s, float* out, uint32_t flags) {
+  if (!s || (s->n > 0 && !out)) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  KRK_TRY(check_flags(flags));
+  std::lock_guard<std::mutex> lk(s->mu);
+  if (s->n)
+    KRK_HIP(hipMemcpyAsync(out, s->e, (size_t)s->n * sizeof(float),
+                           (flags & KRK_DEVICE_PTRS) ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost,
+                           s->stream));
+  if (!(flags & KRK_ASYNC)) KRK_HIP(hipStreamSynchronize(s->stream));
+  return KRK_SUCCESS;
+}
+
+int32_t krk_coo_to_dense(const int64_t* idx, const float* val, int64_t nnz, float* dense, int64_t n,
+                         uint32_t flags) {
+  KRK_TRY(ensure_runtime());
+  KRK_TRY(check_flags(flags));
+  if (n < 0 || nnz < 0 || (n > 0 && !dense) || (nnz > 0 && (!idx || !val))) return KRK_E_ARGUMENT;
+  if (n == 0) return KRK_SUCCESS;
+  hipStream_t st = nullptr;   // owns no object: runs on the null stream
+  const bool host = !(flags & KRK_DEVICE_PTRS);
+  float* d_dense = dense;
+  const long long* d_idx = reinterpret_cast<const long long*>(idx);
+  const float* d_val = val;
+  char* tmp = nullptr;
+  if (host) {
+    const size_t nb = ((size_t)n * 4 + 255) & ~(size_t)255;
+    const size_t ib = ((size_t)nnz * 8 + 255) & ~(size_t)255;
+    KRK_HIP(hipMalloc((void**)&tmp, nb + ib + (size_t)nnz * 4 + 256));
+    d_dense = reinterpret_cast<float*>(tmp);
+    long long* si = reinterpret_cast<long long*>(tmp + nb);
+    float* sv = reinterpret_cast<float*>(tmp + nb + ib);
+    if (nnz) {
+      hipError_t e = hipMemcpy(si, idx, (size_t)nnz * 8, hipMemcpyHostToDevice);
+      if (e == hipSuccess) e = hipMemcpy(sv, val, (size_t)nnz * 4, hipMemcpyHostToDevice);
+      if (e != hipSuccess) {
+        (void)hipFree(tmp);
+        return hip_fail(e, "krk_coo_to_dense staging", __FILE__, __LINE__);
+      }
+    }
+    d_idx = si;
+    d_val = sv;
+  }
+  hipError_t e = hipMemsetAsync(d_dense, 0, (size_t)n * sizeof(float), st);   // t/math.cc:1066 dense.Zero()
+  if (e == hipSuccess && nnz) {
+    hipLaunchKernelGGL(coo_add_kernel, dim3((unsigned)((nnz + kCodecBlock - 1) / kCodecBlock)),
+                       dim3(kCodecBlock), 0, st, d_idx, d_val, nnz, d_dense, n);
+    e = hipGetLastError();
+  }
+  if (e == hipSuccess && host) e = hipMemcpy(dense, d_dense, (size_t)n * sizeof(float), hipMemcpyDeviceToHost);
+  if (e == hipSuccess && !(flags & KRK_ASYNC)) e = hipStreamSynchronize(st);
+  if (tmp) (void)hipFree(tmp);
+  if (e != hipSuccess) return hip_fail(e, "krk_coo_to_dense", __FILE__, __LINE__);
+  return KRK_SUCCESS;
+}
+
+}  // extern "C"

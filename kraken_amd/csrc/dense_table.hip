@@ -1,0 +1,276 @@
+// Dense table: one parameter vector in HBM with its optimizer state, updated by a single fused
+// pass per push. Replaces DenseTable::Pull / ::Push (ps/dense_table.cc:31-43), the whole-tensor
+// Optim::Update chains (ps/optim/*.cc) and COO densification (t/coo_tensor_impl.cc:250-260,
+// t/math.cc:1006-1046).
+#include <cmath>
+#include <new>
+
+#include "krk_internal.h"
+
+struct krk_dense : krk::ObjBase {
+  int64_t n = 0;
+  float* w = nullptr;
+  float* state[KRK_ST_COUNT] = {};   // created on first use, zero filled
+  float* coo_grad = nullptr;         // densified COO gradient
+  int64_t steps = 0;                 // Adam's kSteps (one counter for the whole tensor)
+  bool sgd_started = false;          // momentum buffer exists (first update copies the gradient)
+};
+
+namespace krk {
+
+constexpr int kDenseBlock = 256;
+
+template <int OPT>
+__global__ __launch_bounds__(kDenseBlock) void dense_update_kernel(
+    float* __restrict__ w, float* __restrict__ s0, float* __restrict__ s1, float* __restrict__ s2,
+    const float* __restrict__ grad, int64_t n, float lr, OptimK k, bool first, float bc1, float bc2) {
+  const int64_t n4 = n >> 2;
+  const int64_t stride = (int64_t)gridDim.x * kDenseBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kDenseBlock + threadIdx.x; i < n4; i += stride) {
+    float4 g = reinterpret_cast<const float4*>(grad)[i];
+    float4 ww = reinterpret_cast<float4*>(w)[i];
+    float4 a = s0 ? reinterpret_cast<float4*>(s0)[i] : make_float4(0, 0, 0, 0);
+    float4 b = s1 ? reinterpret_cast<float4*>(s1)[i] : make_float4(0, 0, 0, 0);
+    float4 c = s2 ? reinterpret_cast<float4*>(s2)[i] : make_float4(0, 0, 0, 0);
+    optim_element<OPT>(k, lr, g.x, ww.x, a.x, b.x, c.x, first, bc1, bc2);
+    optim_element<OPT>(k, lr, g.y, ww.y, a.y, b.y, c.y, first, bc1, bc2);
+    optim_element<OPT>(k, lr, g.z, ww.z, a.z, b.z, c.z, first, bc1, bc2);
+    optim_element<OPT>(k, lr, g.w, ww.w, a.w, b.w, c.w, first, bc1, bc2);
+    reinterpret_cast<float4*>(w)[i] = ww;
+    if (s0) reinterpret_cast<float4*>(s0)[i] = a;
+    if (s1) reinterpret_cast<float4*>(s1)[i] = b;
+    if (s2) reinterpret_cast<float4*>(s2)[i] = c;
+  }
+  // tail (n not a multiple of 4)
+  for (int64_t i = (n4 << 2) + (int64_t)blockIdx.x * kDenseBlock + threadIdx.x; i < n; i += stride) {
+    float g = grad[i], ww = w[i];
+    float a = s0 ? s0[i] : 0.0f, b = s1 ? s1[i] : 0.0f, c = s2 ? s2[i] : 0.0f;
+    optim_element<OPT>(k, lr, g, ww, a, b, c, first, bc1, bc2);
+    w[i] = ww;
+    if (s0) s0[i] = a;
+    if (s1) s1[i] = b;
+    if (s2) s2[i] = c;
+  }
+}
+
+// dense[idx[j]] += val[j]; repeated indices add up (t/math.cc:1043).
+__global__ __launch_bounds__(kDenseBlock) void coo_scatter_kernel(const long long* __restrict__ idx,
+                                                                   const float* __restrict__ val,
+                                                                   int64_t nnz, float* __restrict__ dense,
+                                                                   int64_t n, uint32_t* __restrict__ err) {
+  const int64_t j = (int64_t)blockIdx.x * kDenseBlock + threadIdx.x;
+  if (j >= nnz) return;
+  const long long i = idx[j];
+  if (i < 0 || i >= n) {
+    atomicOr(err, 1u);
+    return;
+  }
+  atomicAdd(&dense[i], val[j]);
+}
+
+static unsigned dense_grid(int64_t n) {
+  int64_t blocks = (n / 4 + kDenseBlock - 1) / kDenseBlock;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 256 * 16) blocks = 256 * 16;   // 16 workgroups per CU, grid-stride beyond that
+  return (unsigned)blocks;
+}
+
+static int32_t ensure_state(krk_dense* t, int st) {
+  if (t->state[st]) return KRK_SUCCESS;
+  KRK_HIP(hipMalloc((void**)&t->state[st], (size_t)t->n * sizeof(float)));
+  KRK_HIP(hipMemsetAsync(t->state[st], 0, (size_t)t->n * sizeof(float), t->stream));
+  return KRK_SUCCESS;
+}
+
+// One Optim::Update on the whole tensor with a device-resident gradient.
+static int32_t dense_apply(krk_dense* t, const krk_optim& o, const float* d_grad, float lr) {
+  const uint32_t mask = optim_state_mask(o);
+  for (int st = 1; st < KRK_ST_COUNT; ++st)
+    if (mask & (1u << st)) KRK_TRY(ensure_state(t, st));
+  const OptimK k = make_optim_k(o);
+  const dim3 grid(dense_grid(t->n)), block(kDenseBlock);
+  float *s0 = nullptr, *s1 = nullptr, *s2 = nullptr;
+  bool first = false;
+  float bc1 = 1.0f, bc2 = 1.0f;
+  switch (o.type) {
+    case KRK_SGD:
+      if (o.has_momentum) {
+        s0 = t->state[KRK_ST_MOMENTUM_BUFFER];
+        first = !t->sgd_started;
+        t->sgd_started = true;
+      }
+      hipLaunchKernelGGL((dense_update_kernel<KRK_SGD>), grid, block, 0, t->stream, t->w, s0, s1, s2,
+                         d_grad, t->n, lr, k, first, bc1, bc2);
+      break;
+    case KRK_ADAGRAD:
+      s0 = t->state[KRK_ST_STATE_SUM];
+      hipLaunchKernelGGL((dense_update_kernel<KRK_ADAGRAD>), grid, block, 0, t->stream, t->w, s0, s1,
+                         s2, d_grad, t->n, lr, k, first, bc1, bc2);
+      break;
+    case KRK_ADAM: {
+      s0 = t->state[KRK_ST_FIRST_MOMENT];
+      s1 = t->state[KRK_ST_SECOND_MOMENT];
+      if (o.amsgrad) s2 = t->state[KRK_ST_SECOND_MOMENT_MAX];
+      const int64_t steps = ++t->steps;   // ps/optim/adam.cc:61
+      bc1 = (float)(1.0 - (double)std::pow(o.beta1, (float)steps));   // :63-64, float pow
+      bc2 = (float)(1.0 - (double)std::pow(o.beta2, (float)steps));
+      hipLaunchKernelGGL((dense_update_kernel<KRK_ADAM>), grid, block, 0, t->stream, t->w, s0, s1, s2,
+                         d_grad, t->n, lr, k, first, bc1, bc2);
+      break;
+    }
+    default:
+      s0 = t->state[KRK_ST_SQUARE_AVERAGE];
+      if (o.centered) s1 = t->state[KRK_ST_G_AVE];
+      if (o.has_momentum) s2 = t->state[KRK_ST_MOMENTUM_BUFFER];
+      hipLaunchKernelGGL((dense_update_kernel<KRK_RMSPROP>), grid, block, 0, t->stream, t->w, s0, s1,
+                         s2, d_grad, t->n, lr, k, first, bc1, bc2);
+      break;
+  }
+  KRK_HIP(hipGetLastError());
+  return KRK_SUCCESS;
+}
+
+static int32_t dense_finish(krk_dense* t, uint32_t flags) {
+  if (flags & KRK_ASYNC) return KRK_SUCCESS;
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  return KRK_SUCCESS;
+}
+
+}  // namespace krk
+
+using namespace krk;
+
+static int32_t check_dense(krk_dense* t) {
+  if (!t) {
+    set_error("null dense table handle");
+    return KRK_E_ARGUMENT;
+  }
+  return ensure_runtime();
+}
+
+extern "C" {
+
+int32_t krk_dense_create(const float* val, int64_t n, uint32_t flags, krk_dense** out) {
+  if (!out || n < 0 || (n > 0 && !val)) return KRK_E_ARGUMENT;
+  KRK_TRY(check_flags(flags & ~KRK_ASYNC));
+  KRK_TRY(ensure_runtime());
+  krk_dense* t = new (std::nothrow) krk_dense();
+  if (!t) return KRK_E_DEVICE;
+  t->n = n;
+  int32_t rc = t->open_stream();
+  if (rc == KRK_SUCCESS) {
+    hipError_t e = hipMalloc((void**)&t->w, (size_t)(n ? n : 1) * sizeof(float));
+    if (e == hipSuccess && n)
+      e = hipMemcpyAsync(t->w, val, (size_t)n * sizeof(float),
+                         (flags & KRK_DEVICE_PTRS) ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
+                         t->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(t->stream);
+    if (e != hipSuccess) rc = hip_fail(e, "krk_dense_create", __FILE__, __LINE__);
+  }
+  if (rc != KRK_SUCCESS) {
+    krk_dense_destroy(t);
+    return rc;
+  }
+  *out = t;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dense_destroy(krk_dense* t) {
+  if (!t) return KRK_SUCCESS;
+  if (t->stream) (void)hipStreamSynchronize(t->stream);
+  if (t->w) (void)hipFree(t->w);
+  if (t->coo_grad) (void)hipFree(t->coo_grad);
+  for (auto& s : t->state)
+    if (s) (void)hipFree(s);
+  t->close_stream();
+  delete t;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dense_sync(krk_dense* t) {
+  KRK_TRY(check_dense(t));
+  std::lock_guard<std::mutex> lk(t->mu);
+  return dense_finish(t, 0);
+}
+
+int32_t krk_dense_pull(krk_dense* t, float* out, uint32_t flags) {
+  KRK_TRY(check_dense(t));
+  KRK_TRY(check_flags(flags));
+  if (t->n > 0 && !out) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (t->n)
+    KRK_HIP(hipMemcpyAsync(out, t->w, (size_t)t->n * sizeof(float),
+                           (flags & KRK_DEVICE_PTRS) ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost,
+                           t->stream));
+  return dense_finish(t, flags);
+}
+
+int32_t krk_dense_push(krk_dense* t, const krk_optim* o, const float* grad, int64_t n, float lr,
+                       uint32_t flags) {
+  KRK_TRY(check_dense(t));
+  KRK_TRY(check_flags(flags));
+  if (!o || o->type < KRK_ADAGRAD || o->type > KRK_SGD) return KRK_UNSUPPORTED_OPTIM;
+  if (n < 0 || (n > 0 && !grad)) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (n != t->n) {   // ps/optim/sgd.cc:36-39
+    set_error("gradient has %lld elements, table has %lld", (long long)n, (long long)t->n);
+    return KRK_GRADIENT_UNCOMPATIBLE;
+  }
+  if (n == 0) return KRK_SUCCESS;
+  const float* d_grad;
+  KRK_TRY(t->input(grad, (size_t)n, flags, 0, &d_grad));
+  KRK_TRY(dense_apply(t, *o, d_grad, lr));
+  return dense_finish(t, flags);
+}
+
+int32_t krk_dense_push_coo(krk_dense* t, const krk_optim* o, const int64_t* idx, const float* val,
+                           int64_t nnz, float lr, uint32_t flags) {
+  KRK_TRY(check_dense(t));
+  KRK_TRY(check_flags(flags));
+  if (!o || o->type < KRK_ADAGRAD || o->type > KRK_SGD) return KRK_UNSUPPORTED_OPTIM;
+  if (nnz < 0 || (nnz > 0 && (!idx || !val))) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (nnz == 0) return KRK_SUCCESS;   // ps/optim/adam.cc:26-29 : nothing is touched, not even kSteps
+  if (t->n == 0) return KRK_GRADIENT_UNCOMPATIBLE;
+  if (!t->coo_grad) KRK_HIP(hipMalloc((void**)&t->coo_grad, (size_t)t->n * sizeof(float) + 16));
+  const int64_t* d_idx;
+  const float* d_val;
+  KRK_TRY(t->input(idx, (size_t)nnz, flags, 0, &d_idx));
+  KRK_TRY(t->input(val, (size_t)nnz, flags, 1, &d_val));
+  uint32_t* err = reinterpret_cast<uint32_t*>(t->coo_grad + t->n);
+  KRK_HIP(hipMemsetAsync(t->coo_grad, 0, (size_t)t->n * sizeof(float) + 16, t->stream));
+  hipLaunchKernelGGL(coo_scatter_kernel, dim3((unsigned)((nnz + kDenseBlock - 1) / kDenseBlock)),
+                     dim3(kDenseBlock), 0, t->stream, reinterpret_cast<const long long*>(d_idx), d_val,
+                     nnz, t->coo_grad, t->n, err);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(dense_apply(t, *o, t->coo_grad, lr));
+  return dense_finish(t, flags);
+}
+
+int32_t krk_dense_state(krk_dense* t, int32_t state_type, float* out, uint32_t flags) {
+  KRK_TRY(check_dense(t));
+  KRK_TRY(check_flags(flags));
+  if (state_type < 1 || state_type >= KRK_ST_COUNT || (t->n > 0 && !out)) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (t->n == 0) return KRK_SUCCESS;
+  const size_t bytes = (size_t)t->n * sizeof(float);
+  if (t->state[state_type]) {
+    KRK_HIP(hipMemcpyAsync(out, t->state[state_type], bytes,
+                           (flags & KRK_DEVICE_PTRS) ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost,
+                           t->stream));
+  } else if (flags & KRK_DEVICE_PTRS) {
+    KRK_HIP(hipMemsetAsync(out, 0, bytes, t->stream));
+  } else {
+    memset(out, 0, bytes);
+  }
+  return dense_finish(t, flags);
+}
+
+int32_t krk_dense_steps(krk_dense* t, int64_t* steps) {
+  if (!t || !steps) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  *steps = t->steps;
+  return KRK_SUCCESS;
+}
+
+}  // extern "C"

@@ -1,0 +1,464 @@
+// Runtime plumbing of the table engine: error strings, device selection, harness
+// memory helpers, conf parsing, events and the device-wide scan primitive.
+#include <cmath>
+#include <cstdlib>
+#include <string>
+
+#include "krk_internal.h"
+
+namespace krk {
+
+static thread_local char g_err[512] = "";
+static int g_device = 0;
+static bool g_ready = false;
+static std::mutex g_mu;
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int32_t hip_fail(hipError_t e, const char* what, const char* file, int line) {
+  set_error("HIP error %d (%s) at %s:%d: %s", (int)e, hipGetErrorString(e), file, line, what);
+  return KRK_E_DEVICE;
+}
+
+int current_device() { return g_device; }
+
+static int32_t init_device(int device) {
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= 0) {
+    set_error("no HIP device is visible (hipGetDeviceCount: %s); the table engine has no CPU path",
+              hipGetErrorString(e));
+    return KRK_E_DEVICE;
+  }
+  if (device < 0 || device >= count) {
+    set_error("device %d out of range (%d visible)", device, count);
+    return KRK_E_ARGUMENT;
+  }
+  hipDeviceProp_t prop;
+  KRK_HIP(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    set_error("device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+    return KRK_E_DEVICE;
+  }
+  KRK_HIP(hipSetDevice(device));
+  g_device = device;
+  g_ready = true;
+  return KRK_SUCCESS;
+}
+
+int32_t ensure_runtime() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (!g_ready) KRK_TRY(init_device(g_device));
+  // Worker threads of a server each need the device bound once.
+  KRK_HIP(hipSetDevice(g_device));
+  return KRK_SUCCESS;
+}
+
+int32_t DeviceBuffer::reserve(size_t want) {
+  if (want <= bytes) return KRK_SUCCESS;
+  size_t grow = bytes + bytes / 2;
+  if (want < grow) want = grow;
+  want = (want + 255) & ~(size_t)255;
+  if (ptr) KRK_HIP(hipFree(ptr));
+  ptr = nullptr;
+  bytes = 0;
+  KRK_HIP(hipMalloc(&ptr, want));
+  bytes = want;
+  return KRK_SUCCESS;
+}
+
+void DeviceBuffer::release() {
+  if (ptr) (void)hipFree(ptr);
+  ptr = nullptr;
+  bytes = 0;
+}
+
+OptimK make_optim_k(const krk_optim& o) {
+  OptimK k;
+  k.type = o.type;
+  k.has_wd = o.has_weight_decay;
+  k.has_momentum = o.has_momentum;
+  k.nesterov = o.nesterov;
+  k.amsgrad = o.amsgrad;
+  k.centered = o.centered;
+  k.wd = o.weight_decay;
+  k.momentum = o.momentum;
+  k.one_minus_damp = (float)(1.0 - (double)o.dampening);
+  k.beta1 = o.beta1;
+  k.beta2 = o.beta2;
+  k.one_minus_b1 = (float)(1.0 - (double)o.beta1);
+  k.one_minus_b2 = (float)(1.0 - (double)o.beta2);
+  k.eps = o.eps;
+  k.alpha = o.alpha;
+  k.one_minus_alpha = (float)(1.0 - (double)o.alpha);
+  k.acc0 = o.initial_accumulator;
+  return k;
+}
+
+uint32_t optim_state_mask(const krk_optim& o) {
+  uint32_t m = 0;
+  switch (o.type) {
+    case KRK_SGD:
+      if (o.has_momentum) m |= (1u << KRK_ST_MOMENTUM_BUFFER) | (1u << KRK_ST_STEPS);
+      break;
+    case KRK_ADAGRAD:
+      m |= 1u << KRK_ST_STATE_SUM;
+      break;
+    case KRK_ADAM:
+      m |= (1u << KRK_ST_FIRST_MOMENT) | (1u << KRK_ST_SECOND_MOMENT) | (1u << KRK_ST_STEPS);
+      if (o.amsgrad) m |= 1u << KRK_ST_SECOND_MOMENT_MAX;
+      break;
+    case KRK_RMSPROP:
+      m |= 1u << KRK_ST_SQUARE_AVERAGE;
+      if (o.centered) m |= 1u << KRK_ST_G_AVE;
+      if (o.has_momentum) m |= 1u << KRK_ST_MOMENTUM_BUFFER;
+      break;
+    default:
+      break;
+  }
+  return m;
+}
+
+// ---------------------------------------------------------------------------
+// exclusive scan: block sums -> one-block scan of the sums -> per-block scan + offset
+// ---------------------------------------------------------------------------
+constexpr int kScanThreads = 256;
+constexpr int kScanItems = 8;
+constexpr int kScanTile = kScanThreads * kScanItems;
+
+__device__ inline int block_exclusive_scan(int v, int* lds, int& block_total) {
+  // wave-level inclusive scan, then combine the four wave totals through LDS
+  int lane = threadIdx.x & 63;
+  int wave = threadIdx.x >> 6;
+  int x = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    int y = __shfl_up(x, d, 64);
+    if (lane >= d) x += y;
+  }
+  if (lane == 63) lds[wave] = x;
+  __syncthreads();
+  int base = 0;
+  int tot = 0;
+#pragma unroll
+  for (int w = 0; w < kScanThreads / 64; ++w) {
+    int t = lds[w];
+    if (w < wave) base += t;
+    tot += t;
+  }
+  __syncthreads();
+  block_total = tot;
+  return base + x - v;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_block_sums(const int32_t* __restrict__ in,
+                                                                int64_t n,
+                                                                int32_t* __restrict__ sums) {
+  __shared__ int lds[kScanThreads / 64];
+  int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    int64_t j = base + i;
+    if (j < n) s += in[j];
+  }
+  int tot;
+  block_exclusive_scan(s, lds, tot);
+  if (threadIdx.x == 0) sums[blockIdx.x] = tot;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_of_sums(int32_t* __restrict__ sums, int64_t m,
+                                                             int32_t* __restrict__ total_out) {
+  __shared__ int lds[kScanThreads / 64];
+  int carry = 0;
+  for (int64_t start = 0; start < m; start += kScanThreads) {
+    int64_t j = start + threadIdx.x;
+    int v = j < m ? sums[j] : 0;
+    int tot;
+    int ex = block_exclusive_scan(v, lds, tot);
+    if (j < m) sums[j] = carry + ex;
+    carry += tot;
+  }
+  if (threadIdx.x == 0 && total_out) *total_out = carry;
+}
+
+__global__ __launch_bounds__(kScanThreads) void scan_apply(const int32_t* __restrict__ in,
+                                                           int32_t* __restrict__ out, int64_t n,
+                                                           const int32_t* __restrict__ sums) {
+  __shared__ int lds[kScanThreads / 64];
+  int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  int v[kScanItems];
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    int64_t j = base + i;
+    v[i] = j < n ? in[j] : 0;
+    s += v[i];
+  }
+  int tot;
+  int ex = block_exclusive_scan(s, lds, tot) + sums[blockIdx.x];
+#pragma unroll
+  for (int i = 0; i < kScanItems; ++i) {
+    int64_t j = base + i;
+    if (j < n) out[j] = ex;
+    ex += v[i];
+  }
+}
+
+size_t scan_scratch_bytes(int64_t n) {
+  int64_t blocks = (n + kScanTile - 1) / kScanTile;
+  if (blocks < 1) blocks = 1;
+  return (size_t)blocks * sizeof(int32_t);
+}
+
+int32_t exclusive_scan_i32(const int32_t* in, int32_t* out, int64_t n, int32_t* total_out,
+                           void* scratch, hipStream_t stream) {
+  int64_t blocks = (n + kScanTile - 1) / kScanTile;
+  if (blocks < 1) blocks = 1;
+  int32_t* sums = reinterpret_cast<int32_t*>(scratch);
+  hipLaunchKernelGGL(scan_block_sums, dim3((unsigned)blocks), dim3(kScanThreads), 0, stream, in, n,
+                     sums);
+  hipLaunchKernelGGL(scan_of_sums, dim3(1), dim3(kScanThreads), 0, stream, sums, blocks, total_out);
+  hipLaunchKernelGGL(scan_apply, dim3((unsigned)blocks), dim3(kScanThreads), 0, stream, in, out, n,
+                     sums);
+  KRK_HIP(hipGetLastError());
+  return KRK_SUCCESS;
+}
+
+}  // namespace krk
+
+// ===========================================================================
+// C ABI: runtime, conf parsing, harness helpers, events
+// ===========================================================================
+using namespace krk;
+
+extern "C" {
+
+int32_t krk_runtime_init(int32_t device) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  return init_device(device);
+}
+
+const char* krk_last_error_string(void) { return g_err; }
+
+// ErrorCode::Msg (common/error_code.h:35-93) for the codes this library returns.
+const char* krk_error_message(int32_t code) {
+  switch (code) {
+    case KRK_SUCCESS: return "Success";
+    case KRK_UNSUPPORTED_OPTIM: return "UnSupport optim type";
+    case KRK_INTERFACE_UNIMPLEMENTED: return "UnImplement Interface";
+    case KRK_GRADIENT_UNCOMPATIBLE: return "Uncompatible gradient";
+    case KRK_SPARSE_ID_NOT_EXIST: return "SparseId not exist";
+    case KRK_UNSUPPORTED_INITIALIZER: return "UnSupport initializer type";
+    case KRK_E_DEVICE: return "GPU runtime failure";
+    case KRK_E_ARGUMENT: return "Invalid argument";
+    case KRK_E_CAPACITY: return "Capacity exceeded";
+    default: return "Unrecognized error";
+  }
+}
+
+// ps/optim/optim.cc:23-101
+int32_t krk_optim_defaults(int32_t type, krk_optim* o) {
+  if (!o) return KRK_E_ARGUMENT;
+  memset(o, 0, sizeof(*o));
+  o->type = type;
+  o->beta1 = 0.9f;
+  o->beta2 = 0.999f;
+  o->alpha = 0.99f;
+  switch (type) {
+    case KRK_ADAGRAD: o->eps = 1e-10f; break;
+    case KRK_ADAM:
+    case KRK_RMSPROP:
+    case KRK_SGD: o->eps = 1e-8f; break;
+    default: return KRK_UNSUPPORTED_OPTIM;
+  }
+  return KRK_SUCCESS;
+}
+
+// common/utils.h:55-70 : std::stof, failure leaves the default and reports "absent".
+static bool parse_float(const char* s, float* v) {
+  try {
+    *v = std::stof(std::string(s));
+  } catch (...) {
+    return false;
+  }
+  return true;
+}
+// common/utils.h:72-90 : "true" or "1" (any case) is true, anything else false.
+static bool parse_bool(const char* s) {
+  std::string lv(s);
+  for (auto& c : lv) c = (char)tolower((unsigned char)c);
+  return lv == "true" || lv == "1";
+}
+
+int32_t krk_optim_set(krk_optim* o, const char* key, const char* value) {
+  if (!o || !key || !value) return KRK_E_ARGUMENT;
+  std::string k(key);
+  float f;
+  const int t = o->type;
+  if (k == "weight_decay") {
+    if (parse_float(value, &f)) { o->weight_decay = f; o->has_weight_decay = 1; }
+  } else if (k == "momentum" && (t == KRK_RMSPROP || t == KRK_SGD)) {
+    if (parse_float(value, &f)) { o->momentum = f; o->has_momentum = 1; }
+  } else if (k == "dampening" && t == KRK_SGD) {
+    if (parse_float(value, &f)) { o->dampening = f; o->has_dampening = 1; }
+  } else if (k == "nesterov" && t == KRK_SGD) {
+    o->nesterov = parse_bool(value);
+  } else if (k == "eps" && t != KRK_SGD) {
+    if (parse_float(value, &f)) o->eps = f;
+  } else if (k == "beta1" && t == KRK_ADAM) {
+    if (parse_float(value, &f)) o->beta1 = f;
+  } else if (k == "beta2" && t == KRK_ADAM) {
+    if (parse_float(value, &f)) o->beta2 = f;
+  } else if (k == "amsgrad" && t == KRK_ADAM) {
+    o->amsgrad = parse_bool(value);
+  } else if (k == "alpha" && t == KRK_RMSPROP) {
+    if (parse_float(value, &f)) o->alpha = f;
+  } else if (k == "centered" && t == KRK_RMSPROP) {
+    o->centered = parse_bool(value);
+  } else if (k == "initial_accumulator" && t == KRK_ADAGRAD) {
+    if (parse_float(value, &f)) o->initial_accumulator = f;
+  }
+  return KRK_SUCCESS;
+}
+
+// ps/initializer/initializer.cc:27-58
+int32_t krk_init_defaults(int32_t type, krk_init* i) {
+  if (!i) return KRK_E_ARGUMENT;
+  memset(i, 0, sizeof(*i));
+  i->type = type;
+  switch (type) {
+    case KRK_INIT_CONSTANT: i->a = 0.0f; break;
+    case KRK_INIT_UNIFORM: i->a = 0.0f; i->b = 1.0f; break;
+    case KRK_INIT_NORMAL: i->a = 0.0f; i->b = 1.0f; break;
+    case KRK_INIT_XAVIER_UNIFORM:
+    case KRK_INIT_XAVIER_NORMAL: i->a = 1.0f; break;
+    default: return KRK_UNSUPPORTED_INITIALIZER;
+  }
+  return KRK_SUCCESS;
+}
+
+int32_t krk_init_set(krk_init* i, const char* key, const char* value) {
+  if (!i || !key || !value) return KRK_E_ARGUMENT;
+  std::string k(key);
+  float f;
+  if (k == "seed") {
+    i->seed = strtoull(value, nullptr, 10);
+    return KRK_SUCCESS;
+  }
+  if (!parse_float(value, &f)) return KRK_SUCCESS;
+  switch (i->type) {
+    case KRK_INIT_CONSTANT: if (k == "value") i->a = f; break;
+    case KRK_INIT_UNIFORM: if (k == "lower") i->a = f; else if (k == "upper") i->b = f; break;
+    case KRK_INIT_NORMAL: if (k == "mean") i->a = f; else if (k == "stddev") i->b = f; break;
+    case KRK_INIT_XAVIER_UNIFORM:
+    case KRK_INIT_XAVIER_NORMAL: if (k == "gain") i->a = f; break;
+    default: break;
+  }
+  return KRK_SUCCESS;
+}
+
+int32_t krk_malloc(void** dptr, size_t bytes) {
+  if (!dptr) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  KRK_HIP(hipMalloc(dptr, bytes ? bytes : 1));
+  return KRK_SUCCESS;
+}
+int32_t krk_free(void* dptr) {
+  if (!dptr) return KRK_SUCCESS;
+  KRK_HIP(hipFree(dptr));
+  return KRK_SUCCESS;
+}
+int32_t krk_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+  KRK_TRY(ensure_runtime());
+  if (bytes) KRK_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+  return KRK_SUCCESS;
+}
+int32_t krk_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+  KRK_TRY(ensure_runtime());
+  if (bytes) KRK_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+  return KRK_SUCCESS;
+}
+int32_t krk_memset(void* dptr, int value, size_t bytes) {
+  KRK_TRY(ensure_runtime());
+  if (bytes) KRK_HIP(hipMemset(dptr, value, bytes));
+  return KRK_SUCCESS;
+}
+int32_t krk_device_synchronize(void) {
+  KRK_TRY(ensure_runtime());
+  KRK_HIP(hipDeviceSynchronize());
+  return KRK_SUCCESS;
+}
+int32_t krk_mem_info(size_t* free_bytes, size_t* total_bytes) {
+  KRK_TRY(ensure_runtime());
+  size_t f = 0, t = 0;
+  KRK_HIP(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = f;
+  if (total_bytes) *total_bytes = t;
+  return KRK_SUCCESS;
+}
+
+}  // extern "C"
+
+namespace krk {
+int32_t ObjBase::open_stream() {
+  KRK_TRY(ensure_runtime());
+  KRK_HIP(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+  return KRK_SUCCESS;
+}
+void ObjBase::close_stream() {
+  if (stream) {
+    (void)hipStreamSynchronize(stream);
+    (void)hipStreamDestroy(stream);
+    stream = nullptr;
+  }
+  for (auto& b : stage) b.release();
+}
+}  // namespace krk
+
+struct krk_event {
+  hipEvent_t ev;
+};
+
+extern "C" {
+
+int32_t krk_event_create(krk_event** e) {
+  if (!e) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  krk_event* x = new (std::nothrow) krk_event();
+  if (!x) return KRK_E_DEVICE;
+  hipError_t rc = hipEventCreate(&x->ev);
+  if (rc != hipSuccess) {
+    delete x;
+    return hip_fail(rc, "hipEventCreate", __FILE__, __LINE__);
+  }
+  *e = x;
+  return KRK_SUCCESS;
+}
+int32_t krk_event_destroy(krk_event* e) {
+  if (!e) return KRK_SUCCESS;
+  (void)hipEventDestroy(e->ev);
+  delete e;
+  return KRK_SUCCESS;
+}
+// Every API object begins with an ObjBase, so its stream is reachable from any handle.
+int32_t krk_event_record(krk_event* e, krk_sparse* sparse, krk_dense* dense, krk_dct* dct) {
+  void* h = sparse ? (void*)sparse : dense ? (void*)dense : (void*)dct;
+  if (!e || !h) return KRK_E_ARGUMENT;
+  ObjBase* b = reinterpret_cast<ObjBase*>(h);
+  KRK_HIP(hipEventRecord(e->ev, b->stream));
+  return KRK_SUCCESS;
+}
+int32_t krk_event_elapsed_ms(krk_event* start, krk_event* stop, float* ms) {
+  if (!start || !stop || !ms) return KRK_E_ARGUMENT;
+  KRK_HIP(hipEventSynchronize(stop->ev));
+  KRK_HIP(hipEventElapsedTime(ms, start->ev, stop->ev));
+  return KRK_SUCCESS;
+}
+
+}  // extern "C"

@@ -1,0 +1,778 @@
+// Sparse table: id -> row lookup in an HBM-resident open-addressing index, pull (gather with
+// insert-on-miss) and push (one fused read-modify-write of weight + optimizer state per row).
+//
+// Replaces SparseTable::Pull / ::Push (ps/sparse_table.cc:33-108), the per-row Optim::Update
+// chains (ps/optim/*.cc) and the row initialisers (ps/initializer/*.cc, t/math.cc:333-517).
+//
+// Work mapping: `group` adjacent lanes of a 64-wide wavefront own one id. The group's first
+// lane walks the index (one 16-byte slot load per probe), the row number is broadcast with a
+// wave shuffle, then every lane moves `vec` floats of the record per step, so a dim-16 row is
+// four float4 lanes and sixteen rows share one wavefront instruction.
+#include <cmath>
+#include <new>
+
+#include "sparse_internal.h"
+
+namespace krk {
+
+constexpr int kBlock = 256;
+
+template <int VEC>
+struct VecT;
+template <>
+struct VecT<4> {
+  using type = float4;
+};
+template <>
+struct VecT<1> {
+  using type = float;
+};
+
+template <int VEC>
+__device__ __forceinline__ void vload(const float* p, float (&v)[VEC]) {
+  if constexpr (VEC == 4) {
+    const float4 x = *reinterpret_cast<const float4*>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  } else {
+    v[0] = *p;
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void vstore(float* p, const float (&v)[VEC]) {
+  if constexpr (VEC == 4) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+    *p = v[0];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// pull: gather rows, inserting and initialising the ones that are missing
+// ---------------------------------------------------------------------------
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                      int64_t n, float* __restrict__ out, int dim,
+                                                      int elems, int group, uint32_t base_rows,
+                                                      const uint32_t* __restrict__ base_rows_dev,
+                                                      InitK init) {
+  if (base_rows_dev) base_rows = *base_rows_dev;
+  const int per_block = kBlock / group;
+  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  const int gl = threadIdx.x & (group - 1);
+  const bool active = i < n;
+  const uint64_t id = active ? ids[i] : 0;
+  uint32_t row = kEmptyRow;
+  int owner = 0;
+  if (active && gl == 0) {
+    bool own;
+    row = probe_insert(tv, id, &own);
+    owner = own ? 1 : 0;
+  }
+  row = __shfl(row, 0, group);
+  owner = __shfl(owner, 0, group);
+  if (!active) return;
+  // Rows numbered at or past base_rows were created by this launch: their record may not be
+  // written yet, and their value is a pure function of (seed, id), so it is recomputed.
+  const bool fresh = row == kEmptyRow || row >= base_rows;
+  float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
+  float* dst = out + i * (int64_t)dim;
+  for (int e = gl; e < elems; e += group) {
+    float v[VEC];
+    if (fresh) {
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) v[c] = init_element(init, id, (int64_t)e * VEC + c);
+      if (owner) vstore<VEC>(rec + e * VEC, v);
+    } else {
+      vload<VEC>(rec + e * VEC, v);
+    }
+    vstore<VEC>(dst + e * VEC, v);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// push: per unique id, one fused update of the record
+// ---------------------------------------------------------------------------
+template <int OPT, int VEC>
+__global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                      int64_t n, const float* __restrict__ grads,
+                                                      int dim, int elems, int group, float lr,
+                                                      OptimK k, int c0, int c1off, int c2off,
+                                                      int meta_off) {
+  const int per_block = kBlock / group;
+  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  const int gl = threadIdx.x & (group - 1);
+  const bool active = i < n;
+  uint32_t row = kEmptyRow;
+  if (active && gl == 0) {
+    row = probe_find(tv, ids[i]);
+    if (row == kEmptyRow) atomicOr(&tv.counters[1], kErrMissingId);
+  }
+  row = __shfl(row, 0, group);
+  if (!active || row == kEmptyRow) return;
+  float* rec = tv.recs + (int64_t)row * tv.stride;
+  const float* g = grads + i * (int64_t)dim;
+
+  bool first = false;
+  float bc1 = 1.0f, bc2 = 1.0f;
+  uint64_t steps = 0;
+  if (meta_off >= 0) {
+    const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + meta_off);
+    steps = (uint64_t)meta[0] | ((uint64_t)meta[1] << 32);
+    first = steps == 0;
+    steps += 1;
+    if (OPT == KRK_ADAM) {
+      // ps/optim/adam.cc:61-64 : per-row step counter, float pow, double subtraction
+      bc1 = (float)(1.0 - (double)powf(k.beta1, (float)steps));
+      bc2 = (float)(1.0 - (double)powf(k.beta2, (float)steps));
+    }
+  }
+  for (int e = gl; e < elems; e += group) {
+    float gv[VEC], w[VEC], s0[VEC], s1[VEC], s2[VEC];
+    vload<VEC>(g + e * VEC, gv);
+    vload<VEC>(rec + e * VEC, w);
+    if (c0 >= 0) vload<VEC>(rec + c0 + e * VEC, s0);
+    if (c1off >= 0) vload<VEC>(rec + c1off + e * VEC, s1);
+    if (c2off >= 0) vload<VEC>(rec + c2off + e * VEC, s2);
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) {
+      if (c0 < 0) s0[c] = 0.0f;
+      if (c1off < 0) s1[c] = 0.0f;
+      if (c2off < 0) s2[c] = 0.0f;
+      optim_element<OPT>(k, lr, gv[c], w[c], s0[c], s1[c], s2[c], first, bc1, bc2);
+    }
+    vstore<VEC>(rec + e * VEC, w);
+    if (c0 >= 0) vstore<VEC>(rec + c0 + e * VEC, s0);
+    if (c1off >= 0) vstore<VEC>(rec + c1off + e * VEC, s1);
+    if (c2off >= 0) vstore<VEC>(rec + c2off + e * VEC, s2);
+  }
+  if (meta_off >= 0 && gl == 0) {
+    uint32_t* meta = reinterpret_cast<uint32_t*>(rec + meta_off);
+    meta[0] = (uint32_t)steps;
+    meta[1] = (uint32_t)(steps >> 32);
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void lookup_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                        int64_t n, int32_t* __restrict__ rows) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  const uint32_t r = probe_find(tv, ids[i]);
+  rows[i] = r == kEmptyRow ? -1 : (int32_t)r;
+}
+
+// counters[2] = counters[0]: the row count a following pull starts from, taken in stream order
+__global__ void snapshot_rows_kernel(uint32_t* counters) { counters[2] = counters[0]; }
+
+// import: like pull, but a new row takes its values from the caller
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void import_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                        int64_t n, const float* __restrict__ vals,
+                                                        int dim, int elems, int group) {
+  const int per_block = kBlock / group;
+  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  const int gl = threadIdx.x & (group - 1);
+  const bool active = i < n;
+  uint32_t row = kEmptyRow;
+  int owner = 0;
+  if (active && gl == 0) {
+    bool own;
+    row = probe_insert(tv, ids[i], &own);
+    owner = own ? 1 : 0;
+  }
+  row = __shfl(row, 0, group);
+  owner = __shfl(owner, 0, group);
+  if (!active || !owner) return;
+  float* rec = tv.recs + (int64_t)row * tv.stride;
+  const float* src = vals + i * (int64_t)dim;
+  for (int e = gl; e < elems; e += group) {
+    float v[VEC];
+    vload<VEC>(src + e * VEC, v);
+    vstore<VEC>(rec + e * VEC, v);
+  }
+}
+
+// export: rows in insertion order
+__global__ __launch_bounds__(kBlock) void export_kernel(TableView tv, int64_t rows, int dim,
+                                                        unsigned long long* __restrict__ ids,
+                                                        float* __restrict__ vals, int state_off,
+                                                        float* __restrict__ state, int meta_off,
+                                                        long long* __restrict__ steps) {
+  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t r = t / dim;
+  const int j = (int)(t - r * dim);
+  if (r >= rows) return;
+  const float* rec = tv.recs + r * tv.stride;
+  if (vals) vals[t] = rec[j];
+  if (state) state[t] = state_off >= 0 ? rec[state_off + j] : 0.0f;
+  if (j == 0) {
+    if (ids) ids[r] = tv.row_key[r];
+    if (steps) {
+      long long s = 0;
+      if (meta_off >= 0) {
+        const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + meta_off);
+        s = (long long)((uint64_t)meta[0] | ((uint64_t)meta[1] << 32));
+      }
+      steps[r] = s;
+    }
+  }
+}
+
+// re-index every existing row into a fresh (larger) slot array
+__global__ __launch_bounds__(kBlock) void reindex_kernel(Slot* slots, uint64_t mask,
+                                                         const unsigned long long* __restrict__ row_key,
+                                                         int64_t rows) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r >= rows) return;
+  const unsigned long long id = row_key[r];
+  if (id == kEmptyKey) {
+    slots[mask + 1].key = 0ull;
+    slots[mask + 1].row = (uint32_t)r;
+    return;
+  }
+  uint64_t idx = mix64(id) & mask;
+  for (uint64_t n = 0; n <= mask; ++n) {
+    unsigned long long old = atomicCAS(&slots[idx].key, kEmptyKey, id);
+    if (old == kEmptyKey) {
+      slots[idx].row = (uint32_t)r;
+      return;
+    }
+    idx = (idx + 1) & mask;
+  }
+}
+
+// copy records into a slab with a wider stride (new state columns stay zero)
+__global__ __launch_bounds__(kBlock) void restride_kernel(const float* __restrict__ src,
+                                                          int64_t src_stride, float* __restrict__ dst,
+                                                          int64_t dst_stride, int64_t rows,
+                                                          int copy_floats) {
+  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t r = t / copy_floats;
+  const int j = (int)(t - r * copy_floats);
+  if (r >= rows) return;
+  dst[r * dst_stride + j] = src[r * src_stride + j];
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+static inline unsigned grid_for(int64_t items, int per_block) {
+  return (unsigned)((items + per_block - 1) / per_block);
+}
+
+static int32_t alloc_slots(uint64_t cap, Slot** out, hipStream_t s) {
+  Slot* p = nullptr;
+  KRK_HIP(hipMalloc((void**)&p, (cap + 1) * sizeof(Slot)));
+  hipError_t e = hipMemsetAsync(p, 0xFF, (cap + 1) * sizeof(Slot), s);
+  if (e != hipSuccess) {
+    (void)hipFree(p);
+    return hip_fail(e, "hipMemsetAsync(slots)", __FILE__, __LINE__);
+  }
+  *out = p;
+  return KRK_SUCCESS;
+}
+
+static int32_t grow_rows(krk_sparse* t, int64_t new_cap, int64_t new_stride) {
+  // rows in use must be known exactly before records are moved
+  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  const int64_t rows = t->host_counters[0];
+  t->size_ub = rows;
+  if (new_cap < rows) new_cap = rows;
+  if (new_cap >= (int64_t)kEmptyRow) {
+    set_error("sparse table cannot hold more than 2^32-2 rows");
+    return KRK_E_CAPACITY;
+  }
+  float* nrecs = nullptr;
+  unsigned long long* nkeys = nullptr;
+  const size_t rec_bytes = (size_t)new_cap * (size_t)new_stride * sizeof(float);
+  KRK_HIP(hipMalloc((void**)&nrecs, rec_bytes ? rec_bytes : 16));
+  hipError_t e = hipMalloc((void**)&nkeys, (size_t)(new_cap ? new_cap : 1) * sizeof(unsigned long long));
+  if (e != hipSuccess) {
+    (void)hipFree(nrecs);
+    return hip_fail(e, "hipMalloc(row_key)", __FILE__, __LINE__);
+  }
+  if (new_stride == t->stride) {
+    const size_t used = (size_t)rows * (size_t)t->stride * sizeof(float);
+    if (used) KRK_HIP(hipMemcpyAsync(nrecs, t->recs, used, hipMemcpyDeviceToDevice, t->stream));
+    if (rec_bytes > used)
+      KRK_HIP(hipMemsetAsync(reinterpret_cast<char*>(nrecs) + used, 0, rec_bytes - used, t->stream));
+  } else {
+    KRK_HIP(hipMemsetAsync(nrecs, 0, rec_bytes, t->stream));
+    if (rows) {
+      const int64_t items = rows * t->stride;
+      hipLaunchKernelGGL(restride_kernel, dim3(grid_for(items, kBlock)), dim3(kBlock), 0, t->stream,
+                         t->recs, t->stride, nrecs, new_stride, rows, (int)t->stride);
+      KRK_HIP(hipGetLastError());
+    }
+  }
+  if (rows)
+    KRK_HIP(hipMemcpyAsync(nkeys, t->row_key, (size_t)rows * sizeof(unsigned long long),
+                           hipMemcpyDeviceToDevice, t->stream));
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  if (t->recs) (void)hipFree(t->recs);
+  if (t->row_key) (void)hipFree(t->row_key);
+  t->recs = nrecs;
+  t->row_key = nkeys;
+  t->row_cap = new_cap;
+  t->stride = new_stride;
+  return KRK_SUCCESS;
+}
+
+static int32_t grow_slots(krk_sparse* t, uint64_t new_cap) {
+  Slot* ns = nullptr;
+  KRK_TRY(alloc_slots(new_cap, &ns, t->stream));
+  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  const int64_t rows = t->host_counters[0];
+  t->size_ub = rows;
+  if (rows) {
+    hipLaunchKernelGGL(reindex_kernel, dim3(grid_for(rows, kBlock)), dim3(kBlock), 0, t->stream, ns,
+                       new_cap - 1, t->row_key, rows);
+    KRK_HIP(hipGetLastError());
+  }
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  if (t->slots) (void)hipFree(t->slots);
+  t->slots = ns;
+  t->slot_cap = new_cap;
+  return KRK_SUCCESS;
+}
+
+static uint64_t pow2_at_least(uint64_t x) {
+  uint64_t c = 1024;
+  while (c < x) c <<= 1;
+  return c;
+}
+
+// Room for `extra_rows` more rows: records, row keys, and an index at most half full.
+int32_t sparse_ensure_room(krk_sparse* t, int64_t extra_rows) {
+  int64_t need = t->size_ub + extra_rows;
+  if (need > t->row_cap || (uint64_t)need * 2 > t->slot_cap) {
+    // the bound may be stale (async pulls add their whole request to it): refresh it first
+    KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
+    KRK_HIP(hipStreamSynchronize(t->stream));
+    t->size_ub = t->host_counters[0];
+    need = t->size_ub + extra_rows;
+  }
+  if (need > t->row_cap) {
+    int64_t cap = t->row_cap * 2;
+    if (cap < need) cap = need;
+    if (cap >= (int64_t)kEmptyRow) cap = (int64_t)kEmptyRow - 1;
+    if (cap < need) {
+      set_error("sparse table cannot hold %lld rows", (long long)need);
+      return KRK_E_CAPACITY;
+    }
+    KRK_TRY(grow_rows(t, cap, t->stride));
+  }
+  if ((uint64_t)need * 2 > t->slot_cap) KRK_TRY(grow_slots(t, pow2_at_least((uint64_t)need * 2)));
+  return KRK_SUCCESS;
+}
+
+// Adds the state columns an optimizer needs; existing records are re-strided once.
+int32_t sparse_ensure_columns(krk_sparse* t, uint32_t mask) {
+  int64_t stride = t->stride;
+  bool change = false;
+  int32_t col_off[KRK_ST_COUNT];
+  memcpy(col_off, t->col_off, sizeof(col_off));
+  int32_t meta_off = t->meta_off;
+  // the step counter, when present, stays the last column: re-place it after new columns
+  int64_t body = t->meta_off >= 0 ? t->meta_off : t->stride;
+  for (int st = 1; st < KRK_ST_COUNT; ++st) {
+    if ((mask & (1u << st)) && col_off[st] < 0) {
+      col_off[st] = (int32_t)body;
+      body += t->dim;
+      change = true;
+    }
+  }
+  const bool want_meta = (mask & (1u << KRK_ST_STEPS)) || t->meta_off >= 0;
+  if (want_meta && (t->meta_off < 0 || change)) change = true;
+  if (!change) return KRK_SUCCESS;
+  meta_off = want_meta ? (int32_t)body : -1;
+  stride = body + (want_meta ? t->meta_floats : 0);
+
+  // Move records: weight + old state columns keep their offsets; the step counter moves.
+  const int64_t old_stride = t->stride;
+  const int32_t old_meta = t->meta_off;
+  const int64_t old_body = old_meta >= 0 ? old_meta : old_stride;
+  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  const int64_t rows = t->host_counters[0];
+  t->size_ub = rows;
+  float* nrecs = nullptr;
+  const size_t rec_bytes = (size_t)t->row_cap * (size_t)stride * sizeof(float);
+  KRK_HIP(hipMalloc((void**)&nrecs, rec_bytes ? rec_bytes : 16));
+  KRK_HIP(hipMemsetAsync(nrecs, 0, rec_bytes, t->stream));
+  if (rows) {
+    hipLaunchKernelGGL(restride_kernel, dim3(grid_for(rows * old_body, kBlock)), dim3(kBlock), 0,
+                       t->stream, t->recs, old_stride, nrecs, stride, rows, (int)old_body);
+    if (old_meta >= 0) {
+      hipLaunchKernelGGL(restride_kernel, dim3(grid_for(rows * 2, kBlock)), dim3(kBlock), 0, t->stream,
+                         t->recs + old_meta, old_stride, nrecs + meta_off, stride, rows, 2);
+    }
+    KRK_HIP(hipGetLastError());
+  }
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  if (t->recs) (void)hipFree(t->recs);
+  t->recs = nrecs;
+  t->stride = stride;
+  t->meta_off = meta_off;
+  memcpy(t->col_off, col_off, sizeof(col_off));
+  return KRK_SUCCESS;
+}
+
+void sparse_optim_columns(const krk_sparse* t, const krk_optim& o, int32_t cols[3]) {
+  cols[0] = cols[1] = cols[2] = -1;
+  switch (o.type) {
+    case KRK_SGD:
+      if (o.has_momentum) cols[0] = t->col_off[KRK_ST_MOMENTUM_BUFFER];
+      break;
+    case KRK_ADAGRAD:
+      cols[0] = t->col_off[KRK_ST_STATE_SUM];
+      break;
+    case KRK_ADAM:
+      cols[0] = t->col_off[KRK_ST_FIRST_MOMENT];
+      cols[1] = t->col_off[KRK_ST_SECOND_MOMENT];
+      if (o.amsgrad) cols[2] = t->col_off[KRK_ST_SECOND_MOMENT_MAX];
+      break;
+    case KRK_RMSPROP:
+      cols[0] = t->col_off[KRK_ST_SQUARE_AVERAGE];
+      if (o.centered) cols[1] = t->col_off[KRK_ST_G_AVE];
+      if (o.has_momentum) cols[2] = t->col_off[KRK_ST_MOMENTUM_BUFFER];
+      break;
+    default:
+      break;
+  }
+}
+
+// End of an API call: blocking calls wait, refresh the row count and surface device-side errors.
+int32_t sparse_finish(krk_sparse* t, uint32_t flags) {
+  if (flags & KRK_ASYNC) {
+    t->async_inflight = true;
+    return KRK_SUCCESS;
+  }
+  t->async_inflight = false;
+  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  t->size_ub = t->host_counters[0];
+  const uint32_t err = t->host_counters[1];
+  if (err) {
+    KRK_HIP(hipMemsetAsync(t->counters + 1, 0, sizeof(uint32_t), t->stream));
+    KRK_HIP(hipStreamSynchronize(t->stream));
+    if (err & kErrOverflow) {
+      set_error("sparse table index or row storage overflowed on the device");
+      return KRK_E_CAPACITY;
+    }
+    set_error("push named an id that is not in the table");
+    return KRK_SPARSE_ID_NOT_EXIST;
+  }
+  return KRK_SUCCESS;
+}
+
+static InitK make_init_k(const krk_init& in, int64_t dim) {
+  InitK k;
+  k.seed_mix = splitmix64(in.seed);
+  k.kind = 0;
+  k.p0 = 0.0f;
+  k.p1 = 0.0f;
+  // t/math.cc:24-50 : for a 1-D [dim] tensor fan_out = dim and fan_in = 1;
+  // t/math.cc:476-484, 507-517 : std = gain * sqrt(2.0 / float(fan_in + fan_out)), a = sqrt(3.0) * std
+  const float xstd = (float)((double)in.a * std::sqrt(2.0 / (double)(float)(1 + dim)));
+  switch (in.type) {
+    case KRK_INIT_CONSTANT: k.kind = 0; k.p0 = in.a; break;
+    case KRK_INIT_UNIFORM: k.kind = 1; k.p0 = in.a; k.p1 = in.b; break;
+    case KRK_INIT_NORMAL: k.kind = 2; k.p0 = in.a; k.p1 = in.b; break;
+    case KRK_INIT_XAVIER_UNIFORM: {
+      const float a = (float)(std::sqrt(3.0) * (double)xstd);
+      k.kind = 1; k.p0 = -a; k.p1 = a;
+      break;
+    }
+    case KRK_INIT_XAVIER_NORMAL: k.kind = 2; k.p0 = 0.0f; k.p1 = xstd; break;
+    default: break;
+  }
+  return k;
+}
+
+template <int VEC>
+static void launch_push(krk_sparse* t, const krk_optim& o, const uint64_t* ids, int64_t n,
+                        const float* grads, float lr) {
+  const OptimK k = make_optim_k(o);
+  int32_t cols[3];
+  sparse_optim_columns(t, o, cols);
+  const int per_block = kBlock / t->group;
+  const dim3 grid(grid_for(n, per_block)), block(kBlock);
+  const TableView tv = t->view();
+  const int dim = (int)t->dim;
+  const bool needs_meta = (optim_state_mask(o) >> KRK_ST_STEPS) & 1u;
+  const int meta = needs_meta ? t->meta_off : -1;
+  switch (o.type) {
+    case KRK_SGD:
+      hipLaunchKernelGGL((push_kernel<KRK_SGD, VEC>), grid, block, 0, t->stream, tv, ids, n, grads, dim,
+                         t->elems, t->group, lr, k, cols[0], cols[1], cols[2], meta);
+      break;
+    case KRK_ADAGRAD:
+      hipLaunchKernelGGL((push_kernel<KRK_ADAGRAD, VEC>), grid, block, 0, t->stream, tv, ids, n, grads,
+                         dim, t->elems, t->group, lr, k, cols[0], cols[1], cols[2], meta);
+      break;
+    case KRK_ADAM:
+      hipLaunchKernelGGL((push_kernel<KRK_ADAM, VEC>), grid, block, 0, t->stream, tv, ids, n, grads, dim,
+                         t->elems, t->group, lr, k, cols[0], cols[1], cols[2], meta);
+      break;
+    default:
+      hipLaunchKernelGGL((push_kernel<KRK_RMSPROP, VEC>), grid, block, 0, t->stream, tv, ids, n, grads,
+                         dim, t->elems, t->group, lr, k, cols[0], cols[1], cols[2], meta);
+      break;
+  }
+}
+
+}  // namespace krk
+
+using namespace krk;
+
+static int32_t check_table(krk_sparse* t) {
+  if (!t) {
+    set_error("null sparse table handle");
+    return KRK_E_ARGUMENT;
+  }
+  return ensure_runtime();
+}
+
+static bool valid_optim(const krk_optim* o) {
+  return o && o->type >= KRK_ADAGRAD && o->type <= KRK_SGD;
+}
+
+extern "C" {
+
+int32_t krk_sparse_create(int64_t dim, const krk_init* init, int64_t capacity_hint,
+                          krk_sparse** out) {
+  if (!out || !init || dim <= 0 || dim > (1 << 20) || capacity_hint < 0) {
+    set_error("krk_sparse_create: bad argument (dim=%lld)", (long long)dim);
+    return KRK_E_ARGUMENT;
+  }
+  if (init->type < KRK_INIT_CONSTANT || init->type > KRK_INIT_XAVIER_NORMAL) {
+    set_error("initializer type %d is not supported", init->type);
+    return KRK_UNSUPPORTED_INITIALIZER;   // ps/ps.cc:684-688
+  }
+  KRK_TRY(ensure_runtime());
+  krk_sparse* t = new (std::nothrow) krk_sparse();
+  if (!t) return KRK_E_DEVICE;
+  t->dim = dim;
+  t->vec = (dim % 4 == 0) ? 4 : 1;
+  t->elems = (int)(dim / t->vec);
+  int g = 1;
+  while (g < t->elems && g < kWave) g <<= 1;
+  t->group = g;
+  t->init = *init;
+  t->initk = make_init_k(*init, dim);
+  t->stride = dim;
+  t->meta_floats = t->vec == 4 ? 4 : 2;
+  for (auto& c : t->col_off) c = -1;
+  int32_t rc = t->open_stream();
+  if (rc == KRK_SUCCESS) {
+    hipError_t e = hipMalloc((void**)&t->counters, 16);
+    if (e == hipSuccess) e = hipMemsetAsync(t->counters, 0, 16, t->stream);
+    if (e == hipSuccess) e = hipHostMalloc((void**)&t->host_counters, 16, hipHostMallocDefault);
+    if (e != hipSuccess) rc = hip_fail(e, "krk_sparse_create allocations", __FILE__, __LINE__);
+  }
+  if (rc == KRK_SUCCESS) {
+    int64_t rows = capacity_hint > 0 ? capacity_hint : 4096;
+    rc = sparse_ensure_room(t, rows);
+  }
+  if (rc != KRK_SUCCESS) {
+    krk_sparse_destroy(t);
+    return rc;
+  }
+  *out = t;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_sparse_destroy(krk_sparse* t) {
+  if (!t) return KRK_SUCCESS;
+  if (t->stream) (void)hipStreamSynchronize(t->stream);
+  if (t->slots) (void)hipFree(t->slots);
+  if (t->recs) (void)hipFree(t->recs);
+  if (t->row_key) (void)hipFree(t->row_key);
+  if (t->counters) (void)hipFree(t->counters);
+  if (t->host_counters) (void)hipHostFree(t->host_counters);
+  for (auto& b : t->scratch) b.release();
+  t->close_stream();
+  delete t;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_sparse_dim(krk_sparse* t, int64_t* dim) {
+  if (!t || !dim) return KRK_E_ARGUMENT;
+  *dim = t->dim;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_sparse_size(krk_sparse* t, int64_t* rows) {
+  KRK_TRY(check_table(t));
+  if (!rows) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  t->size_ub = t->host_counters[0];
+  *rows = t->size_ub;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_sparse_reserve(krk_sparse* t, int64_t rows) {
+  KRK_TRY(check_table(t));
+  if (rows < 0) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  const int64_t extra = rows - t->size_ub;
+  return extra > 0 ? sparse_ensure_room(t, extra) : KRK_SUCCESS;
+}
+
+int32_t krk_sparse_sync(krk_sparse* t) {
+  KRK_TRY(check_table(t));
+  std::lock_guard<std::mutex> lk(t->mu);
+  return sparse_finish(t, 0);
+}
+
+int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* out, uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (n < 0 || (n > 0 && (!ids || !out))) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (n == 0) return sparse_finish(t, flags);
+  KRK_TRY(sparse_ensure_room(t, n));
+  const uint64_t* d_ids;
+  float* d_out;
+  KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
+  KRK_TRY(t->output(out, (size_t)n * t->dim, flags, 1, &d_out));
+  const int per_block = kBlock / t->group;
+  // The kernel must know how many rows existed before it started. After a blocking call the
+  // host knows that exactly; while async work is in flight it does not, so the count is
+  // snapshotted on the device in stream order instead.
+  const uint32_t base_rows = (uint32_t)t->host_counters[0];
+  const uint32_t* base_dev = nullptr;
+  if (t->async_inflight || (flags & KRK_ASYNC)) {
+    hipLaunchKernelGGL(snapshot_rows_kernel, dim3(1), dim3(1), 0, t->stream, t->counters);
+    base_dev = t->counters + 2;
+  }
+  const dim3 grid(grid_for(n, per_block)), block(kBlock);
+  if (t->vec == 4) {
+    hipLaunchKernelGGL((pull_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
+                       (int)t->dim, t->elems, t->group, base_rows, base_dev, t->initk);
+  } else {
+    hipLaunchKernelGGL((pull_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
+                       (int)t->dim, t->elems, t->group, base_rows, base_dev, t->initk);
+  }
+  KRK_HIP(hipGetLastError());
+  t->size_ub += n;
+  KRK_TRY(t->output_back(out, (size_t)n * t->dim, flags, 1));
+  return sparse_finish(t, flags);
+}
+
+int32_t krk_sparse_push(krk_sparse* t, const krk_optim* o, const uint64_t* ids, int64_t n,
+                        const float* grads, int64_t grad_dim, float lr, uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (!valid_optim(o)) {
+    set_error("optimizer type is not supported");
+    return KRK_UNSUPPORTED_OPTIM;
+  }
+  if (n < 0 || (n > 0 && (!ids || !grads))) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (n == 0) return sparse_finish(t, flags);
+  if (grad_dim != t->dim) {   // ps/optim/adagrad.cc:29-32
+    set_error("gradient width %lld does not match table dimension %lld", (long long)grad_dim,
+              (long long)t->dim);
+    return KRK_GRADIENT_UNCOMPATIBLE;
+  }
+  KRK_TRY(sparse_ensure_columns(t, optim_state_mask(*o)));
+  const uint64_t* d_ids;
+  const float* d_g;
+  KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
+  KRK_TRY(t->input(grads, (size_t)n * t->dim, flags, 1, &d_g));
+  if (t->vec == 4) {
+    launch_push<4>(t, *o, d_ids, n, d_g, lr);
+  } else {
+    launch_push<1>(t, *o, d_ids, n, d_g, lr);
+  }
+  KRK_HIP(hipGetLastError());
+  return sparse_finish(t, flags);
+}
+
+int32_t krk_sparse_lookup(krk_sparse* t, const uint64_t* ids, int64_t n, int32_t* rows,
+                          uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (n < 0 || (n > 0 && (!ids || !rows))) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (n == 0) return sparse_finish(t, flags);
+  const uint64_t* d_ids;
+  int32_t* d_rows;
+  KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
+  KRK_TRY(t->output(rows, (size_t)n, flags, 1, &d_rows));
+  hipLaunchKernelGGL(lookup_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, t->stream, t->view(),
+                     d_ids, n, d_rows);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(t->output_back(rows, (size_t)n, flags, 1));
+  return sparse_finish(t, flags);
+}
+
+int32_t krk_sparse_import(krk_sparse* t, const uint64_t* ids, int64_t n, const float* vals,
+                          uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (n < 0 || (n > 0 && (!ids || !vals))) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (n == 0) return sparse_finish(t, flags);
+  KRK_TRY(sparse_ensure_room(t, n));
+  const uint64_t* d_ids;
+  const float* d_vals;
+  KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
+  KRK_TRY(t->input(vals, (size_t)n * t->dim, flags, 1, &d_vals));
+  const int per_block = kBlock / t->group;
+  const dim3 grid(grid_for(n, per_block)), block(kBlock);
+  if (t->vec == 4) {
+    hipLaunchKernelGGL((import_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_vals,
+                       (int)t->dim, t->elems, t->group);
+  } else {
+    hipLaunchKernelGGL((import_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, d_vals,
+                       (int)t->dim, t->elems, t->group);
+  }
+  KRK_HIP(hipGetLastError());
+  t->size_ub += n;
+  return sparse_finish(t, flags);
+}
+
+int32_t krk_sparse_export(krk_sparse* t, uint64_t* ids, float* vals, int32_t state_type, float* state,
+                          int64_t* steps, int64_t capacity, int64_t* rows_out, uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;
+  if (state && (state_type < 1 || state_type >= KRK_ST_COUNT)) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  KRK_TRY(sparse_finish(t, 0));
+  const int64_t rows = t->size_ub;
+  if (rows_out) *rows_out = rows;
+  if (rows > capacity) {
+    set_error("export needs room for %lld rows, caller offered %lld", (long long)rows,
+              (long long)capacity);
+    return KRK_E_CAPACITY;
+  }
+  if (rows == 0) return KRK_SUCCESS;
+  unsigned long long* d_ids = nullptr;
+  float* d_vals = nullptr;
+  float* d_state = nullptr;
+  long long* d_steps = nullptr;
+  const size_t cells = (size_t)rows * t->dim;
+  if (ids) KRK_TRY(t->output(reinterpret_cast<unsigned long long*>(ids), (size_t)rows, flags, 0, &d_ids));
+  if (vals) KRK_TRY(t->output(vals, cells, flags, 1, &d_vals));
+  if (state) KRK_TRY(t->output(state, cells, flags, 2, &d_state));
+  if (steps) KRK_TRY(t->output(reinterpret_cast<long long*>(steps), (size_t)rows, flags, 3, &d_steps));
+  const int state_off = state ? t->col_off[state_type] : -1;
+  hipLaunchKernelGGL(export_kernel, dim3(grid_for((int64_t)cells, kBlock)), dim3(kBlock), 0, t->stream,
+                     t->view(), rows, (int)t->dim, d_ids, d_vals, state_off, d_state, t->meta_off,
+                     d_steps);
+  KRK_HIP(hipGetLastError());
+  if (ids) KRK_TRY(t->output_back(reinterpret_cast<unsigned long long*>(ids), (size_t)rows, flags, 0));
+  if (vals) KRK_TRY(t->output_back(vals, cells, flags, 1));
+  if (state) KRK_TRY(t->output_back(state, cells, flags, 2));
+  if (steps) KRK_TRY(t->output_back(reinterpret_cast<long long*>(steps), (size_t)rows, flags, 3));
+  return sparse_finish(t, 0);
+}
+
+}  // extern "C"

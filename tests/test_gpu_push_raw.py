@@ -1,0 +1,130 @@
+"""Worker-side dedup and the fused dedup + segment-reduce + update path against the oracle's
+restatement of Emitter::PullSparseTableImpl / PushSparseTable (worker/emitter.cc:131-149,
+510-531) followed by SparseTable::Push.
+
+Bar: unique ids, their order and the inverse map exact; summed-and-updated values within 1e-5
+relative of the reference order of additions (the GPU adds in a fixed tree, the reference in
+position order), measured against the magnitude of the addends where sums cancel.
+"""
+import numpy as np
+import pytest
+
+from util import OPTIM_CASES, assert_close, make_optims, splitmix64, zipf_ids
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def api():
+    from kraken_amd import api as a
+    a.lib()
+    return a
+
+
+@pytest.mark.parametrize("ids", [
+    [5], [5, 5, 5, 5], [1, 2, 3, 4], [9, 1, 9, 2, 1, 9, 2**64 - 1, 0, 2**64 - 1],
+])
+def test_dedup_small(api, oracle, ids):
+    ids = np.array(ids, dtype=np.uint64)
+    u, inv = api.dedup(ids)
+    ru, rinv = oracle.dedup(ids)
+    assert np.array_equal(u, ru) and np.array_equal(inv, rinv)
+
+
+def test_dedup_empty(api):
+    u, inv = api.dedup(np.zeros(0, np.uint64))
+    assert u.size == 0 and inv.size == 0
+
+
+@pytest.mark.parametrize("n,s,space", [(8192, 1.05, 10**6), (200_000, 1.3, 10**6), (1_000_000, 1.1, 10**7)])
+def test_dedup_zipf_exact(api, oracle, n, s, space):
+    rng = np.random.default_rng(n)
+    ids = zipf_ids(rng, s, space, n)
+    u, inv = api.dedup(ids)
+    ru, rinv = oracle.dedup(ids)
+    assert np.array_equal(u, ru)               # first-occurrence order, bit for bit
+    assert np.array_equal(inv, rinv)
+    assert np.array_equal(u[inv], ids)
+    # device-resident variant
+    d = api.DeviceArray.from_host(ids)
+    du, dinv, cnt = api.dedup(d)
+    assert cnt == ru.size
+    assert np.array_equal(du.to_host()[:cnt], ru) and np.array_equal(dinv.to_host(), rinv)
+
+
+def _cancel_safe_close(got, want, scale, what):
+    """|got - want| <= 1e-5 * (|want| + accumulated magnitude of what was summed)."""
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    tol = 1e-5 * (np.abs(want.astype(np.float64)) + scale) + 1e-7
+    assert (err <= tol).all(), (what, float((err / tol).max()))
+
+
+@pytest.mark.parametrize("name,type_,conf", [c for c in OPTIM_CASES if c[0] in (
+    "sgd", "sgd_damp", "adagrad", "adam", "adam_amsgrad", "rmsprop", "rmsprop_all")],
+    ids=lambda v: v if isinstance(v, str) else None)
+@pytest.mark.parametrize("dim,n,s", [(16, 8192, 1.05), (128, 50_000, 1.3), (100, 3000, 1.3), (8, 300_000, 1.2)])
+def test_push_raw_matches_dedup_sum_then_push(api, oracle, name, type_, conf, dim, n, s):
+    rng = np.random.default_rng(n + dim)
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "9"})
+    t = api.SparseTable(dim, gi)
+    r = oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=9))
+    o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    lr = 0.05
+    for step in range(3):
+        ids = zipf_ids(rng, s, 10**6, n)
+        g = (rng.standard_normal((n, dim)) * 1e-2).astype(np.float32)
+        assert t.Pull(ids)[0] == 0
+        r.pull(ids)
+        assert t.PushRaw(o_gpu, ids, g, lr) == 0
+        u, gs = oracle.dedup_sum(ids, g)
+        assert r.push(o_ref, u, gs, lr) == 0
+    gid, gval, _, gsteps = t.export()
+    rid, rval, _, rsteps = r.export()
+    og, orr = np.argsort(gid), np.argsort(rid)
+    assert np.array_equal(gid[og], rid[orr])
+    if type_ == 1:
+        assert np.array_equal(gsteps[og], rsteps[orr])       # one optimizer step per unique id
+    # an id repeated c times adds c gradients of size ~1e-2: allow for that in the tolerance
+    _cancel_safe_close(gval[og], rval[orr], 0.05, "%s dim %d" % (name, dim))
+
+
+def test_push_raw_single_hot_id_and_all_distinct(api, oracle):
+    """The two extremes of the segmented reduction: one run spanning every tile, and no runs."""
+    dim = 32
+    gi = api.Initializer.create(api.InitializerType.kConstant, {"value": "1"})
+    o_ref, o_gpu = make_optims(oracle, api, 3, {})
+    rng = np.random.default_rng(7)
+    for ids in (np.full(70_000, 12345, dtype=np.uint64),
+                splitmix64(np.arange(70_000, dtype=np.uint64)),
+                np.repeat(splitmix64(np.arange(100, dtype=np.uint64)), 700)):
+        t = api.SparseTable(dim, gi)
+        r = oracle.SparseTable(dim, oracle.init(oracle.INIT_CONSTANT, 1.0))
+        g = (rng.standard_normal((ids.size, dim)) * 1e-2).astype(np.float32)
+        t.Pull(ids)
+        r.pull(ids)
+        assert t.PushRaw(o_gpu, ids, g, 0.5) == 0
+        u, gs = oracle.dedup_sum(ids, g)
+        assert r.push(o_ref, u, gs, 0.5) == 0
+        rc, got = t.Pull(u)
+        _, want = r.pull(u)
+        scale = 0.5 * 1e-2 * np.sqrt(ids.size / u.size)
+        _cancel_safe_close(got, want, scale, "extreme case")
+        # same inputs, same bits: the order of additions is fixed
+        t2 = api.SparseTable(dim, gi)
+        t2.Pull(ids)
+        assert t2.PushRaw(o_gpu, ids, g, 0.5) == 0
+        assert np.array_equal(t2.Pull(u)[1], got)
+
+
+def test_push_raw_missing_id_and_width(api, oracle):
+    gi = api.Initializer.create(api.InitializerType.kConstant, {"value": "2"})
+    t = api.SparseTable(8, gi)
+    t.Pull([1, 2, 3])
+    o = api.Optim.create(api.OptimType.kSGD)
+    g = np.ones((5, 8), np.float32)
+    assert t.PushRaw(o, [1, 1, 2, 77, 77], g, 0.25) == 12
+    rc, rows = t.Pull([1, 2, 3])
+    assert np.array_equal(rows[:, 0], np.float32([2 - 0.5, 2 - 0.25, 2]))
+    assert t.lookup([77])[0] == -1
+    assert t.PushRaw(o, [1, 2], np.ones((2, 4), np.float32), 0.1) == 11
+    assert t.PushRaw(o, [], np.zeros((0, 8), np.float32), 0.1) == 0
