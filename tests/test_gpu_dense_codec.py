@@ -108,7 +108,8 @@ def test_codec_matches_oracle(api, oracle, n, eta):
     for step in range(3):
         g = rng.standard_normal(n).astype(np.float32)
         if step == 1:
-            g[::3] = g[1::3][: g[::3].size]        # ties around the threshold
+            m = g[1::3].size
+            g[::3][:m] = g[1::3]                   # ties around the threshold
         idx, val = bag.MaybeToCoo(2, eta, g)
         ridx, rval = ref.compress(g, life_span=2, eta=eta, exact_select=True)
         assert bag.tau == ref.tau
