@@ -128,6 +128,10 @@ int32_t krk_memcpy_d2h(void* dst, const void* src, size_t bytes);
 int32_t krk_memset(void* dptr, int value, size_t bytes);
 int32_t krk_device_synchronize(void);
 int32_t krk_mem_info(size_t* free_bytes, size_t* total_bytes);
+/* A plain device-to-device streaming copy kernel on the null stream (not synchronised): the
+ * measured bandwidth ceiling, and the known-size kernel byte counters are calibrated against.
+ * Pointers and size must be multiples of 16. */
+int32_t krk_stream_copy(void* dst, const void* src, size_t bytes);
 
 /* ---- sparse table --------------------------------------------------------- */
 typedef struct krk_sparse krk_sparse;
@@ -181,6 +185,31 @@ int32_t krk_sparse_export(krk_sparse* t, uint64_t* ids, float* vals, int32_t sta
                           float* state, int64_t* steps, int64_t capacity, int64_t* rows,
                           uint32_t flags);
 
+/* ---- groups of sparse tables: one combined request, one launch -------------- */
+typedef struct krk_group krk_group;
+/* The tables of a model that are pulled and pushed together
+ * (CombinePullSparseTableRequest / CombinePushSparseTableRequest,
+ * protocol/combine_pull_sparse_table_prot.h:13-33, combine_push_sparse_table_prot.h:12-33).
+ * Members (1..32) must have equal dimension and belong to no other group. While the group
+ * exists its members run on the group's stream, so single-table calls on a member stay
+ * ordered with the group's calls. Destroy the group before its tables. */
+int32_t krk_group_create(krk_sparse** tables, int32_t n, krk_group** out);
+int32_t krk_group_destroy(krk_group* g);
+int32_t krk_group_sync(krk_group* g);
+/* Ps::CombinePullSparseTable (ps/ps_op.cc:370-387): the reference loops over the tables of the
+ * request; here all of them are served by one launch. ids is the concatenation of every
+ * table's ids in member order, offsets[n+1] (host memory, offsets[0] = 0) delimits them, out is
+ * [offsets[n], dim]. Per table the semantics are krk_sparse_pull's. */
+int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets, float* out,
+                       uint32_t flags);
+/* Ps::CombinePushSparseTable (ps/ps_op.cc:456-469) with one optimizer for the whole model
+ * (Ps::CreateModel, ps/ps.cc:604-633). ids unique within each table; grads is
+ * [offsets[n], grad_dim]. Per table the semantics are krk_sparse_push's; the reference
+ * returns at the first failing table, here every table is processed and the first error code
+ * in member order is returned. */
+int32_t krk_group_push(krk_group* g, const krk_optim* o, const uint64_t* ids, const int64_t* offsets,
+                       const float* grads, int64_t grad_dim, float lr, uint32_t flags);
+
 /* Emitter::PullSparseTableImpl's dedup (worker/emitter.cc:131-149): unique ids
  * in first-occurrence order, inv[p] = index of ids[p] in uids. uids and inv
  * hold n entries; *n_unique receives U. */
@@ -233,8 +262,9 @@ int32_t krk_coo_to_dense(const int64_t* idx, const float* val, int64_t nnz, floa
 typedef struct krk_event krk_event;
 int32_t krk_event_create(krk_event** e);
 int32_t krk_event_destroy(krk_event* e);
-/* Exactly one of sparse/dense/dct is non-NULL: the event is recorded on that object's stream. */
-int32_t krk_event_record(krk_event* e, krk_sparse* sparse, krk_dense* dense, krk_dct* dct);
+/* object = a krk_sparse*, krk_group*, krk_dense* or krk_dct*: the event is recorded on that
+ * object's stream, behind the work already enqueued there. */
+int32_t krk_event_record(krk_event* e, void* object);
 int32_t krk_event_elapsed_ms(krk_event* start, krk_event* stop, float* ms);
 
 #ifdef __cplusplus

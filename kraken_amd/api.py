@@ -68,6 +68,7 @@ EXPORTS = {
     "krk_memset": (C.c_int32, [C.c_void_p, C.c_int, C.c_size_t]),
     "krk_device_synchronize": (C.c_int32, []),
     "krk_mem_info": (C.c_int32, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "krk_stream_copy": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "krk_sparse_create": (C.c_int32, [C.c_int64, C.POINTER(krk_init), C.c_int64, C.POINTER(C.c_void_p)]),
     "krk_sparse_destroy": (C.c_int32, [C.c_void_p]),
     "krk_sparse_dim": (C.c_int32, [C.c_void_p, C.POINTER(C.c_int64)]),
@@ -106,7 +107,13 @@ EXPORTS = {
                                      C.c_uint32]),
     "krk_event_create": (C.c_int32, [C.POINTER(C.c_void_p)]),
     "krk_event_destroy": (C.c_int32, [C.c_void_p]),
-    "krk_event_record": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "krk_event_record": (C.c_int32, [C.c_void_p, C.c_void_p]),
+    "krk_group_create": (C.c_int32, [C.POINTER(C.c_void_p), C.c_int32, C.POINTER(C.c_void_p)]),
+    "krk_group_destroy": (C.c_int32, [C.c_void_p]),
+    "krk_group_sync": (C.c_int32, [C.c_void_p]),
+    "krk_group_pull": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32]),
+    "krk_group_push": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_void_p, C.c_void_p,
+                                   C.c_int64, C.c_float, C.c_uint32]),
     "krk_event_elapsed_ms": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "krk_dct2_forward": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_uint32]),
     "krk_dct2_inverse": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_uint32]),
@@ -343,6 +350,59 @@ class SparseTable:
         return ids, vals, st, steps
 
 
+class TableGroup:
+    """The sparse tables of one combined request (Ps::CombinePullSparseTable /
+    CombinePushSparseTable, ps/ps_op.cc:370-387, 456-469): one launch serves all of them."""
+
+    def __init__(self, tables):
+        self.tables = list(tables)
+        self.dimension = self.tables[0].dimension
+        arr = (C.c_void_p * len(self.tables))(*[t.h for t in self.tables])
+        h = C.c_void_p()
+        _check(lib().krk_group_create(arr, len(self.tables), C.byref(h)), "krk_group_create")
+        self.h = h
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().krk_group_destroy(self.h)
+            self.h = None
+
+    __del__ = close
+
+    def sync(self):
+        return lib().krk_group_sync(self.h)
+
+    @staticmethod
+    def _offsets(counts):
+        off = np.zeros(len(counts) + 1, np.int64)
+        np.cumsum(counts, out=off[1:])
+        return off
+
+    def CombinePull(self, ids, offsets, out=None, async_=False):
+        """ids: concatenated per-table ids; offsets: int64[n_tables + 1] -> (code, vals)"""
+        offsets = np.ascontiguousarray(offsets, dtype=np.int64)
+        total = int(offsets[-1])
+        if isinstance(ids, DeviceArray):
+            if out is None:
+                out = DeviceArray((total, self.dimension), np.float32)
+        else:
+            ids = np.ascontiguousarray(ids, dtype=np.uint64)
+            if out is None:
+                out = np.empty((total, self.dimension), np.float32)
+        rc = lib().krk_group_pull(self.h, _ptr(ids), _ptr(offsets), _ptr(out),
+                                  _flags(ids, out, extra=ASYNC if async_ else 0))
+        return rc, out
+
+    def CombinePush(self, optim, ids, offsets, grads, lr, async_=False):
+        offsets = np.ascontiguousarray(offsets, dtype=np.int64)
+        if not isinstance(ids, DeviceArray):
+            ids = np.ascontiguousarray(ids, dtype=np.uint64)
+            grads = np.ascontiguousarray(grads, dtype=np.float32)
+        gd = grads.shape[-1]
+        return lib().krk_group_push(self.h, C.byref(optim.raw), _ptr(ids), _ptr(offsets), _ptr(grads),
+                                    gd, lr, _flags(ids, grads, extra=ASYNC if async_ else 0))
+
+
 class DenseTable:
     """ps/dense_table.h"""
 
@@ -493,10 +553,7 @@ class Event:
         self.h = h
 
     def record(self, obj):
-        s = obj.h if isinstance(obj, SparseTable) else None
-        d = obj.h if isinstance(obj, DenseTable) else None
-        c = obj.h if isinstance(obj, DenseBag) else None
-        _check(lib().krk_event_record(self.h, s, d, c), "krk_event_record")
+        _check(lib().krk_event_record(self.h, obj.h), "krk_event_record")
 
     def elapsed_ms(self, stop):
         ms = C.c_float()

@@ -447,10 +447,9 @@ int32_t krk_event_destroy(krk_event* e) {
   return KRK_SUCCESS;
 }
 // Every API object begins with an ObjBase, so its stream is reachable from any handle.
-int32_t krk_event_record(krk_event* e, krk_sparse* sparse, krk_dense* dense, krk_dct* dct) {
-  void* h = sparse ? (void*)sparse : dense ? (void*)dense : (void*)dct;
-  if (!e || !h) return KRK_E_ARGUMENT;
-  ObjBase* b = reinterpret_cast<ObjBase*>(h);
+int32_t krk_event_record(krk_event* e, void* object) {
+  if (!e || !object) return KRK_E_ARGUMENT;
+  ObjBase* b = reinterpret_cast<ObjBase*>(object);
   KRK_HIP(hipEventRecord(e->ev, b->stream));
   return KRK_SUCCESS;
 }
@@ -462,3 +461,28 @@ int32_t krk_event_elapsed_ms(krk_event* start, krk_event* stop, float* ms) {
 }
 
 }  // extern "C"
+
+// ---------------------------------------------------------------------------
+// A plain streaming copy: the measured ceiling every bandwidth figure is compared with, and the
+// known-size kernel that hardware byte counters are calibrated against.
+// ---------------------------------------------------------------------------
+namespace krk {
+__global__ __launch_bounds__(256) void stream_copy_kernel(const float4* __restrict__ src,
+                                                          float4* __restrict__ dst, int64_t n16) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+}  // namespace krk
+
+extern "C" int32_t krk_stream_copy(void* dst, const void* src, size_t bytes) {
+  KRK_TRY(ensure_runtime());
+  if ((bytes & 15) || ((uintptr_t)dst & 15) || ((uintptr_t)src & 15)) return KRK_E_ARGUMENT;
+  const int64_t n16 = (int64_t)(bytes / 16);
+  if (n16 == 0) return KRK_SUCCESS;
+  int64_t blocks = (n16 + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  hipLaunchKernelGGL(krk::stream_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, nullptr,
+                     reinterpret_cast<const float4*>(src), reinterpret_cast<float4*>(dst), n16);
+  KRK_HIP(hipGetLastError());
+  return KRK_SUCCESS;
+}

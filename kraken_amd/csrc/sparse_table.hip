@@ -2,7 +2,9 @@
 // insert-on-miss) and push (one fused read-modify-write of weight + optimizer state per row).
 //
 // Replaces SparseTable::Pull / ::Push (ps/sparse_table.cc:33-108), the per-row Optim::Update
-// chains (ps/optim/*.cc) and the row initialisers (ps/initializer/*.cc, t/math.cc:333-517).
+// chains (ps/optim/*.cc), the row initialisers (ps/initializer/*.cc, t/math.cc:333-517) and, for
+// a group of tables, the loops of Ps::CombinePullSparseTable / CombinePushSparseTable
+// (ps/ps_op.cc:370-387, 456-469), which become one launch over all tables of the request.
 //
 // Work mapping: `group` adjacent lanes of a 64-wide wavefront own one id. The group's first
 // lane walks the index (one 16-byte slot load per probe), the row number is broadcast with a
@@ -16,17 +18,7 @@
 namespace krk {
 
 constexpr int kBlock = 256;
-
-template <int VEC>
-struct VecT;
-template <>
-struct VecT<4> {
-  using type = float4;
-};
-template <>
-struct VecT<1> {
-  using type = float;
-};
+constexpr int kMaxGroupTables = 32;
 
 template <int VEC>
 __device__ __forceinline__ void vload(const float* p, float (&v)[VEC]) {
@@ -47,38 +39,34 @@ __device__ __forceinline__ void vstore(float* p, const float (&v)[VEC]) {
 }
 
 // ---------------------------------------------------------------------------
-// pull: gather rows, inserting and initialising the ones that are missing
+// pull: gather rows, inserting and initialising the ones that are missing.
+// `i` is this lane group's position in ids/out, gl the lane's index in the group.
 // ---------------------------------------------------------------------------
 template <int VEC>
-__global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, const uint64_t* __restrict__ ids,
-                                                      int64_t n, float* __restrict__ out, int dim,
-                                                      int elems, int group, uint32_t base_rows,
-                                                      const uint32_t* __restrict__ base_rows_dev,
-                                                      InitK init) {
-  if (base_rows_dev) base_rows = *base_rows_dev;
-  const int per_block = kBlock / group;
-  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
-  const int gl = threadIdx.x & (group - 1);
-  const bool active = i < n;
+__device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init,
+                                          const uint64_t* __restrict__ ids, int64_t i, bool active,
+                                          int gl, float* __restrict__ out, int dim, int elems,
+                                          int group) {
   const uint64_t id = active ? ids[i] : 0;
   uint32_t row = kEmptyRow;
-  int owner = 0;
+  int flags = 0;   // bit 0: this group created the row, bit 1: the row was created by this launch
   if (active && gl == 0) {
-    bool own;
-    row = probe_insert(tv, id, &own);
-    owner = own ? 1 : 0;
+    bool own, fresh;
+    row = probe_insert(tv, id, &own, &fresh);
+    flags = (own ? 1 : 0) | (fresh ? 2 : 0);
   }
   row = __shfl(row, 0, group);
-  owner = __shfl(owner, 0, group);
-  if (!active) return;
-  // Rows numbered at or past base_rows were created by this launch: their record may not be
-  // written yet, and their value is a pure function of (seed, id), so it is recomputed.
-  const bool fresh = row == kEmptyRow || row >= base_rows;
+  flags = __shfl(flags, 0, group);
+  if (!active) return;   // callers publish after this returns; nothing below synchronises
+  const bool owner = flags & 1;
+  const bool fresh = flags & 2;
   float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
   float* dst = out + i * (int64_t)dim;
   for (int e = gl; e < elems; e += group) {
     float v[VEC];
     if (fresh) {
+      // the value of a new row is a pure function of (seed, id, element): every group that
+      // meets it computes the same numbers, only the creator stores them
 #pragma unroll
       for (int c = 0; c < VEC; ++c) v[c] = init_element(init, id, (int64_t)e * VEC + c);
       if (owner) vstore<VEC>(rec + e * VEC, v);
@@ -92,16 +80,15 @@ __global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, const uint64
 // ---------------------------------------------------------------------------
 // push: per unique id, one fused update of the record
 // ---------------------------------------------------------------------------
+struct PushCols {
+  int c0, c1, c2, meta;
+};
+
 template <int OPT, int VEC>
-__global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64_t* __restrict__ ids,
-                                                      int64_t n, const float* __restrict__ grads,
-                                                      int dim, int elems, int group, float lr,
-                                                      OptimK k, int c0, int c1off, int c2off,
-                                                      int meta_off) {
-  const int per_block = kBlock / group;
-  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
-  const int gl = threadIdx.x & (group - 1);
-  const bool active = i < n;
+__device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* __restrict__ ids,
+                                          int64_t i, bool active, int gl,
+                                          const float* __restrict__ grads, int dim, int elems,
+                                          int group, float lr, const OptimK& k, const PushCols& pc) {
   uint32_t row = kEmptyRow;
   if (active && gl == 0) {
     row = probe_find(tv, ids[i]);
@@ -115,8 +102,8 @@ __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64
   bool first = false;
   float bc1 = 1.0f, bc2 = 1.0f;
   uint64_t steps = 0;
-  if (meta_off >= 0) {
-    const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + meta_off);
+  if (pc.meta >= 0) {
+    const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + pc.meta);
     steps = (uint64_t)meta[0] | ((uint64_t)meta[1] << 32);
     first = steps == 0;
     steps += 1;
@@ -130,26 +117,110 @@ __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64
     float gv[VEC], w[VEC], s0[VEC], s1[VEC], s2[VEC];
     vload<VEC>(g + e * VEC, gv);
     vload<VEC>(rec + e * VEC, w);
-    if (c0 >= 0) vload<VEC>(rec + c0 + e * VEC, s0);
-    if (c1off >= 0) vload<VEC>(rec + c1off + e * VEC, s1);
-    if (c2off >= 0) vload<VEC>(rec + c2off + e * VEC, s2);
+    if (pc.c0 >= 0) vload<VEC>(rec + pc.c0 + e * VEC, s0);
+    if (pc.c1 >= 0) vload<VEC>(rec + pc.c1 + e * VEC, s1);
+    if (pc.c2 >= 0) vload<VEC>(rec + pc.c2 + e * VEC, s2);
 #pragma unroll
     for (int c = 0; c < VEC; ++c) {
-      if (c0 < 0) s0[c] = 0.0f;
-      if (c1off < 0) s1[c] = 0.0f;
-      if (c2off < 0) s2[c] = 0.0f;
+      if (pc.c0 < 0) s0[c] = 0.0f;
+      if (pc.c1 < 0) s1[c] = 0.0f;
+      if (pc.c2 < 0) s2[c] = 0.0f;
       optim_element<OPT>(k, lr, gv[c], w[c], s0[c], s1[c], s2[c], first, bc1, bc2);
     }
     vstore<VEC>(rec + e * VEC, w);
-    if (c0 >= 0) vstore<VEC>(rec + c0 + e * VEC, s0);
-    if (c1off >= 0) vstore<VEC>(rec + c1off + e * VEC, s1);
-    if (c2off >= 0) vstore<VEC>(rec + c2off + e * VEC, s2);
+    if (pc.c0 >= 0) vstore<VEC>(rec + pc.c0 + e * VEC, s0);
+    if (pc.c1 >= 0) vstore<VEC>(rec + pc.c1 + e * VEC, s1);
+    if (pc.c2 >= 0) vstore<VEC>(rec + pc.c2 + e * VEC, s2);
   }
-  if (meta_off >= 0 && gl == 0) {
-    uint32_t* meta = reinterpret_cast<uint32_t*>(rec + meta_off);
+  if (pc.meta >= 0 && gl == 0) {
+    uint32_t* meta = reinterpret_cast<uint32_t*>(rec + pc.meta);
     meta[0] = (uint32_t)steps;
     meta[1] = (uint32_t)(steps >> 32);
   }
+}
+
+// ---- single-table launches ---------------------------------------------------
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, InitK init,
+                                                      const uint64_t* __restrict__ ids, int64_t n,
+                                                      float* __restrict__ out, int dim, int elems,
+                                                      int group) {
+  const int per_block = kBlock / group;
+  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  pull_body<VEC>(tv, init, ids, i, i < n, threadIdx.x & (group - 1), out, dim, elems, group);
+  publish_rows(tv, gridDim.x);
+}
+
+template <int OPT, int VEC>
+__global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                      int64_t n, const float* __restrict__ grads,
+                                                      int dim, int elems, int group, float lr,
+                                                      OptimK k, PushCols pc) {
+  const int per_block = kBlock / group;
+  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  push_body<OPT, VEC>(tv, ids, i, i < n, threadIdx.x & (group - 1), grads, dim, elems, group, lr, k, pc);
+}
+
+// ---- one launch over several tables of equal row width ------------------------
+// Table t owns workgroups [block_start[t], block_start[t+1]) and the positions
+// [row_start[t], row_start[t+1]) of the concatenated ids / rows.
+struct TableDesc {
+  TableView tv;
+  InitK init;
+  int32_t col_off[KRK_ST_COUNT];
+  int32_t meta_off;
+};
+
+struct GroupCall {
+  int32_t n_tables;
+  uint32_t epoch[kMaxGroupTables];
+  uint32_t block_start[kMaxGroupTables + 1];
+  int64_t row_start[kMaxGroupTables + 1];
+};
+
+__device__ __forceinline__ int find_table(const GroupCall& c) {
+  int t = 0;
+  while (t + 1 < c.n_tables && blockIdx.x >= c.block_start[t + 1]) ++t;
+  return t;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void group_pull_kernel(const TableDesc* __restrict__ descs,
+                                                            GroupCall call,
+                                                            const uint64_t* __restrict__ ids,
+                                                            float* __restrict__ out, int dim, int elems,
+                                                            int group) {
+  const int t = find_table(call);
+  TableView tv = descs[t].tv;
+  tv.epoch = call.epoch[t];
+  const InitK init = descs[t].init;
+  const int per_block = kBlock / group;
+  const int64_t local = (int64_t)(blockIdx.x - call.block_start[t]) * per_block + threadIdx.x / group;
+  const int64_t i = call.row_start[t] + local;
+  pull_body<VEC>(tv, init, ids, i, i < call.row_start[t + 1], threadIdx.x & (group - 1), out, dim,
+                 elems, group);
+  publish_rows(tv, call.block_start[t + 1] - call.block_start[t]);
+}
+
+template <int OPT, int VEC>
+__global__ __launch_bounds__(kBlock) void group_push_kernel(const TableDesc* __restrict__ descs,
+                                                            GroupCall call,
+                                                            const uint64_t* __restrict__ ids,
+                                                            const float* __restrict__ grads, int dim,
+                                                            int elems, int group, float lr, OptimK k,
+                                                            int st0, int st1, int st2, int use_meta) {
+  const int t = find_table(call);
+  const TableView tv = descs[t].tv;
+  PushCols pc;
+  pc.c0 = st0 >= 0 ? descs[t].col_off[st0] : -1;
+  pc.c1 = st1 >= 0 ? descs[t].col_off[st1] : -1;
+  pc.c2 = st2 >= 0 ? descs[t].col_off[st2] : -1;
+  pc.meta = use_meta ? descs[t].meta_off : -1;
+  const int per_block = kBlock / group;
+  const int64_t local = (int64_t)(blockIdx.x - call.block_start[t]) * per_block + threadIdx.x / group;
+  const int64_t i = call.row_start[t] + local;
+  push_body<OPT, VEC>(tv, ids, i, i < call.row_start[t + 1], threadIdx.x & (group - 1), grads, dim,
+                      elems, group, lr, k, pc);
 }
 
 __global__ __launch_bounds__(kBlock) void lookup_kernel(TableView tv, const uint64_t* __restrict__ ids,
@@ -159,9 +230,6 @@ __global__ __launch_bounds__(kBlock) void lookup_kernel(TableView tv, const uint
   const uint32_t r = probe_find(tv, ids[i]);
   rows[i] = r == kEmptyRow ? -1 : (int32_t)r;
 }
-
-// counters[2] = counters[0]: the row count a following pull starts from, taken in stream order
-__global__ void snapshot_rows_kernel(uint32_t* counters) { counters[2] = counters[0]; }
 
 // import: like pull, but a new row takes its values from the caller
 template <int VEC>
@@ -175,20 +243,22 @@ __global__ __launch_bounds__(kBlock) void import_kernel(TableView tv, const uint
   uint32_t row = kEmptyRow;
   int owner = 0;
   if (active && gl == 0) {
-    bool own;
-    row = probe_insert(tv, ids[i], &own);
+    bool own, fresh;
+    row = probe_insert(tv, ids[i], &own, &fresh);
     owner = own ? 1 : 0;
   }
   row = __shfl(row, 0, group);
   owner = __shfl(owner, 0, group);
-  if (!active || !owner) return;
-  float* rec = tv.recs + (int64_t)row * tv.stride;
-  const float* src = vals + i * (int64_t)dim;
-  for (int e = gl; e < elems; e += group) {
-    float v[VEC];
-    vload<VEC>(src + e * VEC, v);
-    vstore<VEC>(rec + e * VEC, v);
+  if (active && owner) {
+    float* rec = tv.recs + (int64_t)row * tv.stride;
+    const float* src = vals + i * (int64_t)dim;
+    for (int e = gl; e < elems; e += group) {
+      float v[VEC];
+      vload<VEC>(src + e * VEC, v);
+      vstore<VEC>(rec + e * VEC, v);
+    }
   }
+  publish_rows(tv, gridDim.x);
 }
 
 // export: rows in insertion order
@@ -217,7 +287,7 @@ __global__ __launch_bounds__(kBlock) void export_kernel(TableView tv, int64_t ro
   }
 }
 
-// re-index every existing row into a fresh (larger) slot array
+// re-index every existing row into a fresh (larger) slot array; launch number 0 = "old row"
 __global__ __launch_bounds__(kBlock) void reindex_kernel(Slot* slots, uint64_t mask,
                                                          const unsigned long long* __restrict__ row_key,
                                                          int64_t rows) {
@@ -226,18 +296,25 @@ __global__ __launch_bounds__(kBlock) void reindex_kernel(Slot* slots, uint64_t m
   const unsigned long long id = row_key[r];
   if (id == kEmptyKey) {
     slots[mask + 1].key = 0ull;
-    slots[mask + 1].row = (uint32_t)r;
+    slots[mask + 1].row_epoch = (unsigned long long)r;
     return;
   }
   uint64_t idx = mix64(id) & mask;
   for (uint64_t n = 0; n <= mask; ++n) {
-    unsigned long long old = atomicCAS(&slots[idx].key, kEmptyKey, id);
+    const unsigned long long old = atomicCAS(&slots[idx].key, kEmptyKey, id);
     if (old == kEmptyKey) {
-      slots[idx].row = (uint32_t)r;
+      slots[idx].row_epoch = (unsigned long long)r;
       return;
     }
     idx = (idx + 1) & mask;
   }
+}
+
+// launch numbers wrapped around: forget them all (every row becomes an "old row")
+__global__ __launch_bounds__(kBlock) void clear_epochs_kernel(Slot* slots, uint64_t count) {
+  const uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= count) return;
+  if (slots[i].key != kEmptyKey) slots[i].row_epoch &= 0xFFFFFFFFull;
 }
 
 // copy records into a slab with a wider stride (new state columns stay zero)
@@ -271,12 +348,16 @@ static int32_t alloc_slots(uint64_t cap, Slot** out, hipStream_t s) {
   return KRK_SUCCESS;
 }
 
-static int32_t grow_rows(krk_sparse* t, int64_t new_cap, int64_t new_stride) {
-  // rows in use must be known exactly before records are moved
+static int32_t refresh_rows(krk_sparse* t) {
   KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
   KRK_HIP(hipStreamSynchronize(t->stream));
-  const int64_t rows = t->host_counters[0];
-  t->size_ub = rows;
+  t->size_ub = t->host_counters[0];
+  return KRK_SUCCESS;
+}
+
+static int32_t grow_rows(krk_sparse* t, int64_t new_cap, int64_t new_stride) {
+  KRK_TRY(refresh_rows(t));   // rows in use must be known exactly before records are moved
+  const int64_t rows = t->size_ub;
   if (new_cap < rows) new_cap = rows;
   if (new_cap >= (int64_t)kEmptyRow) {
     set_error("sparse table cannot hold more than 2^32-2 rows");
@@ -291,20 +372,10 @@ static int32_t grow_rows(krk_sparse* t, int64_t new_cap, int64_t new_stride) {
     (void)hipFree(nrecs);
     return hip_fail(e, "hipMalloc(row_key)", __FILE__, __LINE__);
   }
-  if (new_stride == t->stride) {
-    const size_t used = (size_t)rows * (size_t)t->stride * sizeof(float);
-    if (used) KRK_HIP(hipMemcpyAsync(nrecs, t->recs, used, hipMemcpyDeviceToDevice, t->stream));
-    if (rec_bytes > used)
-      KRK_HIP(hipMemsetAsync(reinterpret_cast<char*>(nrecs) + used, 0, rec_bytes - used, t->stream));
-  } else {
-    KRK_HIP(hipMemsetAsync(nrecs, 0, rec_bytes, t->stream));
-    if (rows) {
-      const int64_t items = rows * t->stride;
-      hipLaunchKernelGGL(restride_kernel, dim3(grid_for(items, kBlock)), dim3(kBlock), 0, t->stream,
-                         t->recs, t->stride, nrecs, new_stride, rows, (int)t->stride);
-      KRK_HIP(hipGetLastError());
-    }
-  }
+  const size_t used = (size_t)rows * (size_t)t->stride * sizeof(float);
+  if (used) KRK_HIP(hipMemcpyAsync(nrecs, t->recs, used, hipMemcpyDeviceToDevice, t->stream));
+  if (rec_bytes > used)
+    KRK_HIP(hipMemsetAsync(reinterpret_cast<char*>(nrecs) + used, 0, rec_bytes - used, t->stream));
   if (rows)
     KRK_HIP(hipMemcpyAsync(nkeys, t->row_key, (size_t)rows * sizeof(unsigned long long),
                            hipMemcpyDeviceToDevice, t->stream));
@@ -314,17 +385,15 @@ static int32_t grow_rows(krk_sparse* t, int64_t new_cap, int64_t new_stride) {
   t->recs = nrecs;
   t->row_key = nkeys;
   t->row_cap = new_cap;
-  t->stride = new_stride;
+  t->layout_version++;
   return KRK_SUCCESS;
 }
 
 static int32_t grow_slots(krk_sparse* t, uint64_t new_cap) {
   Slot* ns = nullptr;
   KRK_TRY(alloc_slots(new_cap, &ns, t->stream));
-  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
-  KRK_HIP(hipStreamSynchronize(t->stream));
-  const int64_t rows = t->host_counters[0];
-  t->size_ub = rows;
+  KRK_TRY(refresh_rows(t));
+  const int64_t rows = t->size_ub;
   if (rows) {
     hipLaunchKernelGGL(reindex_kernel, dim3(grid_for(rows, kBlock)), dim3(kBlock), 0, t->stream, ns,
                        new_cap - 1, t->row_key, rows);
@@ -334,6 +403,7 @@ static int32_t grow_slots(krk_sparse* t, uint64_t new_cap) {
   if (t->slots) (void)hipFree(t->slots);
   t->slots = ns;
   t->slot_cap = new_cap;
+  t->layout_version++;
   return KRK_SUCCESS;
 }
 
@@ -343,14 +413,26 @@ static uint64_t pow2_at_least(uint64_t x) {
   return c;
 }
 
+// Lowers the row bound with the count the device published last: exact as of that launch,
+// plus everything enqueued after it.
+static void tighten_bound(krk_sparse* t) {
+  const unsigned long long pub = __atomic_load_n(t->host_pub, __ATOMIC_ACQUIRE);
+  const uint32_t ep = (uint32_t)(pub >> 32);
+  if (ep == 0 || ep > t->epoch || t->epoch - ep >= 256) return;
+  const int64_t cand = (int64_t)(uint32_t)pub + (int64_t)(t->enq_total - t->enq_at[ep & 255]);
+  if (cand < t->size_ub) t->size_ub = cand;
+}
+
 // Room for `extra_rows` more rows: records, row keys, and an index at most half full.
 int32_t sparse_ensure_room(krk_sparse* t, int64_t extra_rows) {
   int64_t need = t->size_ub + extra_rows;
   if (need > t->row_cap || (uint64_t)need * 2 > t->slot_cap) {
+    tighten_bound(t);
+    need = t->size_ub + extra_rows;
+  }
+  if (need > t->row_cap || (uint64_t)need * 2 > t->slot_cap) {
     // the bound may be stale (async pulls add their whole request to it): refresh it first
-    KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
-    KRK_HIP(hipStreamSynchronize(t->stream));
-    t->size_ub = t->host_counters[0];
+    KRK_TRY(refresh_rows(t));
     need = t->size_ub + extra_rows;
   }
   if (need > t->row_cap) {
@@ -367,14 +449,28 @@ int32_t sparse_ensure_room(krk_sparse* t, int64_t extra_rows) {
   return KRK_SUCCESS;
 }
 
+int32_t sparse_next_epoch(krk_sparse* t, int64_t n) {
+  if (t->epoch >= 0xFFFFFFF0u) {
+    hipLaunchKernelGGL(clear_epochs_kernel, dim3(grid_for((int64_t)t->slot_cap + 1, kBlock)),
+                       dim3(kBlock), 0, t->stream, t->slots, t->slot_cap + 1);
+    KRK_HIP(hipGetLastError());
+    KRK_TRY(refresh_rows(t));   // drains the stream: no launch with an old number is in flight
+    __atomic_store_n(t->host_pub, 0ull, __ATOMIC_RELEASE);
+    t->epoch = 0;
+  }
+  t->epoch += 1;
+  t->enq_total += (uint64_t)n;
+  t->enq_at[t->epoch & 255] = t->enq_total;
+  t->size_ub += n;
+  return KRK_SUCCESS;
+}
+
 // Adds the state columns an optimizer needs; existing records are re-strided once.
 int32_t sparse_ensure_columns(krk_sparse* t, uint32_t mask) {
-  int64_t stride = t->stride;
   bool change = false;
   int32_t col_off[KRK_ST_COUNT];
   memcpy(col_off, t->col_off, sizeof(col_off));
-  int32_t meta_off = t->meta_off;
-  // the step counter, when present, stays the last column: re-place it after new columns
+  // the step counter, when present, stays the last column: it is re-placed after new columns
   int64_t body = t->meta_off >= 0 ? t->meta_off : t->stride;
   for (int st = 1; st < KRK_ST_COUNT; ++st) {
     if ((mask & (1u << st)) && col_off[st] < 0) {
@@ -384,19 +480,16 @@ int32_t sparse_ensure_columns(krk_sparse* t, uint32_t mask) {
     }
   }
   const bool want_meta = (mask & (1u << KRK_ST_STEPS)) || t->meta_off >= 0;
-  if (want_meta && (t->meta_off < 0 || change)) change = true;
+  if (want_meta && t->meta_off < 0) change = true;
   if (!change) return KRK_SUCCESS;
-  meta_off = want_meta ? (int32_t)body : -1;
-  stride = body + (want_meta ? t->meta_floats : 0);
+  const int32_t meta_off = want_meta ? (int32_t)body : -1;
+  const int64_t stride = body + (want_meta ? t->meta_floats : 0);
 
-  // Move records: weight + old state columns keep their offsets; the step counter moves.
   const int64_t old_stride = t->stride;
   const int32_t old_meta = t->meta_off;
   const int64_t old_body = old_meta >= 0 ? old_meta : old_stride;
-  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
-  KRK_HIP(hipStreamSynchronize(t->stream));
-  const int64_t rows = t->host_counters[0];
-  t->size_ub = rows;
+  KRK_TRY(refresh_rows(t));
+  const int64_t rows = t->size_ub;
   float* nrecs = nullptr;
   const size_t rec_bytes = (size_t)t->row_cap * (size_t)stride * sizeof(float);
   KRK_HIP(hipMalloc((void**)&nrecs, rec_bytes ? rec_bytes : 16));
@@ -416,42 +509,43 @@ int32_t sparse_ensure_columns(krk_sparse* t, uint32_t mask) {
   t->stride = stride;
   t->meta_off = meta_off;
   memcpy(t->col_off, col_off, sizeof(col_off));
+  t->layout_version++;
   return KRK_SUCCESS;
 }
 
-void sparse_optim_columns(const krk_sparse* t, const krk_optim& o, int32_t cols[3]) {
-  cols[0] = cols[1] = cols[2] = -1;
+void optim_state_slots(const krk_optim& o, int32_t st[3]) {
+  st[0] = st[1] = st[2] = -1;
   switch (o.type) {
     case KRK_SGD:
-      if (o.has_momentum) cols[0] = t->col_off[KRK_ST_MOMENTUM_BUFFER];
+      if (o.has_momentum) st[0] = KRK_ST_MOMENTUM_BUFFER;
       break;
     case KRK_ADAGRAD:
-      cols[0] = t->col_off[KRK_ST_STATE_SUM];
+      st[0] = KRK_ST_STATE_SUM;
       break;
     case KRK_ADAM:
-      cols[0] = t->col_off[KRK_ST_FIRST_MOMENT];
-      cols[1] = t->col_off[KRK_ST_SECOND_MOMENT];
-      if (o.amsgrad) cols[2] = t->col_off[KRK_ST_SECOND_MOMENT_MAX];
+      st[0] = KRK_ST_FIRST_MOMENT;
+      st[1] = KRK_ST_SECOND_MOMENT;
+      if (o.amsgrad) st[2] = KRK_ST_SECOND_MOMENT_MAX;
       break;
     case KRK_RMSPROP:
-      cols[0] = t->col_off[KRK_ST_SQUARE_AVERAGE];
-      if (o.centered) cols[1] = t->col_off[KRK_ST_G_AVE];
-      if (o.has_momentum) cols[2] = t->col_off[KRK_ST_MOMENTUM_BUFFER];
+      st[0] = KRK_ST_SQUARE_AVERAGE;
+      if (o.centered) st[1] = KRK_ST_G_AVE;
+      if (o.has_momentum) st[2] = KRK_ST_MOMENTUM_BUFFER;
       break;
     default:
       break;
   }
 }
 
-// End of an API call: blocking calls wait, refresh the row count and surface device-side errors.
-int32_t sparse_finish(krk_sparse* t, uint32_t flags) {
-  if (flags & KRK_ASYNC) {
-    t->async_inflight = true;
-    return KRK_SUCCESS;
-  }
-  t->async_inflight = false;
-  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
-  KRK_HIP(hipStreamSynchronize(t->stream));
+void sparse_optim_columns(const krk_sparse* t, const krk_optim& o, int32_t cols[3]) {
+  int32_t st[3];
+  optim_state_slots(o, st);
+  for (int i = 0; i < 3; ++i) cols[i] = st[i] >= 0 ? t->col_off[st[i]] : -1;
+}
+
+// After the stream has drained and counters were copied to host_counters: take the exact row
+// count and turn device-side error bits into a return code.
+int32_t collect_counters(krk_sparse* t) {
   t->size_ub = t->host_counters[0];
   const uint32_t err = t->host_counters[1];
   if (err) {
@@ -465,6 +559,14 @@ int32_t sparse_finish(krk_sparse* t, uint32_t flags) {
     return KRK_SPARSE_ID_NOT_EXIST;
   }
   return KRK_SUCCESS;
+}
+
+// End of an API call: blocking calls wait, refresh the row count and surface device-side errors.
+int32_t sparse_finish(krk_sparse* t, uint32_t flags) {
+  if (flags & KRK_ASYNC) return KRK_SUCCESS;
+  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  return collect_counters(t);
 }
 
 static InitK make_init_k(const krk_init& in, int64_t dim) {
@@ -502,23 +604,23 @@ static void launch_push(krk_sparse* t, const krk_optim& o, const uint64_t* ids, 
   const TableView tv = t->view();
   const int dim = (int)t->dim;
   const bool needs_meta = (optim_state_mask(o) >> KRK_ST_STEPS) & 1u;
-  const int meta = needs_meta ? t->meta_off : -1;
+  PushCols pc{cols[0], cols[1], cols[2], needs_meta ? t->meta_off : -1};
   switch (o.type) {
     case KRK_SGD:
       hipLaunchKernelGGL((push_kernel<KRK_SGD, VEC>), grid, block, 0, t->stream, tv, ids, n, grads, dim,
-                         t->elems, t->group, lr, k, cols[0], cols[1], cols[2], meta);
+                         t->elems, t->group, lr, k, pc);
       break;
     case KRK_ADAGRAD:
       hipLaunchKernelGGL((push_kernel<KRK_ADAGRAD, VEC>), grid, block, 0, t->stream, tv, ids, n, grads,
-                         dim, t->elems, t->group, lr, k, cols[0], cols[1], cols[2], meta);
+                         dim, t->elems, t->group, lr, k, pc);
       break;
     case KRK_ADAM:
       hipLaunchKernelGGL((push_kernel<KRK_ADAM, VEC>), grid, block, 0, t->stream, tv, ids, n, grads, dim,
-                         t->elems, t->group, lr, k, cols[0], cols[1], cols[2], meta);
+                         t->elems, t->group, lr, k, pc);
       break;
     default:
       hipLaunchKernelGGL((push_kernel<KRK_RMSPROP, VEC>), grid, block, 0, t->stream, tv, ids, n, grads,
-                         dim, t->elems, t->group, lr, k, cols[0], cols[1], cols[2], meta);
+                         dim, t->elems, t->group, lr, k, pc);
       break;
   }
 }
@@ -526,6 +628,17 @@ static void launch_push(krk_sparse* t, const krk_optim& o, const uint64_t* ids, 
 }  // namespace krk
 
 using namespace krk;
+
+// Tables of one combined request (CombinePull/PushSparseTable): they share one stream, and a
+// device-resident array of their layouts that is refreshed only when a table has moved.
+struct krk_group : krk::ObjBase {
+  std::vector<krk_sparse*> tables;
+  std::vector<uint64_t> versions;
+  krk::TableDesc* d_descs = nullptr;
+  krk::TableDesc* h_descs = nullptr;   // pinned
+  int64_t dim = 0;
+  int vec = 1, elems = 0, group = 1;
+};
 
 static int32_t check_table(krk_sparse* t) {
   if (!t) {
@@ -538,6 +651,8 @@ static int32_t check_table(krk_sparse* t) {
 static bool valid_optim(const krk_optim* o) {
   return o && o->type >= KRK_ADAGRAD && o->type <= KRK_SGD;
 }
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 extern "C" {
 
@@ -566,10 +681,13 @@ int32_t krk_sparse_create(int64_t dim, const krk_init* init, int64_t capacity_hi
   t->meta_floats = t->vec == 4 ? 4 : 2;
   for (auto& c : t->col_off) c = -1;
   int32_t rc = t->open_stream();
+  t->own_stream = t->stream;
   if (rc == KRK_SUCCESS) {
     hipError_t e = hipMalloc((void**)&t->counters, 16);
     if (e == hipSuccess) e = hipMemsetAsync(t->counters, 0, 16, t->stream);
     if (e == hipSuccess) e = hipHostMalloc((void**)&t->host_counters, 16, hipHostMallocDefault);
+    if (e == hipSuccess) e = hipHostMalloc((void**)&t->host_pub, 8, hipHostMallocCoherent);
+    if (e == hipSuccess) *t->host_pub = 0ull;
     if (e != hipSuccess) rc = hip_fail(e, "krk_sparse_create allocations", __FILE__, __LINE__);
   }
   if (rc == KRK_SUCCESS) {
@@ -586,13 +704,19 @@ int32_t krk_sparse_create(int64_t dim, const krk_init* init, int64_t capacity_hi
 
 int32_t krk_sparse_destroy(krk_sparse* t) {
   if (!t) return KRK_SUCCESS;
+  if (t->member_of) {
+    set_error("destroy the group before its tables");
+    return KRK_E_ARGUMENT;
+  }
   if (t->stream) (void)hipStreamSynchronize(t->stream);
   if (t->slots) (void)hipFree(t->slots);
   if (t->recs) (void)hipFree(t->recs);
   if (t->row_key) (void)hipFree(t->row_key);
   if (t->counters) (void)hipFree(t->counters);
   if (t->host_counters) (void)hipHostFree(t->host_counters);
+  if (t->host_pub) (void)hipHostFree(t->host_pub);
   for (auto& b : t->scratch) b.release();
+  t->stream = t->own_stream;
   t->close_stream();
   delete t;
   return KRK_SUCCESS;
@@ -608,9 +732,7 @@ int32_t krk_sparse_size(krk_sparse* t, int64_t* rows) {
   KRK_TRY(check_table(t));
   if (!rows) return KRK_E_ARGUMENT;
   std::lock_guard<std::mutex> lk(t->mu);
-  KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, t->stream));
-  KRK_HIP(hipStreamSynchronize(t->stream));
-  t->size_ub = t->host_counters[0];
+  KRK_TRY(refresh_rows(t));
   *rows = t->size_ub;
   return KRK_SUCCESS;
 }
@@ -633,6 +755,10 @@ int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* ou
   KRK_TRY(check_table(t));
   KRK_TRY(check_flags(flags));
   if (n < 0 || (n > 0 && (!ids || !out))) return KRK_E_ARGUMENT;
+  if ((flags & KRK_DEVICE_PTRS) && t->vec == 4 && !aligned16(out)) {
+    set_error("device output must be 16-byte aligned");
+    return KRK_E_ARGUMENT;
+  }
   std::lock_guard<std::mutex> lk(t->mu);
   if (n == 0) return sparse_finish(t, flags);
   KRK_TRY(sparse_ensure_room(t, n));
@@ -640,26 +766,17 @@ int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* ou
   float* d_out;
   KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
   KRK_TRY(t->output(out, (size_t)n * t->dim, flags, 1, &d_out));
+  KRK_TRY(sparse_next_epoch(t, n));
   const int per_block = kBlock / t->group;
-  // The kernel must know how many rows existed before it started. After a blocking call the
-  // host knows that exactly; while async work is in flight it does not, so the count is
-  // snapshotted on the device in stream order instead.
-  const uint32_t base_rows = (uint32_t)t->host_counters[0];
-  const uint32_t* base_dev = nullptr;
-  if (t->async_inflight || (flags & KRK_ASYNC)) {
-    hipLaunchKernelGGL(snapshot_rows_kernel, dim3(1), dim3(1), 0, t->stream, t->counters);
-    base_dev = t->counters + 2;
-  }
   const dim3 grid(grid_for(n, per_block)), block(kBlock);
   if (t->vec == 4) {
-    hipLaunchKernelGGL((pull_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
-                       (int)t->dim, t->elems, t->group, base_rows, base_dev, t->initk);
+    hipLaunchKernelGGL((pull_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
+                       (int)t->dim, t->elems, t->group);
   } else {
-    hipLaunchKernelGGL((pull_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
-                       (int)t->dim, t->elems, t->group, base_rows, base_dev, t->initk);
+    hipLaunchKernelGGL((pull_kernel<1>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
+                       (int)t->dim, t->elems, t->group);
   }
   KRK_HIP(hipGetLastError());
-  t->size_ub += n;
   KRK_TRY(t->output_back(out, (size_t)n * t->dim, flags, 1));
   return sparse_finish(t, flags);
 }
@@ -673,6 +790,10 @@ int32_t krk_sparse_push(krk_sparse* t, const krk_optim* o, const uint64_t* ids, 
     return KRK_UNSUPPORTED_OPTIM;
   }
   if (n < 0 || (n > 0 && (!ids || !grads))) return KRK_E_ARGUMENT;
+  if ((flags & KRK_DEVICE_PTRS) && t->vec == 4 && !aligned16(grads)) {
+    set_error("device gradients must be 16-byte aligned");
+    return KRK_E_ARGUMENT;
+  }
   std::lock_guard<std::mutex> lk(t->mu);
   if (n == 0) return sparse_finish(t, flags);
   if (grad_dim != t->dim) {   // ps/optim/adagrad.cc:29-32
@@ -717,6 +838,7 @@ int32_t krk_sparse_import(krk_sparse* t, const uint64_t* ids, int64_t n, const f
   KRK_TRY(check_table(t));
   KRK_TRY(check_flags(flags));
   if (n < 0 || (n > 0 && (!ids || !vals))) return KRK_E_ARGUMENT;
+  if ((flags & KRK_DEVICE_PTRS) && t->vec == 4 && !aligned16(vals)) return KRK_E_ARGUMENT;
   std::lock_guard<std::mutex> lk(t->mu);
   if (n == 0) return sparse_finish(t, flags);
   KRK_TRY(sparse_ensure_room(t, n));
@@ -724,6 +846,7 @@ int32_t krk_sparse_import(krk_sparse* t, const uint64_t* ids, int64_t n, const f
   const float* d_vals;
   KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
   KRK_TRY(t->input(vals, (size_t)n * t->dim, flags, 1, &d_vals));
+  KRK_TRY(sparse_next_epoch(t, n));
   const int per_block = kBlock / t->group;
   const dim3 grid(grid_for(n, per_block)), block(kBlock);
   if (t->vec == 4) {
@@ -734,7 +857,6 @@ int32_t krk_sparse_import(krk_sparse* t, const uint64_t* ids, int64_t n, const f
                        (int)t->dim, t->elems, t->group);
   }
   KRK_HIP(hipGetLastError());
-  t->size_ub += n;
   return sparse_finish(t, flags);
 }
 
@@ -773,6 +895,261 @@ int32_t krk_sparse_export(krk_sparse* t, uint64_t* ids, float* vals, int32_t sta
   if (state) KRK_TRY(t->output_back(state, cells, flags, 2));
   if (steps) KRK_TRY(t->output_back(reinterpret_cast<long long*>(steps), (size_t)rows, flags, 3));
   return sparse_finish(t, 0);
+}
+
+// ---------------------------------------------------------------------------
+// groups of tables: one launch per combined request
+// ---------------------------------------------------------------------------
+int32_t krk_group_create(krk_sparse** tables, int32_t n, krk_group** out) {
+  if (!tables || !out || n <= 0 || n > kMaxGroupTables) {
+    set_error("a group holds 1..%d tables", kMaxGroupTables);
+    return KRK_E_ARGUMENT;
+  }
+  KRK_TRY(ensure_runtime());
+  for (int i = 0; i < n; ++i) {
+    if (!tables[i] || tables[i]->member_of || tables[i]->dim != tables[0]->dim) {
+      set_error("group members must be distinct tables of equal dimension that are in no other group");
+      return KRK_E_ARGUMENT;
+    }
+    for (int j = 0; j < i; ++j)
+      if (tables[j] == tables[i]) return KRK_E_ARGUMENT;
+  }
+  krk_group* g = new (std::nothrow) krk_group();
+  if (!g) return KRK_E_DEVICE;
+  int32_t rc = g->open_stream();
+  if (rc == KRK_SUCCESS) {
+    hipError_t e = hipMalloc((void**)&g->d_descs, sizeof(TableDesc) * kMaxGroupTables);
+    if (e == hipSuccess)
+      e = hipHostMalloc((void**)&g->h_descs, sizeof(TableDesc) * kMaxGroupTables, hipHostMallocDefault);
+    if (e != hipSuccess) rc = hip_fail(e, "krk_group_create", __FILE__, __LINE__);
+  }
+  if (rc != KRK_SUCCESS) {
+    if (g->d_descs) (void)hipFree(g->d_descs);
+    g->close_stream();
+    delete g;
+    return rc;
+  }
+  g->dim = tables[0]->dim;
+  g->vec = tables[0]->vec;
+  g->elems = tables[0]->elems;
+  g->group = tables[0]->group;
+  for (int i = 0; i < n; ++i) {
+    krk_sparse* t = tables[i];
+    std::lock_guard<std::mutex> lk(t->mu);
+    (void)hipStreamSynchronize(t->stream);
+    t->stream = g->stream;   // from now on the table's own calls are ordered with the group's
+    t->member_of = g;
+    g->tables.push_back(t);
+    g->versions.push_back(~0ull);
+  }
+  *out = g;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_group_destroy(krk_group* g) {
+  if (!g) return KRK_SUCCESS;
+  if (g->stream) (void)hipStreamSynchronize(g->stream);
+  for (krk_sparse* t : g->tables) {
+    std::lock_guard<std::mutex> lk(t->mu);
+    t->stream = t->own_stream;
+    t->member_of = nullptr;
+  }
+  if (g->d_descs) (void)hipFree(g->d_descs);
+  if (g->h_descs) (void)hipHostFree(g->h_descs);
+  g->close_stream();
+  delete g;
+  return KRK_SUCCESS;
+}
+
+// Uploads the layouts of tables that moved since the last call.
+static int32_t group_refresh(krk_group* g) {
+  bool dirty = false;
+  for (size_t i = 0; i < g->tables.size(); ++i) {
+    krk_sparse* t = g->tables[i];
+    if (g->versions[i] == t->layout_version) continue;
+    TableDesc& d = g->h_descs[i];
+    d.tv = t->view();
+    d.init = t->initk;
+    memcpy(d.col_off, t->col_off, sizeof(d.col_off));
+    d.meta_off = t->meta_off;
+    g->versions[i] = t->layout_version;
+    dirty = true;
+  }
+  if (dirty) {
+    // in-flight launches read the old array: wait for them before it is overwritten
+    KRK_HIP(hipStreamSynchronize(g->stream));
+    KRK_HIP(hipMemcpyAsync(g->d_descs, g->h_descs, sizeof(TableDesc) * g->tables.size(),
+                           hipMemcpyHostToDevice, g->stream));
+  }
+  return KRK_SUCCESS;
+}
+
+static int32_t group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, int64_t* total) {
+  const int n = (int)g->tables.size();
+  const int per_block = kBlock / g->group;
+  call->n_tables = n;
+  uint64_t blocks = 0;
+  if (offsets[0] != 0) return KRK_E_ARGUMENT;
+  for (int i = 0; i < n; ++i) {
+    const int64_t cnt = offsets[i + 1] - offsets[i];
+    if (cnt < 0) {
+      set_error("offsets must not decrease");
+      return KRK_E_ARGUMENT;
+    }
+    call->block_start[i] = (uint32_t)blocks;
+    call->row_start[i] = offsets[i];
+    blocks += (uint64_t)((cnt + per_block - 1) / per_block);
+  }
+  if (blocks >= 0x7FFFFFFFull) return KRK_E_CAPACITY;
+  call->block_start[n] = (uint32_t)blocks;
+  call->row_start[n] = offsets[n];
+  *total = offsets[n];
+  return KRK_SUCCESS;
+}
+
+struct GroupLock {
+  krk_group* g;
+  explicit GroupLock(krk_group* gg) : g(gg) {
+    g->mu.lock();
+    for (krk_sparse* t : g->tables) t->mu.lock();
+  }
+  ~GroupLock() {
+    for (auto it = g->tables.rbegin(); it != g->tables.rend(); ++it) (*it)->mu.unlock();
+    g->mu.unlock();
+  }
+};
+
+static int32_t group_finish(krk_group* g, uint32_t flags) {
+  if (flags & KRK_ASYNC) return KRK_SUCCESS;
+  // one wait for all members: they share the group's stream
+  for (krk_sparse* t : g->tables)
+    KRK_HIP(hipMemcpyAsync(t->host_counters, t->counters, 16, hipMemcpyDeviceToHost, g->stream));
+  KRK_HIP(hipStreamSynchronize(g->stream));
+  int32_t first = KRK_SUCCESS;
+  for (krk_sparse* t : g->tables) {
+    const int32_t rc = krk::collect_counters(t);
+    if (rc != KRK_SUCCESS && first == KRK_SUCCESS) first = rc;
+  }
+  return first;
+}
+
+int32_t krk_group_sync(krk_group* g) {
+  if (!g) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  GroupLock lk(g);
+  return group_finish(g, 0);
+}
+
+int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets, float* out,
+                       uint32_t flags) {
+  if (!g || !offsets) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  KRK_TRY(check_flags(flags));
+  GroupLock lk(g);
+  GroupCall call;
+  int64_t total = 0;
+  KRK_TRY(group_plan(g, offsets, &call, &total));
+  if (total == 0) return group_finish(g, flags);
+  if (!ids || !out) return KRK_E_ARGUMENT;
+  if ((flags & KRK_DEVICE_PTRS) && g->vec == 4 && !aligned16(out)) return KRK_E_ARGUMENT;
+  for (size_t i = 0; i < g->tables.size(); ++i) {
+    krk_sparse* t = g->tables[i];
+    const int64_t cnt = offsets[i + 1] - offsets[i];
+    if (cnt == 0) {
+      call.epoch[i] = t->epoch;
+      continue;
+    }
+    KRK_TRY(sparse_ensure_room(t, cnt));
+    KRK_TRY(sparse_next_epoch(t, cnt));
+    call.epoch[i] = t->epoch;
+  }
+  KRK_TRY(group_refresh(g));
+  const uint64_t* d_ids;
+  float* d_out;
+  KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
+  KRK_TRY(g->output(out, (size_t)total * g->dim, flags, 1, &d_out));
+  const dim3 grid(call.block_start[call.n_tables]), block(kBlock);
+  if (g->vec == 4) {
+    hipLaunchKernelGGL((group_pull_kernel<4>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
+                       (int)g->dim, g->elems, g->group);
+  } else {
+    hipLaunchKernelGGL((group_pull_kernel<1>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
+                       (int)g->dim, g->elems, g->group);
+  }
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(g->output_back(out, (size_t)total * g->dim, flags, 1));
+  return group_finish(g, flags);
+}
+
+}  // extern "C"
+
+template <int VEC>
+static void launch_group_push(krk_group* g, const krk_optim& o, const GroupCall& call,
+                              const uint64_t* ids, const float* grads, float lr) {
+  const OptimK k = make_optim_k(o);
+  int32_t st[3];
+  optim_state_slots(o, st);
+  const int use_meta = (optim_state_mask(o) >> KRK_ST_STEPS) & 1u;
+  const dim3 grid(call.block_start[call.n_tables]), block(kBlock);
+  const int dim = (int)g->dim;
+  switch (o.type) {
+    case KRK_SGD:
+      hipLaunchKernelGGL((group_push_kernel<KRK_SGD, VEC>), grid, block, 0, g->stream, g->d_descs, call,
+                         ids, grads, dim, g->elems, g->group, lr, k, st[0], st[1], st[2], use_meta);
+      break;
+    case KRK_ADAGRAD:
+      hipLaunchKernelGGL((group_push_kernel<KRK_ADAGRAD, VEC>), grid, block, 0, g->stream, g->d_descs,
+                         call, ids, grads, dim, g->elems, g->group, lr, k, st[0], st[1], st[2], use_meta);
+      break;
+    case KRK_ADAM:
+      hipLaunchKernelGGL((group_push_kernel<KRK_ADAM, VEC>), grid, block, 0, g->stream, g->d_descs, call,
+                         ids, grads, dim, g->elems, g->group, lr, k, st[0], st[1], st[2], use_meta);
+      break;
+    default:
+      hipLaunchKernelGGL((group_push_kernel<KRK_RMSPROP, VEC>), grid, block, 0, g->stream, g->d_descs,
+                         call, ids, grads, dim, g->elems, g->group, lr, k, st[0], st[1], st[2], use_meta);
+      break;
+  }
+}
+
+extern "C" {
+
+int32_t krk_group_push(krk_group* g, const krk_optim* o, const uint64_t* ids, const int64_t* offsets,
+                       const float* grads, int64_t grad_dim, float lr, uint32_t flags) {
+  if (!g || !offsets) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  KRK_TRY(check_flags(flags));
+  if (!valid_optim(o)) {
+    set_error("optimizer type is not supported");
+    return KRK_UNSUPPORTED_OPTIM;
+  }
+  GroupLock lk(g);
+  GroupCall call;
+  int64_t total = 0;
+  KRK_TRY(group_plan(g, offsets, &call, &total));
+  if (total == 0) return group_finish(g, flags);
+  if (!ids || !grads) return KRK_E_ARGUMENT;
+  if ((flags & KRK_DEVICE_PTRS) && g->vec == 4 && !aligned16(grads)) return KRK_E_ARGUMENT;
+  if (grad_dim != g->dim) {
+    set_error("gradient width %lld does not match table dimension %lld", (long long)grad_dim,
+              (long long)g->dim);
+    return KRK_GRADIENT_UNCOMPATIBLE;
+  }
+  const uint32_t mask = optim_state_mask(*o);
+  for (krk_sparse* t : g->tables) KRK_TRY(sparse_ensure_columns(t, mask));
+  KRK_TRY(group_refresh(g));
+  const uint64_t* d_ids;
+  const float* d_g;
+  KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
+  KRK_TRY(g->input(grads, (size_t)total * g->dim, flags, 1, &d_g));
+  for (int i = 0; i < call.n_tables; ++i) call.epoch[i] = 0;
+  if (g->vec == 4) {
+    launch_group_push<4>(g, *o, call, d_ids, d_g, lr);
+  } else {
+    launch_group_push<1>(g, *o, call, d_ids, d_g, lr);
+  }
+  KRK_HIP(hipGetLastError());
+  return group_finish(g, flags);
 }
 
 }  // extern "C"
