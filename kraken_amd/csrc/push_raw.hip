@@ -116,9 +116,11 @@ __global__ __launch_bounds__(kBlock) void rows_of_ids_kernel(TableView tv, const
                                                              int64_t n, uint32_t miss_key,
                                                              uint32_t* __restrict__ keys,
                                                              uint32_t* __restrict__ pos) {
-  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (p >= n) return;
-  uint32_t r = probe_find(tv, ids[p]);
+  const int64_t p = (int64_t)blockIdx.x * (kBlock / kBucket) + threadIdx.x / kBucket;
+  const int gl = threadIdx.x & (kBucket - 1);
+  const bool active = p < n;
+  uint32_t r = probe_find(tv, active ? ids[p] : 0, active, gl, kBucket);
+  if (!active || gl != 0) return;
   if (r == kEmptyRow) {
     atomicOr(&tv.counters[1], kErrMissingId);
     r = miss_key;
@@ -429,8 +431,8 @@ int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* i
   uint32_t* spos = skeys + n;
 
   const TableView tv = t->view();
-  hipLaunchKernelGGL(rows_of_ids_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, t->stream, tv, d_ids,
-                     n, miss_key, keys, pos);
+  hipLaunchKernelGGL(rows_of_ids_kernel, dim3(grid_for(n, kBlock / kBucket)), dim3(kBlock), 0, t->stream,
+                     tv, d_ids, n, miss_key, keys, pos);
   KRK_HIP(hipGetLastError());
   KRK_HIP(rocprim::radix_sort_pairs(t->scratch[1].ptr, sort_bytes, keys, skeys, pos, spos, (size_t)n, 0,
                                     bits, t->stream));

@@ -1,7 +1,8 @@
 // Device-side layout of a sparse table and the probe routines shared by its kernels.
 //
 // HBM layout (one table):
-//   slots   [slot_cap + 1] x 16 B   open-addressing index, linear probing, load <= 1/2:
+//   slots   [slot_cap + 1] x 16 B   open-addressing index, buckets of 4 slots (one 64 B sector),
+//                                   linear probing over buckets, load <= 1/2:
 //                                   {u64 key, u32 row, u32 epoch}. All-ones key = empty; the
 //                                   extra last slot belongs to the one id whose value is all-ones.
 //                                   epoch = number of the launch that created the row.
@@ -10,10 +11,11 @@
 //                                   so a push touches one contiguous record instead of one line
 //                                   per state array.
 //   row_key [row_cap] x 8 B         id of each row (export and re-indexing walk rows, not slots)
-//   counters[4] x 4 B               {rows used, error bits, -, workgroups finished}
-//   host_pub   8 B, pinned host     {rows used, launch number} of the last finished launch that
-//                                   could insert, written by the device so that the host can
-//                                   bound the row count without waiting for the stream
+//   counters[4] x 4 B               {rows used, error bits, -, -}
+//   host_pub   8 B, pinned host     {rows used, launch number}: written by a one-wave kernel that
+//                                   the host enqueues behind an inserting launch when the table
+//                                   is close to full, so that it can bound the row count later
+//                                   without waiting for the stream
 #pragma once
 
 #include <vector>
@@ -40,110 +42,200 @@ struct TableView {
   uint32_t* counters;   // [0] rows used, [1] error bits
   uint32_t row_cap;
   uint32_t epoch;       // number of this launch, for launches that may insert
-  unsigned long long* host_pub;   // pinned host memory, see publish_rows
 };
 
-__device__ __forceinline__ void load_slot(const Slot* s, unsigned long long& key,
-                                          unsigned long long& row_epoch) {
-  const uint4 raw = *reinterpret_cast<const uint4*>(s);
+constexpr int kBucket = 4;   // slots per bucket: one aligned 64-byte sector
+
+__device__ __forceinline__ void unpack_slot(const uint4& raw, unsigned long long& key,
+                                            unsigned long long& row_epoch) {
   key = (unsigned long long)raw.x | ((unsigned long long)raw.y << 32);
   row_epoch = (unsigned long long)raw.z | ((unsigned long long)raw.w << 32);
 }
 
-// id -> row, or kEmptyRow.
-__device__ inline uint32_t probe_find(const TableView& tv, uint64_t id) {
-  unsigned long long key, re;
-  if (id == kEmptyKey) {
-    load_slot(&tv.slots[tv.mask + 1], key, re);
-    return key != kEmptyKey ? (uint32_t)re : kEmptyRow;
-  }
-  uint64_t idx = mix64(id) & tv.mask;
-  for (uint64_t n = 0; n <= tv.mask; ++n) {
-    load_slot(&tv.slots[idx], key, re);
-    if (key == id) return (uint32_t)re;
-    if (key == kEmptyKey) return kEmptyRow;
-    idx = (idx + 1) & tv.mask;
-  }
-  return kEmptyRow;
-}
+// Probing is done by the lane group that owns the id (at least four lanes, all holding the same
+// id). The index is read a bucket at a time: the group's first four lanes load one slot each,
+// which the hardware serves as a single 64-byte request, and two wave ballots tell every lane
+// of the group whether the id or an empty slot was seen. Buckets are tried in linear order
+// from the id's home bucket; a bucket fills from slot 0 upwards and slots are never released,
+// so the first empty slot ends a search. What bounds a launch is the longest chain among its
+// ids; chains are counted in buckets here, a quarter of what slot-by-slot probing walks.
+//
+// Every lane of the wavefront must call these functions together (they use wave-wide ballots
+// and shuffles); lanes without work pass active = false.
 
-// id -> row, claiming a slot and the next free row when absent. *owner is set for the one
-// caller that created the row; *fresh for every caller whose row was created by this launch
-// (its record may not be written yet, so its value must be recomputed, not read). A caller that
-// meets a slot whose creator has not published the row number yet gets kEmptyRow and fresh.
-__device__ inline uint32_t probe_insert(const TableView& tv, uint64_t id, bool* owner, bool* fresh) {
-  *owner = false;
-  *fresh = false;
-  Slot* slot = nullptr;
-  if (id == kEmptyKey) {
-    slot = &tv.slots[tv.mask + 1];
-    const unsigned long long old = atomicCAS(&slot->key, kEmptyKey, 0ull);
-    if (old != kEmptyKey) {
-      const unsigned long long re = __atomic_load_n(&slot->row_epoch, __ATOMIC_RELAXED);
-      *fresh = (uint32_t)re == kEmptyRow || (uint32_t)(re >> 32) == tv.epoch;
-      return (uint32_t)re;
-    }
-  } else {
-    uint64_t idx = mix64(id) & tv.mask;
-    for (uint64_t n = 0; n <= tv.mask; ++n) {
-      unsigned long long key, re;
-      load_slot(&tv.slots[idx], key, re);
-      bool raced = false;
-      if (key == kEmptyKey) {
-        const unsigned long long old = atomicCAS(&tv.slots[idx].key, kEmptyKey, (unsigned long long)id);
-        if (old == kEmptyKey) {
-          slot = &tv.slots[idx];
-          break;
-        }
-        key = old;
-        raced = true;
-      }
-      if (key == id) {
-        // the 16-byte load above may have straddled the creator's update: read the word again
-        if (raced || (uint32_t)re == kEmptyRow)
-          re = __atomic_load_n(&tv.slots[idx].row_epoch, __ATOMIC_RELAXED);
-        *fresh = (uint32_t)re == kEmptyRow || (uint32_t)(re >> 32) == tv.epoch;
-        return (uint32_t)re;
-      }
-      idx = (idx + 1) & tv.mask;
-    }
-    if (!slot) {
-      atomicOr(&tv.counters[1], kErrOverflow);
-      return kEmptyRow;
-    }
+struct ProbeResult {
+  uint32_t row;   // kEmptyRow when absent (find) or when the creator has not published it yet
+  bool owner;     // this group created the row
+  bool fresh;     // the row was created by this launch: recompute its value, do not read it
+};
+
+__device__ __forceinline__ int wave_lane() { return (int)(threadIdx.x & (kWave - 1)); }
+
+// id -> row for every lane of the group, kEmptyRow when absent.
+__device__ inline uint32_t probe_find(const TableView& tv, uint64_t id, bool active, int gl, int group) {
+  const int lane = wave_lane();
+  const int base = lane & ~(group - 1);
+  const uint64_t nb_mask = tv.mask >> 2;
+  uint32_t row = kEmptyRow;
+  bool done = !active;
+  if (active && id == kEmptyKey) {   // the id that equals the empty marker has a slot of its own
+    unsigned long long key, re;
+    unpack_slot(*reinterpret_cast<const uint4*>(&tv.slots[tv.mask + 1]), key, re);
+    row = key != kEmptyKey ? (uint32_t)re : kEmptyRow;
+    done = true;
   }
-  const uint32_t row = atomicAdd(&tv.counters[0], 1u);
-  if (row >= tv.row_cap) {
-    atomicOr(&tv.counters[1], kErrOverflow);
-    return kEmptyRow;
+  uint64_t b = mix64(id) & nb_mask;
+  uint64_t tried = 0;
+  for (;;) {
+    const bool part = !done && gl < kBucket;
+    unsigned long long key = 0, re = 0;
+    if (part) unpack_slot(*reinterpret_cast<const uint4*>(&tv.slots[b * kBucket + gl]), key, re);
+    const unsigned long long m_match = __ballot(part && key == id);
+    const unsigned long long m_empty = __ballot(part && key == kEmptyKey);
+    int src = lane;
+    int action = 0;   // 1 hit, 2 miss, 3 next bucket
+    if (!done) {
+      const uint32_t mm = (uint32_t)(m_match >> base) & 0xFu;
+      const uint32_t me = (uint32_t)(m_empty >> base) & 0xFu;
+      if (mm) {
+        action = 1;
+        src = base + __ffs(mm) - 1;
+      } else {
+        action = me ? 2 : 3;
+      }
+    }
+    const uint32_t r = __shfl((uint32_t)re, src);
+    if (action == 1) {
+      row = r;
+      done = true;
+    } else if (action == 2) {
+      done = true;
+    } else if (action == 3) {
+      b = (b + 1) & nb_mask;
+      if (++tried > nb_mask) done = true;
+    }
+    if (__ballot(!done) == 0ull) break;
   }
-  __atomic_store_n(&slot->row_epoch, (unsigned long long)row | ((unsigned long long)tv.epoch << 32),
-                   __ATOMIC_RELAXED);
-  tv.row_key[row] = id;
-  *owner = true;
-  *fresh = true;
   return row;
 }
 
-// Called by every thread of every workgroup of a launch that may insert, after its inserts.
-// The workgroup that finishes last publishes {rows used, launch number} to pinned host memory:
-// the host then knows the exact row count as of that launch without synchronising, and bounds
-// the current count by adding the sizes of the requests enqueued since.
-__device__ __forceinline__ void publish_rows(const TableView& tv, uint32_t workgroups) {
-  // Every insert of this workgroup took its row number from a returning atomic on counters[0],
-  // so those atomics have been performed once the barrier is passed; the counter of finished
-  // workgroups is bumped with another atomic at the same place. No fence is needed, and none is
-  // wanted: a release fence would write back the whole L2 once per workgroup.
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const uint32_t done = atomicAdd(&tv.counters[3], 1u) + 1u;
-    if (done == workgroups) {
-      atomicExch(&tv.counters[3], 0u);
-      const uint32_t rows = atomicAdd(&tv.counters[0], 0u);
-      __hip_atomic_store(tv.host_pub, (unsigned long long)rows | ((unsigned long long)tv.epoch << 32),
-                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+// id -> row, claiming a slot and the next free row when absent.
+__device__ inline ProbeResult probe_insert(const TableView& tv, uint64_t id, bool active, int gl,
+                                           int group) {
+  const int lane = wave_lane();
+  const int base = lane & ~(group - 1);
+  const uint64_t nb_mask = tv.mask >> 2;
+  ProbeResult res;
+  res.row = kEmptyRow;
+  res.owner = false;
+  res.fresh = false;
+  bool done = !active;
+  const bool special = active && id == kEmptyKey;
+  if (special) {
+    // handled by the group's first lane alone, shared with the others after the loop
+    if (gl == 0) {
+      Slot* slot = &tv.slots[tv.mask + 1];
+      const unsigned long long old = atomicCAS(&slot->key, kEmptyKey, 0ull);
+      if (old != kEmptyKey) {
+        const unsigned long long re = __atomic_load_n(&slot->row_epoch, __ATOMIC_RELAXED);
+        res.row = (uint32_t)re;
+        res.fresh = res.row == kEmptyRow || (uint32_t)(re >> 32) == tv.epoch;
+      } else {
+        const uint32_t row = atomicAdd(&tv.counters[0], 1u);
+        if (row < tv.row_cap) {
+          __atomic_store_n(&slot->row_epoch, (unsigned long long)row | ((unsigned long long)tv.epoch << 32),
+                           __ATOMIC_RELAXED);
+          tv.row_key[row] = id;
+          res.row = row;
+          res.owner = true;
+        } else {
+          atomicOr(&tv.counters[1], kErrOverflow);
+        }
+        res.fresh = true;
+      }
+    }
+    done = true;
+  }
+  uint64_t b = mix64(id) & nb_mask;
+  uint64_t tried = 0;
+  for (;;) {
+    const bool part = !done && gl < kBucket;
+    unsigned long long key = 0, re = 0;
+    Slot* mine = &tv.slots[b * kBucket + (gl < kBucket ? gl : 0)];
+    if (part) unpack_slot(*reinterpret_cast<const uint4*>(mine), key, re);
+    const unsigned long long m_match = __ballot(part && key == id);
+    const unsigned long long m_empty = __ballot(part && key == kEmptyKey);
+    int src = lane;
+    int action = 0;   // 1 hit, 2 try to claim the first empty slot, 3 next bucket
+    if (!done) {
+      const uint32_t mm = (uint32_t)(m_match >> base) & 0xFu;
+      const uint32_t me = (uint32_t)(m_empty >> base) & 0xFu;
+      if (mm) {
+        action = 1;
+        src = base + __ffs(mm) - 1;
+      } else if (me) {
+        action = 2;
+        src = base + __ffs(me) - 1;
+      } else {
+        action = 3;
+      }
+    }
+    unsigned long long cas_old = 0;
+    uint32_t new_row = kEmptyRow;
+    if (action == 2 && lane == src) {
+      cas_old = atomicCAS(&mine->key, kEmptyKey, (unsigned long long)id);
+      if (cas_old == kEmptyKey) {
+        const uint32_t row = atomicAdd(&tv.counters[0], 1u);
+        if (row < tv.row_cap) {
+          __atomic_store_n(&mine->row_epoch, (unsigned long long)row | ((unsigned long long)tv.epoch << 32),
+                           __ATOMIC_RELAXED);
+          tv.row_key[row] = id;
+          new_row = row;
+        } else {
+          atomicOr(&tv.counters[1], kErrOverflow);
+        }
+      } else if (cas_old == id) {
+        re = __atomic_load_n(&mine->row_epoch, __ATOMIC_RELAXED);
+      }
+    } else if (action == 1 && lane == src && (uint32_t)re == kEmptyRow) {
+      // the 16-byte load may have caught the creator between its two stores: read the word again
+      re = __atomic_load_n(&mine->row_epoch, __ATOMIC_RELAXED);
+    }
+    const unsigned long long re_b = __shfl(re, src);
+    const unsigned long long old_b = __shfl(cas_old, src);
+    const uint32_t new_b = __shfl(new_row, src);
+    if (action == 1 || (action == 2 && old_b == id)) {
+      res.row = (uint32_t)re_b;
+      res.fresh = res.row == kEmptyRow || (uint32_t)(re_b >> 32) == tv.epoch;
+      done = true;
+    } else if (action == 2 && old_b == kEmptyKey) {
+      res.row = new_b;
+      res.owner = new_b != kEmptyRow;
+      res.fresh = true;
+      done = true;
+    } else if (action == 3) {
+      b = (b + 1) & nb_mask;
+      if (++tried > nb_mask) {
+        atomicOr(&tv.counters[1], kErrOverflow);
+        res.fresh = true;
+        done = true;
+      }
+    }
+    // action 2 with another id in the slot: somebody else took it, look at the same bucket again
+    if (__ballot(!done) == 0ull) break;
+  }
+  if (group > 1) {
+    // the special id was resolved by the first lane only
+    const uint32_t row0 = __shfl(res.row, base);
+    const int own0 = __shfl((int)res.owner, base);
+    const int fresh0 = __shfl((int)res.fresh, base);
+    if (special) {
+      res.row = row0;
+      res.owner = own0 != 0;
+      res.fresh = fresh0 != 0;
     }
   }
+  return res;
 }
 
 }  // namespace krk
@@ -168,7 +260,8 @@ struct krk_sparse : krk::ObjBase {
   uint32_t* counters = nullptr;       // device
   uint32_t* host_counters = nullptr;  // pinned
   int64_t size_ub = 0;                // upper bound of rows used, exact after a blocking call
-  unsigned long long* host_pub = nullptr;   // pinned, written by the device (publish_rows)
+  unsigned long long* host_pub = nullptr;   // pinned, written by the device (publish_kernel)
+  int64_t last_request = 0;           // size of the last inserting request
   uint64_t enq_total = 0;             // ids handed to inserting launches so far
   uint64_t enq_at[256] = {};          // enq_total right after the launch with number e (mod 256)
   uint32_t epoch = 0;                 // number of the last launch that could insert
@@ -193,7 +286,6 @@ struct krk_sparse : krk::ObjBase {
     tv.counters = counters;
     tv.row_cap = (uint32_t)row_cap;
     tv.epoch = epoch;
-    tv.host_pub = host_pub;
     return tv;
   }
 };
@@ -205,6 +297,10 @@ int32_t sparse_ensure_columns(krk_sparse* t, uint32_t state_mask);
 int32_t sparse_finish(krk_sparse* t, uint32_t flags);
 // A new launch number for a launch that may insert up to n rows into t; call right before it.
 int32_t sparse_next_epoch(krk_sparse* t, int64_t n);
+// True when only a few more requests like the last one fit under the current row bound.
+bool sparse_near_full(const krk_sparse* t);
+// Enqueues the kernel that publishes {rows used, launch number} of each table to the host.
+int32_t sparse_publish(krk_sparse* const* tables, int n, hipStream_t stream);
 // Column offsets an optimizer's three state slots map to (-1 = unused).
 void sparse_optim_columns(const krk_sparse* t, const krk_optim& o, int32_t cols[3]);
 // The three state types an optimizer's slots s0/s1/s2 hold (-1 = unused).

@@ -10,6 +10,7 @@
 // lane walks the index (one 16-byte slot load per probe), the row number is broadcast with a
 // wave shuffle, then every lane moves `vec` floats of the record per step, so a dim-16 row is
 // four float4 lanes and sixteen rows share one wavefront instruction.
+#include <algorithm>
 #include <cmath>
 #include <new>
 
@@ -48,18 +49,11 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
                                           int gl, float* __restrict__ out, int dim, int elems,
                                           int group) {
   const uint64_t id = active ? ids[i] : 0;
-  uint32_t row = kEmptyRow;
-  int flags = 0;   // bit 0: this group created the row, bit 1: the row was created by this launch
-  if (active && gl == 0) {
-    bool own, fresh;
-    row = probe_insert(tv, id, &own, &fresh);
-    flags = (own ? 1 : 0) | (fresh ? 2 : 0);
-  }
-  row = __shfl(row, 0, group);
-  flags = __shfl(flags, 0, group);
-  if (!active) return;   // callers publish after this returns; nothing below synchronises
-  const bool owner = flags & 1;
-  const bool fresh = flags & 2;
+  const ProbeResult pr = probe_insert(tv, id, active, gl, group);
+  if (!active) return;
+  const uint32_t row = pr.row;
+  const bool owner = pr.owner;
+  const bool fresh = pr.fresh;
   float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
   float* dst = out + i * (int64_t)dim;
   for (int e = gl; e < elems; e += group) {
@@ -89,13 +83,12 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
                                           int64_t i, bool active, int gl,
                                           const float* __restrict__ grads, int dim, int elems,
                                           int group, float lr, const OptimK& k, const PushCols& pc) {
-  uint32_t row = kEmptyRow;
-  if (active && gl == 0) {
-    row = probe_find(tv, ids[i]);
-    if (row == kEmptyRow) atomicOr(&tv.counters[1], kErrMissingId);
+  const uint32_t row = probe_find(tv, active ? ids[i] : 0, active, gl, group);
+  if (!active) return;
+  if (row == kEmptyRow) {
+    if (gl == 0) atomicOr(&tv.counters[1], kErrMissingId);
+    return;
   }
-  row = __shfl(row, 0, group);
-  if (!active || row == kEmptyRow) return;
   float* rec = tv.recs + (int64_t)row * tv.stride;
   const float* g = grads + i * (int64_t)dim;
 
@@ -148,7 +141,6 @@ __global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, InitK init,
   const int per_block = kBlock / group;
   const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
   pull_body<VEC>(tv, init, ids, i, i < n, threadIdx.x & (group - 1), out, dim, elems, group);
-  publish_rows(tv, gridDim.x);
 }
 
 template <int OPT, int VEC>
@@ -199,7 +191,6 @@ __global__ __launch_bounds__(kBlock) void group_pull_kernel(const TableDesc* __r
   const int64_t i = call.row_start[t] + local;
   pull_body<VEC>(tv, init, ids, i, i < call.row_start[t + 1], threadIdx.x & (group - 1), out, dim,
                  elems, group);
-  publish_rows(tv, call.block_start[t + 1] - call.block_start[t]);
 }
 
 template <int OPT, int VEC>
@@ -225,10 +216,11 @@ __global__ __launch_bounds__(kBlock) void group_push_kernel(const TableDesc* __r
 
 __global__ __launch_bounds__(kBlock) void lookup_kernel(TableView tv, const uint64_t* __restrict__ ids,
                                                         int64_t n, int32_t* __restrict__ rows) {
-  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i >= n) return;
-  const uint32_t r = probe_find(tv, ids[i]);
-  rows[i] = r == kEmptyRow ? -1 : (int32_t)r;
+  const int64_t i = (int64_t)blockIdx.x * (kBlock / kBucket) + threadIdx.x / kBucket;
+  const int gl = threadIdx.x & (kBucket - 1);
+  const bool active = i < n;
+  const uint32_t r = probe_find(tv, active ? ids[i] : 0, active, gl, kBucket);
+  if (active && gl == 0) rows[i] = r == kEmptyRow ? -1 : (int32_t)r;
 }
 
 // import: like pull, but a new row takes its values from the caller
@@ -240,15 +232,9 @@ __global__ __launch_bounds__(kBlock) void import_kernel(TableView tv, const uint
   const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
   const int gl = threadIdx.x & (group - 1);
   const bool active = i < n;
-  uint32_t row = kEmptyRow;
-  int owner = 0;
-  if (active && gl == 0) {
-    bool own, fresh;
-    row = probe_insert(tv, ids[i], &own, &fresh);
-    owner = own ? 1 : 0;
-  }
-  row = __shfl(row, 0, group);
-  owner = __shfl(owner, 0, group);
+  const ProbeResult pr = probe_insert(tv, active ? ids[i] : 0, active, gl, group);
+  const uint32_t row = pr.row;
+  const bool owner = pr.owner;
   if (active && owner) {
     float* rec = tv.recs + (int64_t)row * tv.stride;
     const float* src = vals + i * (int64_t)dim;
@@ -258,7 +244,23 @@ __global__ __launch_bounds__(kBlock) void import_kernel(TableView tv, const uint
       vstore<VEC>(rec + e * VEC, v);
     }
   }
-  publish_rows(tv, gridDim.x);
+}
+
+// {rows used, launch number} of up to 32 tables -> pinned host memory. Runs behind the launch
+// whose number it carries, so the count is exact as of that launch. The store is a relaxed
+// system-scope atomic: only the value itself has to arrive, nothing is ordered behind it.
+struct PublishArgs {
+  int32_t n;
+  uint32_t epoch[kMaxGroupTables];
+  const uint32_t* counters[kMaxGroupTables];
+  unsigned long long* host_pub[kMaxGroupTables];
+};
+__global__ void publish_kernel(PublishArgs a) {
+  const int i = threadIdx.x;
+  if (i >= a.n) return;
+  const uint32_t rows = a.counters[i][0];
+  __hip_atomic_store(a.host_pub[i], (unsigned long long)rows | ((unsigned long long)a.epoch[i] << 32),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // export: rows in insertion order
@@ -299,14 +301,18 @@ __global__ __launch_bounds__(kBlock) void reindex_kernel(Slot* slots, uint64_t m
     slots[mask + 1].row_epoch = (unsigned long long)r;
     return;
   }
-  uint64_t idx = mix64(id) & mask;
-  for (uint64_t n = 0; n <= mask; ++n) {
-    const unsigned long long old = atomicCAS(&slots[idx].key, kEmptyKey, id);
-    if (old == kEmptyKey) {
-      slots[idx].row_epoch = (unsigned long long)r;
-      return;
+  const uint64_t nb_mask = mask >> 2;
+  uint64_t b = mix64(id) & nb_mask;
+  for (uint64_t n = 0; n <= nb_mask; ++n) {
+    for (int s = 0; s < kBucket; ++s) {
+      Slot* slot = &slots[b * kBucket + s];
+      const unsigned long long old = atomicCAS(&slot->key, kEmptyKey, id);
+      if (old == kEmptyKey) {
+        slot->row_epoch = (unsigned long long)r;
+        return;
+      }
     }
-    idx = (idx + 1) & mask;
+    b = (b + 1) & nb_mask;
   }
 }
 
@@ -462,6 +468,25 @@ int32_t sparse_next_epoch(krk_sparse* t, int64_t n) {
   t->enq_total += (uint64_t)n;
   t->enq_at[t->epoch & 255] = t->enq_total;
   t->size_ub += n;
+  t->last_request = n;
+  return KRK_SUCCESS;
+}
+
+bool sparse_near_full(const krk_sparse* t) {
+  const int64_t room = std::min<int64_t>(t->row_cap, (int64_t)(t->slot_cap / 2)) - t->size_ub;
+  return room < 4 * t->last_request;
+}
+
+int32_t sparse_publish(krk_sparse* const* tables, int n, hipStream_t stream) {
+  PublishArgs a;
+  a.n = n;
+  for (int i = 0; i < n; ++i) {
+    a.epoch[i] = tables[i]->epoch;
+    a.counters[i] = tables[i]->counters;
+    a.host_pub[i] = tables[i]->host_pub;
+  }
+  hipLaunchKernelGGL(publish_kernel, dim3(1), dim3(64), 0, stream, a);
+  KRK_HIP(hipGetLastError());
   return KRK_SUCCESS;
 }
 
@@ -672,7 +697,7 @@ int32_t krk_sparse_create(int64_t dim, const krk_init* init, int64_t capacity_hi
   t->dim = dim;
   t->vec = (dim % 4 == 0) ? 4 : 1;
   t->elems = (int)(dim / t->vec);
-  int g = 1;
+  int g = kBucket;   // at least the four lanes that read an index bucket together
   while (g < t->elems && g < kWave) g <<= 1;
   t->group = g;
   t->init = *init;
@@ -777,6 +802,7 @@ int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* ou
                        (int)t->dim, t->elems, t->group);
   }
   KRK_HIP(hipGetLastError());
+  if ((flags & KRK_ASYNC) && sparse_near_full(t)) KRK_TRY(sparse_publish(&t, 1, t->stream));
   KRK_TRY(t->output_back(out, (size_t)n * t->dim, flags, 1));
   return sparse_finish(t, flags);
 }
@@ -826,8 +852,8 @@ int32_t krk_sparse_lookup(krk_sparse* t, const uint64_t* ids, int64_t n, int32_t
   int32_t* d_rows;
   KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
   KRK_TRY(t->output(rows, (size_t)n, flags, 1, &d_rows));
-  hipLaunchKernelGGL(lookup_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, t->stream, t->view(),
-                     d_ids, n, d_rows);
+  hipLaunchKernelGGL(lookup_kernel, dim3(grid_for(n, kBlock / kBucket)), dim3(kBlock), 0, t->stream,
+                     t->view(), d_ids, n, d_rows);
   KRK_HIP(hipGetLastError());
   KRK_TRY(t->output_back(rows, (size_t)n, flags, 1));
   return sparse_finish(t, flags);
@@ -857,6 +883,7 @@ int32_t krk_sparse_import(krk_sparse* t, const uint64_t* ids, int64_t n, const f
                        (int)t->dim, t->elems, t->group);
   }
   KRK_HIP(hipGetLastError());
+  if ((flags & KRK_ASYNC) && sparse_near_full(t)) KRK_TRY(sparse_publish(&t, 1, t->stream));
   return sparse_finish(t, flags);
 }
 
@@ -1077,6 +1104,11 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
                        (int)g->dim, g->elems, g->group);
   }
   KRK_HIP(hipGetLastError());
+  if (flags & KRK_ASYNC) {
+    bool any = false;
+    for (krk_sparse* t : g->tables) any = any || sparse_near_full(t);
+    if (any) KRK_TRY(sparse_publish(g->tables.data(), (int)g->tables.size(), g->stream));
+  }
   KRK_TRY(g->output_back(out, (size_t)total * g->dim, flags, 1));
   return group_finish(g, flags);
 }
