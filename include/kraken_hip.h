@@ -258,6 +258,17 @@ int32_t krk_dct_residual(krk_dct* s, float* out, uint32_t flags);
 int32_t krk_coo_to_dense(const int64_t* idx, const float* val, int64_t nnz, float* dense,
                          int64_t n, uint32_t flags);
 
+/* ---- blockwise DCT-II (no reference counterpart) --------------------------- */
+/* The reference's "DCT" emitter is the threshold codec above and contains no cosine transform
+ * (worker/dct_emitter.cc:16-43); these two calls exist because this build's target names a
+ * blockwise DCT. x holds n floats, n a multiple of the block length 256. forward writes, for
+ * each block, the first `keep` coefficients of its orthonormal DCT-II (scipy.fft.dct(type=2,
+ * norm="ortho")) to coeff[n / 256, keep]; inverse rebuilds n floats from them (DCT-III with
+ * the missing coefficients taken as zero). keep is 64, 128, 192 or 256; 256 round-trips
+ * exactly up to fp32 rounding, 64 is the emitter's default retention 1 - eta = 0.25. */
+int32_t krk_dct2_forward(const float* x, float* coeff, int64_t n, int32_t keep, uint32_t flags);
+int32_t krk_dct2_inverse(const float* coeff, float* x, int64_t n, int32_t keep, uint32_t flags);
+
 /* ---- timing (HIP events on an object's own stream) ------------------------ */
 typedef struct krk_event krk_event;
 int32_t krk_event_create(krk_event** e);

@@ -93,23 +93,31 @@ __global__ void select_begin_kernel(uint32_t* sel, uint32_t k) {
   sel[1] = k;
 }
 
-// Per tile of kCodecTile consecutive elements: how many have |g+e| >= tau.
+// A tile is kCodecTile consecutive elements; inside it each wavefront owns 512 consecutive
+// elements and reads them as eight rows of 64, so every load and store is fully coalesced and
+// the output order is still the input order: within a row a lane's rank is the number of kept
+// elements in lower lanes (one ballot and a population count), rows and waves are offset by
+// running totals.
+
+// Per tile: how many elements have |g+e| >= tau.
 __global__ __launch_bounds__(kCodecBlock) void emit_count_kernel(const float* __restrict__ g,
                                                                  const float* __restrict__ e, int64_t n,
                                                                  const uint32_t* __restrict__ sel,
                                                                  int32_t* __restrict__ tile_counts) {
   __shared__ int wave_sum[kCodecBlock / 64];
   const uint32_t tau_bits = sel[2];
-  const int64_t base = (int64_t)blockIdx.x * kCodecTile + (int64_t)threadIdx.x * kCodecItems;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int64_t base = (int64_t)blockIdx.x * kCodecTile + (int64_t)wave * (64 * kCodecItems) + lane;
   int c = 0;
 #pragma unroll
-  for (int i = 0; i < kCodecItems; ++i) {
-    const int64_t j = base + i;
+  for (int k = 0; k < kCodecItems; ++k) {
+    const int64_t j = base + (int64_t)k * 64;
     if (j < n) c += abs_bits(g[j] + e[j]) >= tau_bits ? 1 : 0;
   }
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) c += __shfl_down(c, d, 64);
-  if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = c;
+  if (lane == 0) wave_sum[wave] = c;
   __syncthreads();
   if (threadIdx.x == 0) {
     int s = 0;
@@ -126,43 +134,37 @@ __global__ __launch_bounds__(kCodecBlock) void emit_write_kernel(
     long long* __restrict__ idx, float* __restrict__ val, float* __restrict__ e_next) {
   __shared__ int wave_sum[kCodecBlock / 64];
   const uint32_t tau_bits = sel[2];
-  const int64_t base = (int64_t)blockIdx.x * kCodecTile + (int64_t)threadIdx.x * kCodecItems;
-  float f[kCodecItems];
-  bool keep[kCodecItems];
-  int c = 0;
-#pragma unroll
-  for (int i = 0; i < kCodecItems; ++i) {
-    const int64_t j = base + i;
-    f[i] = j < n ? g[j] + e[j] : 0.0f;
-    keep[i] = j < n && abs_bits(f[i]) >= tau_bits;
-    c += keep[i] ? 1 : 0;
-  }
-  // exclusive scan of the per-thread counts across the workgroup
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  int x = c;
+  const int64_t base = (int64_t)blockIdx.x * kCodecTile + (int64_t)wave * (64 * kCodecItems) + lane;
+  float f[kCodecItems];
+  unsigned long long masks[kCodecItems];
+  int wave_total = 0;
 #pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int y = __shfl_up(x, d, 64);
-    if (lane >= d) x += y;
+  for (int k = 0; k < kCodecItems; ++k) {
+    const int64_t j = base + (int64_t)k * 64;
+    f[k] = j < n ? g[j] + e[j] : 0.0f;
+    masks[k] = __ballot(j < n && abs_bits(f[k]) >= tau_bits);
+    wave_total += __popcll(masks[k]);
   }
-  if (lane == 63) wave_sum[wave] = x;
+  if (lane == 0) wave_sum[wave] = wave_total;
   __syncthreads();
-  int off = tile_offsets[blockIdx.x] + x - c;
+  int off = tile_offsets[blockIdx.x];
 #pragma unroll
   for (int w = 0; w < kCodecBlock / 64; ++w)
     if (w < wave) off += wave_sum[w];
+  const unsigned long long below = (1ull << lane) - 1ull;
 #pragma unroll
-  for (int i = 0; i < kCodecItems; ++i) {
-    const int64_t j = base + i;
-    if (j < n) {
-      if (keep[i]) {
-        idx[off] = j;
-        val[off] = f[i];
-        ++off;
-      }
-      e_next[j] = keep[i] ? 0.0f : f[i];   // t/math.cc:1098-1123 : |x| < th keeps x
+  for (int k = 0; k < kCodecItems; ++k) {
+    const int64_t j = base + (int64_t)k * 64;
+    const bool keep = (masks[k] >> lane) & 1ull;
+    if (keep) {
+      const int at = off + __popcll(masks[k] & below);
+      idx[at] = j;
+      val[at] = f[k];
     }
+    if (j < n) e_next[j] = keep ? 0.0f : f[k];   // t/math.cc:1098-1123 : |x| < th keeps x
+    off += __popcll(masks[k]);
   }
 }
 
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(kCodecBlock) void coo_add_kernel(const long long* _
   const int64_t j = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x;
   if (j >= nnz) return;
   const long long i = idx[j];
-  if (i >= 0 && i < n) atomicAdd(&dense[i], val[j]);
+  if (i >= 0 && i < n) unsafeAtomicAdd(&dense[i], val[j]);   // hardware fp32 add, no CAS loop
 }
 
 static unsigned stream_grid(int64_t n) {

@@ -65,7 +65,7 @@ __global__ __launch_bounds__(kDenseBlock) void coo_scatter_kernel(const long lon
     atomicOr(err, 1u);
     return;
   }
-  atomicAdd(&dense[i], val[j]);
+  unsafeAtomicAdd(&dense[i], val[j]);   // hardware fp32 add, no CAS loop
 }
 
 static unsigned dense_grid(int64_t n) {

@@ -58,25 +58,47 @@ __global__ __launch_bounds__(kBlock) void dedup_claim_kernel(DSlot* slots, uint6
                                                              const uint64_t* __restrict__ ids, int64_t n,
                                                              uint32_t* __restrict__ slot_of) {
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (p >= n) return;
-  const unsigned long long id = ids[p];
-  uint64_t idx;
-  if (id == kEmptyKey) {
-    idx = mask + 1;   // the all-ones id owns the extra last slot
-  } else {
-    idx = mix64(id) & mask;
-    for (uint64_t t = 0; t <= mask; ++t) {
-      unsigned long long key = __atomic_load_n(&slots[idx].key, __ATOMIC_RELAXED);
-      if (key == kEmptyKey) {
-        const unsigned long long old = atomicCAS(&slots[idx].key, kEmptyKey, id);
-        key = old == kEmptyKey ? id : old;
-      }
-      if (key == id) break;
-      idx = (idx + 1) & mask;
-    }
+  const bool active = p < n;
+  const unsigned long long id = active ? ids[p] : 0ull;
+  const int lane = (int)(threadIdx.x & (kWave - 1));
+  // Equal ids inside one wavefront are folded first: positions grow with the lane number, so
+  // the lowest lane holding an id also holds its smallest position in this wave. Only that lane
+  // goes to the index; the others take the slot number from it. An id that fills a quarter of
+  // the request then costs one atomic per wave instead of sixteen.
+  int leader = lane;
+  unsigned long long todo = __ballot(active);
+  while (todo) {
+    const int first = __ffsll((unsigned long long)todo) - 1;
+    const unsigned int lo = __builtin_amdgcn_readlane((unsigned int)id, first);
+    const unsigned int hi = __builtin_amdgcn_readlane((unsigned int)(id >> 32), first);
+    const unsigned long long lid = (unsigned long long)lo | ((unsigned long long)hi << 32);
+    const bool same = active && id == lid;
+    if (same) leader = first;
+    todo &= ~__ballot(same);
   }
-  atomicMin(&slots[idx].minpos, (uint32_t)p);
-  slot_of[p] = (uint32_t)idx;
+  uint64_t idx = 0;
+  if (active && leader == lane) {
+    if (id == kEmptyKey) {
+      idx = mask + 1;   // the all-ones id owns the extra last slot
+    } else {
+      idx = mix64(id) & mask;
+      for (uint64_t t = 0; t <= mask; ++t) {
+        unsigned long long key = __atomic_load_n(&slots[idx].key, __ATOMIC_RELAXED);
+        if (key == kEmptyKey) {
+          const unsigned long long old = atomicCAS(&slots[idx].key, kEmptyKey, id);
+          key = old == kEmptyKey ? id : old;
+        }
+        if (key == id) break;
+        idx = (idx + 1) & mask;
+      }
+    }
+    // minpos only ever decreases, so a stale read can at worst cause a redundant atomic; later
+    // waves mostly find a smaller position already there and skip it.
+    if (__builtin_nontemporal_load(&slots[idx].minpos) > (uint32_t)p)
+      atomicMin(&slots[idx].minpos, (uint32_t)p);
+  }
+  const uint32_t shared_idx = __shfl((uint32_t)idx, leader);
+  if (active) slot_of[p] = shared_idx;
 }
 
 __global__ __launch_bounds__(kBlock) void dedup_flag_kernel(const DSlot* __restrict__ slots,
@@ -185,21 +207,47 @@ __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, con
 // keys[cnt] ascending (entries >= empty_from are holes). LEVEL0: the value of entry j is gradient
 // row pos[j]; otherwise it is vals[j, :]. Each tile of `tile` entries writes carry slots 2t
 // (run entering from the left) and 2t+1 (run leaving to the right).
+//
+// A workgroup first stages the keys (and positions) of all its tiles in LDS with coalesced loads,
+// including one neighbour on each side, so the walk itself only waits for value rows; those are
+// requested kPrefetch entries ahead of where the sums are.
+constexpr int kPrefetch = 4;
+
 template <int OPT, int VEC, bool LEVEL0>
 __global__ __launch_bounds__(kBlock) void segreduce_kernel(
     TableView tv, const uint32_t* __restrict__ keys, const uint32_t* __restrict__ pos,
     const float* __restrict__ vals, int64_t cnt, int tile, uint32_t empty_from,
     uint32_t* __restrict__ keys_out, float* __restrict__ vals_out, int dim, int elems, int group,
     ApplyArgs args) {
+  extern __shared__ uint32_t lds[];
   const int per_block = kBlock / group;
+  const int span = per_block * tile;                       // entries staged by this workgroup
+  const int64_t first = (int64_t)blockIdx.x * span;        // global index of lds_keys[1]
+  uint32_t* lds_keys = lds;                                // [span + 2], shifted by one
+  uint32_t* lds_pos = lds + span + 2;                      // [span]
+  for (int i = threadIdx.x; i < span + 2; i += kBlock) {
+    const int64_t j = first + i - 1;
+    lds_keys[i] = (j >= 0 && j < cnt) ? keys[j] : kNoRow;
+  }
+  if (LEVEL0) {
+    for (int i = threadIdx.x; i < span; i += kBlock) {
+      const int64_t j = first + i;
+      lds_pos[i] = j < cnt ? pos[j] : 0u;
+    }
+  }
+  __syncthreads();
+
   const int64_t t = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
   const int gl = threadIdx.x & (group - 1);
   const int64_t a = t * tile;
   if (a >= cnt) return;
   const int64_t b = a + tile < cnt ? a + tile : cnt;
-  const uint32_t left_key = a > 0 ? keys[a - 1] : kNoRow;
-  const uint32_t right_key = b < cnt ? keys[b] : kNoRow;
+  const int la = (int)(a - first);                          // tile's first entry, LDS-relative
+  const int lb = (int)(b - first);
+  const uint32_t left_key = lds_keys[la];                   // entry a - 1
+  const uint32_t right_key = lds_keys[lb + 1];              // entry b
   const bool leader = gl == 0;
+  uint32_t carry_key0 = kNoRow, carry_key1 = kNoRow;        // what this tile leaves in the carry list
 
   for (int e0 = 0; e0 < elems; e0 += group) {
     const int e = e0 + gl;
@@ -208,51 +256,70 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
     float acc[VEC];
 #pragma unroll
     for (int c = 0; c < VEC; ++c) acc[c] = 0.0f;
-    uint32_t run_key = keys[a];
-    int64_t run_start = a;
-    for (int64_t j = a; j <= b; ++j) {
-      const uint32_t key = j < b ? keys[j] : kNoRow;
-      if (j == b || key != run_key) {
-        // close the run [run_start, j)
-        if (run_key < empty_from) {
-          const bool open_left = run_start == a && left_key == run_key;
-          const bool open_right = j == b && right_key == run_key;
-          if (!open_left && !open_right) {
-            apply_row<OPT, VEC>(tv, run_key, acc, e, lane_on, leader, last_chunk, args);
-          } else {
-            const int64_t slot = open_left ? 2 * t : 2 * t + 1;
-            if (lane_on) vstore<VEC>(vals_out + slot * dim + e * VEC, acc);
-            if (leader) keys_out[slot] = run_key;
-            if (open_left && open_right) {
-              // the run covers the whole tile: keep the carry list contiguous with a zero piece
-              float z[VEC];
-#pragma unroll
-              for (int c = 0; c < VEC; ++c) z[c] = 0.0f;
-              if (lane_on) vstore<VEC>(vals_out + (slot + 1) * dim + e * VEC, z);
-              if (leader) keys_out[slot + 1] = run_key;
-            }
-          }
-        }
-        if (j == b) break;
-        run_key = key;
-        run_start = j;
-#pragma unroll
-        for (int c = 0; c < VEC; ++c) acc[c] = 0.0f;
+    uint32_t run_key = lds_keys[la + 1];
+    int run_start = la;
+
+    // closes the run [run_start, end) of run_key
+    auto close_run = [&](int end) {
+      if (run_key >= empty_from) return;
+      const bool open_left = run_start == la && left_key == run_key;
+      const bool open_right = end == lb && right_key == run_key;
+      if (!open_left && !open_right) {
+        apply_row<OPT, VEC>(tv, run_key, acc, e, lane_on, leader, last_chunk, args);
+        return;
       }
-      if (key < empty_from && lane_on) {
-        float v[VEC];
-        const float* src = LEVEL0 ? vals + (int64_t)pos[j] * dim : vals + j * dim;
-        vload<VEC>(src + e * VEC, v);
+      const int64_t slot = open_left ? 2 * t : 2 * t + 1;
+      if (lane_on) vstore<VEC>(vals_out + slot * dim + e * VEC, acc);
+      if (open_left) carry_key0 = run_key; else carry_key1 = run_key;
+      if (open_left && open_right) {
+        // the run covers the whole tile: keep the carry list contiguous with a zero piece
+        float z[VEC];
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) z[c] = 0.0f;
+        if (lane_on) vstore<VEC>(vals_out + (slot + 1) * dim + e * VEC, z);
+        carry_key1 = run_key;
+      }
+    };
+
+    for (int j0 = la; j0 < lb; j0 += kPrefetch) {
+      float v[kPrefetch][VEC];
+      uint32_t k[kPrefetch];
+#pragma unroll
+      for (int u = 0; u < kPrefetch; ++u) {
+        const int j = j0 + u;
+        k[u] = j < lb ? lds_keys[j + 1] : kNoRow;
+        if (j < lb && k[u] < empty_from && lane_on) {
+          const float* src = LEVEL0 ? vals + (int64_t)lds_pos[j] * dim : vals + (first + j) * dim;
+          vload<VEC>(src + e * VEC, v[u]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) v[u][c] = 0.0f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kPrefetch; ++u) {
+        const int j = j0 + u;
+        if (j >= lb) break;
+        if (k[u] != run_key) {
+          close_run(j);
+          run_key = k[u];
+          run_start = j;
+        }
         if (j == run_start) {
           // the first addend is copied, not added to zero (worker/emitter.cc:527 clones it)
 #pragma unroll
-          for (int c = 0; c < VEC; ++c) acc[c] = v[c];
+          for (int c = 0; c < VEC; ++c) acc[c] = v[u][c];
         } else {
 #pragma unroll
-          for (int c = 0; c < VEC; ++c) acc[c] = acc[c] + v[c];
+          for (int c = 0; c < VEC; ++c) acc[c] = acc[c] + v[u][c];
         }
       }
     }
+    close_run(lb);
+  }
+  if (leader && keys_out) {
+    keys_out[2 * t] = carry_key0;
+    keys_out[2 * t + 1] = carry_key1;
   }
 }
 
@@ -264,12 +331,15 @@ static void launch_segreduce(bool level0, const TableView& tv, const uint32_t* k
   const int per_block = kBlock / t->group;
   const int64_t tiles = (cnt + tile - 1) / tile;
   const dim3 grid(grid_for(tiles, per_block)), block(kBlock);
+  const size_t lds_bytes = (size_t)(2 * per_block * tile + 2) * sizeof(uint32_t);
   if (level0) {
-    hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, true>), grid, block, 0, stream, tv, keys, pos, vals,
-                       cnt, tile, empty_from, keys_out, vals_out, (int)t->dim, t->elems, t->group, args);
+    hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, true>), grid, block, lds_bytes, stream, tv, keys, pos,
+                       vals, cnt, tile, empty_from, keys_out, vals_out, (int)t->dim, t->elems, t->group,
+                       args);
   } else {
-    hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, false>), grid, block, 0, stream, tv, keys, pos, vals,
-                       cnt, tile, empty_from, keys_out, vals_out, (int)t->dim, t->elems, t->group, args);
+    hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, false>), grid, block, lds_bytes, stream, tv, keys, pos,
+                       vals, cnt, tile, empty_from, keys_out, vals_out, (int)t->dim, t->elems, t->group,
+                       args);
   }
 }
 
@@ -317,8 +387,8 @@ int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, 
   KRK_TRY(check_flags(flags));
   if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;   // the count comes back by value
   if (n < 0 || !n_unique || (n > 0 && (!ids || !uids))) return KRK_E_ARGUMENT;
-  if (n >= (int64_t)0x7FFFFFFF) {
-    set_error("krk_dedup handles fewer than 2^31 ids per call");
+  if (n > ((int64_t)1 << 30)) {
+    set_error("krk_dedup handles at most 2^30 ids per call");
     return KRK_E_CAPACITY;
   }
   KRK_TRY(ensure_runtime());
@@ -334,12 +404,12 @@ int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, 
   const bool host = !(flags & KRK_DEVICE_PTRS);
   // one allocation: slots | slot_of | flag | rank | scan scratch | total | (staged ids, uids, inv)
   size_t total = slots_b + 3 * n4 + scan_b + 256 + (host ? 3 * n8 : 0);
-  char* base = nullptr;
-  KRK_HIP(hipMalloc((void**)&base, total));
-  struct Free {
-    char* p;
-    ~Free() { (void)hipFree(p); }
-  } guard{base};
+  // work space is kept between calls (the call blocks, so one buffer under a lock is enough)
+  static std::mutex pool_mu;
+  static DeviceBuffer pool;
+  std::lock_guard<std::mutex> pool_lock(pool_mu);
+  KRK_TRY(pool.reserve(total));
+  char* base = pool.as<char>();
   char* cur = base;
   DSlot* slots = reinterpret_cast<DSlot*>(cur); cur += slots_b;
   uint32_t* slot_of = reinterpret_cast<uint32_t*>(cur); cur += n4;
@@ -464,7 +534,6 @@ int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* i
     if (tiles > 1) {
       okeys = ckeys[which];
       ovals = cvals[which];
-      KRK_HIP(hipMemsetAsync(okeys, 0xFF, (size_t)(2 * tiles) * sizeof(uint32_t), t->stream));
     }
     if (t->vec == 4) {
       dispatch_segreduce<4>(o->type, level0, tv, in_keys, spos, in_vals, cnt, tile, empty_from, okeys,
@@ -480,7 +549,7 @@ int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* i
     cnt = 2 * tiles;
     level0 = false;
     which ^= 1;
-    tile = 16;
+    tile = 16;   // carry lists are short: short tiles keep many lane groups busy
   }
   return sparse_finish(t, flags);
 }

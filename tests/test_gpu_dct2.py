@@ -1,0 +1,78 @@
+"""Blockwise DCT-II on the matrix cores. The reference has no cosine transform (its "DCT"
+emitter is the threshold codec), so there is no reference output to match: the transform is
+pinned by the library definition scipy.fft.dct(type=2, norm="ortho") on blocks of 256, by the
+orthonormality of the basis (Parseval) and by the round trip. Tolerance: fp32 accumulation of
+256 products, 2e-5 relative to the block's norm."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dct2():
+    from kraken_amd import api, dct2 as d
+    api.lib()
+    return d
+
+
+def _ref(x, keep):
+    fft = pytest.importorskip("scipy.fft")
+    return fft.dct(x.reshape(-1, 256).astype(np.float64), type=2, norm="ortho", axis=1)[:, :keep]
+
+
+@pytest.mark.parametrize("blocks", [1, 3, 128, 1000])
+@pytest.mark.parametrize("keep", [64, 128, 256])
+def test_forward_matches_scipy(dct2, blocks, keep):
+    rng = np.random.default_rng(blocks + keep)
+    x = rng.standard_normal(blocks * 256).astype(np.float32)
+    got = dct2.forward(x, keep)
+    want = _ref(x, keep)
+    scale = np.linalg.norm(x.reshape(-1, 256), axis=1, keepdims=True)
+    assert np.abs(got - want).max() <= 2e-5 * scale.max()
+    assert (np.abs(got - want) <= 2e-5 * scale + 1e-7).all()
+
+
+def test_known_vectors(dct2):
+    """Closed forms: a constant block has only the k = 0 coefficient (= c * sqrt(256));
+    a single cosine of the basis maps to a single coefficient."""
+    x = np.full(256, 0.5, np.float32)
+    y = dct2.forward(x, 256)[0]
+    assert abs(y[0] - 0.5 * 16.0) < 1e-5 and np.abs(y[1:]).max() < 1e-5
+    j = np.arange(256)
+    k = 37
+    x = (np.sqrt(2.0 / 256) * np.cos(np.pi * (2 * j + 1) * k / 512.0)).astype(np.float32)
+    y = dct2.forward(x, 256)[0]
+    assert abs(y[k] - 1.0) < 1e-5 and np.abs(np.delete(y, k)).max() < 1e-5
+
+
+def test_round_trip_and_parseval(dct2):
+    rng = np.random.default_rng(1)
+    n = 4096 * 256
+    x = rng.standard_normal(n).astype(np.float32)
+    y = dct2.forward(x, 256)
+    assert abs(np.sum(y.astype(np.float64) ** 2) / np.sum(x.astype(np.float64) ** 2) - 1.0) < 1e-5
+    back = dct2.inverse(y, n, 256)
+    assert np.abs(back - x).max() < 2e-5 * 16
+    # truncated: inverse(keep) equals the inverse of the zero-padded coefficients
+    y64 = dct2.forward(x, 64)
+    assert np.array_equal(y64, y[:, :64])
+    fft = pytest.importorskip("scipy.fft")
+    pad = np.zeros((n // 256, 256))
+    pad[:, :64] = y64
+    want = fft.idct(pad, type=2, norm="ortho", axis=1).ravel()
+    got = dct2.inverse(y64, n, 64)
+    assert np.abs(got - want).max() < 2e-5 * 16
+
+
+def test_device_pointers_and_arguments(dct2):
+    from kraken_amd import api
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal(512 * 256).astype(np.float32)
+    d = api.DeviceArray.from_host(x)
+    y = dct2.forward(d, 64)
+    assert np.array_equal(y.to_host(), dct2.forward(x, 64))
+    with pytest.raises(api.KrakenHipError):
+        dct2.forward(x[:100], 64)
+    with pytest.raises(api.KrakenHipError):
+        dct2.forward(x, 50)
