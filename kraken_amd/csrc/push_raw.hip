@@ -387,7 +387,7 @@ int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, 
   KRK_TRY(check_flags(flags));
   if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;   // the count comes back by value
   if (n < 0 || !n_unique || (n > 0 && (!ids || !uids))) return KRK_E_ARGUMENT;
-  if (n > ((int64_t)1 << 30)) {
+  if (n > ((int64_t)1 << 30)) {   // one thread per id, and slot numbers are 32 bits wide
     set_error("krk_dedup handles at most 2^30 ids per call");
     return KRK_E_CAPACITY;
   }
@@ -458,8 +458,8 @@ int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* i
     return KRK_UNSUPPORTED_OPTIM;
   }
   if (n < 0 || (n > 0 && (!ids || !grads))) return KRK_E_ARGUMENT;
-  if (n >= (int64_t)0x7FFFFFFF) {
-    set_error("krk_sparse_push_raw handles fewer than 2^31 ids per call");
+  if (n > ((int64_t)1 << 28)) {
+    set_error("krk_sparse_push_raw handles at most 2^28 ids per call; split the request");
     return KRK_E_CAPACITY;
   }
   std::lock_guard<std::mutex> lk(t->mu);

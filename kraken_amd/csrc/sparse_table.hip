@@ -6,10 +6,11 @@
 // a group of tables, the loops of Ps::CombinePullSparseTable / CombinePushSparseTable
 // (ps/ps_op.cc:370-387, 456-469), which become one launch over all tables of the request.
 //
-// Work mapping: `group` adjacent lanes of a 64-wide wavefront own one id. The group's first
-// lane walks the index (one 16-byte slot load per probe), the row number is broadcast with a
-// wave shuffle, then every lane moves `vec` floats of the record per step, so a dim-16 row is
-// four float4 lanes and sixteen rows share one wavefront instruction.
+// Work mapping: `group` adjacent lanes (at least four) of a 64-wide wavefront own one id. Four
+// of them read an index bucket together (one 64-byte request per probe step) and wave ballots
+// give every lane of the group the row number; then every lane moves `vec` floats of the
+// record per step, so a dim-16 row is four float4 lanes and sixteen rows share one wavefront
+// instruction.
 #include <algorithm>
 #include <cmath>
 #include <new>
@@ -269,22 +270,24 @@ __global__ __launch_bounds__(kBlock) void export_kernel(TableView tv, int64_t ro
                                                         float* __restrict__ vals, int state_off,
                                                         float* __restrict__ state, int meta_off,
                                                         long long* __restrict__ steps) {
-  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t r = t / dim;
-  const int j = (int)(t - r * dim);
-  if (r >= rows) return;
-  const float* rec = tv.recs + r * tv.stride;
-  if (vals) vals[t] = rec[j];
-  if (state) state[t] = state_off >= 0 ? rec[state_off + j] : 0.0f;
-  if (j == 0) {
-    if (ids) ids[r] = tv.row_key[r];
-    if (steps) {
-      long long s = 0;
-      if (meta_off >= 0) {
-        const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + meta_off);
-        s = (long long)((uint64_t)meta[0] | ((uint64_t)meta[1] << 32));
+  const int64_t total = rows * dim;
+  const int64_t step = (int64_t)gridDim.x * kBlock;   // grid-stride: see restride_kernel
+  for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < total; t += step) {
+    const int64_t r = t / dim;
+    const int j = (int)(t - r * dim);
+    const float* rec = tv.recs + r * tv.stride;
+    if (vals) vals[t] = rec[j];
+    if (state) state[t] = state_off >= 0 ? rec[state_off + j] : 0.0f;
+    if (j == 0) {
+      if (ids) ids[r] = tv.row_key[r];
+      if (steps) {
+        long long s = 0;
+        if (meta_off >= 0) {
+          const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + meta_off);
+          s = (long long)((uint64_t)meta[0] | ((uint64_t)meta[1] << 32));
+        }
+        steps[r] = s;
       }
-      steps[r] = s;
     }
   }
 }
@@ -328,11 +331,14 @@ __global__ __launch_bounds__(kBlock) void restride_kernel(const float* __restric
                                                           int64_t src_stride, float* __restrict__ dst,
                                                           int64_t dst_stride, int64_t rows,
                                                           int copy_floats) {
-  const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t r = t / copy_floats;
-  const int j = (int)(t - r * copy_floats);
-  if (r >= rows) return;
-  dst[r * dst_stride + j] = src[r * src_stride + j];
+  // grid-stride: a launch cannot carry more than 2^32 work-items, a large table has more floats
+  const int64_t total = rows * copy_floats;
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < total; t += step) {
+    const int64_t r = t / copy_floats;
+    const int j = (int)(t - r * copy_floats);
+    dst[r * dst_stride + j] = src[r * src_stride + j];
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -341,6 +347,19 @@ __global__ __launch_bounds__(kBlock) void restride_kernel(const float* __restric
 static inline unsigned grid_for(int64_t items, int per_block) {
   return (unsigned)((items + per_block - 1) / per_block);
 }
+
+// Workgroups for a grid-stride kernel over `items`: enough to fill the chip many times over,
+// never so many that workgroups x 256 passes the 2^32 work-items one launch can carry.
+static inline unsigned strided_grid(int64_t items) {
+  int64_t blocks = (items + kBlock - 1) / kBlock;
+  const int64_t cap = 1 << 20;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
+// Ids one launch of a `group`-lanes-per-id kernel may take so that ids x group stays below 2^31.
+static inline int64_t max_ids_per_launch(int group) { return ((int64_t)1 << 31) / group - kBlock; }
 
 static int32_t alloc_slots(uint64_t cap, Slot** out, hipStream_t s) {
   Slot* p = nullptr;
@@ -520,10 +539,10 @@ int32_t sparse_ensure_columns(krk_sparse* t, uint32_t mask) {
   KRK_HIP(hipMalloc((void**)&nrecs, rec_bytes ? rec_bytes : 16));
   KRK_HIP(hipMemsetAsync(nrecs, 0, rec_bytes, t->stream));
   if (rows) {
-    hipLaunchKernelGGL(restride_kernel, dim3(grid_for(rows * old_body, kBlock)), dim3(kBlock), 0,
+    hipLaunchKernelGGL(restride_kernel, dim3(strided_grid(rows * old_body)), dim3(kBlock), 0,
                        t->stream, t->recs, old_stride, nrecs, stride, rows, (int)old_body);
     if (old_meta >= 0) {
-      hipLaunchKernelGGL(restride_kernel, dim3(grid_for(rows * 2, kBlock)), dim3(kBlock), 0, t->stream,
+      hipLaunchKernelGGL(restride_kernel, dim3(strided_grid(rows * 2)), dim3(kBlock), 0, t->stream,
                          t->recs + old_meta, old_stride, nrecs + meta_off, stride, rows, 2);
     }
     KRK_HIP(hipGetLastError());
@@ -784,6 +803,11 @@ int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* ou
     set_error("device output must be 16-byte aligned");
     return KRK_E_ARGUMENT;
   }
+  if (n > max_ids_per_launch(t->group)) {
+    set_error("at most %lld ids per call for this row width; split the request",
+              (long long)max_ids_per_launch(t->group));
+    return KRK_E_CAPACITY;
+  }
   std::lock_guard<std::mutex> lk(t->mu);
   if (n == 0) return sparse_finish(t, flags);
   KRK_TRY(sparse_ensure_room(t, n));
@@ -820,6 +844,11 @@ int32_t krk_sparse_push(krk_sparse* t, const krk_optim* o, const uint64_t* ids, 
     set_error("device gradients must be 16-byte aligned");
     return KRK_E_ARGUMENT;
   }
+  if (n > max_ids_per_launch(t->group)) {
+    set_error("at most %lld ids per call for this row width; split the request",
+              (long long)max_ids_per_launch(t->group));
+    return KRK_E_CAPACITY;
+  }
   std::lock_guard<std::mutex> lk(t->mu);
   if (n == 0) return sparse_finish(t, flags);
   if (grad_dim != t->dim) {   // ps/optim/adagrad.cc:29-32
@@ -846,6 +875,11 @@ int32_t krk_sparse_lookup(krk_sparse* t, const uint64_t* ids, int64_t n, int32_t
   KRK_TRY(check_table(t));
   KRK_TRY(check_flags(flags));
   if (n < 0 || (n > 0 && (!ids || !rows))) return KRK_E_ARGUMENT;
+  if (n > max_ids_per_launch(kBucket)) {
+    set_error("at most %lld ids per call for this row width; split the request",
+              (long long)max_ids_per_launch(kBucket));
+    return KRK_E_CAPACITY;
+  }
   std::lock_guard<std::mutex> lk(t->mu);
   if (n == 0) return sparse_finish(t, flags);
   const uint64_t* d_ids;
@@ -865,6 +899,11 @@ int32_t krk_sparse_import(krk_sparse* t, const uint64_t* ids, int64_t n, const f
   KRK_TRY(check_flags(flags));
   if (n < 0 || (n > 0 && (!ids || !vals))) return KRK_E_ARGUMENT;
   if ((flags & KRK_DEVICE_PTRS) && t->vec == 4 && !aligned16(vals)) return KRK_E_ARGUMENT;
+  if (n > max_ids_per_launch(t->group)) {
+    set_error("at most %lld ids per call for this row width; split the request",
+              (long long)max_ids_per_launch(t->group));
+    return KRK_E_CAPACITY;
+  }
   std::lock_guard<std::mutex> lk(t->mu);
   if (n == 0) return sparse_finish(t, flags);
   KRK_TRY(sparse_ensure_room(t, n));
@@ -913,7 +952,7 @@ int32_t krk_sparse_export(krk_sparse* t, uint64_t* ids, float* vals, int32_t sta
   if (state) KRK_TRY(t->output(state, cells, flags, 2, &d_state));
   if (steps) KRK_TRY(t->output(reinterpret_cast<long long*>(steps), (size_t)rows, flags, 3, &d_steps));
   const int state_off = state ? t->col_off[state_type] : -1;
-  hipLaunchKernelGGL(export_kernel, dim3(grid_for((int64_t)cells, kBlock)), dim3(kBlock), 0, t->stream,
+  hipLaunchKernelGGL(export_kernel, dim3(strided_grid((int64_t)cells)), dim3(kBlock), 0, t->stream,
                      t->view(), rows, (int)t->dim, d_ids, d_vals, state_off, d_state, t->meta_off,
                      d_steps);
   KRK_HIP(hipGetLastError());
@@ -1027,7 +1066,10 @@ static int32_t group_plan(krk_group* g, const int64_t* offsets, GroupCall* call,
     call->row_start[i] = offsets[i];
     blocks += (uint64_t)((cnt + per_block - 1) / per_block);
   }
-  if (blocks >= 0x7FFFFFFFull) return KRK_E_CAPACITY;
+  if (blocks * (uint64_t)kBlock >= 0x7FFFFFFFull) {
+    set_error("combined request too large for one launch; split it");
+    return KRK_E_CAPACITY;
+  }
   call->block_start[n] = (uint32_t)blocks;
   call->row_start[n] = offsets[n];
   *total = offsets[n];
