@@ -9,8 +9,8 @@
 //
 // Shape of the work: Y[M, N] = X[M, K] * Basis[K, N] with M = n / 256 blocks. Forward: K = 256,
 // N = keep. Inverse: K = keep, N = 256. A workgroup keeps its 64-column basis tile resident in
-// LDS, walks over row tiles of 128 blocks, stages X through LDS in 32-wide slices and feeds
-// v_mfma_f32_32x32x2_f32: four wavefronts, each owning a 32 x 64 piece of the output tile.
+// LDS, walks over row tiles of 256 blocks, stages X through LDS in 32-wide slices and feeds
+// v_mfma_f32_32x32x2_f32: eight wavefronts, each owning a 32 x 64 piece of the output tile.
 #include <cmath>
 #include <mutex>
 
@@ -19,10 +19,12 @@
 namespace krk {
 
 constexpr int kDctB = 256;      // block length
-constexpr int kTileM = 128;     // rows (blocks) per output tile
+constexpr int kThreads = 512;   // eight wavefronts: two per SIMD, so one can wait while one multiplies
+constexpr int kTileM = 256;     // rows (blocks) per output tile: 32 per wavefront
 constexpr int kTileN = 64;      // basis columns per workgroup
 constexpr int kSliceK = 32;     // reduction slice staged per step
 constexpr int kXsLd = kSliceK + 1;   // padded: a column read by 32 lanes hits 32 banks
+constexpr int kStageVec = (kTileM * kSliceK / 4) / kThreads;   // float4 loads per thread per slice
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -40,10 +42,14 @@ __global__ void dct2_basis_kernel(float* __restrict__ fwd, float* __restrict__ i
 
 // Y[M, N] = X[M, K] * Bm[K, N]; ldx / ldb / ldy are row strides in floats. K is a multiple of 32,
 // N a multiple of 64 (both <= 256). grid.x workgroups share the row tiles, grid.y = N / 64.
-__global__ __launch_bounds__(256) void dct2_gemm_kernel(const float* __restrict__ X, int64_t ldx,
-                                                        const float* __restrict__ Bm, int ldb,
-                                                        float* __restrict__ Y, int64_t ldy, int64_t M,
-                                                        int K) {
+//
+// Pipeline per 32-wide slice of the reduction: the next slice of X is requested from HBM into
+// registers, the current slice (already in LDS) is multiplied, and only then are the registers
+// written to the other LDS buffer, so the memory latency sits behind 32 matrix instructions.
+__global__ __launch_bounds__(kThreads) void dct2_gemm_kernel(const float* __restrict__ X, int64_t ldx,
+                                                             const float* __restrict__ Bm, int ldb,
+                                                             float* __restrict__ Y, int64_t ldy,
+                                                             int64_t M, int K) {
   extern __shared__ float lds[];
   float* Bs = lds;                                  // [K][kTileN], resident for the whole launch
   float* Xs = lds + (size_t)K * kTileN;             // 2 x [kTileM][kXsLd]
@@ -52,7 +58,7 @@ __global__ __launch_bounds__(256) void dct2_gemm_kernel(const float* __restrict_
   const int wave = tid >> 6;
   const int n0 = blockIdx.y * kTileN;
 
-  for (int i = tid; i < K * (kTileN / 4); i += 256) {
+  for (int i = tid; i < K * (kTileN / 4); i += kThreads) {
     const int r = i / (kTileN / 4);
     const int c4 = i - r * (kTileN / 4);
     reinterpret_cast<float4*>(Bs)[i] = *reinterpret_cast<const float4*>(Bm + (size_t)r * ldb + n0 + c4 * 4);
@@ -63,25 +69,33 @@ __global__ __launch_bounds__(256) void dct2_gemm_kernel(const float* __restrict_
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
     const int64_t m0 = tile * kTileM;
     v16f acc0 = {0}, acc1 = {0};
-    // stage slice 0
-    auto stage = [&](int slice, int buf) {
-      float* dst = Xs + buf * (kTileM * kXsLd);
+    float4 regs[kStageVec];
+    auto fetch = [&](int slice) {
 #pragma unroll
-      for (int it = 0; it < (kTileM * kSliceK / 4) / 256; ++it) {
-        const int i = it * 256 + tid;            // float4 index inside the slice
+      for (int it = 0; it < kStageVec; ++it) {
+        const int i = it * kThreads + tid;       // float4 index inside the slice
         const int r = i >> 3;                    // 8 float4 per 32-float row piece
         const int c4 = i & 7;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (m0 + r < M) v = *reinterpret_cast<const float4*>(X + (m0 + r) * ldx + slice * kSliceK + c4 * 4);
-        float* d = dst + r * kXsLd + c4 * 4;
-        d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+        regs[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (m0 + r < M)
+          regs[it] = *reinterpret_cast<const float4*>(X + (m0 + r) * ldx + slice * kSliceK + c4 * 4);
       }
     };
-    stage(0, 0);
+    auto park = [&](int buf) {
+      float* dst = Xs + buf * (kTileM * kXsLd);
+#pragma unroll
+      for (int it = 0; it < kStageVec; ++it) {
+        const int i = it * kThreads + tid;
+        float* d = dst + (i >> 3) * kXsLd + (i & 7) * 4;
+        d[0] = regs[it].x; d[1] = regs[it].y; d[2] = regs[it].z; d[3] = regs[it].w;
+      }
+    };
+    fetch(0);
+    park(0);
     __syncthreads();
     for (int s = 0; s < slices; ++s) {
       const int buf = s & 1;
-      if (s + 1 < slices) stage(s + 1, buf ^ 1);
+      if (s + 1 < slices) fetch(s + 1);
       const float* xs = Xs + buf * (kTileM * kXsLd) + (wave * 32 + (lane & 31)) * kXsLd + (lane >> 5);
       const float* bs = Bs + (size_t)(s * kSliceK + (lane >> 5)) * kTileN + (lane & 31);
 #pragma unroll
@@ -92,6 +106,7 @@ __global__ __launch_bounds__(256) void dct2_gemm_kernel(const float* __restrict_
         acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b0, acc0, 0, 0, 0);
         acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b1, acc1, 0, 0, 0);
       }
+      if (s + 1 < slices) park(buf ^ 1);
       __syncthreads();
     }
     // accumulator element i of lane l is C[(i / 4) * 8 + (l / 32) * 4 + i % 4][l % 32]
@@ -159,12 +174,12 @@ static int32_t dct2_run(const float* in, float* out, int64_t n, int32_t keep, ui
   const float* basis = forward ? g_basis_fwd : g_basis_inv;
   const size_t lds_bytes = sizeof(float) * ((size_t)K * kTileN + 2 * kTileM * kXsLd);
   const int64_t tiles = (M + kTileM - 1) / kTileM;
-  int64_t gx = tiles < 256 * 2 / (N / kTileN) ? tiles : 256 * 2 / (N / kTileN);   // ~2 workgroups per CU
+  int64_t gx = tiles < 256 / (N / kTileN) ? tiles : 256 / (N / kTileN);   // one workgroup per CU
   if (gx < 1) gx = 1;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(dct2_gemm_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (e == hipSuccess) {
-    hipLaunchKernelGGL(dct2_gemm_kernel, dim3((unsigned)gx, (unsigned)(N / kTileN)), dim3(256), lds_bytes, s,
+    hipLaunchKernelGGL(dct2_gemm_kernel, dim3((unsigned)gx, (unsigned)(N / kTileN)), dim3(kThreads), lds_bytes, s,
                        d_in, (int64_t)K, basis, kDctB, d_out, (int64_t)N, M, K);
     e = hipGetLastError();
   }

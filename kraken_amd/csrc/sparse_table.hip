@@ -84,6 +84,13 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
                                           int64_t i, bool active, int gl,
                                           const float* __restrict__ grads, int dim, int elems,
                                           int group, float lr, const OptimK& k, const PushCols& pc) {
+  // The gradient row does not depend on the index: its first slice is requested before the
+  // probe so that it travels while the probe waits for its bucket.
+  const float* g = grads + i * (int64_t)dim;
+  float g_first[VEC];
+#pragma unroll
+  for (int c = 0; c < VEC; ++c) g_first[c] = 0.0f;
+  if (active && gl < elems) vload<VEC>(g + gl * VEC, g_first);
   const uint32_t row = probe_find(tv, active ? ids[i] : 0, active, gl, group);
   if (!active) return;
   if (row == kEmptyRow) {
@@ -91,7 +98,6 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
     return;
   }
   float* rec = tv.recs + (int64_t)row * tv.stride;
-  const float* g = grads + i * (int64_t)dim;
 
   bool first = false;
   float bc1 = 1.0f, bc2 = 1.0f;
@@ -109,7 +115,12 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
   }
   for (int e = gl; e < elems; e += group) {
     float gv[VEC], w[VEC], s0[VEC], s1[VEC], s2[VEC];
-    vload<VEC>(g + e * VEC, gv);
+    if (e == gl) {
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) gv[c] = g_first[c];
+    } else {
+      vload<VEC>(g + e * VEC, gv);
+    }
     vload<VEC>(rec + e * VEC, w);
     if (pc.c0 >= 0) vload<VEC>(rec + pc.c0 + e * VEC, s0);
     if (pc.c1 >= 0) vload<VEC>(rec + pc.c1 + e * VEC, s1);
