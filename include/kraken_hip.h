@@ -167,6 +167,34 @@ int32_t krk_sparse_push(krk_sparse* t, const krk_optim* o, const uint64_t* ids, 
  * grads is [n, grad_dim]. */
 int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* ids, int64_t n,
                             const float* grads, int64_t grad_dim, float lr, uint32_t flags);
+
+/* ---- multi-hot fields: Pull / Push fused with the worker's jagged pooling ---
+ * A field holds `bags` bags; bag i owns ids[offsets[i] .. offsets[i+1]), offsets is
+ * [bags + 1], starts at 0 and ends at n (checked when the pointers are host pointers;
+ * device offsets are clamped to [0, n] and ids outside every bag are ignored).
+ * weights is NULL or [n]: the per-id factors of JaggedTensor.weights()
+ * (pytorch/jagged_embedding.py:41-45). */
+#define KRK_POOL_SUM 0
+#define KRK_POOL_MEAN 1
+/* SparseTable::Pull (ps/sparse_table.cc:33-75, ids inserted when absent) followed by
+ * jagged::SumForward / MeanForward (pytorch/py/jagged_ops.cc:14-56, 206-236) in one pass:
+ * out[i] = row(first id) (* weight), then the bag's other rows added in position order; mean
+ * multiplies by (float)(1.0 / float(len)); an empty bag yields patch_value. out is
+ * [bags, dim]. The n pulled rows are never written out. Rows wider than 256 floats (64 when
+ * dim is not a multiple of 4) return 10. */
+int32_t krk_sparse_pull_pooled(krk_sparse* t, const uint64_t* ids, int64_t n, const int64_t* offsets,
+                               int64_t bags, const float* weights, int32_t mode, float patch_value,
+                               float* out, uint32_t flags);
+/* The backward of the above fused with krk_sparse_push_raw: position p of bag i carries the
+ * gradient bag_grads[i] (sum) or bag_grads[i] * (float)(1.0 / float(len)) (mean,
+ * pytorch/py/jagged_ops.cc:303-334), times weights[p] when given; gradients of equal ids are
+ * summed and each row is updated once, as in krk_sparse_push_raw. The [n, dim] per-position
+ * gradient is never materialised. For the sum this is the transpose of the forward, which is
+ * what pytorch/py/jagged_ops.cc:148-160 is meant to be (as written it fills only the first row
+ * of each bag). bag_grads is [bags, grad_dim]. */
+int32_t krk_sparse_push_pooled(krk_sparse* t, const krk_optim* o, const uint64_t* ids, int64_t n,
+                               const int64_t* offsets, int64_t bags, const float* weights, int32_t mode,
+                               const float* bag_grads, int64_t grad_dim, float lr, uint32_t flags);
 /* id -> row lookup alone (ParallelSkipList::HitSlot + SkipList::Find,
  * common/parallel_skip_list.h:100-102, common/skip_list.h:315-324):
  * rows[i] = dense row index of ids[i], or -1 when absent. Row indices are
@@ -274,7 +302,8 @@ typedef struct krk_event krk_event;
 int32_t krk_event_create(krk_event** e);
 int32_t krk_event_destroy(krk_event* e);
 /* object = a krk_sparse*, krk_group*, krk_dense* or krk_dct*: the event is recorded on that
- * object's stream, behind the work already enqueued there. */
+ * object's stream, behind the work already enqueued there. NULL = the null stream, where the
+ * calls that own no object (krk_dedup, krk_dct2_*, krk_coo_to_dense, krk_stream_copy) run. */
 int32_t krk_event_record(krk_event* e, void* object);
 int32_t krk_event_elapsed_ms(krk_event* start, krk_event* stop, float* ms);
 

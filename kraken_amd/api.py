@@ -80,6 +80,11 @@ EXPORTS = {
                                     C.c_int64, C.c_float, C.c_uint32]),
     "krk_sparse_push_raw": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_int64,
                                         C.c_void_p, C.c_int64, C.c_float, C.c_uint32]),
+    "krk_sparse_pull_pooled": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64,
+                                           C.c_void_p, C.c_int32, C.c_float, C.c_void_p, C.c_uint32]),
+    "krk_sparse_push_pooled": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_int64,
+                                           C.c_void_p, C.c_int64, C.c_void_p, C.c_int32, C.c_void_p,
+                                           C.c_int64, C.c_float, C.c_uint32]),
     "krk_sparse_lookup": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_uint32]),
     "krk_sparse_import": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_uint32]),
     "krk_sparse_export": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p,
@@ -315,6 +320,42 @@ class SparseTable:
     def PushRaw(self, optim, ids, grads, lr, async_=False):
         """Emitter::PushSparseTable's dedup + sum fused with Push: ids may repeat."""
         return self.Push(optim, ids, grads, lr, async_=async_, raw=True)
+
+    _POOL = {"sum": 0, "mean": 1}
+
+    def PullPooled(self, ids, offsets, mode="sum", patch_value=0.0, weights=None, out=None, async_=False):
+        """JaggedEmbedding.forward (pytorch/jagged_embedding.py:32-52) in one launch: Pull of the
+        bags' ids fused with jagged sum / mean. -> (code, [bags, dim]). Host arrays or
+        DeviceArrays (all of one kind)."""
+        dev = isinstance(ids, DeviceArray)
+        if not dev:
+            ids = np.ascontiguousarray(ids, dtype=np.uint64)
+            offsets = np.ascontiguousarray(offsets, dtype=np.int64)
+            if weights is not None:
+                weights = np.ascontiguousarray(weights, dtype=np.float32)
+        bags = offsets.size - 1
+        if out is None:
+            out = DeviceArray((bags, self.dimension), np.float32) if dev else \
+                np.empty((bags, self.dimension), np.float32)
+        rc = lib().krk_sparse_pull_pooled(self.h, _ptr(ids), ids.size, _ptr(offsets), bags, _ptr(weights),
+                                          self._POOL[mode], patch_value, _ptr(out),
+                                          _flags(ids, out, extra=ASYNC if async_ else 0))
+        return rc, out
+
+    def PushPooled(self, optim, ids, offsets, bag_grads, lr, mode="sum", weights=None, async_=False):
+        """The backward of PullPooled fused with PushRaw: bag_grads is [bags, dim]."""
+        dev = isinstance(ids, DeviceArray)
+        if not dev:
+            ids = np.ascontiguousarray(ids, dtype=np.uint64)
+            offsets = np.ascontiguousarray(offsets, dtype=np.int64)
+            bag_grads = np.ascontiguousarray(bag_grads, dtype=np.float32)
+            if weights is not None:
+                weights = np.ascontiguousarray(weights, dtype=np.float32)
+        bags = offsets.size - 1
+        gd = bag_grads.shape[-1] if len(bag_grads.shape) > 1 else bag_grads.size // max(bags, 1)
+        return lib().krk_sparse_push_pooled(self.h, C.byref(optim.raw), _ptr(ids), ids.size, _ptr(offsets),
+                                            bags, _ptr(weights), self._POOL[mode], _ptr(bag_grads), gd, lr,
+                                            _flags(ids, bag_grads, extra=ASYNC if async_ else 0))
 
     def lookup(self, ids):
         if isinstance(ids, DeviceArray):
@@ -553,7 +594,8 @@ class Event:
         self.h = h
 
     def record(self, obj):
-        _check(lib().krk_event_record(self.h, obj.h), "krk_event_record")
+        # obj None: the null stream, where the calls that own no object (dedup, dct2) run
+        _check(lib().krk_event_record(self.h, obj.h if obj is not None else None), "krk_event_record")
 
     def elapsed_ms(self, stop):
         ms = C.c_float()

@@ -8,9 +8,9 @@
 // each block (keep = B * (1 - eta) = 64 for the emitter's default eta = 0.75) is the compression.
 //
 // Shape of the work: Y[M, N] = X[M, K] * Basis[K, N] with M = n / 256 blocks. Forward: K = 256,
-// N = keep. Inverse: K = keep, N = 256. A workgroup keeps its 64-column basis tile resident in
-// LDS, walks over row tiles of 256 blocks, stages X through LDS in 32-wide slices and feeds
-// v_mfma_f32_32x32x2_f32: eight wavefronts, each owning a 32 x 64 piece of the output tile.
+// N = keep. Inverse: K = keep, N = 256. A workgroup keeps a 64- or 128-column basis tile resident
+// in LDS and walks over row tiles of 256 blocks; each of its eight wavefronts owns 32 rows, holds
+// their X values in registers and feeds v_mfma_f32_32x32x2_f32.
 #include <cmath>
 #include <mutex>
 
@@ -19,12 +19,9 @@
 namespace krk {
 
 constexpr int kDctB = 256;      // block length
-constexpr int kThreads = 512;   // eight wavefronts: two per SIMD, so one can wait while one multiplies
+constexpr int kThreads = 512;   // eight wavefronts, two per SIMD
 constexpr int kTileM = 256;     // rows (blocks) per output tile: 32 per wavefront
-constexpr int kTileN = 64;      // basis columns per workgroup
-constexpr int kSliceK = 32;     // reduction slice staged per step
-constexpr int kXsLd = kSliceK + 1;   // padded: a column read by 32 lanes hits 32 banks
-constexpr int kStageVec = (kTileM * kSliceK / 4) / kThreads;   // float4 loads per thread per slice
+constexpr int kSliceK = 32;     // reduction slice held in registers per step
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
@@ -41,84 +38,106 @@ __global__ void dct2_basis_kernel(float* __restrict__ fwd, float* __restrict__ i
 }
 
 // Y[M, N] = X[M, K] * Bm[K, N]; ldx / ldb / ldy are row strides in floats. K is a multiple of 32,
-// N a multiple of 64 (both <= 256). grid.x workgroups share the row tiles, grid.y = N / 64.
+// N a multiple of 32 * NT. grid.x workgroups share the row tiles, grid.y = N / (32 * NT).
 //
-// Pipeline per 32-wide slice of the reduction: the next slice of X is requested from HBM into
-// registers, the current slice (already in LDS) is multiplied, and only then are the registers
-// written to the other LDS buffer, so the memory latency sits behind 32 matrix instructions.
+// The basis tile [K][32 * NT] sits in LDS for the whole launch and is only read. X never
+// passes through LDS: the matrix instruction takes, per lane (r = lane % 32, h = lane / 32),
+// one value A[r][k_h] for its two reduction indices k_0, k_1, and the order in which the
+// reduction indices are consumed is free as long as the basis rows follow it. So lane (r, h)
+// loads the 16 consecutive floats X[row r][32 s + 16 h ...] of slice s as four float4 and
+// step j multiplies them against basis rows 32 s + 16 h + j. Wavefronts never wait on each
+// other inside the loop; the next slice's loads are in flight while this one multiplies.
+template <int NT>
 __global__ __launch_bounds__(kThreads) void dct2_gemm_kernel(const float* __restrict__ X, int64_t ldx,
                                                              const float* __restrict__ Bm, int ldb,
                                                              float* __restrict__ Y, int64_t ldy,
                                                              int64_t M, int K) {
-  extern __shared__ float lds[];
-  float* Bs = lds;                                  // [K][kTileN], resident for the whole launch
-  float* Xs = lds + (size_t)K * kTileN;             // 2 x [kTileM][kXsLd]
+  constexpr int kTileN = 32 * NT;
+  extern __shared__ float Bs[];                     // [K][kTileN]
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  const int r = lane & 31;
+  const int h = lane >> 5;
   const int n0 = blockIdx.y * kTileN;
 
   for (int i = tid; i < K * (kTileN / 4); i += kThreads) {
-    const int r = i / (kTileN / 4);
-    const int c4 = i - r * (kTileN / 4);
-    reinterpret_cast<float4*>(Bs)[i] = *reinterpret_cast<const float4*>(Bm + (size_t)r * ldb + n0 + c4 * 4);
+    const int br = i / (kTileN / 4);
+    const int c4 = i - br * (kTileN / 4);
+    reinterpret_cast<float4*>(Bs)[i] = *reinterpret_cast<const float4*>(Bm + (size_t)br * ldb + n0 + c4 * 4);
   }
+  __syncthreads();
 
   const int64_t tiles = (M + kTileM - 1) / kTileM;
   const int slices = K / kSliceK;
+  // Rows past the end are clamped, not masked: row r of X only reaches row r of Y, and those
+  // rows are never stored, so the loads carry no branch.
+  auto row_ptr = [&](int64_t tile) {
+    int64_t row = tile * kTileM + wave * 32 + r;
+    if (row >= M) row = M - 1;
+    return X + row * ldx + 16 * h;
+  };
+  const float* bs = Bs + (size_t)(16 * h) * kTileN + r;
+  const float* xrow = row_ptr(blockIdx.x);
+  // X runs two slices ahead of the multiplies (K >= 64, so a tile has at least two slices).
+  float4 cur[4], nx1[4], nx2[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    cur[q] = reinterpret_cast<const float4*>(xrow)[q];
+    nx1[q] = reinterpret_cast<const float4*>(xrow + kSliceK)[q];
+  }
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int64_t m0 = tile * kTileM;
-    v16f acc0 = {0}, acc1 = {0};
-    float4 regs[kStageVec];
-    auto fetch = [&](int slice) {
+    // the tile after this one (or this one again at the end: its values are then unused)
+    const float* xnext = row_ptr(tile + gridDim.x < tiles ? tile + gridDim.x : tile);
+    v16f acc[NT];
 #pragma unroll
-      for (int it = 0; it < kStageVec; ++it) {
-        const int i = it * kThreads + tid;       // float4 index inside the slice
-        const int r = i >> 3;                    // 8 float4 per 32-float row piece
-        const int c4 = i & 7;
-        regs[it] = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (m0 + r < M)
-          regs[it] = *reinterpret_cast<const float4*>(X + (m0 + r) * ldx + slice * kSliceK + c4 * 4);
-      }
-    };
-    auto park = [&](int buf) {
-      float* dst = Xs + buf * (kTileM * kXsLd);
+    for (int t = 0; t < NT; ++t) acc[t] = v16f{0};
+    float bcur[NT], bnxt[NT];
 #pragma unroll
-      for (int it = 0; it < kStageVec; ++it) {
-        const int i = it * kThreads + tid;
-        float* d = dst + (i >> 3) * kXsLd + (i & 7) * 4;
-        d[0] = regs[it].x; d[1] = regs[it].y; d[2] = regs[it].z; d[3] = regs[it].w;
-      }
-    };
-    fetch(0);
-    park(0);
-    __syncthreads();
+    for (int t = 0; t < NT; ++t) bcur[t] = bs[32 * t];
     for (int s = 0; s < slices; ++s) {
-      const int buf = s & 1;
-      if (s + 1 < slices) fetch(s + 1);
-      const float* xs = Xs + buf * (kTileM * kXsLd) + (wave * 32 + (lane & 31)) * kXsLd + (lane >> 5);
-      const float* bs = Bs + (size_t)(s * kSliceK + (lane >> 5)) * kTileN + (lane & 31);
+      // slice s + 2 of this tile, or one of the first two slices of the next tile
+      const float* ahead = s + 2 < slices ? xrow + (s + 2) * kSliceK : xnext + (s + 2 - slices) * kSliceK;
 #pragma unroll
-      for (int kk = 0; kk < kSliceK; kk += 2) {
-        const float a = xs[kk];
-        const float b0 = bs[kk * kTileN];
-        const float b1 = bs[kk * kTileN + 32];
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b0, acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b1, acc1, 0, 0, 0);
+      for (int q = 0; q < 4; ++q) nx2[q] = reinterpret_cast<const float4*>(ahead)[q];
+      __builtin_amdgcn_sched_barrier(0);   // keep the requests ahead of the multiplies
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float a4[4] = {cur[q].x, cur[q].y, cur[q].z, cur[q].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          // basis values of the following step are requested before this step multiplies
+          const int step = s * 16 + q * 4 + e + 1;
+          const float* brow = bs + (size_t)((step >> 4) * kSliceK + (step & 15)) * kTileN;
+          const bool more = step < slices * 16;
+#pragma unroll
+          for (int t = 0; t < NT; ++t) bnxt[t] = brow[more ? 32 * t : 32 * t - kSliceK * kTileN];
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[e], bcur[t], acc[t], 0, 0, 0);
+#pragma unroll
+          for (int t = 0; t < NT; ++t) bcur[t] = bnxt[t];
+        }
       }
-      if (s + 1 < slices) park(buf ^ 1);
-      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        cur[q] = nx1[q];
+        nx1[q] = nx2[q];
+      }
     }
     // accumulator element i of lane l is C[(i / 4) * 8 + (l / 32) * 4 + i % 4][l % 32]
+    const int64_t base = tile * kTileM + wave * 32;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int r = wave * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-      if (m0 + r < M) {
-        float* y = Y + (m0 + r) * ldy + n0 + (lane & 31);
-        y[0] = acc0[i];
-        y[32] = acc1[i];
+      const int64_t orow = base + (i >> 2) * 8 + h * 4 + (i & 3);
+      if (orow < M) {
+        float* y = Y + orow * ldy + n0 + r;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) y[32 * t] = acc[t][i];
       }
     }
+    xrow = xnext;
   }
 }
 
@@ -142,7 +161,7 @@ static int32_t ensure_basis(hipStream_t s) {
 static int32_t dct2_run(const float* in, float* out, int64_t n, int32_t keep, uint32_t flags, bool forward) {
   KRK_TRY(ensure_runtime());
   KRK_TRY(check_flags(flags));
-  if (n < 0 || n % kDctB != 0 || keep <= 0 || keep > kDctB || keep % kTileN != 0 || (n > 0 && (!in || !out))) {
+  if (n < 0 || n % kDctB != 0 || keep <= 0 || keep > kDctB || keep % 64 != 0 || (n > 0 && (!in || !out))) {
     set_error("dct2: n must be a multiple of 256 and keep one of 64, 128, 192, 256");
     return KRK_E_ARGUMENT;
   }
@@ -172,14 +191,19 @@ static int32_t dct2_run(const float* in, float* out, int64_t n, int32_t keep, ui
   const int K = forward ? kDctB : keep;
   const int N = forward ? keep : kDctB;
   const float* basis = forward ? g_basis_fwd : g_basis_inv;
-  const size_t lds_bytes = sizeof(float) * ((size_t)K * kTileN + 2 * kTileM * kXsLd);
+  const int nt = (N % 128 == 0) ? 4 : 2;          // 128-column tiles where the width allows
+  const int tile_n = 32 * nt;
+  const size_t lds_bytes = sizeof(float) * (size_t)K * tile_n;
   const int64_t tiles = (M + kTileM - 1) / kTileM;
-  int64_t gx = tiles < 256 / (N / kTileN) ? tiles : 256 / (N / kTileN);   // one workgroup per CU
+  const int64_t per_cu = lds_bytes <= 64 * 1024 ? 2 : 1;   // workgroups that fit one CU's LDS
+  int64_t gx = 256 * per_cu / (N / tile_n);
+  if (gx > tiles) gx = tiles;
   if (gx < 1) gx = 1;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(dct2_gemm_kernel),
+  auto kernel = nt == 4 ? dct2_gemm_kernel<4> : dct2_gemm_kernel<2>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (e == hipSuccess) {
-    hipLaunchKernelGGL(dct2_gemm_kernel, dim3((unsigned)gx, (unsigned)(N / kTileN)), dim3(kThreads), lds_bytes, s,
+    hipLaunchKernelGGL(kernel, dim3((unsigned)gx, (unsigned)(N / tile_n)), dim3(kThreads), lds_bytes, s,
                        d_in, (int64_t)K, basis, kDctB, d_out, (int64_t)N, M, K);
     e = hipGetLastError();
   }

@@ -448,9 +448,9 @@ int32_t krk_event_destroy(krk_event* e) {
 }
 // Every API object begins with an ObjBase, so its stream is reachable from any handle.
 int32_t krk_event_record(krk_event* e, void* object) {
-  if (!e || !object) return KRK_E_ARGUMENT;
+  if (!e) return KRK_E_ARGUMENT;
   ObjBase* b = reinterpret_cast<ObjBase*>(object);
-  KRK_HIP(hipEventRecord(e->ev, b->stream));
+  KRK_HIP(hipEventRecord(e->ev, b ? b->stream : nullptr));
   return KRK_SUCCESS;
 }
 int32_t krk_event_elapsed_ms(krk_event* start, krk_event* stop, float* ms) {

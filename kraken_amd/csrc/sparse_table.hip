@@ -155,6 +155,119 @@ __global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, InitK init,
   pull_body<VEC>(tv, init, ids, i, i < n, threadIdx.x & (group - 1), out, dim, elems, group);
 }
 
+// ---------------------------------------------------------------------------
+// pooled pull: Pull fused with the worker's jagged sum / mean (pytorch/py/jagged_ops.cc:14-56,
+// 206-236, called from pytorch/jagged_embedding.py:32-52), in two launches.
+//   1. every position is probed on its own (four lanes per id, all positions in flight at once);
+//      ids that are not in the table are inserted and their creator initialises the record, as
+//      in pull_body; the row number of each position goes to a scratch array (a position that
+//      meets a row while its creator is still numbering it leaves the entry open).
+//   2. one lane group per bag adds the bag's records in position order: the first row is copied,
+//      the others are added to it, exactly the reference's order, so the pooled row is
+//      bit-identical to pooling the pulled rows on the host. The loads of a bag do not depend
+//      on each other and are issued four at a time.
+// The n pulled rows themselves are never written anywhere.
+// ---------------------------------------------------------------------------
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pooled_probe_kernel(TableView tv, InitK init,
+                                                              const uint64_t* __restrict__ ids, int64_t n,
+                                                              uint32_t* __restrict__ rows, int elems) {
+  const int64_t p = (int64_t)blockIdx.x * (kBlock / kBucket) + threadIdx.x / kBucket;
+  const int gl = threadIdx.x & (kBucket - 1);
+  const bool active = p < n;
+  const uint64_t id = active ? ids[p] : 0;
+  const ProbeResult pr = probe_insert(tv, id, active, gl, kBucket);
+  if (!active) return;
+  if (pr.fresh && pr.owner && pr.row != kEmptyRow) {
+    float* rec = tv.recs + (int64_t)pr.row * tv.stride;
+    for (int e = gl; e < elems; e += kBucket) {
+      float v[VEC];
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) v[c] = init_element(init, id, (int64_t)e * VEC + c);
+      vstore<VEC>(rec + e * VEC, v);
+    }
+  }
+  if (gl == 0) rows[p] = pr.row;
+}
+
+constexpr int kPoolAhead = 4;   // records of one bag requested together
+
+// One lane looking an id up by itself (no votes): the rare second look of pooled_sum_kernel.
+__device__ inline uint32_t probe_find_alone(const TableView& tv, uint64_t id) {
+  if (id == kEmptyKey) {
+    const Slot* s = &tv.slots[tv.mask + 1];
+    return __atomic_load_n(&s->key, __ATOMIC_RELAXED) != kEmptyKey
+               ? (uint32_t)__atomic_load_n(&s->row_epoch, __ATOMIC_RELAXED) : kEmptyRow;
+  }
+  const uint64_t nb_mask = tv.mask >> 2;
+  uint64_t b = mix64(id) & nb_mask;
+  for (uint64_t tried = 0; tried <= nb_mask; ++tried) {
+    for (int i = 0; i < kBucket; ++i) {
+      const Slot* s = &tv.slots[b * kBucket + i];
+      const unsigned long long key = __atomic_load_n(&s->key, __ATOMIC_RELAXED);
+      if (key == id) return (uint32_t)__atomic_load_n(&s->row_epoch, __ATOMIC_RELAXED);
+      if (key == kEmptyKey) return kEmptyRow;
+    }
+    b = (b + 1) & nb_mask;
+  }
+  return kEmptyRow;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pooled_sum_kernel(TableView tv, const uint32_t* __restrict__ rows,
+                                                            const uint64_t* __restrict__ ids,
+                                                            int64_t n, const long long* __restrict__ offsets,
+                                                            int64_t bags, const float* __restrict__ weights,
+                                                            int mean, float patch, float* __restrict__ out,
+                                                            int dim, int elems, int group) {
+  const int per_block = kBlock / group;
+  const int64_t bag = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  const int gl = threadIdx.x & (group - 1);
+  if (bag >= bags || gl >= elems) return;      // the host only launches this with elems <= group
+  long long lo = offsets[bag], hi = offsets[bag + 1];
+  if (lo < 0) lo = 0;
+  if (hi > n) hi = n;
+  float acc[VEC];
+#pragma unroll
+  for (int c = 0; c < VEC; ++c) acc[c] = patch;
+  for (long long j0 = lo; j0 < hi; j0 += kPoolAhead) {
+    float v[kPoolAhead][VEC];
+    float w[kPoolAhead];
+#pragma unroll
+    for (int u = 0; u < kPoolAhead; ++u) {
+      const long long j = j0 + u;
+      uint32_t row = j < hi ? rows[j] : kEmptyRow;
+      // A position that met its id while another position's group was still creating the row
+      // could not learn the row number in the first launch; by now it is in the index.
+      if (j < hi && row == kEmptyRow) row = probe_find_alone(tv, ids[j]);
+      w[u] = (weights && j < hi) ? weights[j] : 1.0f;
+      if (row != kEmptyRow) {
+        vload<VEC>(tv.recs + (int64_t)row * tv.stride + gl * VEC, v[u]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) v[u][c] = 0.0f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kPoolAhead; ++u) {
+      const long long j = j0 + u;
+      if (j >= hi) break;
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) {
+        // pytorch/jagged_embedding.py:41-45 scales the rows before pooling
+        const float x = weights ? v[u][c] * w[u] : v[u][c];
+        acc[c] = j == lo ? x : acc[c] + x;
+      }
+    }
+  }
+  if (mean && hi > lo) {
+    const float ratio = (float)(1.0 / (double)(float)(hi - lo));   // jagged_ops.cc:219
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) acc[c] = acc[c] * ratio;
+  }
+  vstore<VEC>(out + bag * (int64_t)dim + gl * VEC, acc);
+}
+
 template <int OPT, int VEC>
 __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64_t* __restrict__ ids,
                                                       int64_t n, const float* __restrict__ grads,
@@ -839,6 +952,67 @@ int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* ou
   KRK_HIP(hipGetLastError());
   if ((flags & KRK_ASYNC) && sparse_near_full(t)) KRK_TRY(sparse_publish(&t, 1, t->stream));
   KRK_TRY(t->output_back(out, (size_t)n * t->dim, flags, 1));
+  return sparse_finish(t, flags);
+}
+
+int32_t krk_sparse_pull_pooled(krk_sparse* t, const uint64_t* ids, int64_t n, const int64_t* offsets,
+                               int64_t bags, const float* weights, int32_t mode, float patch_value,
+                               float* out, uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (n < 0 || bags < 0 || (mode != KRK_POOL_SUM && mode != KRK_POOL_MEAN) || !offsets ||
+      (n > 0 && !ids) || (bags > 0 && !out))
+    return KRK_E_ARGUMENT;
+  if (t->elems > t->group) {
+    set_error("pooled pull supports rows of at most %d floats for this layout", 64 * t->vec);
+    return KRK_INTERFACE_UNIMPLEMENTED;
+  }
+  if ((flags & KRK_DEVICE_PTRS) && t->vec == 4 && !aligned16(out)) {
+    set_error("device output must be 16-byte aligned");
+    return KRK_E_ARGUMENT;
+  }
+  if (bags > max_ids_per_launch(t->group) || n > max_ids_per_launch(kBucket)) {
+    set_error("at most %lld bags per call for this row width; split the request",
+              (long long)max_ids_per_launch(t->group));
+    return KRK_E_CAPACITY;
+  }
+  if (!(flags & KRK_DEVICE_PTRS) && (offsets[0] != 0 || offsets[bags] != n)) {
+    set_error("offsets must start at 0 and end at the number of ids");
+    return KRK_E_ARGUMENT;
+  }
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (bags == 0) return sparse_finish(t, flags);
+  KRK_TRY(sparse_ensure_room(t, n));
+  const uint64_t* d_ids = nullptr;
+  const long long* d_off;
+  const float* d_w = nullptr;
+  float* d_out;
+  if (n > 0) KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
+  KRK_TRY(t->input(reinterpret_cast<const long long*>(offsets), (size_t)bags + 1, flags, 1, &d_off));
+  if (weights && n > 0) KRK_TRY(t->input(weights, (size_t)n, flags, 2, &d_w));
+  KRK_TRY(t->output(out, (size_t)bags * t->dim, flags, 3, &d_out));
+  KRK_TRY(sparse_next_epoch(t, n));
+  KRK_TRY(t->scratch[5].reserve((size_t)(n > 0 ? n : 1) * sizeof(uint32_t)));
+  uint32_t* rows = t->scratch[5].as<uint32_t>();
+  const int per_block = kBlock / t->group;
+  const dim3 probe_grid(grid_for(n, kBlock / kBucket)), grid(grid_for(bags, per_block)), block(kBlock);
+  const int mean = mode == KRK_POOL_MEAN;
+  if (t->vec == 4) {
+    if (n > 0)
+      hipLaunchKernelGGL((pooled_probe_kernel<4>), probe_grid, block, 0, t->stream, t->view(), t->initk, d_ids,
+                         n, rows, t->elems);
+    hipLaunchKernelGGL((pooled_sum_kernel<4>), grid, block, 0, t->stream, t->view(), rows, d_ids, n, d_off, bags, d_w,
+                       mean, patch_value, d_out, (int)t->dim, t->elems, t->group);
+  } else {
+    if (n > 0)
+      hipLaunchKernelGGL((pooled_probe_kernel<1>), probe_grid, block, 0, t->stream, t->view(), t->initk, d_ids,
+                         n, rows, t->elems);
+    hipLaunchKernelGGL((pooled_sum_kernel<1>), grid, block, 0, t->stream, t->view(), rows, d_ids, n, d_off, bags, d_w,
+                       mean, patch_value, d_out, (int)t->dim, t->elems, t->group);
+  }
+  KRK_HIP(hipGetLastError());
+  if ((flags & KRK_ASYNC) && sparse_near_full(t)) KRK_TRY(sparse_publish(&t, 1, t->stream));
+  KRK_TRY(t->output_back(out, (size_t)bags * t->dim, flags, 3));
   return sparse_finish(t, flags);
 }
 

@@ -100,6 +100,10 @@ def lib():
         "kro_dense_value": (vp, [vp]),
         "kro_dedup": (i64, [pu, i64, pu, pi]),
         "kro_dedup_sum": (i64, [pu, i64, pf, i64, pu, pf]),
+        "kro_jagged_sum_forward": (None, [pf, i64, pi, i64, f32, pf]),
+        "kro_jagged_mean_forward": (None, [pf, i64, pi, i64, f32, pf]),
+        "kro_jagged_sum_backward": (None, [pi, i64, pf, i64, pf]),
+        "kro_jagged_mean_backward": (None, [pi, i64, pf, i64, pf]),
         "kro_abs": (None, [pf, pf, i64]),
         "kro_topk_chunked": (None, [pf, i64, pf, i64, i64]),
         "kro_topk": (None, [pf, i64, pf, i64, i64]),
@@ -143,6 +147,26 @@ def ref_lib():
                                C.POINTER(C.c_float), i64]
     L.ref_map_keys.restype = i64
     L.ref_map_keys.argtypes = [C.c_void_p, C.POINTER(u64)]
+    return L
+
+
+_REF_JAGGED_PATH = os.path.join(_HERE, "_ref", "libkraken_ref_jagged.so")
+
+
+def ref_jagged_lib():
+    """The reference's own jagged pooling loops (pytorch/py/jagged_ops.cc) compiled in place,
+    or None when absent."""
+    if not os.path.exists(_REF_JAGGED_PATH):
+        return None
+    L = C.CDLL(_REF_JAGGED_PATH)
+    i64, f32 = C.c_int64, C.c_float
+    pf, pi = C.POINTER(f32), C.POINTER(i64)
+    for name in ("ref_jagged_sum_forward", "ref_jagged_mean_forward"):
+        getattr(L, name).restype = None
+        getattr(L, name).argtypes = [pf, i64, pi, i64, f32, pf]
+    for name in ("ref_jagged_sum_backward", "ref_jagged_mean_backward"):
+        getattr(L, name).restype = None
+        getattr(L, name).argtypes = [pi, i64, pf, i64, pf]
     return L
 
 
@@ -306,6 +330,30 @@ def dedup_sum(ids, grads):
     u = lib().kro_dedup_sum(_p(ids, C.c_uint64), ids.size, _p(grads, C.c_float), dim,
                             _p(uids, C.c_uint64), _p(out, C.c_float))
     return uids[:u].copy(), out[:u].copy()
+
+
+def jagged_forward(values, offsets, mode="sum", patch_value=0.0):
+    """pytorch/py/jagged_ops.cc SumForward / MeanForward on [rows, col] values."""
+    values = _f32(values)
+    offsets = np.ascontiguousarray(offsets, np.int64)
+    col = values.shape[-1]
+    k = offsets.size - 1
+    out = np.empty((k, col), np.float32)
+    fn = lib().kro_jagged_sum_forward if mode == "sum" else lib().kro_jagged_mean_forward
+    fn(_p(values, C.c_float), col, _p(offsets, C.c_int64), k, patch_value, _p(out, C.c_float))
+    return out
+
+
+def jagged_backward(offsets, grads, mode="sum"):
+    """Gradient of jagged_forward with respect to the values: [offsets[-1], col]."""
+    grads = _f32(grads)
+    offsets = np.ascontiguousarray(offsets, np.int64)
+    col = grads.shape[-1]
+    k = offsets.size - 1
+    out = np.zeros((int(offsets[-1]), col), np.float32)
+    fn = lib().kro_jagged_sum_backward if mode == "sum" else lib().kro_jagged_mean_backward
+    fn(_p(offsets, C.c_int64), k, _p(grads, C.c_float), col, _p(out, C.c_float))
+    return out
 
 
 def init_row(init_, id_, dim):

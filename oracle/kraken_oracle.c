@@ -828,6 +828,63 @@ int64_t kro_dedup_sum(const uint64_t* ids, int64_t n, const float* grads, int64_
 }
 
 /* ========================================================================== */
+/* jagged pooling                                                             */
+/* ========================================================================== */
+
+/* pytorch/py/jagged_ops.cc:14-56 (the AVX2 variant :59-110 does the same fp32 adds) */
+void kro_jagged_sum_forward(const float* v, int64_t col, const int64_t* offsets, int64_t k,
+                            float patch_value, float* out) {
+  for (int64_t i = 0; i < k; ++i) {
+    float* o = out + i * col;
+    if (offsets[i + 1] <= offsets[i]) {
+      for (int64_t l = 0; l < col; ++l) o[l] = patch_value;
+      continue;
+    }
+    memcpy(o, v + offsets[i] * col, sizeof(float) * (size_t)col);
+    for (int64_t j = offsets[i] + 1; j < offsets[i + 1]; ++j) {
+      const float* r = v + j * col;
+      for (int64_t l = 0; l < col; ++l) o[l] += r[l];
+    }
+  }
+}
+
+/* pytorch/py/jagged_ops.cc:206-236 : `T ratio = 1.0 / T(len)` divides in double */
+static float jagged_ratio(int64_t len) {
+  return (float)(1.0 / (double)(float)len);
+}
+
+void kro_jagged_mean_forward(const float* v, int64_t col, const int64_t* offsets, int64_t k,
+                             float patch_value, float* out) {
+  kro_jagged_sum_forward(v, col, offsets, k, patch_value, out);
+  for (int64_t i = 0; i < k; ++i) {
+    if (offsets[i + 1] <= offsets[i]) continue;
+    const float ratio = jagged_ratio(offsets[i + 1] - offsets[i]);
+    float* o = out + i * col;
+    for (int64_t l = 0; l < col; ++l) o[l] *= ratio;
+  }
+}
+
+void kro_jagged_sum_backward(const int64_t* offsets, int64_t k, const float* grads, int64_t col,
+                             float* vgrads) {
+  for (int64_t i = 0; i < k; ++i)
+    for (int64_t j = offsets[i]; j < offsets[i + 1]; ++j)
+      memcpy(vgrads + j * col, grads + i * col, sizeof(float) * (size_t)col);
+}
+
+/* pytorch/py/jagged_ops.cc:303-334 */
+void kro_jagged_mean_backward(const int64_t* offsets, int64_t k, const float* grads, int64_t col,
+                              float* vgrads) {
+  for (int64_t i = 0; i < k; ++i) {
+    if (offsets[i + 1] <= offsets[i]) continue;
+    const float ratio = jagged_ratio(offsets[i + 1] - offsets[i]);
+    float* first = vgrads + offsets[i] * col;
+    for (int64_t l = 0; l < col; ++l) first[l] = grads[i * col + l] * ratio;
+    for (int64_t j = offsets[i] + 1; j < offsets[i + 1]; ++j)
+      memcpy(vgrads + j * col, first, sizeof(float) * (size_t)col);
+  }
+}
+
+/* ========================================================================== */
 /* threshold codec                                                            */
 /* ========================================================================== */
 

@@ -164,6 +164,24 @@ int64_t kro_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv);
 int64_t kro_dedup_sum(const uint64_t* ids, int64_t n, const float* grads,
                       int64_t dim, uint64_t* uids, float* out);
 
+/* ---- jagged (multi-hot) pooling ------------------------------------------- */
+/* pytorch/py/jagged_ops.cc:14-56 : out[i] = v[offsets[i]] copied, then the bag's other
+ * rows added in position order; an empty bag gets patch_value. v [rows, col], out [k, col]. */
+void kro_jagged_sum_forward(const float* v, int64_t col, const int64_t* offsets, int64_t k,
+                            float patch_value, float* out);
+/* pytorch/py/jagged_ops.cc:206-236 : the sum, then times (float)(1.0 / float(len)). */
+void kro_jagged_mean_forward(const float* v, int64_t col, const int64_t* offsets, int64_t k,
+                             float patch_value, float* out);
+/* Derivative of the sum: every row of bag i receives grads[i]. This is NOT what
+ * pytorch/py/jagged_ops.cc:148-160 does: its destination pointer never advances, so only
+ * the first row of a bag is written and the others stay uninitialised. The intended
+ * semantics (the transpose of the forward) is what is stated here. */
+void kro_jagged_sum_backward(const int64_t* offsets, int64_t k, const float* grads, int64_t col,
+                             float* vgrads);
+/* pytorch/py/jagged_ops.cc:303-334 : every row of bag i receives grads[i] * ratio. */
+void kro_jagged_mean_backward(const int64_t* offsets, int64_t k, const float* grads, int64_t col,
+                              float* vgrads);
+
 /* ---- threshold ("DCT") codec --------------------------------------------- */
 void kro_abs(const float* x, float* y, int64_t n);            /* t/math.cc:540-546 */
 /* t/math.cc:564-626 with t_num workers: chunk stride n / t_num, elements past

@@ -451,3 +451,87 @@ def test_dense_table_and_coo(oracle):
     # repeated COO indices accumulate (t/math.cc:1043 "Should add the r maybe same")
     d = oracle.coo_to_dense([3, 3, 5], [1.0, 2.0, 4.0], 8)
     assert np.array_equal(d, np.array([0, 0, 0, 3, 0, 4, 0, 0], np.float32))
+
+
+# --------------------------------------------------------------------------- #
+# jagged pooling vs the compiled reference, a library routine and autograd
+# --------------------------------------------------------------------------- #
+
+def _jagged_cases():
+    for c in json.load(open(os.path.join(GOLDEN, "ref_jagged.json")))["cases"]:
+        col = c["col"]
+        off = np.array(c["offsets"], np.int64)
+        yield (c, col, off, np.array(c["values"], np.float32).reshape(-1, col),
+               np.array(c["grads"], np.float32).reshape(-1, col))
+
+
+def test_jagged_forward_matches_reference_vectors(oracle):
+    for c, col, off, v, g in _jagged_cases():
+        for mode in ("sum", "mean"):
+            want = np.array(c[mode + "_forward"], np.float32).reshape(-1, col)
+            got = oracle.jagged_forward(v, off, mode, c["patch_value"])
+            assert np.array_equal(got, want), (mode, col)
+
+
+def test_jagged_backward_matches_reference_vectors(oracle):
+    for c, col, off, v, g in _jagged_cases():
+        want = np.array(c["mean_backward"], np.float32).reshape(-1, col)
+        got = oracle.jagged_backward(off, g, "mean")
+        live = want != np.float32(c["sentinel"])      # rows of non-empty bags
+        assert live.all()
+        assert np.array_equal(got, want)
+        # the reference's SumBackward only ever writes the first row of a bag; where it wrote,
+        # the oracle agrees, and everywhere else the oracle holds the bag's gradient
+        ref = np.array(c["sum_backward"], np.float32).reshape(-1, col)
+        got = oracle.jagged_backward(off, g, "sum")
+        firsts = off[:-1][off[1:] > off[:-1]]
+        wrote = np.zeros(ref.shape[0], bool)
+        wrote[firsts] = True
+        assert np.array_equal(got[wrote], ref[wrote])
+        assert (ref[~wrote] == np.float32(c["sentinel"])).all()
+        bag_of = np.repeat(np.arange(off.size - 1), np.diff(off))
+        assert np.array_equal(got, g[bag_of])
+
+
+def test_jagged_matches_torch_segment_reduce_and_autograd(oracle):
+    """Independent of the reference build: torch.segment_reduce for the forward, autograd of
+    an index_add formulation for the backward (the transpose the reference's SumBackward was
+    meant to be)."""
+    import torch
+    rng = np.random.default_rng(9)
+    lengths = rng.integers(0, 9, size=40)
+    off = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
+    # values on a binary grid: every order of summation gives the same fp32 result
+    v = (rng.integers(-512, 513, size=(int(off[-1]), 6)) / 256.0).astype(np.float32)
+    tv = torch.tensor(v, requires_grad=True)
+    for mode in ("sum", "mean"):
+        want = torch.segment_reduce(tv, mode, offsets=torch.tensor(off))
+        got = oracle.jagged_forward(v, off, mode, 0.5)
+        nonempty = lengths > 0
+        np.testing.assert_allclose(got[nonempty], want.detach().numpy()[nonempty], rtol=1e-6, atol=0)
+        assert (got[~nonempty] == 0.5).all()
+        g = (rng.integers(-64, 65, size=(lengths.size, 6)) / 64.0).astype(np.float32)
+        bag_of = torch.tensor(np.repeat(np.arange(lengths.size), lengths))
+        pooled = torch.zeros(lengths.size, 6).index_add(0, bag_of, tv)
+        if mode == "mean":
+            pooled = pooled / torch.tensor(np.maximum(lengths, 1), dtype=torch.float32)[:, None]
+        (gv,) = torch.autograd.grad(pooled, tv, torch.tensor(g))
+        np.testing.assert_allclose(oracle.jagged_backward(off, g, mode), gv.numpy(), rtol=1e-6, atol=0)
+
+
+def test_jagged_matches_reference_live(oracle):
+    L = oracle.ref_jagged_lib()
+    if L is None:
+        pytest.skip("oracle/_ref not built (reference tree absent)")
+    import ctypes as C
+    rng = np.random.default_rng(10)
+    lengths = rng.integers(0, 30, size=200)
+    off = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
+    for col in (3, 8, 32):
+        v = rng.standard_normal((int(off[-1]), col)).astype(np.float32)
+        for mode in ("sum", "mean"):
+            want = np.empty((lengths.size, col), np.float32)
+            getattr(L, "ref_jagged_%s_forward" % mode)(
+                v.ctypes.data_as(C.POINTER(C.c_float)), col, off.ctypes.data_as(C.POINTER(C.c_int64)),
+                lengths.size, -1.5, want.ctypes.data_as(C.POINTER(C.c_float)))
+            assert np.array_equal(oracle.jagged_forward(v, off, mode, -1.5), want)
