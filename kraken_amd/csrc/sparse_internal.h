@@ -71,17 +71,27 @@ struct ProbeResult {
 
 __device__ __forceinline__ int wave_lane() { return (int)(threadIdx.x & (kWave - 1)); }
 
-// id -> row for every lane of the group, kEmptyRow when absent.
-__device__ inline uint32_t probe_find(const TableView& tv, uint64_t id, bool active, int gl, int group) {
+// What a search that never writes reports: whether the id has a slot, and the slot's second
+// word (row number in the low half, number of the launch that created the row in the high half).
+struct FindResult {
+  bool found;
+  unsigned long long row_epoch;
+};
+
+__device__ inline FindResult probe_find_slot(const TableView& tv, uint64_t id, bool active, int gl,
+                                             int group) {
   const int lane = wave_lane();
   const int base = lane & ~(group - 1);
   const uint64_t nb_mask = tv.mask >> 2;
-  uint32_t row = kEmptyRow;
+  FindResult res;
+  res.found = false;
+  res.row_epoch = ~0ull;
   bool done = !active;
   if (active && id == kEmptyKey) {   // the id that equals the empty marker has a slot of its own
     unsigned long long key, re;
     unpack_slot(*reinterpret_cast<const uint4*>(&tv.slots[tv.mask + 1]), key, re);
-    row = key != kEmptyKey ? (uint32_t)re : kEmptyRow;
+    res.found = key != kEmptyKey;
+    if (res.found) res.row_epoch = re;
     done = true;
   }
   uint64_t b = mix64(id) & nb_mask;
@@ -104,9 +114,10 @@ __device__ inline uint32_t probe_find(const TableView& tv, uint64_t id, bool act
         action = me ? 2 : 3;
       }
     }
-    const uint32_t r = __shfl((uint32_t)re, src);
+    const unsigned long long r = __shfl(re, src);
     if (action == 1) {
-      row = r;
+      res.found = true;
+      res.row_epoch = r;
       done = true;
     } else if (action == 2) {
       done = true;
@@ -116,7 +127,13 @@ __device__ inline uint32_t probe_find(const TableView& tv, uint64_t id, bool act
     }
     if (__ballot(!done) == 0ull) break;
   }
-  return row;
+  return res;
+}
+
+// id -> row for every lane of the group, kEmptyRow when absent.
+__device__ inline uint32_t probe_find(const TableView& tv, uint64_t id, bool active, int gl, int group) {
+  const FindResult f = probe_find_slot(tv, id, active, gl, group);
+  return f.found ? (uint32_t)f.row_epoch : kEmptyRow;
 }
 
 // id -> row, claiming a slot and the next free row when absent.

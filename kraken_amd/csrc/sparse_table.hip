@@ -50,7 +50,18 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
                                           int gl, float* __restrict__ out, int dim, int elems,
                                           int group) {
   const uint64_t id = active ? ids[i] : 0;
-  const ProbeResult pr = probe_insert(tv, id, active, gl, group);
+  // Most ids are resident: a search that never writes settles them, and only a wavefront that
+  // holds a missing id goes through the claiming search as well.
+  const FindResult f = probe_find_slot(tv, id, active, gl, group);
+  ProbeResult pr;
+  pr.row = (uint32_t)f.row_epoch;
+  pr.owner = false;
+  pr.fresh = pr.row == kEmptyRow || (uint32_t)(f.row_epoch >> 32) == tv.epoch;
+  const bool miss = active && !f.found;
+  if (__any(miss)) {
+    const ProbeResult q = probe_insert(tv, id, miss, gl, group);
+    if (miss) pr = q;
+  }
   if (!active) return;
   const uint32_t row = pr.row;
   const bool owner = pr.owner;
