@@ -212,6 +212,27 @@ int32_t krk_sparse_import(krk_sparse* t, const uint64_t* ids, int64_t n, const f
 int32_t krk_sparse_export(krk_sparse* t, uint64_t* ids, float* vals, int32_t state_type,
                           float* state, int64_t* steps, int64_t capacity, int64_t* rows,
                           uint32_t flags);
+/* Ps::TryFetchSparseValues (ps/ps.cc:914-935) and the transfer-out walk (ps/ps.cc:289-321):
+ * the Values of the ids that exist; nothing is inserted. found[i] = 1 where ids[i] is present;
+ * vals / state are [n, dim] (zero rows for absent ids), steps is [n]. Any output may be NULL.
+ * Blocking. */
+int32_t krk_sparse_fetch(krk_sparse* t, const uint64_t* ids, int64_t n, uint8_t* found, float* vals,
+                         int32_t state_type, float* state, int64_t* steps, uint32_t flags);
+/* The rest of a Value for rows brought in with krk_sparse_import (transfer-in ps/ps.cc:789-792,
+ * checkpoint load checkpoint/checkpoint.cc:620-645): one optimizer state [n, dim] and / or the
+ * per-row step counters [n]. Either may be NULL. An id that is not in the table returns 12 and
+ * leaves the other rows written. A row whose counter is 0 counts as never updated: SGD then
+ * seeds its momentum buffer from the next gradient (ps/optim/sgd.cc:46-47), so a loader gives
+ * rows that carry state a counter of at least 1. */
+int32_t krk_sparse_import_state(krk_sparse* t, const uint64_t* ids, int64_t n, int32_t state_type,
+                                const float* state, const int64_t* steps, uint32_t flags);
+/* The clean-up after a cluster change (ps/ps.cc:92-109: SkipList::Remove on every row routed
+ * elsewhere). The routing decision stays on the host: it reads the ids (krk_sparse_export),
+ * picks those that go and hands them here. Ids that are not present are ignored; *erased (may
+ * be NULL) receives how many rows went. Rows stay densely numbered, so the row numbers
+ * krk_sparse_lookup reports change. Costs a pass over the whole index; blocking. */
+int32_t krk_sparse_erase(krk_sparse* t, const uint64_t* ids, int64_t n, int64_t* erased,
+                         uint32_t flags);
 
 /* ---- groups of sparse tables: one combined request, one launch -------------- */
 typedef struct krk_group krk_group;

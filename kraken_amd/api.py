@@ -89,6 +89,11 @@ EXPORTS = {
     "krk_sparse_import": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_uint32]),
     "krk_sparse_export": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p,
                                       C.c_void_p, C.c_int64, C.POINTER(C.c_int64), C.c_uint32]),
+    "krk_sparse_fetch": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32,
+                                     C.c_void_p, C.c_void_p, C.c_uint32]),
+    "krk_sparse_import_state": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p,
+                                            C.c_void_p, C.c_uint32]),
+    "krk_sparse_erase": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(C.c_int64), C.c_uint32]),
     "krk_dedup": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64),
                               C.c_uint32]),
     "krk_dense_create": (C.c_int32, [C.c_void_p, C.c_int64, C.c_uint32, C.POINTER(C.c_void_p)]),
@@ -375,6 +380,38 @@ class SparseTable:
             vals = np.ascontiguousarray(vals, dtype=np.float32)
         _check(lib().krk_sparse_import(self.h, _ptr(ids), ids.size, _ptr(vals), _flags(ids, vals)),
                "krk_sparse_import")
+
+    def fetch(self, ids, state_type=None):
+        """Ps::TryFetchSparseValues (ps/ps.cc:914-935): nothing is inserted.
+        -> found[n] bool, vals[n, dim], state[n, dim] or None, steps[n]"""
+        ids = np.ascontiguousarray(ids, dtype=np.uint64)
+        n = ids.size
+        found = np.zeros(n, np.uint8)
+        vals = np.empty((n, self.dimension), np.float32)
+        steps = np.empty(n, np.int64)
+        st = np.empty((n, self.dimension), np.float32) if state_type is not None else None
+        _check(lib().krk_sparse_fetch(self.h, _ptr(ids), n, _ptr(found), _ptr(vals),
+                                      state_type if state_type is not None else 1, _ptr(st), _ptr(steps), 0),
+               "krk_sparse_fetch")
+        return found.astype(bool), vals, st, steps
+
+    def load_state(self, ids, state_type=None, state=None, steps=None):
+        """Optimizer state / step counters of rows brought in with load(); returns the code."""
+        ids = np.ascontiguousarray(ids, dtype=np.uint64)
+        if state is not None:
+            state = np.ascontiguousarray(state, dtype=np.float32)
+        if steps is not None:
+            steps = np.ascontiguousarray(steps, dtype=np.int64)
+        return lib().krk_sparse_import_state(self.h, _ptr(ids), ids.size,
+                                             state_type if state_type is not None else 1,
+                                             _ptr(state), _ptr(steps), 0)
+
+    def erase(self, ids):
+        """The clean-up of ps/ps.cc:92-109 for the listed ids; returns how many rows went."""
+        ids = np.ascontiguousarray(ids, dtype=np.uint64)
+        gone = C.c_int64()
+        _check(lib().krk_sparse_erase(self.h, _ptr(ids), ids.size, C.byref(gone), 0), "krk_sparse_erase")
+        return gone.value
 
     def export(self, state_type=None):
         """-> ids[rows], vals[rows, dim], state[rows, dim] or None, steps[rows] (insertion order)"""

@@ -427,6 +427,132 @@ __global__ __launch_bounds__(kBlock) void export_kernel(TableView tv, int64_t ro
   }
 }
 
+// fetch: the rows of the ids that exist, nothing inserted (ps/ps.cc:914-935)
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void fetch_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                       int64_t n, unsigned char* __restrict__ found,
+                                                       float* __restrict__ vals, int state_off,
+                                                       float* __restrict__ state, int meta_off,
+                                                       long long* __restrict__ steps, int dim, int elems,
+                                                       int group) {
+  const int per_block = kBlock / group;
+  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  const int gl = threadIdx.x & (group - 1);
+  const bool active = i < n;
+  const uint32_t row = probe_find(tv, active ? ids[i] : 0, active, gl, group);
+  if (!active) return;
+  const bool hit = row != kEmptyRow;
+  const float* rec = hit ? tv.recs + (int64_t)row * tv.stride : nullptr;
+  if (gl == 0) {
+    if (found) found[i] = hit ? 1 : 0;
+    if (steps) {
+      long long s = 0;
+      if (hit && meta_off >= 0) {
+        const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + meta_off);
+        s = (long long)((uint64_t)meta[0] | ((uint64_t)meta[1] << 32));
+      }
+      steps[i] = s;
+    }
+  }
+  for (int e = gl; e < elems; e += group) {
+    float v[VEC];
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) v[c] = 0.0f;
+    if (vals) {
+      if (hit) vload<VEC>(rec + e * VEC, v);
+      vstore<VEC>(vals + i * (int64_t)dim + e * VEC, v);
+    }
+    if (state) {
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) v[c] = 0.0f;
+      if (hit && state_off >= 0) vload<VEC>(rec + state_off + e * VEC, v);
+      vstore<VEC>(state + i * (int64_t)dim + e * VEC, v);
+    }
+  }
+}
+
+// import_state: optimizer state and step counters of rows that exist (checkpoint load,
+// transfer-in: checkpoint/checkpoint.cc:620-645 inserts whole Values)
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void import_state_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                              int64_t n, int state_off,
+                                                              const float* __restrict__ state, int meta_off,
+                                                              const long long* __restrict__ steps, int dim,
+                                                              int elems, int group) {
+  const int per_block = kBlock / group;
+  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  const int gl = threadIdx.x & (group - 1);
+  const bool active = i < n;
+  const uint32_t row = probe_find(tv, active ? ids[i] : 0, active, gl, group);
+  if (!active) return;
+  if (row == kEmptyRow) {
+    if (gl == 0) atomicOr(&tv.counters[1], kErrMissingId);
+    return;
+  }
+  float* rec = tv.recs + (int64_t)row * tv.stride;
+  if (state) {
+    for (int e = gl; e < elems; e += group) {
+      float v[VEC];
+      vload<VEC>(state + i * (int64_t)dim + e * VEC, v);
+      vstore<VEC>(rec + state_off + e * VEC, v);
+    }
+  }
+  if (steps && gl == 0) {
+    uint32_t* meta = reinterpret_cast<uint32_t*>(rec + meta_off);
+    const unsigned long long s = (unsigned long long)steps[i];
+    meta[0] = (uint32_t)s;
+    meta[1] = (uint32_t)(s >> 32);
+  }
+}
+
+// ---- erase -------------------------------------------------------------------
+// Rows are kept dense: the rows that go leave holes, and the live rows at the tail move into
+// the holes below the new row count. Sources lie at or above that count, destinations below
+// it, so all moves can run at once. The index is rebuilt from the row keys afterwards.
+__global__ __launch_bounds__(kBlock) void erase_mark_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                            int64_t n, int32_t* __restrict__ dead) {
+  const int64_t i = (int64_t)blockIdx.x * (kBlock / kBucket) + threadIdx.x / kBucket;
+  const int gl = threadIdx.x & (kBucket - 1);
+  const bool active = i < n;
+  const uint32_t r = probe_find(tv, active ? ids[i] : 0, active, gl, kBucket);
+  if (active && gl == 0 && r != kEmptyRow) dead[r] = 1;   // an id listed twice writes the same 1
+}
+
+// dead_before[r] = dead rows among [0, r). keep = rows that stay.
+__global__ __launch_bounds__(kBlock) void erase_plan_kernel(const int32_t* __restrict__ dead,
+                                                            const int32_t* __restrict__ dead_before,
+                                                            int64_t rows, int64_t keep,
+                                                            uint32_t* __restrict__ holes,
+                                                            uint32_t* __restrict__ movers) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r >= rows) return;
+  if (r < keep) {
+    if (dead[r]) holes[dead_before[r]] = (uint32_t)r;
+  } else if (!dead[r]) {
+    // live rows among [keep, r): all rows there minus the dead ones there
+    const int64_t dead_below_keep = dead_before[keep];
+    movers[(r - keep) - (dead_before[r] - dead_below_keep)] = (uint32_t)r;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void erase_move_kernel(TableView tv, const uint32_t* __restrict__ holes,
+                                                            const uint32_t* __restrict__ movers,
+                                                            int64_t count) {
+  const int64_t total = count * tv.stride;
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x; t < total; t += step) {
+    const int64_t k = t / tv.stride;
+    const int64_t j = t - k * tv.stride;
+    const int64_t src = movers[k], dst = holes[k];
+    tv.recs[dst * tv.stride + j] = tv.recs[src * tv.stride + j];
+    if (j == 0) tv.row_key[dst] = tv.row_key[src];
+  }
+}
+
+__global__ void set_row_count_kernel(uint32_t* counters, uint32_t rows) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) counters[0] = rows;
+}
+
 // re-index every existing row into a fresh (larger) slot array; launch number 0 = "old row"
 __global__ __launch_bounds__(kBlock) void reindex_kernel(Slot* slots, uint64_t mask,
                                                          const unsigned long long* __restrict__ row_key,
@@ -1157,6 +1283,166 @@ int32_t krk_sparse_export(krk_sparse* t, uint64_t* ids, float* vals, int32_t sta
   if (state) KRK_TRY(t->output_back(state, cells, flags, 2));
   if (steps) KRK_TRY(t->output_back(reinterpret_cast<long long*>(steps), (size_t)rows, flags, 3));
   return sparse_finish(t, 0);
+}
+
+int32_t krk_sparse_fetch(krk_sparse* t, const uint64_t* ids, int64_t n, uint8_t* found, float* vals,
+                         int32_t state_type, float* state, int64_t* steps, uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;
+  if (n < 0 || (n > 0 && !ids)) return KRK_E_ARGUMENT;
+  if (state && (state_type < 1 || state_type >= KRK_ST_COUNT)) return KRK_E_ARGUMENT;
+  if (n > max_ids_per_launch(t->group)) {
+    set_error("at most %lld ids per call for this row width; split the request",
+              (long long)max_ids_per_launch(t->group));
+    return KRK_E_CAPACITY;
+  }
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (n == 0) return sparse_finish(t, 0);
+  const bool host = !(flags & KRK_DEVICE_PTRS);
+  const size_t cells = (size_t)n * t->dim;
+  // the four staging buffers of a table carry ids, values, state; flags and counters of a
+  // host call travel through the work space instead
+  const uint64_t* d_ids;
+  float* d_vals = nullptr;
+  float* d_state = nullptr;
+  unsigned char* d_found = found;
+  long long* d_steps = reinterpret_cast<long long*>(steps);
+  KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
+  if (vals) KRK_TRY(t->output(vals, cells, flags, 1, &d_vals));
+  if (state) KRK_TRY(t->output(state, cells, flags, 2, &d_state));
+  if (host && (found || steps)) {
+    const size_t steps_bytes = (size_t)n * sizeof(long long);
+    KRK_TRY(t->scratch[5].reserve(steps_bytes + (size_t)n + 16));
+    d_steps = steps ? t->scratch[5].as<long long>() : nullptr;
+    d_found = found ? reinterpret_cast<unsigned char*>(t->scratch[5].as<char>() + steps_bytes) : nullptr;
+  }
+  const int per_block = kBlock / t->group;
+  const dim3 grid(grid_for(n, per_block)), block(kBlock);
+  const int state_off = state ? t->col_off[state_type] : -1;
+  if (t->vec == 4) {
+    hipLaunchKernelGGL((fetch_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_found, d_vals,
+                       state_off, d_state, t->meta_off, d_steps, (int)t->dim, t->elems, t->group);
+  } else {
+    hipLaunchKernelGGL((fetch_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, d_found, d_vals,
+                       state_off, d_state, t->meta_off, d_steps, (int)t->dim, t->elems, t->group);
+  }
+  KRK_HIP(hipGetLastError());
+  if (vals) KRK_TRY(t->output_back(vals, cells, flags, 1));
+  if (state) KRK_TRY(t->output_back(state, cells, flags, 2));
+  if (host && steps)
+    KRK_HIP(hipMemcpyAsync(steps, d_steps, (size_t)n * sizeof(long long), hipMemcpyDeviceToHost, t->stream));
+  if (host && found) KRK_HIP(hipMemcpyAsync(found, d_found, (size_t)n, hipMemcpyDeviceToHost, t->stream));
+  return sparse_finish(t, 0);
+}
+
+int32_t krk_sparse_import_state(krk_sparse* t, const uint64_t* ids, int64_t n, int32_t state_type,
+                                const float* state, const int64_t* steps, uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (n < 0 || (n > 0 && !ids)) return KRK_E_ARGUMENT;
+  if (state && (state_type < 1 || state_type >= KRK_ST_COUNT)) return KRK_E_ARGUMENT;
+  if (n > max_ids_per_launch(t->group)) {
+    set_error("at most %lld ids per call for this row width; split the request",
+              (long long)max_ids_per_launch(t->group));
+    return KRK_E_CAPACITY;
+  }
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (n == 0 || (!state && !steps)) return sparse_finish(t, flags);
+  uint32_t mask = 0;
+  if (state) mask |= 1u << state_type;
+  if (steps) mask |= 1u << KRK_ST_STEPS;
+  KRK_TRY(sparse_ensure_columns(t, mask));
+  const uint64_t* d_ids;
+  const float* d_state = nullptr;
+  const long long* d_steps = nullptr;
+  KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
+  if (state) KRK_TRY(t->input(state, (size_t)n * t->dim, flags, 1, &d_state));
+  if (steps) KRK_TRY(t->input(reinterpret_cast<const long long*>(steps), (size_t)n, flags, 2, &d_steps));
+  const int per_block = kBlock / t->group;
+  const dim3 grid(grid_for(n, per_block)), block(kBlock);
+  const int state_off = state ? t->col_off[state_type] : -1;
+  if (t->vec == 4) {
+    hipLaunchKernelGGL((import_state_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, state_off,
+                       d_state, t->meta_off, d_steps, (int)t->dim, t->elems, t->group);
+  } else {
+    hipLaunchKernelGGL((import_state_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, state_off,
+                       d_state, t->meta_off, d_steps, (int)t->dim, t->elems, t->group);
+  }
+  KRK_HIP(hipGetLastError());
+  return sparse_finish(t, flags);
+}
+
+int32_t krk_sparse_erase(krk_sparse* t, const uint64_t* ids, int64_t n, int64_t* erased, uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;   // the count comes back by value
+  if (n < 0 || (n > 0 && !ids)) return KRK_E_ARGUMENT;
+  if (n > max_ids_per_launch(kBucket)) {
+    set_error("at most %lld ids per call; split the request", (long long)max_ids_per_launch(kBucket));
+    return KRK_E_CAPACITY;
+  }
+  if (erased) *erased = 0;
+  std::lock_guard<std::mutex> lk(t->mu);
+  KRK_TRY(sparse_finish(t, 0));        // drains the stream and reports what earlier calls left
+  KRK_TRY(refresh_rows(t));
+  const int64_t rows = t->size_ub;
+  if (n == 0 || rows == 0) return KRK_SUCCESS;
+  const uint64_t* d_ids;
+  KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
+  // work space: dead[rows] | dead_before[rows] | holes[rows] | movers[rows] | scan scratch | total
+  const size_t r4 = ((size_t)rows * 4 + 255) & ~(size_t)255;
+  const size_t scan_b = (scan_scratch_bytes(rows) + 255) & ~(size_t)255;
+  KRK_TRY(t->scratch[5].reserve(4 * r4 + scan_b + 256));
+  char* base = t->scratch[5].as<char>();
+  int32_t* dead = reinterpret_cast<int32_t*>(base);
+  int32_t* dead_before = reinterpret_cast<int32_t*>(base + r4);
+  uint32_t* holes = reinterpret_cast<uint32_t*>(base + 2 * r4);
+  uint32_t* movers = reinterpret_cast<uint32_t*>(base + 3 * r4);
+  void* scan_tmp = base + 4 * r4;
+  int32_t* d_total = reinterpret_cast<int32_t*>(base + 4 * r4 + scan_b);
+  KRK_HIP(hipMemsetAsync(dead, 0, (size_t)rows * 4, t->stream));
+  const TableView tv = t->view();
+  hipLaunchKernelGGL(erase_mark_kernel, dim3(grid_for(n, kBlock / kBucket)), dim3(kBlock), 0, t->stream, tv,
+                     d_ids, n, dead);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(exclusive_scan_i32(dead, dead_before, rows, d_total, scan_tmp, t->stream));
+  int32_t gone = 0;
+  KRK_HIP(hipMemcpyAsync(&gone, d_total, sizeof(gone), hipMemcpyDeviceToHost, t->stream));
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  if (erased) *erased = gone;
+  if (gone == 0) return KRK_SUCCESS;
+  const int64_t keep = rows - gone;
+  if (keep > 0) {
+    hipLaunchKernelGGL(erase_plan_kernel, dim3(grid_for(rows, kBlock)), dim3(kBlock), 0, t->stream, dead,
+                       dead_before, rows, keep, holes, movers);
+    // as many live rows sit at or above `keep` as dead ones below it; that count is
+    // dead_before[keep], known only on the device, and at most min(gone, keep)
+    int32_t to_move = 0;
+    KRK_HIP(hipMemcpyAsync(&to_move, dead_before + keep, sizeof(to_move), hipMemcpyDeviceToHost, t->stream));
+    KRK_HIP(hipStreamSynchronize(t->stream));
+    if (to_move > 0) {
+      hipLaunchKernelGGL(erase_move_kernel, dim3(strided_grid((int64_t)to_move * t->stride)), dim3(kBlock), 0,
+                         t->stream, tv, holes, movers, (int64_t)to_move);
+    }
+    KRK_HIP(hipGetLastError());
+  }
+  // rows at and above `keep` are free again: a row that is created later must find zeroed
+  // optimizer state and a zero step counter there, as in a slab that was never used
+  KRK_HIP(hipMemsetAsync(t->recs + keep * t->stride, 0, (size_t)gone * (size_t)t->stride * sizeof(float),
+                         t->stream));
+  // the index is rebuilt from the keys of the rows that remain
+  KRK_HIP(hipMemsetAsync(t->slots, 0xFF, (t->slot_cap + 1) * sizeof(Slot), t->stream));
+  if (keep > 0) {
+    hipLaunchKernelGGL(reindex_kernel, dim3(grid_for(keep, kBlock)), dim3(kBlock), 0, t->stream, t->slots,
+                       t->slot_cap - 1, t->row_key, keep);
+  }
+  hipLaunchKernelGGL(set_row_count_kernel, dim3(1), dim3(64), 0, t->stream, t->counters, (uint32_t)keep);
+  KRK_HIP(hipGetLastError());
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  t->size_ub = keep;
+  t->layout_version++;
+  return KRK_SUCCESS;
 }
 
 // ---------------------------------------------------------------------------

@@ -92,6 +92,8 @@ def lib():
         "kro_sparse_load": (None, [vp, pu, i64, pf]),
         "kro_sparse_export": (i64, [vp, pu, pf, i32, pf, pi]),
         "kro_sparse_contains": (i32, [vp, u64]),
+        "kro_sparse_erase": (i64, [vp, pu, i64]),
+        "kro_sparse_fetch": (i64, [vp, pu, i64, C.POINTER(C.c_uint8), pf]),
         "kro_dense_create": (vp, [pf, i64]),
         "kro_dense_destroy": (None, [vp]),
         "kro_dense_pull": (i32, [vp, pf]),
@@ -261,6 +263,18 @@ class SparseTable:
 
     def contains(self, id_):
         return bool(lib().kro_sparse_contains(self.h, int(id_)))
+
+    def erase(self, ids):
+        ids = _u64(ids)
+        return lib().kro_sparse_erase(self.h, _p(ids, C.c_uint64), ids.size)
+
+    def fetch(self, ids):
+        """-> found[n] bool, vals[n, dim] (rows of absent ids are zero)"""
+        ids = _u64(ids)
+        found = np.zeros(ids.size, np.uint8)
+        vals = np.zeros((ids.size, self.dim), np.float32)
+        lib().kro_sparse_fetch(self.h, _p(ids, C.c_uint64), ids.size, _p(found, C.c_uint8), _p(vals, C.c_float))
+        return found.astype(bool), vals
 
     def export(self, state_type=None):
         n = len(self)

@@ -523,6 +523,20 @@ static int sl_insert(skiplist* s, uint64_t key, kro_value* value) {
   s->count++;
   return 1;
 }
+/* common/skip_list.h:336-359 : unlink the node on every level whose predecessor points at
+ * it, then free it. */
+static int sl_remove(skiplist* s, uint64_t key) {
+  sl_node* prev[SL_MAX_HEIGHT];
+  sl_node* x = sl_find_ge(s, key, prev);
+  if (x == NULL || x->key != key) return 0;
+  for (size_t i = 0; i < s->max_height; ++i) {
+    if (prev[i]->next[i] == x) prev[i]->next[i] = x->next[i];
+  }
+  kro_value_destroy(x->value);
+  free(x);
+  s->count--;
+  return 1;
+}
 static void sl_clear(skiplist* s) {
   sl_node* x = s->head->next[0];
   while (x) {
@@ -697,6 +711,31 @@ int64_t kro_sparse_export(const kro_sparse* t, uint64_t* ids, float* vals, int32
     }
   }
   return k;
+}
+
+/* ps/ps.cc:92-109 : the clean-up after a cluster change walks every slot under its unique
+ * lock and removes the rows that are routed elsewhere. The routing decision is the caller's;
+ * this removes the listed ids and returns how many were present. */
+int64_t kro_sparse_erase(kro_sparse* t, const uint64_t* ids, int64_t n) {
+  int64_t removed = 0;
+  for (int64_t i = 0; i < n; ++i) removed += sl_remove(&t->lists[kro_hit_slot(ids[i])], ids[i]);
+  return removed;
+}
+
+/* ps/ps.cc:914-935 (TryFetchSparseValues) : values of the ids that exist, nothing inserted.
+ * found[i] = 1 and vals[i] filled where id i is present; other rows of vals are left alone. */
+int64_t kro_sparse_fetch(const kro_sparse* t, const uint64_t* ids, int64_t n, uint8_t* found,
+                         float* vals) {
+  int64_t hits = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    const sl_node* x = sl_find(&t->lists[kro_hit_slot(ids[i])], ids[i]);
+    found[i] = x != NULL;
+    if (x) {
+      memcpy(vals + i * t->dim, x->value->val->p, sizeof(float) * (size_t)t->dim);
+      ++hits;
+    }
+  }
+  return hits;
 }
 
 /* ========================================================================== */

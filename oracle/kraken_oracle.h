@@ -136,6 +136,12 @@ int64_t kro_sparse_export(const kro_sparse* t, uint64_t* ids, float* vals,
                           int32_t state_type, float* state, int64_t* steps);
 /* 1 if id is present. */
 int32_t kro_sparse_contains(const kro_sparse* t, uint64_t id);
+/* ps/ps.cc:92-109 with common/skip_list.h:336-359 : remove the listed ids; returns how many
+ * were present. */
+int64_t kro_sparse_erase(kro_sparse* t, const uint64_t* ids, int64_t n);
+/* ps/ps.cc:914-935 : values of the ids that exist, nothing inserted. Returns the hits. */
+int64_t kro_sparse_fetch(const kro_sparse* t, const uint64_t* ids, int64_t n, uint8_t* found,
+                         float* vals);
 /* Thread-safe variants that take the per-slot lock like the reference does;
  * used by the multi-threaded CPU baseline. */
 int32_t kro_sparse_pull_mt(kro_sparse* t, const uint64_t* ids, int64_t n, float* out);

@@ -56,6 +56,29 @@ void ref_map_find(void* m, const uint64_t* ids, int64_t n, uint8_t* hit, float* 
   }
 }
 
+// The clean-up walk of ps/ps.cc:92-109 with the routing decision replaced by a list of ids to
+// drop: every slot under its unique handler, SkipList::Remove on the rows that go. Returns how
+// many rows were removed.
+int64_t ref_map_erase(void* m, const uint64_t* ids, int64_t n) {
+  Map* map = static_cast<Map*>(m);
+  std::unordered_map<uint64_t, bool> drop;
+  for (int64_t i = 0; i < n; ++i) drop[ids[i]] = true;
+  int64_t removed = 0;
+  for (size_t s = 0; s < map->slot_count(); ++s) {
+    auto h = map->UniqueSkipListHandler(s);
+    auto it = h.skip_list.Begin();
+    while (it.Valid()) {
+      if (drop.count(it.key())) {
+        it = h.skip_list.Remove(it);
+        ++removed;
+      } else {
+        it.Next();
+      }
+    }
+  }
+  return removed;
+}
+
 // Keys in slot-major, key-ascending order (the order the checkpoint writer walks).
 int64_t ref_map_keys(void* m, uint64_t* ids) {
   Map* map = static_cast<Map*>(m);

@@ -85,7 +85,50 @@ def test_container_matches_reference_live(oracle):
     assert rc == 0 and np.array_equal(rows, got[hit == 1])
     for k, h in zip(probe[500:520], hit[500:520]):
         assert t.contains(int(k)) == bool(h)
+    # SkipList::Remove through the clean-up walk of ps/ps.cc:92-109: same rows go, the rest keep
+    # their order and their values
+    L.ref_map_erase.restype = C.c_int64
+    L.ref_map_erase.argtypes = [C.c_void_p, C.POINTER(C.c_uint64), C.c_int64]
+    drop = np.concatenate([ids[::3], rng.integers(0, 2**64, size=300, dtype=np.uint64)])
+    removed = L.ref_map_erase(m, drop.ctypes.data_as(C.POINTER(C.c_uint64)), drop.size)
+    assert t.erase(drop) == removed
+    n = L.ref_map_keys(m, order.ctypes.data_as(C.POINTER(C.c_uint64)))
+    eid, ev, _, _ = t.export()
+    assert n == eid.size == fresh - removed and np.array_equal(order[:n], eid)
+    L.ref_map_find(m, probe.ctypes.data_as(C.POINTER(C.c_uint64)), probe.size,
+                   hit.ctypes.data_as(C.POINTER(C.c_uint8)),
+                   got.ctypes.data_as(C.POINTER(C.c_float)), 3)
+    found, rows = t.fetch(probe)
+    assert np.array_equal(found, hit == 1) and np.array_equal(rows[found], got[hit == 1])
+    assert len(t) == n                                   # fetch inserts nothing
     L.ref_map_destroy(m)
+
+
+def test_erase_and_fetch_against_a_python_dict(oracle):
+    """No reference needed: the table is a map, erase and fetch are map operations."""
+    rng = np.random.default_rng(6)
+    ids = rng.integers(0, 5000, size=4000).astype(np.uint64)
+    vals = rng.standard_normal((ids.size, 2)).astype(np.float32)
+    t = oracle.SparseTable(2, oracle.init(oracle.INIT_CONSTANT, 0.0))
+    t.load(ids, vals)
+    model = {}
+    for k, v in zip(ids.tolist(), vals):
+        model.setdefault(k, v)
+    for round_ in range(3):
+        drop = rng.integers(0, 5000, size=700).astype(np.uint64)
+        want = sum(1 for k in set(drop.tolist()) if k in model)
+        assert t.erase(drop) == want
+        for k in drop.tolist():
+            model.pop(k, None)
+        assert len(t) == len(model)
+        probe = rng.integers(0, 5000, size=900).astype(np.uint64)
+        found, rows = t.fetch(probe)
+        for k, f, r in zip(probe.tolist(), found, rows):
+            assert f == (k in model)
+            if f:
+                assert np.array_equal(r, model[k])
+        eid, _, _, _ = t.export()
+        assert sorted(eid.tolist()) == sorted(model)
 
 
 # --------------------------------------------------------------------------- #
