@@ -47,6 +47,7 @@ extern "C" {
 #define KRK_E_DEVICE (-2)       /* a HIP call failed, or no usable GPU            */
 #define KRK_E_ARGUMENT (-3)     /* null handle, negative size, bad flag           */
 #define KRK_E_CAPACITY (-4)     /* output buffer too small / table cannot grow    */
+#define KRK_E_IO (-5)           /* a table file could not be opened, read or written */
 
 /* kraken/common/info.h:46-72 */
 enum { KRK_ADAGRAD = 0, KRK_ADAM = 1, KRK_RMSPROP = 2, KRK_SGD = 3 };
@@ -218,6 +219,10 @@ int32_t krk_sparse_export(krk_sparse* t, uint64_t* ids, float* vals, int32_t sta
  * Blocking. */
 int32_t krk_sparse_fetch(krk_sparse* t, const uint64_t* ids, int64_t n, uint8_t* found, float* vals,
                          int32_t state_type, float* state, int64_t* steps, uint32_t flags);
+/* Which parts of a Value the table's rows carry besides the weights (common/info.h:74-92):
+ * bit st is set when optimizer state st exists, bit 0 when rows keep a step counter. What a
+ * checkpoint writer has to walk (checkpoint/checkpoint.cc:465-509). */
+int32_t krk_sparse_states(krk_sparse* t, uint32_t* mask);
 /* The rest of a Value for rows brought in with krk_sparse_import (transfer-in ps/ps.cc:789-792,
  * checkpoint load checkpoint/checkpoint.cc:620-645): one optimizer state [n, dim] and / or the
  * per-row step counters [n]. Either may be NULL. An id that is not in the table returns 12 and
@@ -233,6 +238,21 @@ int32_t krk_sparse_import_state(krk_sparse* t, const uint64_t* ids, int64_t n, i
  * krk_sparse_lookup reports change. Costs a pass over the whole index; blocking. */
 int32_t krk_sparse_erase(krk_sparse* t, const uint64_t* ids, int64_t n, int64_t* erased,
                          uint32_t flags);
+
+/* ---- table files ------------------------------------------------------------- */
+/* Checkpoint::SaveSparseTable (checkpoint/checkpoint.cc:465-509): the table as a *.sparse file in
+ * the reference's byte layout (common/serialize.h), rows grouped by id % 8 and ascending inside
+ * a group, each a Value (weights, the optimizer states the row carries, Adam's step counter).
+ * table_id and name are the ones the reference's Table holds (ps/table.h:13-19). */
+int32_t krk_sparse_save_file(krk_sparse* t, const char* path, uint64_t table_id, const char* name);
+/* Checkpoint::LoadSparseTable (checkpoint/checkpoint.cc:586-649): inserts the file's rows. The
+ * file must describe this table (type, id, name, dimension, element type, initializer type),
+ * otherwise KRK_E_ARGUMENT. keep (may be NULL = every row) stands for the routing test
+ * node_id == router.Hit(utils::Hash(table_id, sparse_id)) of line 640: a row is taken when it
+ * returns non-zero. *rows_loaded (may be NULL) receives the rows taken. */
+typedef int32_t (*krk_keep_fn)(uint64_t sparse_id, void* ctx);
+int32_t krk_sparse_load_file(krk_sparse* t, const char* path, uint64_t table_id, const char* name,
+                             krk_keep_fn keep, void* keep_ctx, int64_t* rows_loaded);
 
 /* ---- groups of sparse tables: one combined request, one launch -------------- */
 typedef struct krk_group krk_group;
@@ -284,6 +304,22 @@ int32_t krk_dense_push_coo(krk_dense* t, const krk_optim* o, const int64_t* idx,
 /* Optimizer state for parity dumps; zeros when never created. */
 int32_t krk_dense_state(krk_dense* t, int32_t state_type, float* out, uint32_t flags);
 int32_t krk_dense_steps(krk_dense* t, int64_t* steps);
+int32_t krk_dense_size(krk_dense* t, int64_t* n);
+/* Same bit mask as krk_sparse_states for the dense table's one Value. */
+int32_t krk_dense_states(krk_dense* t, uint32_t* mask);
+/* Restores one optimizer state [n] (may be NULL) and / or Adam's step counter (steps < 0
+ * leaves it) of a table built from a saved Value (checkpoint/checkpoint.cc:535-557). */
+int32_t krk_dense_import_state(krk_dense* t, int32_t state_type, const float* state, int64_t steps,
+                               uint32_t flags);
+/* Checkpoint::SaveDenseTable / LoadDenseTable (checkpoint/checkpoint.cc:444-463, 535-557): a
+ * *.dense file holds the table's type, id, name and Value. shape/rank give the tensor shape to
+ * record (rank 0 = one dimension of n elements). Loading creates the table; *rank holds the
+ * capacity of `shape` on entry and the file's rank on return; name receives at most
+ * name_cap - 1 characters. table_id, name, shape and rank may be NULL. */
+int32_t krk_dense_save_file(krk_dense* t, const char* path, uint64_t table_id, const char* name,
+                            const int64_t* shape, int32_t rank);
+int32_t krk_dense_load_file(const char* path, krk_dense** out, uint64_t* table_id, char* name,
+                            size_t name_cap, int64_t* shape, int32_t* rank);
 
 /* ---- threshold ("DCT") gradient codec -------------------------------------- */
 typedef struct krk_dct krk_dct;

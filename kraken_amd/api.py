@@ -22,7 +22,7 @@ INTERFACE_UNIMPLEMENTED = 10
 GRADIENT_UNCOMPATIBLE = 11
 SPARSE_ID_NOT_EXIST = 12
 UNSUPPORTED_INITIALIZER = 13
-E_DEVICE, E_ARGUMENT, E_CAPACITY = -2, -3, -4
+E_DEVICE, E_ARGUMENT, E_CAPACITY, E_IO = -2, -3, -4, -5
 
 
 class OptimType:          # common/info.h:46-51
@@ -93,6 +93,17 @@ EXPORTS = {
                                      C.c_void_p, C.c_void_p, C.c_uint32]),
     "krk_sparse_import_state": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p,
                                             C.c_void_p, C.c_uint32]),
+    "krk_sparse_states": (C.c_int32, [C.c_void_p, C.POINTER(C.c_uint32)]),
+    "krk_dense_states": (C.c_int32, [C.c_void_p, C.POINTER(C.c_uint32)]),
+    "krk_dense_import_state": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_uint32]),
+    "krk_sparse_save_file": (C.c_int32, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_char_p]),
+    "krk_sparse_load_file": (C.c_int32, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_char_p, C.c_void_p, C.c_void_p,
+                                         C.POINTER(C.c_int64)]),
+    "krk_dense_size": (C.c_int32, [C.c_void_p, C.POINTER(C.c_int64)]),
+    "krk_dense_save_file": (C.c_int32, [C.c_void_p, C.c_char_p, C.c_uint64, C.c_char_p, C.POINTER(C.c_int64),
+                                        C.c_int32]),
+    "krk_dense_load_file": (C.c_int32, [C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_uint64), C.c_char_p,
+                                        C.c_size_t, C.POINTER(C.c_int64), C.POINTER(C.c_int32)]),
     "krk_sparse_erase": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(C.c_int64), C.c_uint32]),
     "krk_dedup": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64),
                               C.c_uint32]),
@@ -406,6 +417,21 @@ class SparseTable:
                                              state_type if state_type is not None else 1,
                                              _ptr(state), _ptr(steps), 0)
 
+    def save(self, path, table_id, name):
+        """Checkpoint::SaveSparseTable (checkpoint/checkpoint.cc:465-509); returns the code."""
+        return lib().krk_sparse_save_file(self.h, os.fsencode(path), table_id, name.encode())
+
+    def load_file(self, path, table_id, name, keep=None):
+        """Checkpoint::LoadSparseTable (checkpoint/checkpoint.cc:586-649). keep(id) -> bool plays
+        the routing test of line 640. -> (code, rows taken)"""
+        KEEP = C.CFUNCTYPE(C.c_int32, C.c_uint64, C.c_void_p)
+        cb = KEEP(lambda id_, ctx: 1 if keep(id_) else 0) if keep is not None else None
+        taken = C.c_int64()
+        rc = lib().krk_sparse_load_file(self.h, os.fsencode(path), table_id, name.encode(),
+                                        C.cast(cb, C.c_void_p) if cb is not None else None, None,
+                                        C.byref(taken))
+        return rc, taken.value
+
     def erase(self, ids):
         """The clean-up of ps/ps.cc:92-109 for the listed ids; returns how many rows went."""
         ids = np.ascontiguousarray(ids, dtype=np.uint64)
@@ -505,6 +531,30 @@ class DenseTable:
 
     def sync(self):
         return lib().krk_dense_sync(self.h)
+
+    def save(self, path, table_id, name, shape=None):
+        """Checkpoint::SaveDenseTable (checkpoint/checkpoint.cc:444-463); returns the code."""
+        shape = np.ascontiguousarray(shape if shape is not None else [], dtype=np.int64)
+        return lib().krk_dense_save_file(self.h, os.fsencode(path), table_id, name.encode(),
+                                         shape.ctypes.data_as(C.POINTER(C.c_int64)), shape.size)
+
+    @classmethod
+    def from_file(cls, path):
+        """Checkpoint::LoadDenseTable (checkpoint/checkpoint.cc:535-557)
+        -> (code, table or None, table id, name, shape)"""
+        h, tid, rank = C.c_void_p(), C.c_uint64(), C.c_int32(16)
+        name = C.create_string_buffer(1024)
+        shape = (C.c_int64 * 16)()
+        rc = lib().krk_dense_load_file(os.fsencode(path), C.byref(h), C.byref(tid), name, 1024, shape,
+                                       C.byref(rank))
+        if rc != 0:
+            return rc, None, None, None, None
+        t = cls.__new__(cls)
+        t.h = h
+        n = C.c_int64()
+        _check(lib().krk_dense_size(h, C.byref(n)), "krk_dense_size")
+        t.n = n.value
+        return 0, t, tid.value, name.value.decode(), list(shape[:rank.value])
 
     def Pull(self, out=None):
         if out is None:

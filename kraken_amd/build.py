@@ -18,7 +18,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libkraken_hip.so")
 
 SOURCES = ["runtime.hip", "sparse_table.hip", "push_raw.hip", "dense_table.hip", "codec.hip",
-           "dct2.hip"]
+           "dct2.hip", "checkpoint.hip"]
 
 # -ffp-contract=off: the reference rounds after every elementwise op (one Eigen pass per op),
 # so a fused multiply-add would change results. The packed-fp32 feature is switched off because

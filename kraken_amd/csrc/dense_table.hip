@@ -266,6 +266,41 @@ int32_t krk_dense_state(krk_dense* t, int32_t state_type, float* out, uint32_t f
   return dense_finish(t, flags);
 }
 
+int32_t krk_dense_size(krk_dense* t, int64_t* n) {
+  if (!t || !n) return KRK_E_ARGUMENT;
+  *n = t->n;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dense_states(krk_dense* t, uint32_t* mask) {
+  if (!t || !mask) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  uint32_t m = t->steps > 0 ? 1u : 0u;
+  for (int st = 1; st < KRK_ST_COUNT; ++st) {
+    if (t->state[st]) m |= 1u << st;   // states are created by the first update that needs them
+  }
+  *mask = m;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dense_import_state(krk_dense* t, int32_t state_type, const float* state, int64_t steps,
+                               uint32_t flags) {
+  KRK_TRY(check_dense(t));
+  KRK_TRY(check_flags(flags));
+  if (state && (state_type < 1 || state_type >= KRK_ST_COUNT)) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (state && t->n > 0) {
+    KRK_TRY(ensure_state(t, state_type));
+    KRK_HIP(hipMemcpyAsync(t->state[state_type], state, (size_t)t->n * sizeof(float),
+                           (flags & KRK_DEVICE_PTRS) ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
+                           t->stream));
+    if (state_type == KRK_ST_MOMENTUM_BUFFER) t->sgd_started = true;
+  }
+  if (steps >= 0) t->steps = steps;
+  // a host source buffer may be reused by the caller as soon as this returns
+  return dense_finish(t, (flags & KRK_DEVICE_PTRS) ? flags : (flags & ~KRK_ASYNC));
+}
+
 int32_t krk_dense_steps(krk_dense* t, int64_t* steps) {
   if (!t || !steps) return KRK_E_ARGUMENT;
   std::lock_guard<std::mutex> lk(t->mu);

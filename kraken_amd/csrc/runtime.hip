@@ -258,6 +258,7 @@ const char* krk_error_message(int32_t code) {
     case KRK_E_DEVICE: return "GPU runtime failure";
     case KRK_E_ARGUMENT: return "Invalid argument";
     case KRK_E_CAPACITY: return "Capacity exceeded";
+    case KRK_E_IO: return "Table file error";
     default: return "Unrecognized error";
   }
 }

@@ -1285,6 +1285,18 @@ int32_t krk_sparse_export(krk_sparse* t, uint64_t* ids, float* vals, int32_t sta
   return sparse_finish(t, 0);
 }
 
+int32_t krk_sparse_states(krk_sparse* t, uint32_t* mask) {
+  KRK_TRY(check_table(t));
+  if (!mask) return KRK_E_ARGUMENT;
+  std::lock_guard<std::mutex> lk(t->mu);
+  uint32_t m = t->meta_off >= 0 ? 1u : 0u;
+  for (int st = 1; st < KRK_ST_COUNT; ++st) {
+    if (t->col_off[st] >= 0) m |= 1u << st;
+  }
+  *mask = m;
+  return KRK_SUCCESS;
+}
+
 int32_t krk_sparse_fetch(krk_sparse* t, const uint64_t* ids, int64_t n, uint8_t* found, float* vals,
                          int32_t state_type, float* state, int64_t* steps, uint32_t flags) {
   KRK_TRY(check_table(t));

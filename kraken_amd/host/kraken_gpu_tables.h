@@ -213,6 +213,11 @@ class DenseTable : public Table {
       : Table(TableType::kDense, id, name), size_(val.Size()) {
     create_code_ = krk_dense_create(val.Data(), val.Size(), 0, &h_);
   }
+  // Adopts a table the library built (krk_dense_load_file).
+  DenseTable(uint64_t id, const std::string& name, krk_dense* adopted)
+      : Table(TableType::kDense, id, name), size_(0), h_(adopted) {
+    if (krk_dense_size(h_, &size_) != KRK_SUCCESS) create_code_ = KRK_E_ARGUMENT;
+  }
   ~DenseTable() override { krk_dense_destroy(h_); }
   DenseTable(const DenseTable&) = delete;
   DenseTable& operator=(const DenseTable&) = delete;

@@ -11,6 +11,7 @@
 #include <cstring>
 #include <random>
 
+#include "kraken_gpu_checkpoint.h"
 #include "kraken_gpu_tables.h"
 
 using namespace kraken_gpu;
@@ -134,6 +135,29 @@ int main(int argc, char** argv) {
     w -= 0.1f * (gi / (std::sqrt(sum) + 1e-10f));
     EXPECT(FloatEq(vals[0][i], w));
   }
+  // checkpoint/checkpoint.cc:444-509, 535-649 : through *.sparse / *.dense files and on
+  const char* tmp = std::getenv("TMPDIR");
+  const std::string dir = tmp ? tmp : "/tmp";
+  const std::string sparse_path = dir + "/krk_host_test.sparse", dense_path = dir + "/krk_host_test.dense";
+  EXPECT(io::SaveSparseTable(sparse_path, &s2));
+  SparseTable s3(3, "SparseTable1", 4, Initializer::Create(InitializerType::kConstant, {{"value", "1"}}));
+  EXPECT(io::LoadSparseTable(sparse_path, &s3, [](uint64_t id) { return id == 5; }));
+  SparseTable other(4, "SparseTable1", 4, Initializer::Create(InitializerType::kConstant, {{"value", "1"}}));
+  EXPECT(!io::LoadSparseTable(sparse_path, &other));          // another table id: refused (:611-616)
+  EXPECT(s2.Push(adagrad.get(), {5}, g, 0.1f) == 0);
+  EXPECT(s3.Push(adagrad.get(), {5}, g, 0.1f) == 0);          // carries on with the saved state_sum
+  std::vector<Tensor> a, b;
+  EXPECT(s2.Pull({5}, &a) == 0 && s3.Pull({5}, &b) == 0);
+  for (int i = 0; i < 4; ++i) EXPECT(a[0][i] == b[0][i]);
+  EXPECT(io::SaveDenseTable(dense_path, &dense, {10, 10}));
+  std::unique_ptr<DenseTable> dense2 = io::LoadDenseTable(dense_path);
+  EXPECT(dense2 && dense2->id() == 0 && dense2->name() == "DensTable0");
+  Tensor x, y;
+  EXPECT(dense2 && dense.Pull(&x) == 0 && dense2->Pull(&y) == 0 && x.Size() == y.Size());
+  for (int i = 0; i < 100 && dense2; ++i) EXPECT(x[i] == y[i]);
+  EXPECT(!io::LoadDenseTable(sparse_path));                    // a sparse file is no dense table
+  std::remove(sparse_path.c_str());
+  std::remove(dense_path.c_str());
   std::printf("%s\n", failures ? "FAILED" : "table interface ok");
   return failures ? 1 : 0;
 }

@@ -18,7 +18,8 @@ def _build():
         build.build(verbose=False)
     src = os.path.join(ROOT, "tests", "host", "table_interface_test.cc")
     if os.path.exists(EXE) and os.path.getmtime(EXE) > max(
-            os.path.getmtime(src), os.path.getmtime(os.path.join(lib_dir, "host", "kraken_gpu_tables.h"))):
+            os.path.getmtime(src), os.path.getmtime(os.path.join(lib_dir, "host", "kraken_gpu_tables.h")),
+            os.path.getmtime(os.path.join(lib_dir, "host", "kraken_gpu_checkpoint.h"))):
         return
     subprocess.check_call(["g++", "-std=c++17", "-O2", "-Wall", "-I" + os.path.join(ROOT, "include"),
                            "-I" + os.path.join(lib_dir, "host"), src, "-o", EXE, "-L" + lib_dir,
