@@ -11,7 +11,7 @@
 //                                   so a push touches one contiguous record instead of one line
 //                                   per state array.
 //   row_key [row_cap] x 8 B         id of each row (export and re-indexing walk rows, not slots)
-//   counters[4] x 4 B               {rows used, error bits, -, -}
+//   counters[4] x 4 B               {rows used, error bits, missing-id queue length x 2}
 //   host_pub   8 B, pinned host     {rows used, launch number}: written by a one-wave kernel that
 //                                   the host enqueues behind an inserting launch when the table
 //                                   is close to full, so that it can bound the row count later
@@ -283,6 +283,7 @@ struct krk_sparse : krk::ObjBase {
   uint64_t enq_at[256] = {};          // enq_total right after the launch with number e (mod 256)
   uint32_t epoch = 0;                 // number of the last launch that could insert
   uint64_t layout_version = 0;        // bumped whenever slots, records or columns move
+  int pull_parity = 0;                // which of counters[2..3] the next two-launch pull queues into
 
   int32_t col_off[KRK_ST_COUNT];      // float offset of each state column in a record, -1 = absent
   int32_t meta_off = -1;              // float offset of the step counter (two u32), -1 = absent

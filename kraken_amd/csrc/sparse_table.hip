@@ -21,6 +21,23 @@ namespace krk {
 
 constexpr int kBlock = 256;
 constexpr int kMaxGroupTables = 32;
+constexpr int64_t kTwoLaunchPull = 1 << 18;   // ids from which a pull runs as two launches
+constexpr int kMissingGrid = 2048;            // workgroups of the launch that inserts missing ids
+
+// VEC initial values of a new row, evaluated one after the other: the loop stays rolled so that
+// the double-precision Box-Muller of the rare branch is live once, not VEC times, and the
+// kernels that carry it keep their occupancy (the pulls are bound by the reads in flight).
+template <int VEC>
+__device__ __forceinline__ void init_vec(const InitK& init, uint64_t id, int64_t first, float (&v)[VEC]) {
+#pragma unroll
+  for (int c = 0; c < VEC; ++c) v[c] = 0.0f;
+#pragma unroll 1
+  for (int c = 0; c < VEC; ++c) {
+    const float x = init_element(init, id, first + c);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) v[k] = k == c ? x : v[k];
+  }
+}
 
 template <int VEC>
 __device__ __forceinline__ void vload(const float* p, float (&v)[VEC]) {
@@ -73,8 +90,7 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
     if (fresh) {
       // the value of a new row is a pure function of (seed, id, element): every group that
       // meets it computes the same numbers, only the creator stores them
-#pragma unroll
-      for (int c = 0; c < VEC; ++c) v[c] = init_element(init, id, (int64_t)e * VEC + c);
+      init_vec<VEC>(init, id, (int64_t)e * VEC, v);
       if (owner) vstore<VEC>(rec + e * VEC, v);
     } else {
       vload<VEC>(rec + e * VEC, v);
@@ -166,6 +182,64 @@ __global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, InitK init,
   pull_body<VEC>(tv, init, ids, i, i < n, threadIdx.x & (group - 1), out, dim, elems, group);
 }
 
+// ---- large pulls in two launches ------------------------------------------------
+// A large pull is bound by the random reads in flight, i.e. by wavefronts per SIMD, and the
+// claiming search plus the initialiser of new rows cost pull_kernel a quarter of them. So a
+// large request first runs a kernel that only searches and copies (eight wavefronts per SIMD)
+// and queues the positions whose id is missing; a second, small launch walks that queue with
+// pull_body. In steady state the queue is empty and the second launch ends at once.
+// counters[2 + parity] counts the queue; the second launch clears the other parity's counter
+// for the request after it (same stream, so that request's first kernel has not started).
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                               int64_t n, float* __restrict__ out,
+                                                               uint32_t* __restrict__ todo, int parity, int dim,
+                                                               int elems, int group) {
+  const int per_block = kBlock / group;
+  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  const int gl = threadIdx.x & (group - 1);
+  const bool active = i < n;
+  const uint32_t row = probe_find(tv, active ? ids[i] : 0, active, gl, group);
+  // one atomic per wavefront reserves queue entries for all of its missing ids
+  const bool queue = active && row == kEmptyRow && gl == 0;
+  const unsigned long long votes = __ballot(queue);
+  if (votes) {
+    const int lane = wave_lane();
+    const int first = __ffsll(votes) - 1;
+    uint32_t base = 0;
+    if (lane == first) base = atomicAdd(&tv.counters[2 + parity], (uint32_t)__popcll(votes));
+    base = __shfl(base, first);
+    if (queue) todo[base + (uint32_t)__popcll(votes & ((1ull << lane) - 1ull))] = (uint32_t)i;
+  }
+  if (!active || row == kEmptyRow) return;
+  const float* rec = tv.recs + (int64_t)row * tv.stride;
+  float* dst = out + i * (int64_t)dim;
+  for (int e = gl; e < elems; e += group) {
+    float v[VEC];
+    vload<VEC>(rec + e * VEC, v);
+    vstore<VEC>(dst + e * VEC, v);
+  }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pull_missing_kernel(TableView tv, InitK init,
+                                                              const uint64_t* __restrict__ ids,
+                                                              float* __restrict__ out,
+                                                              const uint32_t* __restrict__ todo, int parity,
+                                                              int dim, int elems, int group) {
+  const uint32_t count = __atomic_load_n(&tv.counters[2 + parity], __ATOMIC_RELAXED);
+  if (blockIdx.x == 0 && threadIdx.x == 0) tv.counters[2 + (parity ^ 1)] = 0u;
+  const int per_block = kBlock / group;
+  const uint32_t stride = gridDim.x * per_block;
+  const int gl = threadIdx.x & (group - 1);
+  // block-uniform trip count: pull_body votes across the wavefront
+  for (uint32_t k0 = blockIdx.x * per_block; k0 < count; k0 += stride) {
+    const uint32_t k = k0 + threadIdx.x / group;
+    const bool active = k < count;
+    pull_body<VEC>(tv, init, ids, active ? (int64_t)todo[k] : 0, active, gl, out, dim, elems, group);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // pooled pull: Pull fused with the worker's jagged sum / mean (pytorch/py/jagged_ops.cc:14-56,
 // 206-236, called from pytorch/jagged_embedding.py:32-52), in two launches.
@@ -193,8 +267,7 @@ __global__ __launch_bounds__(kBlock) void pooled_probe_kernel(TableView tv, Init
     float* rec = tv.recs + (int64_t)pr.row * tv.stride;
     for (int e = gl; e < elems; e += kBucket) {
       float v[VEC];
-#pragma unroll
-      for (int c = 0; c < VEC; ++c) v[c] = init_element(init, id, (int64_t)e * VEC + c);
+      init_vec<VEC>(init, id, (int64_t)e * VEC, v);
       vstore<VEC>(rec + e * VEC, v);
     }
   }
@@ -1079,7 +1152,24 @@ int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* ou
   KRK_TRY(sparse_next_epoch(t, n));
   const int per_block = kBlock / t->group;
   const dim3 grid(grid_for(n, per_block)), block(kBlock);
-  if (t->vec == 4) {
+  if (n >= kTwoLaunchPull) {
+    KRK_TRY(t->scratch[5].reserve((size_t)n * sizeof(uint32_t)));
+    uint32_t* todo = t->scratch[5].as<uint32_t>();
+    const int parity = t->pull_parity;
+    t->pull_parity ^= 1;
+    const dim3 small(kMissingGrid);
+    if (t->vec == 4) {
+      hipLaunchKernelGGL((pull_resident_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
+                         parity, (int)t->dim, t->elems, t->group);
+      hipLaunchKernelGGL((pull_missing_kernel<4>), small, block, 0, t->stream, t->view(), t->initk, d_ids, d_out,
+                         todo, parity, (int)t->dim, t->elems, t->group);
+    } else {
+      hipLaunchKernelGGL((pull_resident_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
+                         parity, (int)t->dim, t->elems, t->group);
+      hipLaunchKernelGGL((pull_missing_kernel<1>), small, block, 0, t->stream, t->view(), t->initk, d_ids, d_out,
+                         todo, parity, (int)t->dim, t->elems, t->group);
+    }
+  } else if (t->vec == 4) {
     hipLaunchKernelGGL((pull_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
                        (int)t->dim, t->elems, t->group);
   } else {
