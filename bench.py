@@ -296,6 +296,10 @@ def main():
         sys.exit(2)
     cfg = WORKLOADS[args.workload]
     dt, rows, roofline, batches = run_gpu(cfg, args.steps, args.warmup)
+    # the same achieved figure against what a plain copy kernel moves on this very box
+    ceiling = copy_calibration(nbytes=1 << 28, reps=10)["copy_gbs_read_plus_write"]
+    roofline["copy_ceiling"] = ceiling
+    roofline["frac_of_copy_ceiling"] = roofline["achieved"] / ceiling
     value = rows / dt
     dim = cfg["dim"]
     S = state_arrays(cfg["optim"])

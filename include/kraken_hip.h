@@ -15,6 +15,10 @@
  * then only enqueued on the table's stream and a failure is reported by the
  * next blocking call or by the object's *_sync() function.
  *
+ * Stream capture: do not record these calls into a HIP graph. Every launch that may insert
+ * rows carries a launch number chosen on the host, and a replayed launch would present an old
+ * number, under which rows created since would be taken for rows still being created.
+ *
  * Threading: any number of host threads may call into one table; calls on one
  * table are serialised (the reference takes a unique lock per slot for Pull
  * and Push alike, ps/sparse_table.cc:48,88, and a unique lock for a dense
@@ -284,6 +288,18 @@ int32_t krk_group_push(krk_group* g, const krk_optim* o, const uint64_t* ids, co
  * hold n entries; *n_unique receives U. */
 int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv,
                   int64_t* n_unique, uint32_t flags);
+
+/* Emitter::PushSparseTable's dedup + sum as a call of its own (worker/emitter.cc:510-531), for a
+ * worker whose server is elsewhere: uids as krk_dedup, sums[u, :] = the gradient rows of unique
+ * id u added in position order starting from a copy of the first. grads is [n, dim]; sums needs
+ * room for n rows, *n_unique of them are written. inv may be NULL. Blocking. */
+int32_t krk_dedup_sum(const uint64_t* ids, int64_t n, const float* grads, int64_t dim, uint64_t* uids,
+                      int64_t* inv, float* sums, int64_t* n_unique, uint32_t flags);
+/* The re-expansion after a pull of unique ids (worker/emitter.cc:162-182): out[p, :] =
+ * rows[inv[p], :]. rows is [n_rows, dim], out [n, dim]. An index outside rows returns
+ * KRK_E_ARGUMENT (those output rows are zero). Blocking. */
+int32_t krk_expand_rows(const float* rows, int64_t n_rows, const int64_t* inv, int64_t n, int64_t dim,
+                        float* out, uint32_t flags);
 
 /* ---- dense table ---------------------------------------------------------- */
 typedef struct krk_dense krk_dense;

@@ -107,6 +107,10 @@ EXPORTS = {
     "krk_sparse_erase": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(C.c_int64), C.c_uint32]),
     "krk_dedup": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64),
                               C.c_uint32]),
+    "krk_dedup_sum": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
+                                  C.c_void_p, C.POINTER(C.c_int64), C.c_uint32]),
+    "krk_expand_rows": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p,
+                                    C.c_uint32]),
     "krk_dense_create": (C.c_int32, [C.c_void_p, C.c_int64, C.c_uint32, C.POINTER(C.c_void_p)]),
     "krk_dense_destroy": (C.c_int32, [C.c_void_p]),
     "krk_dense_sync": (C.c_int32, [C.c_void_p]),
@@ -604,6 +608,37 @@ def dedup(ids):
     if isinstance(ids, DeviceArray):
         return uids, inv, u.value
     return uids[:u.value].copy(), inv
+
+
+def dedup_sum(ids, grads):
+    """Emitter::PushSparseTable's dedup + sum (worker/emitter.cc:510-531)
+    -> (uids, inv, sums[U, dim]); device inputs give device outputs plus U."""
+    dev = isinstance(ids, DeviceArray)
+    if not dev:
+        ids = np.ascontiguousarray(ids, dtype=np.uint64)
+        grads = np.ascontiguousarray(grads, dtype=np.float32)
+    n = ids.size
+    dim = grads.shape[-1]
+    mk = (lambda shape, dt: DeviceArray(shape, dt)) if dev else (lambda shape, dt: np.empty(shape, dt))
+    uids, inv, sums = mk(max(n, 1), np.uint64), mk(max(n, 1), np.int64), mk((max(n, 1), dim), np.float32)
+    u = C.c_int64()
+    _check(lib().krk_dedup_sum(_ptr(ids), n, _ptr(grads), dim, _ptr(uids), _ptr(inv), _ptr(sums), C.byref(u),
+                               _flags(ids, grads, uids)), "krk_dedup_sum")
+    if dev:
+        return uids, inv, sums, u.value
+    return uids[:u.value].copy(), inv[:n], sums[:u.value].copy()
+
+
+def expand_rows(rows, inv):
+    """The re-expansion of worker/emitter.cc:162-182: out[p] = rows[inv[p]]; returns (code, out)."""
+    dev = isinstance(rows, DeviceArray)
+    if not dev:
+        rows = np.ascontiguousarray(rows, dtype=np.float32)
+        inv = np.ascontiguousarray(inv, dtype=np.int64)
+    n, dim = inv.size, rows.shape[-1]
+    out = DeviceArray((n, dim), np.float32) if dev else np.empty((n, dim), np.float32)
+    rc = lib().krk_expand_rows(_ptr(rows), rows.shape[0], _ptr(inv), n, dim, _ptr(out), _flags(rows, inv, out))
+    return rc, out
 
 
 class DenseBag:

@@ -202,11 +202,19 @@ struct ApplyArgs {
   int c0, c1, c2, meta_off;
 };
 
+// What a closed run does with its sum: one of the four optimizers, or (stand-alone dedup + sum)
+// just store it as row `row` of the output.
+constexpr int kOptStore = 4;
+
 template <int OPT, int VEC>
 __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, const float (&gsum)[VEC],
                                           int e, bool lane_on, bool leader, bool last_chunk,
                                           const ApplyArgs& a) {
   float* rec = tv.recs + (int64_t)row * tv.stride;
+  if constexpr (OPT == kOptStore) {
+    if (lane_on) vstore<VEC>(rec + e * VEC, gsum);
+    return;
+  }
   bool first = false;
   float bc1 = 1.0f, bc2 = 1.0f;
   uint64_t steps = 0;
@@ -391,10 +399,16 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
   }
 }
 
+// Row width and lane mapping of a reduction: a table's, or those of a stand-alone call.
+struct ReduceShape {
+  int64_t dim;
+  int vec, elems, group;
+};
+
 template <int OPT, int VEC>
 static void launch_segreduce(bool level0, const TableView& tv, const uint32_t* keys, const uint32_t* pos,
                              const float* vals, int64_t cnt, int tile, uint32_t empty_from,
-                             uint32_t* keys_out, float* vals_out, const krk_sparse* t,
+                             uint32_t* keys_out, float* vals_out, const ReduceShape* t,
                              const ApplyArgs& args, const PooledSrc& ps, hipStream_t stream) {
   const int per_block = kBlock / t->group;
   const int64_t tiles = (cnt + tile - 1) / tile;
@@ -415,9 +429,13 @@ template <int VEC>
 static void dispatch_segreduce(int opt, bool level0, const TableView& tv, const uint32_t* keys,
                                const uint32_t* pos, const float* vals, int64_t cnt, int tile,
                                uint32_t empty_from, uint32_t* keys_out, float* vals_out,
-                               const krk_sparse* t, const ApplyArgs& args, const PooledSrc& ps,
+                               const ReduceShape* t, const ApplyArgs& args, const PooledSrc& ps,
                                hipStream_t stream) {
   switch (opt) {
+    case kOptStore:
+      launch_segreduce<kOptStore, VEC>(level0, tv, keys, pos, vals, cnt, tile, empty_from, keys_out,
+                                       vals_out, t, args, ps, stream);
+      break;
     case KRK_SGD:
       launch_segreduce<KRK_SGD, VEC>(level0, tv, keys, pos, vals, cnt, tile, empty_from, keys_out,
                                      vals_out, t, args, ps, stream);
@@ -445,64 +463,45 @@ static int pick_tile(int64_t cnt) {
   return 8;
 }
 
-// Positions -> rows -> stable sort by row -> tiled segmented reduction fused with the update.
-// d_vals holds one gradient row per sort payload (per position, or per bag for pooled pushes).
-// The caller holds the table's lock and has made the optimizer's columns exist.
-static int32_t push_sorted(krk_sparse* t, const krk_optim* o, const uint64_t* d_ids, int64_t n,
-                           const float* d_g, float lr, const uint32_t* bag_of, bool payload_is_bag,
-                           const PooledSrc& ps) {
-  // sort key width: rows are < row_cap; one value above them marks a missing id
-  uint32_t miss_key = 1;
-  int bits = 1;
-  while ((int64_t)miss_key < t->row_cap) {
-    miss_key <<= 1;
-    ++bits;
-  }
+// Stable sort of (key, payload) by key, then the tiled segmented reduction: every run of equal
+// keys is summed in payload order and handed to apply_row<opt> once. `fill(keys, payload)`
+// enqueues the kernel that writes the n unsorted pairs; keys >= miss_key are skipped. d_vals
+// holds one value row per payload. scratch[0..4] is the caller's work space.
+template <typename Fill>
+static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, DeviceBuffer* scratch,
+                               const TableView& tv, int opt, int64_t n, uint32_t miss_key, int bits,
+                               const float* d_vals, const ApplyArgs& args, const PooledSrc& ps, Fill fill) {
   const int tile0 = pick_tile(n);
   const int64_t tiles0 = (n + tile0 - 1) / tile0;
   const size_t n4 = (size_t)n * sizeof(uint32_t);
   size_t sort_bytes = 0;
   KRK_HIP(rocprim::radix_sort_pairs(nullptr, sort_bytes, (uint32_t*)nullptr, (uint32_t*)nullptr,
-                                    (uint32_t*)nullptr, (uint32_t*)nullptr, (size_t)n, 0, bits,
-                                    t->stream));
+                                    (uint32_t*)nullptr, (uint32_t*)nullptr, (size_t)n, 0, bits, stream));
   const size_t carry_entries = (size_t)(2 * tiles0);
-  KRK_TRY(t->scratch[0].reserve(4 * n4));                       // keys, pos, sorted keys, sorted pos
-  KRK_TRY(t->scratch[1].reserve(sort_bytes));
-  KRK_TRY(t->scratch[2].reserve(carry_entries * sizeof(uint32_t) * 2));              // carry keys A|B
-  KRK_TRY(t->scratch[3].reserve(carry_entries * (size_t)t->dim * sizeof(float)));    // carry vals A
-  KRK_TRY(t->scratch[4].reserve((carry_entries / 2 + 16) * (size_t)t->dim * sizeof(float)));  // B
-  uint32_t* keys = t->scratch[0].as<uint32_t>();
+  KRK_TRY(scratch[0].reserve(4 * n4));                       // keys, payload, sorted keys, sorted payload
+  KRK_TRY(scratch[1].reserve(sort_bytes));
+  KRK_TRY(scratch[2].reserve(carry_entries * sizeof(uint32_t) * 2));              // carry keys A|B
+  KRK_TRY(scratch[3].reserve(carry_entries * (size_t)sh.dim * sizeof(float)));    // carry vals A
+  KRK_TRY(scratch[4].reserve((carry_entries / 2 + 16) * (size_t)sh.dim * sizeof(float)));  // B
+  uint32_t* keys = scratch[0].as<uint32_t>();
   uint32_t* pos = keys + n;
   uint32_t* skeys = pos + n;
   uint32_t* spos = skeys + n;
 
-  const TableView tv = t->view();
-  hipLaunchKernelGGL(rows_of_ids_kernel, dim3(grid_for(n, kBlock / kBucket)), dim3(kBlock), 0, t->stream,
-                     tv, d_ids, n, miss_key, bag_of, payload_is_bag, keys, pos);
+  fill(keys, pos);
   KRK_HIP(hipGetLastError());
-  KRK_HIP(rocprim::radix_sort_pairs(t->scratch[1].ptr, sort_bytes, keys, skeys, pos, spos, (size_t)n, 0,
-                                    bits, t->stream));
+  KRK_HIP(rocprim::radix_sort_pairs(scratch[1].ptr, sort_bytes, keys, skeys, pos, spos, (size_t)n, 0, bits,
+                                    stream));
 
-  ApplyArgs args;
-  args.lr = lr;
-  args.k = make_optim_k(*o);
-  int32_t cols[3];
-  sparse_optim_columns(t, *o, cols);
-  args.c0 = cols[0];
-  args.c1 = cols[1];
-  args.c2 = cols[2];
-  args.meta_off = ((optim_state_mask(*o) >> KRK_ST_STEPS) & 1u) ? t->meta_off : -1;
-
-  // level 0 reads gradients through the sorted positions; later levels read the carry list
-  uint32_t* ckeys[2] = {t->scratch[2].as<uint32_t>(), t->scratch[2].as<uint32_t>() + carry_entries};
-  float* cvals[2] = {t->scratch[3].as<float>(), t->scratch[4].as<float>()};
+  // level 0 reads value rows through the sorted payloads; later levels read the carry list
+  uint32_t* ckeys[2] = {scratch[2].as<uint32_t>(), scratch[2].as<uint32_t>() + carry_entries};
+  float* cvals[2] = {scratch[3].as<float>(), scratch[4].as<float>()};
   const uint32_t* in_keys = skeys;
-  const float* in_vals = d_g;
+  const float* in_vals = d_vals;
   int64_t cnt = n;
   int tile = tile0;
   bool level0 = true;
   int which = 0;
-  uint32_t empty_from = miss_key;
   for (;;) {
     const int64_t tiles = (cnt + tile - 1) / tile;
     uint32_t* okeys = nullptr;
@@ -511,12 +510,12 @@ static int32_t push_sorted(krk_sparse* t, const krk_optim* o, const uint64_t* d_
       okeys = ckeys[which];
       ovals = cvals[which];
     }
-    if (t->vec == 4) {
-      dispatch_segreduce<4>(o->type, level0, tv, in_keys, spos, in_vals, cnt, tile, empty_from, okeys,
-                            ovals, t, args, ps, t->stream);
+    if (sh.vec == 4) {
+      dispatch_segreduce<4>(opt, level0, tv, in_keys, spos, in_vals, cnt, tile, miss_key, okeys, ovals, &sh,
+                            args, ps, stream);
     } else {
-      dispatch_segreduce<1>(o->type, level0, tv, in_keys, spos, in_vals, cnt, tile, empty_from, okeys,
-                            ovals, t, args, ps, t->stream);
+      dispatch_segreduce<1>(opt, level0, tv, in_keys, spos, in_vals, cnt, tile, miss_key, okeys, ovals, &sh,
+                            args, ps, stream);
     }
     KRK_HIP(hipGetLastError());
     if (tiles <= 1) break;
@@ -530,11 +529,132 @@ static int32_t push_sorted(krk_sparse* t, const krk_optim* o, const uint64_t* d_
   return KRK_SUCCESS;
 }
 
+// Positions -> rows -> sort_and_reduce fused with the optimizer. d_g holds one gradient row per
+// sort payload (per position, or per bag for pooled pushes). The caller holds the table's lock
+// and has made the optimizer's columns exist.
+static int32_t push_sorted(krk_sparse* t, const krk_optim* o, const uint64_t* d_ids, int64_t n,
+                           const float* d_g, float lr, const uint32_t* bag_of, bool payload_is_bag,
+                           const PooledSrc& ps) {
+  // sort key width: rows are < row_cap; one value above them marks a missing id
+  uint32_t miss_key = 1;
+  int bits = 1;
+  while ((int64_t)miss_key < t->row_cap) {
+    miss_key <<= 1;
+    ++bits;
+  }
+  ApplyArgs args;
+  args.lr = lr;
+  args.k = make_optim_k(*o);
+  int32_t cols[3];
+  sparse_optim_columns(t, *o, cols);
+  args.c0 = cols[0];
+  args.c1 = cols[1];
+  args.c2 = cols[2];
+  args.meta_off = ((optim_state_mask(*o) >> KRK_ST_STEPS) & 1u) ? t->meta_off : -1;
+  const TableView tv = t->view();
+  const ReduceShape sh{t->dim, t->vec, t->elems, t->group};
+  return sort_and_reduce(sh, t->stream, t->scratch, tv, o->type, n, miss_key, bits, d_g, args, ps,
+                         [&](uint32_t* keys, uint32_t* pos) {
+                           hipLaunchKernelGGL(rows_of_ids_kernel, dim3(grid_for(n, kBlock / kBucket)),
+                                              dim3(kBlock), 0, t->stream, tv, d_ids, n, miss_key, bag_of,
+                                              payload_is_bag, keys, pos);
+                         });
+}
+
+// stand-alone dedup + sum: (unique index, position) pairs for the sort
+__global__ __launch_bounds__(kBlock) void dedup_pairs_kernel(const DSlot* __restrict__ slots,
+                                                             const uint32_t* __restrict__ slot_of, int64_t n,
+                                                             uint32_t* __restrict__ keys,
+                                                             uint32_t* __restrict__ pos) {
+  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (p >= n) return;
+  keys[p] = slots[slot_of[p]].uidx;
+  pos[p] = (uint32_t)p;
+}
+
+// worker/emitter.cc:162-182 : rows of the unique ids back to one row per position
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void expand_rows_kernel(const float* __restrict__ rows,
+                                                             const long long* __restrict__ inv, int64_t n,
+                                                             int64_t n_rows, float* __restrict__ out, int dim,
+                                                             int elems, uint32_t* __restrict__ err) {
+  const int64_t total = n * elems;
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += step) {
+    const int64_t p = i / elems;
+    const int e = (int)(i - p * elems);
+    const long long u = inv[p];
+    float v[VEC];
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) v[c] = 0.0f;
+    if (u >= 0 && u < n_rows) {
+      vload<VEC>(rows + u * dim + e * VEC, v);
+    } else if (e == 0) {
+      atomicOr(err, 1u);
+    }
+    vstore<VEC>(out + p * dim + e * VEC, v);
+  }
+}
+
 }  // namespace krk
 
 using namespace krk;
 
 extern "C" {
+
+// The stand-alone dedup calls block and own no table: their work space is kept between calls
+// under one lock, and they run on the null stream.
+static std::mutex g_dedup_mu;
+static DeviceBuffer g_dedup_pool;
+static DeviceBuffer g_dedup_reduce[5];
+
+struct DedupWork {
+  DSlot* slots;
+  uint64_t cap;
+  uint32_t* slot_of;
+  int32_t* flag;
+  int32_t* rank;
+  void* scan_tmp;
+  int32_t* d_total;
+  char* extra;   // `extra_bytes` more for the caller (staged host arguments)
+};
+
+static size_t round256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+static int32_t dedup_layout(int64_t n, size_t extra_bytes, DedupWork* w) {
+  uint64_t cap = 1024;
+  while (cap < (uint64_t)n * 2) cap <<= 1;
+  const size_t slots_b = (cap + 1) * sizeof(DSlot);
+  const size_t n4 = round256((size_t)n * 4);
+  const size_t scan_b = round256(scan_scratch_bytes(n));
+  KRK_TRY(g_dedup_pool.reserve(slots_b + 3 * n4 + scan_b + 256 + extra_bytes));
+  char* cur = g_dedup_pool.as<char>();
+  w->slots = reinterpret_cast<DSlot*>(cur); cur += slots_b;
+  w->cap = cap;
+  w->slot_of = reinterpret_cast<uint32_t*>(cur); cur += n4;
+  w->flag = reinterpret_cast<int32_t*>(cur); cur += n4;
+  w->rank = reinterpret_cast<int32_t*>(cur); cur += n4;
+  w->scan_tmp = cur; cur += scan_b;
+  w->d_total = reinterpret_cast<int32_t*>(cur); cur += 256;
+  w->extra = cur;
+  return KRK_SUCCESS;
+}
+
+// unique ids in first-occurrence order into d_uids, every position's slot into w.slot_of (the
+// slot then holds the id's index in the unique list); *u = number of unique ids
+static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, uint64_t* d_uids, hipStream_t s,
+                          int32_t* u) {
+  KRK_HIP(hipMemsetAsync(w.slots, 0xFF, (w.cap + 1) * sizeof(DSlot), s));
+  const dim3 grid(grid_for(n, kBlock)), block(kBlock);
+  hipLaunchKernelGGL(dedup_claim_kernel, grid, block, 0, s, w.slots, w.cap - 1, d_ids, n, w.slot_of);
+  hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, w.slots, w.slot_of, n, w.flag);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
+  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids);
+  KRK_HIP(hipGetLastError());
+  KRK_HIP(hipMemcpy(u, w.d_total, sizeof(*u), hipMemcpyDeviceToHost));
+  return KRK_SUCCESS;
+}
 
 int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, int64_t* n_unique,
                   uint32_t flags) {
@@ -548,57 +668,172 @@ int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, 
   KRK_TRY(ensure_runtime());
   *n_unique = 0;
   if (n == 0) return KRK_SUCCESS;
-
-  uint64_t cap = 1024;
-  while (cap < (uint64_t)n * 2) cap <<= 1;
-  const size_t slots_b = (cap + 1) * sizeof(DSlot);
-  const size_t n4 = ((size_t)n * 4 + 255) & ~(size_t)255;
-  const size_t n8 = ((size_t)n * 8 + 255) & ~(size_t)255;
-  const size_t scan_b = (scan_scratch_bytes(n) + 255) & ~(size_t)255;
   const bool host = !(flags & KRK_DEVICE_PTRS);
-  // one allocation: slots | slot_of | flag | rank | scan scratch | total | (staged ids, uids, inv)
-  size_t total = slots_b + 3 * n4 + scan_b + 256 + (host ? 3 * n8 : 0);
-  // work space is kept between calls (the call blocks, so one buffer under a lock is enough)
-  static std::mutex pool_mu;
-  static DeviceBuffer pool;
-  std::lock_guard<std::mutex> pool_lock(pool_mu);
-  KRK_TRY(pool.reserve(total));
-  char* base = pool.as<char>();
-  char* cur = base;
-  DSlot* slots = reinterpret_cast<DSlot*>(cur); cur += slots_b;
-  uint32_t* slot_of = reinterpret_cast<uint32_t*>(cur); cur += n4;
-  int32_t* flag = reinterpret_cast<int32_t*>(cur); cur += n4;
-  int32_t* rank = reinterpret_cast<int32_t*>(cur); cur += n4;
-  void* scan_tmp = cur; cur += scan_b;
-  int32_t* d_total = reinterpret_cast<int32_t*>(cur); cur += 256;
+  const size_t n8 = round256((size_t)n * 8);
+  std::lock_guard<std::mutex> pool_lock(g_dedup_mu);
+  DedupWork w;
+  KRK_TRY(dedup_layout(n, host ? 3 * n8 : 0, &w));
   const uint64_t* d_ids = ids;
   uint64_t* d_uids = uids;
   long long* d_inv = reinterpret_cast<long long*>(inv);
   if (host) {
-    uint64_t* s_ids = reinterpret_cast<uint64_t*>(cur); cur += n8;
-    d_uids = reinterpret_cast<uint64_t*>(cur); cur += n8;
-    d_inv = reinterpret_cast<long long*>(cur); cur += n8;
+    uint64_t* s_ids = reinterpret_cast<uint64_t*>(w.extra);
+    d_uids = reinterpret_cast<uint64_t*>(w.extra + n8);
+    d_inv = reinterpret_cast<long long*>(w.extra + 2 * n8);
     KRK_HIP(hipMemcpy(s_ids, ids, (size_t)n * 8, hipMemcpyHostToDevice));
     d_ids = s_ids;
   }
-  hipStream_t s = nullptr;   // the null stream: this call owns no table and blocks anyway
-  KRK_HIP(hipMemsetAsync(slots, 0xFF, slots_b, s));
-  const dim3 grid(grid_for(n, kBlock)), block(kBlock);
-  hipLaunchKernelGGL(dedup_claim_kernel, grid, block, 0, s, slots, cap - 1, d_ids, n, slot_of);
-  hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, slots, slot_of, n, flag);
-  KRK_HIP(hipGetLastError());
-  KRK_TRY(exclusive_scan_i32(flag, rank, n, d_total, scan_tmp, s));
-  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, slots, slot_of, rank, d_ids, n, d_uids);
-  if (inv) hipLaunchKernelGGL(dedup_inv_kernel, grid, block, 0, s, slots, slot_of, n, d_inv);
-  KRK_HIP(hipGetLastError());
+  hipStream_t s = nullptr;
   int32_t u = 0;
-  KRK_HIP(hipMemcpy(&u, d_total, sizeof(u), hipMemcpyDeviceToHost));
+  KRK_TRY(dedup_core(w, d_ids, n, d_uids, s, &u));
+  if (inv) {
+    hipLaunchKernelGGL(dedup_inv_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, w.slots, w.slot_of, n,
+                       d_inv);
+    KRK_HIP(hipGetLastError());
+  }
   *n_unique = u;
   if (host) {
     KRK_HIP(hipMemcpy(uids, d_uids, (size_t)u * 8, hipMemcpyDeviceToHost));
     if (inv) KRK_HIP(hipMemcpy(inv, d_inv, (size_t)n * 8, hipMemcpyDeviceToHost));
   }
   KRK_HIP(hipStreamSynchronize(s));
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dedup_sum(const uint64_t* ids, int64_t n, const float* grads, int64_t dim, uint64_t* uids,
+                      int64_t* inv, float* sums, int64_t* n_unique, uint32_t flags) {
+  KRK_TRY(check_flags(flags));
+  if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;   // the count comes back by value
+  if (n < 0 || dim <= 0 || !n_unique || (n > 0 && (!ids || !grads || !uids || !sums))) return KRK_E_ARGUMENT;
+  if (n > ((int64_t)1 << 28)) {
+    set_error("krk_dedup_sum handles at most 2^28 ids per call; split the request");
+    return KRK_E_CAPACITY;
+  }
+  KRK_TRY(ensure_runtime());
+  *n_unique = 0;
+  if (n == 0) return KRK_SUCCESS;
+  ReduceShape sh;
+  sh.dim = dim;
+  sh.vec = dim % 4 == 0 ? 4 : 1;
+  sh.elems = (int)(dim / sh.vec);
+  sh.group = 4;
+  while (sh.group < sh.elems && sh.group < 64) sh.group <<= 1;
+  const bool host = !(flags & KRK_DEVICE_PTRS);
+  if (!host && sh.vec == 4 && ((((uintptr_t)grads) | ((uintptr_t)sums)) & 15)) {
+    set_error("device gradients and sums must be 16-byte aligned");
+    return KRK_E_ARGUMENT;
+  }
+  const size_t n8 = round256((size_t)n * 8);
+  const size_t rows_b = round256((size_t)n * (size_t)dim * sizeof(float));
+  std::lock_guard<std::mutex> pool_lock(g_dedup_mu);
+  DedupWork w;
+  KRK_TRY(dedup_layout(n, host ? 3 * n8 + 2 * rows_b : 0, &w));
+  const uint64_t* d_ids = ids;
+  const float* d_g = grads;
+  uint64_t* d_uids = uids;
+  long long* d_inv = reinterpret_cast<long long*>(inv);
+  float* d_sums = sums;
+  if (host) {
+    uint64_t* s_ids = reinterpret_cast<uint64_t*>(w.extra);
+    d_uids = reinterpret_cast<uint64_t*>(w.extra + n8);
+    d_inv = reinterpret_cast<long long*>(w.extra + 2 * n8);
+    float* s_g = reinterpret_cast<float*>(w.extra + 3 * n8);
+    d_sums = reinterpret_cast<float*>(w.extra + 3 * n8 + rows_b);
+    KRK_HIP(hipMemcpy(s_ids, ids, (size_t)n * 8, hipMemcpyHostToDevice));
+    KRK_HIP(hipMemcpy(s_g, grads, (size_t)n * (size_t)dim * sizeof(float), hipMemcpyHostToDevice));
+    d_ids = s_ids;
+    d_g = s_g;
+  }
+  hipStream_t s = nullptr;
+  int32_t u = 0;
+  KRK_TRY(dedup_core(w, d_ids, n, d_uids, s, &u));
+  if (inv) {
+    hipLaunchKernelGGL(dedup_inv_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, w.slots, w.slot_of, n,
+                       d_inv);
+    KRK_HIP(hipGetLastError());
+  }
+  // positions sorted by unique index (stable: position order inside a run, as
+  // worker/emitter.cc:527-529 adds them), every run summed and stored as row `index` of sums
+  uint32_t miss_key = 1;
+  int bits = 1;
+  while ((int64_t)miss_key < (int64_t)u) {
+    miss_key <<= 1;
+    ++bits;
+  }
+  TableView tv{};
+  tv.recs = d_sums;
+  tv.stride = dim;
+  ApplyArgs args{};
+  args.c0 = args.c1 = args.c2 = args.meta_off = -1;
+  const DSlot* slots = w.slots;
+  const uint32_t* slot_of = w.slot_of;
+  KRK_TRY(sort_and_reduce(sh, s, g_dedup_reduce, tv, kOptStore, n, miss_key, bits, d_g, args,
+                          PooledSrc{nullptr, nullptr}, [&](uint32_t* keys, uint32_t* pos) {
+                            hipLaunchKernelGGL(dedup_pairs_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s,
+                                               slots, slot_of, n, keys, pos);
+                          }));
+  *n_unique = u;
+  if (host) {
+    KRK_HIP(hipMemcpy(uids, d_uids, (size_t)u * 8, hipMemcpyDeviceToHost));
+    if (inv) KRK_HIP(hipMemcpy(inv, d_inv, (size_t)n * 8, hipMemcpyDeviceToHost));
+    KRK_HIP(hipMemcpy(sums, d_sums, (size_t)u * (size_t)dim * sizeof(float), hipMemcpyDeviceToHost));
+  }
+  KRK_HIP(hipStreamSynchronize(s));
+  return KRK_SUCCESS;
+}
+
+int32_t krk_expand_rows(const float* rows, int64_t n_rows, const int64_t* inv, int64_t n, int64_t dim,
+                        float* out, uint32_t flags) {
+  KRK_TRY(check_flags(flags));
+  if (n < 0 || n_rows < 0 || dim <= 0 || (n > 0 && (!rows || !inv || !out))) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  if (n == 0) return KRK_SUCCESS;
+  const int vec = dim % 4 == 0 ? 4 : 1;
+  const int elems = (int)(dim / vec);
+  const bool host = !(flags & KRK_DEVICE_PTRS);
+  if (!host && vec == 4 && ((((uintptr_t)rows) | ((uintptr_t)out)) & 15)) {
+    set_error("device rows and output must be 16-byte aligned");
+    return KRK_E_ARGUMENT;
+  }
+  const size_t in_b = round256((size_t)n_rows * (size_t)dim * sizeof(float));
+  const size_t inv_b = round256((size_t)n * 8);
+  const size_t out_b = round256((size_t)n * (size_t)dim * sizeof(float));
+  std::lock_guard<std::mutex> pool_lock(g_dedup_mu);
+  KRK_TRY(g_dedup_pool.reserve(256 + (host ? in_b + inv_b + out_b : 0)));
+  char* base = g_dedup_pool.as<char>();
+  uint32_t* d_err = reinterpret_cast<uint32_t*>(base);
+  const float* d_rows = rows;
+  const long long* d_inv = reinterpret_cast<const long long*>(inv);
+  float* d_out = out;
+  hipStream_t s = nullptr;
+  if (host) {
+    float* s_rows = reinterpret_cast<float*>(base + 256);
+    long long* s_inv = reinterpret_cast<long long*>(base + 256 + in_b);
+    d_out = reinterpret_cast<float*>(base + 256 + in_b + inv_b);
+    KRK_HIP(hipMemcpy(s_rows, rows, (size_t)n_rows * (size_t)dim * sizeof(float), hipMemcpyHostToDevice));
+    KRK_HIP(hipMemcpy(s_inv, inv, (size_t)n * 8, hipMemcpyHostToDevice));
+    d_rows = s_rows;
+    d_inv = s_inv;
+  }
+  KRK_HIP(hipMemsetAsync(d_err, 0, 4, s));
+  int64_t blocks = (n * elems + kBlock - 1) / kBlock;
+  if (blocks > 256 * 64) blocks = 256 * 64;   // grid-stride beyond that
+  if (vec == 4) {
+    hipLaunchKernelGGL((expand_rows_kernel<4>), dim3((unsigned)blocks), dim3(kBlock), 0, s, d_rows, d_inv, n,
+                       n_rows, d_out, (int)dim, elems, d_err);
+  } else {
+    hipLaunchKernelGGL((expand_rows_kernel<1>), dim3((unsigned)blocks), dim3(kBlock), 0, s, d_rows, d_inv, n,
+                       n_rows, d_out, (int)dim, elems, d_err);
+  }
+  KRK_HIP(hipGetLastError());
+  uint32_t err = 0;
+  KRK_HIP(hipMemcpy(&err, d_err, 4, hipMemcpyDeviceToHost));
+  if (host) KRK_HIP(hipMemcpy(out, d_out, (size_t)n * (size_t)dim * sizeof(float), hipMemcpyDeviceToHost));
+  KRK_HIP(hipStreamSynchronize(s));
+  if (err) {
+    set_error("an index lies outside the %lld rows", (long long)n_rows);
+    return KRK_E_ARGUMENT;
+  }
   return KRK_SUCCESS;
 }
 

@@ -159,3 +159,45 @@ def test_push_raw_missing_id_and_width(api, oracle):
     assert t.lookup([77])[0] == -1
     assert t.PushRaw(o, [1, 2], np.ones((2, 4), np.float32), 0.1) == 11
     assert t.PushRaw(o, [], np.zeros((0, 8), np.float32), 0.1) == 0
+
+
+@pytest.mark.parametrize("dim", [1, 6, 16, 128])
+@pytest.mark.parametrize("n,s,space", [(1, 1.05, 10), (9, 1.05, 4), (8192, 1.05, 10**6), (300_000, 1.3, 10**6)])
+def test_dedup_sum_standalone(api, oracle, dim, n, s, space):
+    """Emitter::PushSparseTable's dedup + sum as a call of its own: unique ids, inverse map and
+    (on a binary grid, where the order of additions cannot matter) the summed rows all exact."""
+    rng = np.random.default_rng(dim * 1000 + n)
+    ids = zipf_ids(rng, s, space, n)
+    g = (rng.integers(-64, 65, size=(n, dim)) / 4096.0).astype(np.float32)
+    u, inv, sums = api.dedup_sum(ids, g)
+    ru, rs = oracle.dedup_sum(ids, g)
+    _, rinv = oracle.dedup(ids)
+    assert np.array_equal(u, ru) and np.array_equal(inv, rinv)
+    assert np.array_equal(sums, rs)
+    # the pull side's re-expansion (worker/emitter.cc:162-182) undoes the dedup
+    rc, back = api.expand_rows(sums, inv)
+    assert rc == 0 and np.array_equal(back, rs[rinv])
+
+
+def test_dedup_sum_random_gradients_and_device_arrays(api, oracle):
+    rng = np.random.default_rng(77)
+    n, dim = 500_000, 32
+    ids = zipf_ids(rng, 1.2, 10**6, n)
+    g = rng.standard_normal((n, dim)).astype(np.float32)
+    d_u, d_inv, d_sums, count = api.dedup_sum(api.DeviceArray.from_host(ids), api.DeviceArray.from_host(g))
+    ru, rinv = oracle.dedup(ids)
+    assert count == ru.size
+    assert np.array_equal(d_u.to_host()[:count], ru) and np.array_equal(d_inv.to_host(), rinv)
+    exact = np.zeros((count, dim), np.float64)
+    np.add.at(exact, rinv, g.astype(np.float64))
+    mass = np.zeros((count, dim), np.float64)
+    np.add.at(mass, rinv, np.abs(g).astype(np.float64))
+    got = d_sums.to_host()[:count]
+    # fp32 summation in a fixed tree: error bounded by a few ulps of the summed magnitudes
+    assert (np.abs(got - exact) <= 4e-7 * mass + 1e-30).all()
+    rc, d_back = api.expand_rows(d_sums, d_inv)
+    assert rc == 0 and np.array_equal(d_back.to_host(), got[rinv])
+    bad = rinv.copy()
+    bad[5] = count + 3
+    rc, _ = api.expand_rows(got, bad)
+    assert rc == api.E_ARGUMENT
