@@ -114,15 +114,29 @@ def run_gpu(cfg, steps, warmup, n_batches=32):
         dev.append((api.DeviceArray.from_host(ids), api.DeviceArray.from_host(g),
                     api.DeviceArray((ids.size, dim), np.float32), off, ids.size))
 
+    # several tables: one combined request per step (one launch each way); a single table
+    # is called directly, as a server with one sparse table would
+    def pull(d_ids, off, d_out):
+        if single:
+            tables[0].Pull(d_ids, out=d_out, async_=True)
+        else:
+            group.CombinePull(d_ids, off, out=d_out, async_=True)
+
+    def push(d_ids, off, d_g):
+        if single:
+            tables[0].Push(optim, d_ids, d_g, lr, async_=True)
+        else:
+            group.CombinePush(optim, d_ids, off, d_g, lr, async_=True)
+
     def step(i):
         d_ids, d_g, d_out, off, _ = dev[i % n_batches]
-        group.CombinePull(d_ids, off, out=d_out, async_=True)
-        group.CombinePush(optim, d_ids, off, d_g, lr, async_=True)
+        pull(d_ids, off, d_out)
+        push(d_ids, off, d_g)
         if dense is not None:
             dense.Push(dense_opt, d_dense_g[i % n_batches], 1e-3, async_=True)
 
     def sync_all():
-        rc = group.sync()
+        rc = owner.sync()
         if rc != 0:
             raise RuntimeError("sparse tables reported error %d" % rc)
         if dense is not None:
@@ -143,7 +157,9 @@ def run_gpu(cfg, steps, warmup, n_batches=32):
             t.sync()
             d.free()
     scratch.free()
-    group = api.TableGroup(tables)
+    single = len(tables) == 1
+    group = None if single else api.TableGroup(tables)
+    owner = tables[0] if single else group          # whose stream the step's launches run on
     for i in range(n_batches):
         step(i)
     sync_all()
@@ -168,16 +184,16 @@ def run_gpu(cfg, steps, warmup, n_batches=32):
     for kind in ("push", "pull"):
         for timed in (False, True):
             if timed:
-                e0.record(group)
+                e0.record(owner)
             for j in range(reps):
                 d_ids, d_g, d_out, off, _ = dev[j % n_batches]
                 if kind == "push":
-                    group.CombinePush(optim, d_ids, off, d_g, lr, async_=True)
+                    push(d_ids, off, d_g)
                 else:
-                    group.CombinePull(d_ids, off, out=d_out, async_=True)
+                    pull(d_ids, off, d_out)
             if timed:
-                e1.record(group)
-            group.sync()
+                e1.record(owner)
+            owner.sync()
         ms = e0.elapsed_ms(e1) / reps
         u = float(np.mean([dev[j % n_batches][4] for j in range(reps)]))
         if kind == "push":
@@ -188,7 +204,7 @@ def run_gpu(cfg, steps, warmup, n_batches=32):
     push_bytes = push_u * (8 + 4 * dim + 8 * dim * (1 + S) + extra)
     pull_bytes = pull_u * (8 + 8 * dim)
     roofline = {
-        "bound": "hbm", "kernel": "group_push_kernel<%s,4>" % cfg["optim"],
+        "bound": "hbm", "kernel": "%spush_kernel<%s,4>" % ("" if single else "group_", cfg["optim"]),
         "achieved": push_bytes / (push_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": push_bytes / (push_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
         "bytes_per_launch": push_bytes, "us_per_launch": push_ms * 1e3,
@@ -297,7 +313,7 @@ def main():
     cfg = WORKLOADS[args.workload]
     dt, rows, roofline, batches = run_gpu(cfg, args.steps, args.warmup)
     # the same achieved figure against what a plain copy kernel moves on this very box
-    ceiling = copy_calibration(nbytes=1 << 28, reps=10)["copy_gbs_read_plus_write"]
+    ceiling = copy_calibration(nbytes=1 << 30, reps=10)["copy_gbs_read_plus_write"]
     roofline["copy_ceiling"] = ceiling
     roofline["frac_of_copy_ceiling"] = roofline["achieved"] / ceiling
     value = rows / dt
