@@ -231,7 +231,7 @@ def test_device_pointers_and_async(api, oracle):
 
 
 def test_config1_plumbing(api, oracle):
-    """BASELINE config 1 in full: one table, dim 8, 100k preloaded rows N(0, 0.01) seed 0,
+    """The first benchmark configuration in full: one table, dim 8, 100k preloaded rows N(0, 0.01) seed 0,
     100 steps of 1024 x 26 uniform ids, pull then push N(0, 1e-2) grads, SGD lr 0.01; the whole
     final table is compared. Duplicate ids inside a step are reduced worker-side in the
     reference (emitter.cc:516-531): the oracle side uses its dedup_sum, the GPU side PushRaw."""

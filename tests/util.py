@@ -23,7 +23,7 @@ def zipf_ranks(rng, s, space, size):
 
 
 def zipf_ids(rng, s, space, size):
-    """BASELINE config ids: splitmix64 of a Zipf rank."""
+    """Ids of the benchmark configurations: splitmix64 of a Zipf rank."""
     return splitmix64(zipf_ranks(rng, s, space, size))
 
 
