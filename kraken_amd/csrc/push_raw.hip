@@ -54,36 +54,58 @@ struct DSlot {
   uint32_t uidx;     // its index in the unique list
 };
 
-__global__ __launch_bounds__(kBlock) void dedup_claim_kernel(DSlot* slots, uint64_t mask,
-                                                             const uint64_t* __restrict__ ids, int64_t n,
-                                                             uint32_t* __restrict__ slot_of) {
-  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+// Equal ids are folded inside the workgroup first, through a small hash table in LDS: the lane
+// that claims an LDS entry speaks for every position of that id in the workgroup's 1024
+// consecutive positions (the entry collects their smallest position), and only it goes to the
+// request-wide index. An id that fills a quarter of the request then costs one global probe
+// and at most one atomic per workgroup instead of 256, and a workgroup of all-distinct ids pays
+// one LDS atomic per lane rather than a vote per distinct id.
+constexpr int kDedupBlock = 1024;
+constexpr int kDedupLds = 2048;   // entries: at most half full
+
+__global__ __launch_bounds__(kDedupBlock) void dedup_claim_kernel(DSlot* slots, uint64_t mask,
+                                                                  const uint64_t* __restrict__ ids, int64_t n,
+                                                                  uint32_t* __restrict__ slot_of) {
+  __shared__ unsigned long long lkey[kDedupLds + 1];   // the last entry belongs to the all-ones id
+  __shared__ uint32_t lmin[kDedupLds + 1];
+  __shared__ uint32_t lidx[kDedupLds + 1];
+  for (int i = threadIdx.x; i <= kDedupLds; i += kDedupBlock) {
+    lkey[i] = kEmptyKey;
+    lmin[i] = 0xFFFFFFFFu;
+  }
+  __syncthreads();
+  const int64_t p = (int64_t)blockIdx.x * kDedupBlock + threadIdx.x;
   const bool active = p < n;
   const unsigned long long id = active ? ids[p] : 0ull;
-  const int lane = (int)(threadIdx.x & (kWave - 1));
-  // Equal ids inside one wavefront are folded first: positions grow with the lane number, so
-  // the lowest lane holding an id also holds its smallest position in this wave. Only that lane
-  // goes to the index; the others take the slot number from it. An id that fills a quarter of
-  // the request then costs one atomic per wave instead of sixteen.
-  int leader = lane;
-  unsigned long long todo = __ballot(active);
-  while (todo) {
-    const int first = __ffsll((unsigned long long)todo) - 1;
-    const unsigned int lo = __builtin_amdgcn_readlane((unsigned int)id, first);
-    const unsigned int hi = __builtin_amdgcn_readlane((unsigned int)(id >> 32), first);
-    const unsigned long long lid = (unsigned long long)lo | ((unsigned long long)hi << 32);
-    const bool same = active && id == lid;
-    if (same) leader = first;
-    todo &= ~__ballot(same);
+  int entry = kDedupLds;
+  bool owner = false;
+  if (active) {
+    if (id == kEmptyKey) {
+      owner = atomicCAS(&lkey[kDedupLds], kEmptyKey, 0ull) == kEmptyKey;
+    } else {
+      entry = (int)(mix64(id) >> 32) & (kDedupLds - 1);   // high bits: the index below uses the low ones
+      for (;;) {
+        const unsigned long long old = atomicCAS(&lkey[entry], kEmptyKey, id);
+        if (old == kEmptyKey || old == id) {
+          owner = old == kEmptyKey;
+          break;
+        }
+        entry = (entry + 1) & (kDedupLds - 1);
+      }
+    }
+    atomicMin(&lmin[entry], (uint32_t)p);
   }
-  uint64_t idx = 0;
-  if (active && leader == lane) {
+  __syncthreads();
+  if (owner) {
+    uint64_t idx;
     if (id == kEmptyKey) {
       idx = mask + 1;   // the all-ones id owns the extra last slot
     } else {
       idx = mix64(id) & mask;
       for (uint64_t t = 0; t <= mask; ++t) {
-        unsigned long long key = __atomic_load_n(&slots[idx].key, __ATOMIC_RELAXED);
+        // A plain (cacheable) load: a key never changes once it is set, so a hit is final.
+        // A stale "empty" only costs the CAS below.
+        unsigned long long key = slots[idx].key;
         if (key == kEmptyKey) {
           const unsigned long long old = atomicCAS(&slots[idx].key, kEmptyKey, id);
           key = old == kEmptyKey ? id : old;
@@ -92,13 +114,14 @@ __global__ __launch_bounds__(kBlock) void dedup_claim_kernel(DSlot* slots, uint6
         idx = (idx + 1) & mask;
       }
     }
-    // minpos only ever decreases, so a stale read can at worst cause a redundant atomic; later
-    // waves mostly find a smaller position already there and skip it.
-    if (__builtin_nontemporal_load(&slots[idx].minpos) > (uint32_t)p)
-      atomicMin(&slots[idx].minpos, (uint32_t)p);
+    // minpos only ever decreases, so a stale (cached) read can at worst cause a redundant
+    // atomic; later workgroups mostly find a smaller position already there and skip it.
+    const uint32_t first = lmin[entry];
+    if (slots[idx].minpos > first) atomicMin(&slots[idx].minpos, first);
+    lidx[entry] = (uint32_t)idx;
   }
-  const uint32_t shared_idx = __shfl((uint32_t)idx, leader);
-  if (active) slot_of[p] = shared_idx;
+  __syncthreads();
+  if (active) slot_of[p] = lidx[entry];
 }
 
 __global__ __launch_bounds__(kBlock) void dedup_flag_kernel(const DSlot* __restrict__ slots,
@@ -646,7 +669,8 @@ static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, 
                           int32_t* u) {
   KRK_HIP(hipMemsetAsync(w.slots, 0xFF, (w.cap + 1) * sizeof(DSlot), s));
   const dim3 grid(grid_for(n, kBlock)), block(kBlock);
-  hipLaunchKernelGGL(dedup_claim_kernel, grid, block, 0, s, w.slots, w.cap - 1, d_ids, n, w.slot_of);
+  hipLaunchKernelGGL(dedup_claim_kernel, dim3(grid_for(n, kDedupBlock)), dim3(kDedupBlock), 0, s, w.slots,
+                     w.cap - 1, d_ids, n, w.slot_of);
   hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, w.slots, w.slot_of, n, w.flag);
   KRK_HIP(hipGetLastError());
   KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
