@@ -153,6 +153,12 @@ int32_t krk_sparse_size(krk_sparse* t, int64_t* rows);
 int32_t krk_sparse_reserve(krk_sparse* t, int64_t rows);
 /* Waits for enqueued work and returns the first deferred error (then clears it). */
 int32_t krk_sparse_sync(krk_sparse* t);
+/* Makes the table enqueue its work on the caller's HIP stream (a hipStream_t) instead of its
+ * own, so that KRK_ASYNC calls are ordered with the caller's other work on that stream: a
+ * training framework passes the stream its tensors are produced and consumed on. NULL returns
+ * to the table's own stream. Work already enqueued is waited for first. The stream must outlive
+ * its use by the table; tables that belong to a group cannot switch. No reference counterpart. */
+int32_t krk_sparse_set_stream(krk_sparse* t, void* stream);
 
 /* SparseTable::Pull (ps/sparse_table.cc:33-75): out[i,:] = row of ids[i];
  * a missing id is inserted with the table's initializer and returned. ids may

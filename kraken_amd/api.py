@@ -75,6 +75,7 @@ EXPORTS = {
     "krk_sparse_size": (C.c_int32, [C.c_void_p, C.POINTER(C.c_int64)]),
     "krk_sparse_reserve": (C.c_int32, [C.c_void_p, C.c_int64]),
     "krk_sparse_sync": (C.c_int32, [C.c_void_p]),
+    "krk_sparse_set_stream": (C.c_int32, [C.c_void_p, C.c_void_p]),
     "krk_sparse_pull": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_uint32]),
     "krk_sparse_push": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_int64, C.c_void_p,
                                     C.c_int64, C.c_float, C.c_uint32]),

@@ -1100,6 +1100,21 @@ int32_t krk_sparse_destroy(krk_sparse* t) {
   return KRK_SUCCESS;
 }
 
+int32_t krk_sparse_set_stream(krk_sparse* t, void* stream) {
+  KRK_TRY(check_table(t));
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (t->member_of) {
+    set_error("a group member runs on its group's stream");
+    return KRK_E_ARGUMENT;
+  }
+  hipStream_t next = stream ? reinterpret_cast<hipStream_t>(stream) : t->own_stream;
+  if (next == t->stream) return KRK_SUCCESS;
+  // what is enqueued on the old stream must be complete before work on the new one may follow
+  KRK_TRY(sparse_finish(t, 0));
+  t->stream = next;
+  return KRK_SUCCESS;
+}
+
 int32_t krk_sparse_dim(krk_sparse* t, int64_t* dim) {
   if (!t || !dim) return KRK_E_ARGUMENT;
   *dim = t->dim;

@@ -1,0 +1,145 @@
+"""The reference's worker-side embedding modules on GPU tensors.
+
+`kraken/pytorch/embedding.py` and `jagged_embedding.py` wrap an autograd Function around
+`kraken_native.pull_sparse_table / push_sparse_table`, which reject device tensors
+(pytorch/py/pytorch.cc:42,102,116,188) and send the request to a server. Here the table lives on
+the same GPU as the tensors: forward is one pull (or one pooled pull) straight into a torch
+tensor, backward is one fused dedup + sum + optimizer step on the gradient torch hands over.
+Nothing is copied to the host and nothing is synchronised: the table enqueues its kernels on
+torch's current stream.
+
+PyTorch is plumbing here (it owns the tensors and the stream); the arithmetic is the table
+engine's. Importing this module needs torch; nothing else in the package does.
+"""
+import ctypes as C
+
+import torch
+
+from . import api
+
+
+def _stream_ptr():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ids_ptr(indices):
+    """int64 indices are the uint64 ids bit for bit (worker/emitter.cc:126 casts the same way)."""
+    if indices.dtype != torch.int64 or not indices.is_cuda:
+        raise TypeError("indices must be an int64 CUDA tensor")
+    indices = indices.contiguous()
+    return indices, C.c_void_p(indices.data_ptr())
+
+
+class GpuSparseTable(torch.nn.Parameter):
+    """pytorch/sparse_table.py: a Parameter that stands for the table so that autograd calls the
+    Function's backward. The rows are not in this tensor but in the engine's table."""
+
+    def __new__(cls, dimension, initializer=None, optim=None, lr=0.01, capacity_hint=0):
+        self = super().__new__(cls, torch.empty(0), requires_grad=True)
+        self._dimension = int(dimension)
+        self._table = api.SparseTable(dimension, initializer or api.Initializer.create(
+            api.InitializerType.kNormal, {}), capacity_hint=capacity_hint)
+        self._optim = optim or api.Optim.create(api.OptimType.kSGD)
+        self.lr = float(lr)
+        return self
+
+    def dimension(self):
+        return self._dimension
+
+    def table(self):
+        return self._table
+
+    def _on_current_stream(self):
+        api._check(api.lib().krk_sparse_set_stream(self._table.h, _stream_ptr()), "krk_sparse_set_stream")
+        return self._table.h
+
+
+class EmbeddingFunction(torch.autograd.Function):
+    """pytorch/embedding.py:9-23"""
+
+    @staticmethod
+    def forward(ctx, sparse_table, indices):
+        ids, p_ids = _ids_ptr(indices)
+        dim = sparse_table.dimension()
+        out = torch.empty(tuple(indices.shape) + (dim,), dtype=torch.float32, device=indices.device)
+        h = sparse_table._on_current_stream()
+        api._check(api.lib().krk_sparse_pull(h, p_ids, ids.numel(), C.c_void_p(out.data_ptr()),
+                                             api.DEVICE_PTRS | api.ASYNC), "krk_sparse_pull")
+        ctx.table = sparse_table
+        ctx.save_for_backward(ids)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        (ids,) = ctx.saved_tensors
+        t = ctx.table
+        grad = grad.contiguous().to(torch.float32)
+        h = t._on_current_stream()
+        api._check(api.lib().krk_sparse_push_raw(h, C.byref(t._optim.raw), C.c_void_p(ids.data_ptr()), ids.numel(),
+                                                 C.c_void_p(grad.data_ptr()), t.dimension(), t.lr,
+                                                 api.DEVICE_PTRS | api.ASYNC), "krk_sparse_push_raw")
+        return None, None
+
+
+class Embedding(torch.nn.Module):
+    """pytorch/embedding.py:26-43 with the table on the GPU. The optimizer step of the rows is
+    part of backward (the reference applies it on the server when the push arrives)."""
+
+    def __init__(self, dimension, initializer=None, optim=None, lr=0.01, capacity_hint=0):
+        super().__init__()
+        self.sparse_table = GpuSparseTable(dimension, initializer, optim, lr, capacity_hint)
+
+    def forward(self, indices):
+        return EmbeddingFunction.apply(self.sparse_table, indices)
+
+
+class JaggedEmbeddingFunction(torch.autograd.Function):
+    """pytorch/jagged_embedding_funcs.py over pytorch/py/jagged_ops.cc, fused with the table."""
+
+    @staticmethod
+    def forward(ctx, sparse_table, indices, offsets, weights, mode, patch_value):
+        ids, p_ids = _ids_ptr(indices)
+        if offsets.dtype != torch.int64 or not offsets.is_cuda:
+            raise TypeError("offsets must be an int64 CUDA tensor")
+        offsets = offsets.contiguous()
+        w = weights.contiguous().to(torch.float32) if weights is not None else None
+        bags = offsets.numel() - 1
+        out = torch.empty((bags, sparse_table.dimension()), dtype=torch.float32, device=indices.device)
+        h = sparse_table._on_current_stream()
+        api._check(api.lib().krk_sparse_pull_pooled(
+            h, p_ids, ids.numel(), C.c_void_p(offsets.data_ptr()), bags,
+            C.c_void_p(w.data_ptr()) if w is not None else None, mode, patch_value, C.c_void_p(out.data_ptr()),
+            api.DEVICE_PTRS | api.ASYNC), "krk_sparse_pull_pooled")
+        ctx.table, ctx.mode, ctx.weights = sparse_table, mode, w
+        ctx.save_for_backward(ids, offsets)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        ids, offsets = ctx.saved_tensors
+        t, w = ctx.table, ctx.weights
+        grad = grad.contiguous().to(torch.float32)
+        h = t._on_current_stream()
+        api._check(api.lib().krk_sparse_push_pooled(
+            h, C.byref(t._optim.raw), C.c_void_p(ids.data_ptr()), ids.numel(), C.c_void_p(offsets.data_ptr()),
+            offsets.numel() - 1, C.c_void_p(w.data_ptr()) if w is not None else None, ctx.mode,
+            C.c_void_p(grad.data_ptr()), t.dimension(), t.lr, api.DEVICE_PTRS | api.ASYNC), "krk_sparse_push_pooled")
+        return None, None, None, None, None, None
+
+
+class JaggedEmbedding(torch.nn.Module):
+    """pytorch/jagged_embedding.py:10-52: values / offsets / optional weights of a jagged batch,
+    pooled per bag with sum or mean; an empty bag yields patch_value."""
+
+    def __init__(self, dimension, initializer=None, optim=None, lr=0.01, mode="sum", patch_value=0.0,
+                 capacity_hint=0):
+        super().__init__()
+        if mode not in ("sum", "mean"):
+            raise ValueError("JaggedEmbedding's mode only support sum/mean.")
+        self.sparse_table = GpuSparseTable(dimension, initializer, optim, lr, capacity_hint)
+        self._mode = 0 if mode == "sum" else 1
+        self._patch_value = float(patch_value)
+
+    def forward(self, values, offsets, weights=None):
+        return JaggedEmbeddingFunction.apply(self.sparse_table, values, offsets, weights, self._mode,
+                                             self._patch_value)

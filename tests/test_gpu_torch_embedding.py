@@ -1,0 +1,106 @@
+"""The worker-side embedding modules (kraken/pytorch/embedding.py, jagged_embedding.py) on GPU
+tensors: forward values and the rows after backward agree with the oracle fed with the very
+gradient torch's autograd produced."""
+import numpy as np
+import pytest
+
+from util import assert_close, make_optims
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def mods():
+    if not torch.cuda.is_available():
+        pytest.skip("torch sees no GPU")
+    from kraken_amd import api, torch_embedding
+    api.lib()
+    return api, torch_embedding
+
+
+def _init(api, oracle, seed):
+    return (api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": str(seed)}),
+            oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=seed))
+
+
+def test_embedding_forward_backward(mods, oracle):
+    api, te = mods
+    dim = 16
+    gi, oi = _init(api, oracle, 3)
+    o_ref, o_gpu = make_optims(oracle, api, 0, {})
+    emb = te.Embedding(dim, initializer=gi, optim=o_gpu, lr=0.05)
+    head = torch.nn.Linear(dim, 1, bias=False).cuda()
+    ref = oracle.SparseTable(dim, oi)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    for step in range(3):
+        idx = torch.randint(0, 500, (64, 7), generator=g).cuda()        # a batch of 7 fields, with repeats
+        out = emb(idx)
+        ids = idx.cpu().numpy().astype(np.uint64).ravel()
+        u, inv = oracle.dedup(ids)
+        rc, rows = ref.pull(u)
+        assert_close(out.detach().cpu().numpy().reshape(-1, dim), rows[inv], "forward %d" % step, rtol=1e-6)
+        out.retain_grad()
+        loss = head(out).square().sum()
+        loss.backward()
+        grad = out.grad.detach().cpu().numpy().reshape(-1, dim)
+        assert np.abs(grad).sum() > 0
+        u2, gs = oracle.dedup_sum(ids, grad)
+        assert ref.push(o_ref, u2, gs, 0.05) == 0
+        assert emb.sparse_table.grad is None                            # the rows are not in the Parameter
+    torch.cuda.synchronize()
+    t = emb.sparse_table.table()
+    rid, rval, _, _ = ref.export()
+    assert len(t) == len(ref)
+    # sums of fp32 gradients in two orders: compared at the tolerance of the values they move
+    assert_close(t.Pull(rid)[1], rval, "rows after three steps", rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("mode", ["sum", "mean"])
+@pytest.mark.parametrize("weighted", [False, True])
+def test_jagged_embedding_forward_backward(mods, oracle, mode, weighted):
+    api, te = mods
+    dim = 8
+    gi, oi = _init(api, oracle, 9)
+    o_ref, o_gpu = make_optims(oracle, api, 3, {})                      # plain SGD: linear in the summed gradient
+    emb = te.JaggedEmbedding(dim, initializer=gi, optim=o_gpu, lr=0.5, mode=mode, patch_value=0.25)
+    ref = oracle.SparseTable(dim, oi)
+    rng = np.random.default_rng(1)
+    for step in range(2):
+        lengths = rng.integers(0, 6, size=200)
+        off = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
+        ids = rng.integers(0, 300, size=int(off[-1])).astype(np.uint64)
+        w = (2.0 ** rng.integers(-1, 2, size=ids.size)).astype(np.float32) if weighted else None
+        out = emb(torch.from_numpy(ids.astype(np.int64)).cuda(), torch.from_numpy(off).cuda(),
+                  torch.from_numpy(w).cuda() if weighted else None)
+        u, inv = oracle.dedup(ids)
+        rows = ref.pull(u)[1][inv]
+        if weighted:
+            rows = rows * w[:, None]
+        want = oracle.jagged_forward(rows, off, mode, 0.25)
+        if step == 0 or mode == "sum":
+            # the bag is added up in the reference's order: identical bits (after a mean step
+            # the rows themselves carry sums of inexact addends and agree to rounding only)
+            assert np.array_equal(out.detach().cpu().numpy(), want)
+        else:
+            assert_close(out.detach().cpu().numpy(), want, "pooled forward", rtol=1e-5, atol=1e-6)
+        coef = (rng.integers(-8, 9, size=(lengths.size, dim)) / 16.0).astype(np.float32)
+        (out * torch.from_numpy(coef).cuda()).sum().backward()
+        vg = oracle.jagged_backward(off, coef, mode)
+        if weighted:
+            vg = vg * w[:, None]
+        u2, gs = oracle.dedup_sum(ids, vg)
+        assert ref.push(o_ref, u2, gs, 0.5) == 0
+    torch.cuda.synchronize()
+    rid, rval, _, _ = ref.export()
+    assert_close(emb.sparse_table.table().Pull(rid)[1], rval, "rows after two steps", rtol=1e-5, atol=1e-6)
+
+
+def test_rejects_host_tensors(mods):
+    api, te = mods
+    emb = te.Embedding(4)
+    with pytest.raises(TypeError):
+        emb(torch.zeros(3, dtype=torch.int64))
+    with pytest.raises(TypeError):
+        emb(torch.zeros(3, dtype=torch.int32).cuda())
