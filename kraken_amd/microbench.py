@@ -1,0 +1,240 @@
+"""Per-kernel timings of the table engine at the sizes of the benchmark configurations.
+
+    python -m kraken_amd.microbench [tables] [raw] [pooled] [codec] [dense] [dct2] [copy]
+
+Every figure is the average of back-to-back launches between two HIP events recorded on the
+stream the kernels run on, with inputs resident in HBM; bandwidths are algorithmic bytes
+(stated per line) over that time. With no argument all sections run (about a minute). This is
+the program the rocprofv3 summaries of the individual kernels are taken from.
+"""
+import sys
+
+import numpy as np
+
+from . import api
+
+
+def splitmix64(x):
+    with np.errstate(over="ignore"):
+        z = np.asarray(x, dtype=np.uint64) + np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+
+def zipf_ranks(rng, s, space, size):
+    w = 1.0 / np.arange(1, space + 1, dtype=np.float64) ** s
+    cdf = np.cumsum(w)
+    cdf /= cdf[-1]
+    return np.searchsorted(cdf, rng.random(size)).astype(np.uint64)
+
+
+def timed(owner, fn, reps=10, sync=None):
+    """Average seconds per call of fn between two events on owner's stream (None: null stream)."""
+    sync = sync or (owner.sync if owner is not None else api.synchronize)
+    fn()
+    sync()
+    e0, e1 = api.Event(), api.Event()
+    e0.record(owner)
+    for _ in range(reps):
+        fn()
+    e1.record(owner)
+    sync()
+    return e0.elapsed_ms(e1) / reps * 1e-3
+
+
+def prefill(t, rows, dim, chunk=1 << 22):
+    scratch = api.DeviceArray((min(chunk, rows), dim), np.float32)
+    t.reserve(rows + rows // 8)
+    for lo in range(0, rows, chunk):
+        d = api.DeviceArray.from_host(splitmix64(np.arange(lo, min(lo + chunk, rows), dtype=np.uint64)))
+        t.Pull(d, out=scratch, async_=True)
+        t.sync()
+        d.free()
+    scratch.free()
+
+
+def tables():
+    print("# lookup / pull / push of U unique resident ids, table of 4e6 rows")
+    print("#   bytes: lookup 20U, pull U(8+8D), push U(8+4D+8D(1+S)) (+16U Adam)")
+    init = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "0"})
+    rows = 4 * 10**6
+    for dim, u, optim_name in ((16, 98_600, "adagrad"), (16, 10**6, "adagrad"), (32, 10**6, "adagrad"),
+                               (64, 10**6, "adagrad"), (128, 10**6, "adagrad"), (32, 10**6, "adam")):
+        t = api.SparseTable(dim, init, capacity_hint=rows)
+        prefill(t, rows, dim)
+        rng = np.random.default_rng(0)
+        sets = []
+        for _ in range(4):
+            ids = splitmix64(rng.choice(rows, size=u, replace=False).astype(np.uint64))
+            sets.append((api.DeviceArray.from_host(ids),
+                         api.DeviceArray.from_host((rng.standard_normal((u, dim)) * 1e-2).astype(np.float32)),
+                         api.DeviceArray((u, dim), np.float32), api.DeviceArray(u, np.int32)))
+        o = api.Optim.create({"adagrad": 0, "adam": 1}[optim_name])
+        S = {"adagrad": 1, "adam": 2}[optim_name]
+        k = [0]
+
+        def nxt():
+            k[0] += 1
+            return sets[k[0] % 4]
+
+        def lookup():
+            d_ids, _, _, d_rows = nxt()
+            api.lib().krk_sparse_lookup(t.h, api._ptr(d_ids), u, api._ptr(d_rows), api.DEVICE_PTRS | api.ASYNC)
+
+        def pull():
+            d_ids, _, d_out, _ = nxt()
+            t.Pull(d_ids, out=d_out, async_=True)
+
+        def push():
+            d_ids, d_g, _, _ = nxt()
+            t.Push(o, d_ids, d_g, 0.01, async_=True)
+
+        tl, tp, tq = timed(t, lookup, 20), timed(t, pull, 20), timed(t, push, 20)
+        bl, bp = 20 * u, u * (8 + 8 * dim)
+        bq = u * (8 + 4 * dim + 8 * dim * (1 + S) + (16 if optim_name == "adam" else 0))
+        print("dim %3d U %8d %-7s | lookup %7.1f us %5.0f GB/s | pull %7.1f us %5.0f GB/s | push %7.1f us %5.0f GB/s"
+              % (dim, u, optim_name, tl * 1e6, bl / tl / 1e9, tp * 1e6, bp / tp / 1e9, tq * 1e6, bq / tq / 1e9),
+              flush=True)
+        for s in sets:
+            for a in s:
+                a.free()
+        t.close()
+
+
+def raw():
+    print("# push_raw (dedup + duplicate-gradient sum + update fused) and stand-alone dedup of N ids")
+    print("#   bytes: U(8+4D+8D(1+S)) + 8N + 4DN")
+    init = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01"})
+    for dim, space, n, s, optim in ((16, 10**6, 8192, 1.05, 0), (16, 10**6, 212_992, 1.05, 0),
+                                    (128, 2 * 10**7, 1 << 20, 1.3, 2), (32, 10**7, 2_000_000, 1.1, 1)):
+        rng = np.random.default_rng(0)
+        t = api.SparseTable(dim, init, capacity_hint=min(space, 3 * 10**7))
+        ids = splitmix64(zipf_ranks(rng, s, space, n))
+        u = np.unique(ids).size
+        d_ids = api.DeviceArray.from_host(ids)
+        d_g = api.DeviceArray.from_host((rng.standard_normal((n, dim)) * 1e-2).astype(np.float32))
+        d_out = api.DeviceArray((n, dim), np.float32)
+        t.Pull(d_ids, out=d_out, async_=True)
+        assert t.sync() == 0
+        o = api.Optim.create(optim, {"alpha": "0.9"} if optim == 2 else {})
+        S = {0: 1, 1: 2, 2: 1}[optim]
+        dt = timed(t, lambda: t.PushRaw(o, d_ids, d_g, 0.01, async_=True))
+        dp = timed(t, lambda: t.Pull(d_ids, out=d_out, async_=True))
+        alg = u * (8 + 4 * dim + 8 * dim * (1 + S)) + 8 * n + 4 * dim * n
+        uids, inv = api.DeviceArray(n, np.uint64), api.DeviceArray(n, np.int64)
+        cnt = api.C.c_int64()
+
+        def dedup():
+            api.lib().krk_dedup(api._ptr(d_ids), n, api._ptr(uids), api._ptr(inv), api.C.byref(cnt),
+                                api.DEVICE_PTRS)
+        dd = timed(None, dedup, 5)
+        print("dim %3d N %8d U %7d zipf %.2f | push_raw %7.1f us %5.0f GB/s | pull of the N ids %7.1f us | "
+              "dedup (blocking call) %7.1f us" % (dim, n, u, s, dt * 1e6, alg / dt / 1e9, dp * 1e6, dd * 1e6),
+              flush=True)
+        for a in (d_ids, d_g, d_out, uids, inv):
+            a.free()
+        t.close()
+
+
+def pooled():
+    print("# multi-hot field of the DeepFM shape: 65536 samples x 13 fields, 1..20 ids per bag, dim 32,")
+    print("# table of 1e7 rows, Zipf 1.1")
+    space, dim, samples = 10**7, 32, 65536
+    rng = np.random.default_rng(0)
+    init = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "3"})
+    t = api.SparseTable(dim, init, capacity_hint=space)
+    prefill(t, space, dim)
+    bags = samples * 13
+    lengths = rng.integers(1, 21, size=bags)
+    off = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
+    n = int(off[-1])
+    d_ids = api.DeviceArray.from_host(splitmix64(zipf_ranks(rng, 1.1, space, n)))
+    d_off = api.DeviceArray.from_host(off)
+    d_g = api.DeviceArray.from_host((rng.standard_normal((bags, dim)) * 1e-3).astype(np.float32))
+    d_out = api.DeviceArray((bags, dim), np.float32)
+    d_rows = api.DeviceArray((n, dim), np.float32)
+    opt = api.Optim.create(api.OptimType.kAdam)
+    print("bags %d ids %d" % (bags, n), flush=True)
+    for name, fn in (
+            ("pull of every id -> [n, dim]", lambda: t.Pull(d_ids, out=d_rows, async_=True)),
+            ("pooled pull (mean) -> [bags, dim]", lambda: t.PullPooled(d_ids, d_off, "mean", out=d_out, async_=True)),
+            ("push_raw of [n, dim] gradients", lambda: t.PushRaw(opt, d_ids, d_rows, 1e-3, async_=True)),
+            ("pooled push (mean)", lambda: t.PushPooled(opt, d_ids, d_off, d_g, 1e-3, mode="mean", async_=True)),
+            ("pooled push (sum)", lambda: t.PushPooled(opt, d_ids, d_off, d_g, 1e-3, mode="sum", async_=True))):
+        print("%-36s %8.1f us" % (name, timed(t, fn, 5) * 1e6), flush=True)
+    t.close()
+
+
+def codec():
+    print("# threshold codec, eta 0.75: bytes compress 12n + 12nnz, decode 4n + 16nnz")
+    for n in (1 << 20, 4096 * 16384):
+        rng = np.random.default_rng(1)
+        d_g = api.DeviceArray.from_host(rng.standard_normal(n).astype(np.float32))
+        bag = api.DenseBag(n)
+        idx, val = api.DeviceArray(n, np.int64), api.DeviceArray(n, np.float32)
+        nnz = bag.MaybeToCoo(1000, 0.75, d_g, idx, val)[2]
+        dt = timed(bag, lambda: bag.MaybeToCoo(1000, 0.75, d_g, idx, val), 5, sync=api.synchronize)
+        dense = api.DeviceArray(n, np.float32)
+
+        def decode():
+            api.lib().krk_coo_to_dense(api._ptr(idx), api._ptr(val), nnz, api._ptr(dense), n, api.DEVICE_PTRS)
+        dd = timed(None, decode, 5)
+        print("n %9d nnz %9d | compress (stale threshold) %7.1f us %5.0f GB/s | decode (blocking call) %7.1f us "
+              "%5.0f GB/s" % (n, nnz, dt * 1e6, (12 * n + 12 * nnz) / dt / 1e9, dd * 1e6,
+                              (4 * n + 16 * nnz) / dd / 1e9), flush=True)
+        for a in (d_g, idx, val, dense):
+            a.free()
+
+
+def dense():
+    print("# dense table, Adam: bytes 28P")
+    for p in (150_000, 1 << 26):
+        t = api.DenseTable(np.zeros(p, np.float32))
+        o = api.Optim.create(api.OptimType.kAdam)
+        g = api.DeviceArray.from_host(np.ones(p, np.float32))
+        dt = timed(t, lambda: t.Push(o, g, 1e-3, async_=True), 50)
+        print("P %9d | push %7.1f us %5.0f GB/s" % (p, dt * 1e6, 28 * p / dt / 1e9), flush=True)
+        g.free()
+        t.close()
+
+
+def dct():
+    print("# blockwise DCT-II, block 256, n = 4096 x 16384: 2 n keep flop, 4 (n + n keep / 256) bytes")
+    n = 4096 * 16384
+    x = api.DeviceArray.from_host(np.random.default_rng(0).standard_normal(n).astype(np.float32))
+    for keep in (64, 128, 256):
+        y = api.DeviceArray((n // 256, keep), np.float32)
+        back = api.DeviceArray(n, np.float32)
+        fl = api.DEVICE_PTRS | api.ASYNC
+        for name, fn in (
+                ("forward", lambda: api.lib().krk_dct2_forward(api._ptr(x), api._ptr(y), n, keep, fl)),
+                ("inverse", lambda: api.lib().krk_dct2_inverse(api._ptr(y), api._ptr(back), n, keep, fl))):
+            dt = timed(None, fn, 10)
+            print("keep %3d %s | %7.1f us %6.1f TFLOP/s %5.0f GB/s" % (
+                keep, name, dt * 1e6, 2.0 * n * keep / dt / 1e12, 4.0 * (n + n // 256 * keep) / dt / 1e9), flush=True)
+        y.free()
+        back.free()
+
+
+def copy():
+    nbytes = 1 << 30
+    a, b = api.DeviceArray(nbytes // 4, np.float32), api.DeviceArray(nbytes // 4, np.float32)
+    api.lib().krk_memset(api._ptr(a), 1, nbytes)
+    dt = timed(None, lambda: api.lib().krk_stream_copy(api._ptr(b), api._ptr(a), nbytes), 20)
+    print("# plain copy of 1 GiB: %.1f us, %.0f GB/s read + write" % (dt * 1e6, 2 * nbytes / dt / 1e9), flush=True)
+
+
+SECTIONS = {"copy": copy, "tables": tables, "raw": raw, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct}
+
+
+def main(argv):
+    rc = api.lib().krk_runtime_init(0)
+    if rc != 0:
+        raise RuntimeError("no usable GPU: " + api.lib().krk_last_error_string().decode())
+    for name in argv or list(SECTIONS):
+        SECTIONS[name]()
+
+
+if __name__ == "__main__":
+    main(sys.argv[1:])
