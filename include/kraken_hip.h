@@ -288,6 +288,17 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
  * in member order is returned. */
 int32_t krk_group_push(krk_group* g, const krk_optim* o, const uint64_t* ids, const int64_t* offsets,
                        const float* grads, int64_t grad_dim, float lr, uint32_t flags);
+/* Emitter::CombinePushSparseTable's dedup + duplicate-gradient sum over (table, id) pairs
+ * (worker/emitter.cc:552-606) fused with krk_group_push: ids may repeat within a table, the
+ * gradients of equal ids are summed in position order and the optimizer runs once per distinct
+ * row. One sort and one segmented reduction serve all members. The members' row capacities and
+ * the member count must fit a 32-bit sort key together (KRK_E_CAPACITY otherwise: 32 tables of
+ * up to 2^26 rows each, fewer tables for larger ones), at most 2^28 ids per call. Errors as
+ * krk_group_push. */
+int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids, const int64_t* offsets,
+                           const float* grads, int64_t grad_dim, float lr, uint32_t flags);
+/* krk_sparse_set_stream for a group and all its members. */
+int32_t krk_group_set_stream(krk_group* g, void* stream);
 
 /* Emitter::PullSparseTableImpl's dedup (worker/emitter.cc:131-149): unique ids
  * in first-occurrence order, inv[p] = index of ids[p] in uids. uids and inv

@@ -140,6 +140,9 @@ EXPORTS = {
     "krk_group_pull": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32]),
     "krk_group_push": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_void_p, C.c_void_p,
                                    C.c_int64, C.c_float, C.c_uint32]),
+    "krk_group_push_raw": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.c_int64, C.c_float, C.c_uint32]),
+    "krk_group_set_stream": (C.c_int32, [C.c_void_p, C.c_void_p]),
     "krk_event_elapsed_ms": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "krk_dct2_forward": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_uint32]),
     "krk_dct2_inverse": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_uint32]),
@@ -502,14 +505,19 @@ class TableGroup:
                                   _flags(ids, out, extra=ASYNC if async_ else 0))
         return rc, out
 
-    def CombinePush(self, optim, ids, offsets, grads, lr, async_=False):
+    def CombinePush(self, optim, ids, offsets, grads, lr, async_=False, raw=False):
         offsets = np.ascontiguousarray(offsets, dtype=np.int64)
         if not isinstance(ids, DeviceArray):
             ids = np.ascontiguousarray(ids, dtype=np.uint64)
             grads = np.ascontiguousarray(grads, dtype=np.float32)
         gd = grads.shape[-1]
-        return lib().krk_group_push(self.h, C.byref(optim.raw), _ptr(ids), _ptr(offsets), _ptr(grads),
-                                    gd, lr, _flags(ids, grads, extra=ASYNC if async_ else 0))
+        fn = lib().krk_group_push_raw if raw else lib().krk_group_push
+        return fn(self.h, C.byref(optim.raw), _ptr(ids), _ptr(offsets), _ptr(grads),
+                  gd, lr, _flags(ids, grads, extra=ASYNC if async_ else 0))
+
+    def CombinePushRaw(self, optim, ids, offsets, grads, lr, async_=False):
+        """Emitter::CombinePushSparseTable's dedup + sum fused with CombinePush: ids may repeat."""
+        return self.CombinePush(optim, ids, offsets, grads, lr, async_=async_, raw=True)
 
 
 class DenseTable:

@@ -185,6 +185,33 @@ __global__ __launch_bounds__(kBlock) void rows_of_ids_kernel(TableView tv, const
   pos[p] = payload_is_bag ? bag : (uint32_t)p;
 }
 
+// The same for a combined request: position p belongs to the member whose [row_start, row_start
+// of the next) holds it; its key is (member << row_bits) | row. A missing id raises the error
+// on its own member.
+__global__ __launch_bounds__(kBlock) void group_rows_of_ids_kernel(const TableDesc* __restrict__ descs,
+                                                                   GroupCall call,
+                                                                   const uint64_t* __restrict__ ids, int64_t n,
+                                                                   int row_bits, uint32_t miss_key,
+                                                                   uint32_t* __restrict__ keys,
+                                                                   uint32_t* __restrict__ pos) {
+  const int64_t p = (int64_t)blockIdx.x * (kBlock / kBucket) + threadIdx.x / kBucket;
+  const int gl = threadIdx.x & (kBucket - 1);
+  const bool active = p < n;
+  int m = 0;
+  while (active && m + 1 < call.n_tables && p >= call.row_start[m + 1]) ++m;
+  const TableView tv = descs[m].tv;
+  uint32_t r = probe_find(tv, active ? ids[p] : 0, active, gl, kBucket);
+  if (!active || gl != 0) return;
+  if (r == kEmptyRow) {
+    atomicOr(&tv.counters[1], kErrMissingId);
+    r = miss_key;
+  } else {
+    r |= (uint32_t)m << row_bits;
+  }
+  keys[p] = r;
+  pos[p] = (uint32_t)p;
+}
+
 // ---- pooled pushes: from bag offsets to per-position bag numbers ----------------
 __global__ __launch_bounds__(kBlock) void fill_u32_kernel(uint32_t* __restrict__ dst, int64_t n, uint32_t v) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -286,6 +313,9 @@ __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, con
 // requested four entries ahead of where the sums are. Carry levels use short tiles: the lists
 // are short, so short tiles keep many lane groups busy (tiles of 32 with eight entries in
 // flight save one or two dependent launches but measured slower, 442 vs 432 us at 1M ids).
+// Running the last, short levels in one launch of a single workgroup (barrier between levels)
+// was measured too: on one CU every level pays its dependent memory round trips one after the
+// other, 36 us against four launches of about 8 us for the tail of an 8192-id request.
 constexpr int kPrefetch = 4;
 constexpr int kPrefetchCarry = 4;
 constexpr int kCarryTile = 16;
@@ -297,40 +327,25 @@ struct PooledSrc {
   const float* weight;
 };
 
-template <int OPT, int VEC, bool LEVEL0>
-__global__ __launch_bounds__(kBlock) void segreduce_kernel(
-    TableView tv, const uint32_t* __restrict__ keys, const uint32_t* __restrict__ pos,
-    const float* __restrict__ vals, int64_t cnt, int tile, uint32_t empty_from,
-    uint32_t* __restrict__ keys_out, float* __restrict__ vals_out, int dim, int elems, int group,
-    ApplyArgs args, PooledSrc ps) {
-  extern __shared__ uint32_t lds[];
-  const int per_block = kBlock / group;
-  const int span = per_block * tile;                       // entries staged by this workgroup
-  const int64_t first = (int64_t)blockIdx.x * span;        // global index of lds_keys[1]
-  uint32_t* lds_keys = lds;                                // [span + 2], shifted by one
-  uint32_t* lds_pos = lds + span + 2;                      // [span]
-  float* lds_w = reinterpret_cast<float*>(lds + 2 * span + 2);   // [span], weighted bags only
-  for (int i = threadIdx.x; i < span + 2; i += kBlock) {
-    const int64_t j = first + i - 1;
-    lds_keys[i] = (j >= 0 && j < cnt) ? keys[j] : kNoRow;
-  }
-  const bool weighted = LEVEL0 && ps.weight != nullptr;
-  if (LEVEL0) {
-    for (int i = threadIdx.x; i < span; i += kBlock) {
-      const int64_t j = first + i;
-      uint32_t p = j < cnt ? pos[j] : 0u;
-      if (weighted) {
-        // the payload is the position: it names the weight and, through bag_of, the row
-        lds_w[i] = j < cnt ? ps.weight[p] : 0.0f;
-        const uint32_t b = j < cnt ? ps.bag_of[p] : 0u;
-        p = b == kNoBag ? 0u : b;
-      }
-      lds_pos[i] = p;
-    }
-  }
-  __syncthreads();
+// Combined pushes (GROUPED): a key is (member number << row_bits) | row, and a closed run takes
+// its member's record layout from descs. st0..st2 are the state types of the optimizer's three
+// slots (-1 = unused); the column each lives in differs from member to member.
+struct GroupSrc {
+  const TableDesc* descs;
+  int row_bits;
+  int st0, st1, st2;
+  int use_meta;
+};
 
-  const int64_t t = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+// One tile: entries [t * tile, (t + 1) * tile) of the sequence, walked by the `group` lanes that
+// call this together. lds_keys[i] holds the key of entry first + i - 1 (so both neighbours of
+// the tile are there), lds_pos / lds_w the payloads and weights of entry first + i.
+template <int OPT, int VEC, bool LEVEL0, bool GROUPED>
+__device__ __forceinline__ void reduce_tile(
+    int64_t t, int64_t first, const uint32_t* lds_keys, const uint32_t* lds_pos, const float* lds_w,
+    bool weighted, const TableView& tv, const float* __restrict__ vals, int64_t cnt, int tile,
+    uint32_t empty_from, uint32_t* __restrict__ keys_out, float* __restrict__ vals_out, int dim, int elems,
+    int group, const ApplyArgs& args, const GroupSrc& gs) {
   const int gl = threadIdx.x & (group - 1);
   const int64_t a = t * tile;
   if (a >= cnt) return;
@@ -358,7 +373,21 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
       const bool open_left = run_start == la && left_key == run_key;
       const bool open_right = end == lb && right_key == run_key;
       if (!open_left && !open_right) {
-        apply_row<OPT, VEC>(tv, run_key, acc, e, lane_on, leader, last_chunk, args);
+        if constexpr (GROUPED) {
+          const TableDesc& d = gs.descs[run_key >> gs.row_bits];
+          TableView member = tv;
+          member.recs = d.tv.recs;
+          member.stride = d.tv.stride;
+          ApplyArgs aa = args;
+          aa.c0 = gs.st0 >= 0 ? d.col_off[gs.st0] : -1;
+          aa.c1 = gs.st1 >= 0 ? d.col_off[gs.st1] : -1;
+          aa.c2 = gs.st2 >= 0 ? d.col_off[gs.st2] : -1;
+          aa.meta_off = gs.use_meta ? d.meta_off : -1;
+          apply_row<OPT, VEC>(member, run_key & ((1u << gs.row_bits) - 1u), acc, e, lane_on, leader,
+                              last_chunk, aa);
+        } else {
+          apply_row<OPT, VEC>(tv, run_key, acc, e, lane_on, leader, last_chunk, args);
+        }
         return;
       }
       const int64_t slot = open_left ? 2 * t : 2 * t + 1;
@@ -422,6 +451,43 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
   }
 }
 
+template <int OPT, int VEC, bool LEVEL0, bool GROUPED>
+__global__ __launch_bounds__(kBlock) void segreduce_kernel(
+    TableView tv, const uint32_t* __restrict__ keys, const uint32_t* __restrict__ pos,
+    const float* __restrict__ vals, int64_t cnt, int tile, uint32_t empty_from,
+    uint32_t* __restrict__ keys_out, float* __restrict__ vals_out, int dim, int elems, int group,
+    ApplyArgs args, PooledSrc ps, GroupSrc gs) {
+  extern __shared__ uint32_t lds[];
+  const int per_block = kBlock / group;
+  const int span = per_block * tile;                       // entries staged by this workgroup
+  const int64_t first = (int64_t)blockIdx.x * span;        // global index of lds_keys[1]
+  uint32_t* lds_keys = lds;                                // [span + 2], shifted by one
+  uint32_t* lds_pos = lds + span + 2;                      // [span]
+  float* lds_w = reinterpret_cast<float*>(lds + 2 * span + 2);   // [span], weighted bags only
+  for (int i = threadIdx.x; i < span + 2; i += kBlock) {
+    const int64_t j = first + i - 1;
+    lds_keys[i] = (j >= 0 && j < cnt) ? keys[j] : kNoRow;
+  }
+  const bool weighted = LEVEL0 && ps.weight != nullptr;
+  if (LEVEL0) {
+    for (int i = threadIdx.x; i < span; i += kBlock) {
+      const int64_t j = first + i;
+      uint32_t p = j < cnt ? pos[j] : 0u;
+      if (weighted) {
+        // the payload is the position: it names the weight and, through bag_of, the row
+        lds_w[i] = j < cnt ? ps.weight[p] : 0.0f;
+        const uint32_t b = j < cnt ? ps.bag_of[p] : 0u;
+        p = b == kNoBag ? 0u : b;
+      }
+      lds_pos[i] = p;
+    }
+  }
+  __syncthreads();
+  const int64_t t = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  reduce_tile<OPT, VEC, LEVEL0, GROUPED>(t, first, lds_keys, lds_pos, lds_w, weighted, tv, vals, cnt, tile,
+                                         empty_from, keys_out, vals_out, dim, elems, group, args, gs);
+}
+
 // Row width and lane mapping of a reduction: a table's, or those of a stand-alone call.
 struct ReduceShape {
   int64_t dim;
@@ -432,19 +498,36 @@ template <int OPT, int VEC>
 static void launch_segreduce(bool level0, const TableView& tv, const uint32_t* keys, const uint32_t* pos,
                              const float* vals, int64_t cnt, int tile, uint32_t empty_from,
                              uint32_t* keys_out, float* vals_out, const ReduceShape* t,
-                             const ApplyArgs& args, const PooledSrc& ps, hipStream_t stream) {
+                             const ApplyArgs& args, const PooledSrc& ps, const GroupSrc* gs,
+                             hipStream_t stream) {
   const int per_block = kBlock / t->group;
   const int64_t tiles = (cnt + tile - 1) / tile;
   const dim3 grid(grid_for(tiles, per_block)), block(kBlock);
   const size_t lds_bytes = (size_t)(3 * per_block * tile + 2) * sizeof(uint32_t);
+  const PooledSrc none{nullptr, nullptr};
+  if constexpr (OPT != kOptStore) {
+    if (gs) {
+      if (level0) {
+        hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, true, true>), grid, block, lds_bytes, stream, tv, keys,
+                           pos, vals, cnt, tile, empty_from, keys_out, vals_out, (int)t->dim, t->elems,
+                           t->group, args, ps, *gs);
+      } else {
+        hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, false, true>), grid, block, lds_bytes, stream, tv, keys,
+                           pos, vals, cnt, tile, empty_from, keys_out, vals_out, (int)t->dim, t->elems,
+                           t->group, args, none, *gs);
+      }
+      return;
+    }
+  }
+  const GroupSrc plain{nullptr, 0, -1, -1, -1, 0};
   if (level0) {
-    hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, true>), grid, block, lds_bytes, stream, tv, keys, pos,
+    hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, true, false>), grid, block, lds_bytes, stream, tv, keys, pos,
                        vals, cnt, tile, empty_from, keys_out, vals_out, (int)t->dim, t->elems, t->group,
-                       args, ps);
+                       args, ps, plain);
   } else {
-    hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, false>), grid, block, lds_bytes, stream, tv, keys, pos,
+    hipLaunchKernelGGL((segreduce_kernel<OPT, VEC, false, false>), grid, block, lds_bytes, stream, tv, keys, pos,
                        vals, cnt, tile, empty_from, keys_out, vals_out, (int)t->dim, t->elems, t->group,
-                       args, PooledSrc{nullptr, nullptr});
+                       args, none, plain);
   }
 }
 
@@ -453,27 +536,27 @@ static void dispatch_segreduce(int opt, bool level0, const TableView& tv, const 
                                const uint32_t* pos, const float* vals, int64_t cnt, int tile,
                                uint32_t empty_from, uint32_t* keys_out, float* vals_out,
                                const ReduceShape* t, const ApplyArgs& args, const PooledSrc& ps,
-                               hipStream_t stream) {
+                               const GroupSrc* gs, hipStream_t stream) {
   switch (opt) {
     case kOptStore:
       launch_segreduce<kOptStore, VEC>(level0, tv, keys, pos, vals, cnt, tile, empty_from, keys_out,
-                                       vals_out, t, args, ps, stream);
+                                       vals_out, t, args, ps, gs, stream);
       break;
     case KRK_SGD:
       launch_segreduce<KRK_SGD, VEC>(level0, tv, keys, pos, vals, cnt, tile, empty_from, keys_out,
-                                     vals_out, t, args, ps, stream);
+                                     vals_out, t, args, ps, gs, stream);
       break;
     case KRK_ADAGRAD:
       launch_segreduce<KRK_ADAGRAD, VEC>(level0, tv, keys, pos, vals, cnt, tile, empty_from, keys_out,
-                                         vals_out, t, args, ps, stream);
+                                         vals_out, t, args, ps, gs, stream);
       break;
     case KRK_ADAM:
       launch_segreduce<KRK_ADAM, VEC>(level0, tv, keys, pos, vals, cnt, tile, empty_from, keys_out,
-                                      vals_out, t, args, ps, stream);
+                                      vals_out, t, args, ps, gs, stream);
       break;
     default:
       launch_segreduce<KRK_RMSPROP, VEC>(level0, tv, keys, pos, vals, cnt, tile, empty_from, keys_out,
-                                         vals_out, t, args, ps, stream);
+                                         vals_out, t, args, ps, gs, stream);
       break;
   }
 }
@@ -516,7 +599,8 @@ static hipError_t sort_pairs(void* tmp, size_t& tmp_bytes, uint32_t* keys, uint3
 template <typename Fill>
 static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, DeviceBuffer* scratch,
                                const TableView& tv, int opt, int64_t n, uint32_t miss_key, int bits,
-                               const float* d_vals, const ApplyArgs& args, const PooledSrc& ps, Fill fill) {
+                               const float* d_vals, const ApplyArgs& args, const PooledSrc& ps,
+                               const GroupSrc* gs, Fill fill) {
   const int tile0 = pick_tile(n);
   const int64_t tiles0 = (n + tile0 - 1) / tile0;
   const size_t n4 = (size_t)n * sizeof(uint32_t);
@@ -556,10 +640,10 @@ static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, Device
     }
     if (sh.vec == 4) {
       dispatch_segreduce<4>(opt, level0, tv, in_keys, spos, in_vals, cnt, tile, miss_key, okeys, ovals, &sh,
-                            args, ps, stream);
+                            args, ps, gs, stream);
     } else {
       dispatch_segreduce<1>(opt, level0, tv, in_keys, spos, in_vals, cnt, tile, miss_key, okeys, ovals, &sh,
-                            args, ps, stream);
+                            args, ps, gs, stream);
     }
     KRK_HIP(hipGetLastError());
     if (tiles <= 1) break;
@@ -597,7 +681,7 @@ static int32_t push_sorted(krk_sparse* t, const krk_optim* o, const uint64_t* d_
   args.meta_off = ((optim_state_mask(*o) >> KRK_ST_STEPS) & 1u) ? t->meta_off : -1;
   const TableView tv = t->view();
   const ReduceShape sh{t->dim, t->vec, t->elems, t->group};
-  return sort_and_reduce(sh, t->stream, t->scratch, tv, o->type, n, miss_key, bits, d_g, args, ps,
+  return sort_and_reduce(sh, t->stream, t->scratch, tv, o->type, n, miss_key, bits, d_g, args, ps, nullptr,
                          [&](uint32_t* keys, uint32_t* pos) {
                            hipLaunchKernelGGL(rows_of_ids_kernel, dim3(grid_for(n, kBlock / kBucket)),
                                               dim3(kBlock), 0, t->stream, tv, d_ids, n, miss_key, bag_of,
@@ -813,7 +897,7 @@ int32_t krk_dedup_sum(const uint64_t* ids, int64_t n, const float* grads, int64_
   const DSlot* slots = w.slots;
   const uint32_t* slot_of = w.slot_of;
   KRK_TRY(sort_and_reduce(sh, s, g_dedup_reduce, tv, kOptStore, n, miss_key, bits, d_g, args,
-                          PooledSrc{nullptr, nullptr}, [&](uint32_t* keys, uint32_t* pos) {
+                          PooledSrc{nullptr, nullptr}, nullptr, [&](uint32_t* keys, uint32_t* pos) {
                             hipLaunchKernelGGL(dedup_pairs_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s,
                                                slots, slot_of, n, keys, pos);
                           }));
@@ -911,6 +995,69 @@ int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* i
 
   KRK_TRY(push_sorted(t, o, d_ids, n, d_g, lr, nullptr, false, PooledSrc{nullptr, nullptr}));
   return sparse_finish(t, flags);
+}
+
+int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids, const int64_t* offsets,
+                           const float* grads, int64_t grad_dim, float lr, uint32_t flags) {
+  if (!g || !offsets) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  KRK_TRY(check_flags(flags));
+  if (!o || o->type < KRK_ADAGRAD || o->type > KRK_SGD) {
+    set_error("optimizer type is not supported");
+    return KRK_UNSUPPORTED_OPTIM;
+  }
+  GroupLock lk(g);
+  GroupCall call;
+  int64_t total = 0;
+  KRK_TRY(group_plan(g, offsets, &call, &total));
+  if (total == 0) return group_finish(g, flags);
+  if (!ids || !grads) return KRK_E_ARGUMENT;
+  if (total > ((int64_t)1 << 28)) {
+    set_error("krk_group_push_raw handles at most 2^28 ids per call; split the request");
+    return KRK_E_CAPACITY;
+  }
+  if (grad_dim != g->dim) {
+    set_error("gradient width %lld does not match table dimension %lld", (long long)grad_dim,
+              (long long)g->dim);
+    return KRK_GRADIENT_UNCOMPATIBLE;
+  }
+  const uint32_t mask = optim_state_mask(*o);
+  for (krk_sparse* t : g->tables) KRK_TRY(sparse_ensure_columns(t, mask));
+  KRK_TRY(group_refresh(g));
+  // sort key: member number above the row number; one value above every key marks a missing id
+  int row_bits = 1;
+  for (krk_sparse* t : g->tables)
+    while (((int64_t)1 << row_bits) < t->row_cap) ++row_bits;
+  const int n_tables = (int)g->tables.size();
+  int member_bits = 1;
+  while ((1 << member_bits) <= n_tables) ++member_bits;
+  if (row_bits + member_bits > 32) {
+    set_error("combined push with repeats: %d tables of up to 2^%d rows do not fit a 32-bit sort key",
+              n_tables, row_bits);
+    return KRK_E_CAPACITY;
+  }
+  const uint32_t miss_key = (uint32_t)n_tables << row_bits;
+  const uint64_t* d_ids;
+  const float* d_g;
+  KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
+  KRK_TRY(g->input(grads, (size_t)total * g->dim, flags, 1, &d_g));
+  ApplyArgs args;
+  args.lr = lr;
+  args.k = make_optim_k(*o);
+  args.c0 = args.c1 = args.c2 = args.meta_off = -1;     // taken per member from its layout
+  int32_t st[3];
+  optim_state_slots(*o, st);
+  const GroupSrc gs{g->d_descs, row_bits, st[0], st[1], st[2], (int)((mask >> KRK_ST_STEPS) & 1u)};
+  TableView none{};
+  const ReduceShape sh{g->dim, g->vec, g->elems, g->group};
+  KRK_TRY(sort_and_reduce(sh, g->stream, g->scratch, none, o->type, total, miss_key, row_bits + member_bits,
+                          d_g, args, PooledSrc{nullptr, nullptr}, &gs, [&](uint32_t* keys, uint32_t* pos) {
+                            hipLaunchKernelGGL(group_rows_of_ids_kernel,
+                                               dim3(grid_for(total, kBlock / kBucket)), dim3(kBlock), 0,
+                                               g->stream, g->d_descs, call, d_ids, total, row_bits, miss_key,
+                                               keys, pos);
+                          }));
+  return group_finish(g, flags);
 }
 
 int32_t krk_sparse_push_pooled(krk_sparse* t, const krk_optim* o, const uint64_t* ids, int64_t n,

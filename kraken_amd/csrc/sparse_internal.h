@@ -309,6 +309,61 @@ struct krk_sparse : krk::ObjBase {
 };
 
 namespace krk {
+constexpr int kMaxGroupTables = 32;
+
+// What a kernel of a combined request needs to know about one member table.
+struct TableDesc {
+  TableView tv;
+  InitK init;
+  int32_t col_off[KRK_ST_COUNT];
+  int32_t meta_off;
+};
+
+// One combined request: the launch number of each member, and where each member's ids start,
+// in workgroups of the one-launch kernels (block_start) and in positions (row_start).
+struct GroupCall {
+  int32_t n_tables;
+  uint32_t epoch[kMaxGroupTables];
+  uint32_t block_start[kMaxGroupTables + 1];
+  int64_t row_start[kMaxGroupTables + 1];
+};
+}  // namespace krk
+
+// Tables of one combined request (CombinePull/PushSparseTable): they share one stream, and a
+// device-resident array of their layouts that is refreshed only when a table has moved.
+struct krk_group : krk::ObjBase {
+  std::vector<krk_sparse*> tables;
+  std::vector<uint64_t> versions;
+  krk::TableDesc* d_descs = nullptr;
+  krk::TableDesc* h_descs = nullptr;   // pinned
+  int64_t dim = 0;
+  int vec = 1, elems = 0, group = 1;
+  hipStream_t own_stream = nullptr;    // the stream created with the group
+  krk::DeviceBuffer scratch[5];        // push_raw work space
+};
+
+namespace krk {
+// Takes the group's lock and then every member's, in member order.
+struct GroupLock {
+  krk_group* g;
+  explicit GroupLock(krk_group* gg) : g(gg) {
+    g->mu.lock();
+    for (krk_sparse* t : g->tables) t->mu.lock();
+  }
+  ~GroupLock() {
+    for (auto it = g->tables.rbegin(); it != g->tables.rend(); ++it) (*it)->mu.unlock();
+    g->mu.unlock();
+  }
+  GroupLock(const GroupLock&) = delete;
+  GroupLock& operator=(const GroupLock&) = delete;
+};
+// Checks the offsets of a combined request and lays its members out over the grid.
+int32_t group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, int64_t* total);
+// Uploads the layouts of members that moved since the last call.
+int32_t group_refresh(krk_group* g);
+// Blocking calls: waits for the group's stream and reports the first member's error.
+int32_t group_finish(krk_group* g, uint32_t flags);
+
 // Host-side pieces shared between the table's translation units.
 int32_t sparse_ensure_room(krk_sparse* t, int64_t extra_rows);
 int32_t sparse_ensure_columns(krk_sparse* t, uint32_t state_mask);

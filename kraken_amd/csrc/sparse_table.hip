@@ -20,7 +20,6 @@
 namespace krk {
 
 constexpr int kBlock = 256;
-constexpr int kMaxGroupTables = 32;
 constexpr int64_t kTwoLaunchPull = 1 << 18;   // ids from which a pull runs as two launches
 constexpr int kMissingGrid = 2048;            // workgroups of the launch that inserts missing ids
 
@@ -365,20 +364,6 @@ __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64
 // ---- one launch over several tables of equal row width ------------------------
 // Table t owns workgroups [block_start[t], block_start[t+1]) and the positions
 // [row_start[t], row_start[t+1]) of the concatenated ids / rows.
-struct TableDesc {
-  TableView tv;
-  InitK init;
-  int32_t col_off[KRK_ST_COUNT];
-  int32_t meta_off;
-};
-
-struct GroupCall {
-  int32_t n_tables;
-  uint32_t epoch[kMaxGroupTables];
-  uint32_t block_start[kMaxGroupTables + 1];
-  int64_t row_start[kMaxGroupTables + 1];
-};
-
 __device__ __forceinline__ int find_table(const GroupCall& c) {
   int t = 0;
   while (t + 1 < c.n_tables && blockIdx.x >= c.block_start[t + 1]) ++t;
@@ -1007,17 +992,6 @@ static void launch_push(krk_sparse* t, const krk_optim& o, const uint64_t* ids, 
 
 using namespace krk;
 
-// Tables of one combined request (CombinePull/PushSparseTable): they share one stream, and a
-// device-resident array of their layouts that is refreshed only when a table has moved.
-struct krk_group : krk::ObjBase {
-  std::vector<krk_sparse*> tables;
-  std::vector<uint64_t> versions;
-  krk::TableDesc* d_descs = nullptr;
-  krk::TableDesc* h_descs = nullptr;   // pinned
-  int64_t dim = 0;
-  int vec = 1, elems = 0, group = 1;
-};
-
 static int32_t check_table(krk_sparse* t) {
   if (!t) {
     set_error("null sparse table handle");
@@ -1594,6 +1568,7 @@ int32_t krk_group_create(krk_sparse** tables, int32_t n, krk_group** out) {
     delete g;
     return rc;
   }
+  g->own_stream = g->stream;
   g->dim = tables[0]->dim;
   g->vec = tables[0]->vec;
   g->elems = tables[0]->elems;
@@ -1621,13 +1596,30 @@ int32_t krk_group_destroy(krk_group* g) {
   }
   if (g->d_descs) (void)hipFree(g->d_descs);
   if (g->h_descs) (void)hipHostFree(g->h_descs);
+  for (auto& b : g->scratch) b.release();
+  g->stream = g->own_stream;
   g->close_stream();
   delete g;
   return KRK_SUCCESS;
 }
 
+int32_t krk_group_set_stream(krk_group* g, void* stream) {
+  if (!g) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  GroupLock lk(g);
+  hipStream_t next = stream ? reinterpret_cast<hipStream_t>(stream) : g->own_stream;
+  if (next == g->stream) return KRK_SUCCESS;
+  // what is enqueued on the old stream must be complete before work on the new one may follow
+  KRK_TRY(group_finish(g, 0));
+  g->stream = next;
+  for (krk_sparse* t : g->tables) t->stream = next;
+  return KRK_SUCCESS;
+}
+
+}  // extern "C"
+
 // Uploads the layouts of tables that moved since the last call.
-static int32_t group_refresh(krk_group* g) {
+int32_t krk::group_refresh(krk_group* g) {
   bool dirty = false;
   for (size_t i = 0; i < g->tables.size(); ++i) {
     krk_sparse* t = g->tables[i];
@@ -1649,7 +1641,7 @@ static int32_t group_refresh(krk_group* g) {
   return KRK_SUCCESS;
 }
 
-static int32_t group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, int64_t* total) {
+int32_t krk::group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, int64_t* total) {
   const int n = (int)g->tables.size();
   const int per_block = kBlock / g->group;
   call->n_tables = n;
@@ -1675,19 +1667,7 @@ static int32_t group_plan(krk_group* g, const int64_t* offsets, GroupCall* call,
   return KRK_SUCCESS;
 }
 
-struct GroupLock {
-  krk_group* g;
-  explicit GroupLock(krk_group* gg) : g(gg) {
-    g->mu.lock();
-    for (krk_sparse* t : g->tables) t->mu.lock();
-  }
-  ~GroupLock() {
-    for (auto it = g->tables.rbegin(); it != g->tables.rend(); ++it) (*it)->mu.unlock();
-    g->mu.unlock();
-  }
-};
-
-static int32_t group_finish(krk_group* g, uint32_t flags) {
+int32_t krk::group_finish(krk_group* g, uint32_t flags) {
   if (flags & KRK_ASYNC) return KRK_SUCCESS;
   // one wait for all members: they share the group's stream
   for (krk_sparse* t : g->tables)
@@ -1700,6 +1680,8 @@ static int32_t group_finish(krk_group* g, uint32_t flags) {
   }
   return first;
 }
+
+extern "C" {
 
 int32_t krk_group_sync(krk_group* g) {
   if (!g) return KRK_E_ARGUMENT;

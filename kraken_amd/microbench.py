@@ -1,6 +1,6 @@
 """Per-kernel timings of the table engine at the sizes of the benchmark configurations.
 
-    python -m kraken_amd.microbench [tables] [raw] [pooled] [codec] [dense] [dct2] [copy]
+    python -m kraken_amd.microbench [copy] [tables] [raw] [combined] [pooled] [codec] [dense] [dct2] [copy]
 
 Every figure is the average of back-to-back launches between two HIP events recorded on the
 stream the kernels run on, with inputs resident in HBM; bandwidths are algorithmic bytes
@@ -137,6 +137,42 @@ def raw():
         t.close()
 
 
+def combined():
+    print("# Wide&Deep step with the worker side on the device: 26 tables of 1e6 rows, 8192 Zipf 1.05 ids")
+    print("# per table with repeats, dim 16, Adagrad")
+    n_tables, space, batch, dim = 26, 10**6, 8192, 16
+    init = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01"})
+    rng = np.random.default_rng(0)
+    tables = [api.SparseTable(dim, init, capacity_hint=space) for _ in range(n_tables)]
+    for t in tables:
+        prefill(t, space, dim)
+    grp = api.TableGroup(tables)
+    per = [splitmix64(zipf_ranks(rng, 1.05, space, batch)) for _ in range(n_tables)]
+    off = grp._offsets([batch] * n_tables)
+    n = n_tables * batch
+    u = sum(np.unique(p).size for p in per)
+    d_ids = api.DeviceArray.from_host(np.concatenate(per))
+    d_one = [api.DeviceArray.from_host(p) for p in per]
+    d_g = api.DeviceArray.from_host((rng.standard_normal((n, dim)) * 1e-2).astype(np.float32))
+    d_g1 = api.DeviceArray.from_host((rng.standard_normal((batch, dim)) * 1e-2).astype(np.float32))
+    d_out = api.DeviceArray((n, dim), np.float32)
+    o = api.Optim.create(api.OptimType.kAdagrad)
+    print("ids %d, distinct (table, id) pairs %d" % (n, u), flush=True)
+
+    def per_table():
+        for t, d in zip(tables, d_one):
+            t.PushRaw(o, d, d_g1, 0.01, async_=True)
+
+    for name, fn in (
+            ("combined pull of all ids", lambda: grp.CombinePull(d_ids, off, out=d_out, async_=True)),
+            ("combined push with repeats", lambda: grp.CombinePushRaw(o, d_ids, off, d_g, 0.01, async_=True)),
+            ("push_raw table by table (26 calls)", per_table)):
+        print("%-36s %8.1f us" % (name, timed(grp, fn, 10) * 1e6), flush=True)
+    grp.close()
+    for t in tables:
+        t.close()
+
+
 def pooled():
     print("# multi-hot field of the DeepFM shape: 65536 samples x 13 fields, 1..20 ids per bag, dim 32,")
     print("# table of 1e7 rows, Zipf 1.1")
@@ -225,7 +261,7 @@ def copy():
     print("# plain copy of 1 GiB: %.1f us, %.0f GB/s read + write" % (dt * 1e6, 2 * nbytes / dt / 1e9), flush=True)
 
 
-SECTIONS = {"copy": copy, "tables": tables, "raw": raw, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct}
+SECTIONS = {"copy": copy, "tables": tables, "raw": raw, "combined": combined, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct}
 
 
 def main(argv):

@@ -143,3 +143,103 @@ class JaggedEmbedding(torch.nn.Module):
     def forward(self, values, offsets, weights=None):
         return JaggedEmbeddingFunction.apply(self.sparse_table, values, offsets, weights, self._mode,
                                              self._patch_value)
+
+
+class GpuCombineSparseTable(torch.nn.Parameter):
+    """pytorch/combine_sparse_table.py: the tables of one combined request. Tables of equal
+    dimension form one group of the engine (one launch serves a group); the reference allows
+    mixed dimensions, which gives one group per distinct dimension here."""
+
+    def __new__(cls, dimensions, initializers=None, optim=None, lr=0.01, capacity_hint=0):
+        self = super().__new__(cls, torch.empty(0), requires_grad=True)
+        if initializers is not None and len(initializers) != len(dimensions):
+            raise ValueError("dimensions and initializers must have the same length")
+        self._dimensions = [int(d) for d in dimensions]
+        self._tables = [
+            api.SparseTable(d, (initializers[i] if initializers else None) or api.Initializer.create(
+                api.InitializerType.kNormal, {}), capacity_hint=capacity_hint)
+            for i, d in enumerate(self._dimensions)]
+        self._members = {}                        # dimension -> positions of its tables in the request
+        for i, d in enumerate(self._dimensions):
+            self._members.setdefault(d, []).append(i)
+        self._groups = {d: api.TableGroup([self._tables[i] for i in idx]) for d, idx in self._members.items()}
+        self._optim = optim or api.Optim.create(api.OptimType.kSGD)
+        self.lr = float(lr)
+        return self
+
+    def dimensions(self):
+        return self._dimensions
+
+    def tables(self):
+        return self._tables
+
+    def _on_current_stream(self, dim):
+        g = self._groups[dim]
+        api._check(api.lib().krk_group_set_stream(g.h, _stream_ptr()), "krk_group_set_stream")
+        return g.h
+
+
+def _group_offsets(counts):
+    off = (C.c_int64 * (len(counts) + 1))()
+    for i, c in enumerate(counts):
+        off[i + 1] = off[i] + c
+    return off
+
+
+class CombineEmbeddingFunction(torch.autograd.Function):
+    """pytorch/combine_embedding.py:10-31 over Emitter::CombinePullSparseTable /
+    CombinePushSparseTable (worker/emitter.cc:185-283, 552-632): ids may repeat, within a table
+    and across tables."""
+
+    @staticmethod
+    def forward(ctx, table, *indices):
+        if len(indices) != len(table.dimensions()):
+            raise ValueError("one index tensor per table")
+        outs = [None] * len(indices)
+        saved = []
+        for dim, members in table._members.items():
+            parts = [_ids_ptr(indices[i])[0].reshape(-1) for i in members]
+            ids = torch.cat(parts) if len(parts) > 1 else parts[0]
+            off = _group_offsets([p.numel() for p in parts])
+            out = torch.empty((ids.numel(), dim), dtype=torch.float32, device=ids.device)
+            h = table._on_current_stream(dim)
+            api._check(api.lib().krk_group_pull(h, C.c_void_p(ids.data_ptr()), off, C.c_void_p(out.data_ptr()),
+                                                api.DEVICE_PTRS | api.ASYNC), "krk_group_pull")
+            for k, i in enumerate(members):
+                outs[i] = out[off[k]:off[k + 1]].view(tuple(indices[i].shape) + (dim,))
+            saved.append(ids)
+        ctx.table = table
+        ctx.counts = [x.numel() for x in indices]
+        ctx.save_for_backward(*saved)
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        t = ctx.table
+        for ids, (dim, members) in zip(ctx.saved_tensors, t._members.items()):
+            counts = [ctx.counts[i] for i in members]
+            # an output the loss never used has no gradient: its rows get zeros
+            parts = [grads[i].reshape(-1, dim).to(torch.float32) if grads[i] is not None
+                     else torch.zeros((c, dim), dtype=torch.float32, device=ids.device)
+                     for i, c in zip(members, counts)]
+            g = (torch.cat(parts) if len(parts) > 1 else parts[0]).contiguous()
+            off = _group_offsets(counts)
+            h = t._on_current_stream(dim)
+            api._check(api.lib().krk_group_push_raw(h, C.byref(t._optim.raw), C.c_void_p(ids.data_ptr()), off,
+                                                    C.c_void_p(g.data_ptr()), dim, t.lr,
+                                                    api.DEVICE_PTRS | api.ASYNC), "krk_group_push_raw")
+        return (None,) * (1 + len(grads))
+
+
+class CombineEmbedding(torch.nn.Module):
+    """pytorch/combine_embedding.py:34-55: one call pulls every table's rows, one backward pushes
+    every table's gradients."""
+
+    def __init__(self, dimensions, initializers=None, optim=None, lr=0.01, capacity_hint=0):
+        super().__init__()
+        self.combine_sparse_table = GpuCombineSparseTable(dimensions, initializers, optim, lr, capacity_hint)
+
+    def forward(self, indices):
+        if len(indices) != len(self.combine_sparse_table.dimensions()):
+            raise ValueError("one index tensor per table")
+        return list(CombineEmbeddingFunction.apply(self.combine_sparse_table, *indices))

@@ -113,3 +113,108 @@ def test_group_errors_and_async(api, oracle):
     assert np.array_equal(d_out.to_host()[:3], np.full((3, 8), np.float32(0.5)))
     assert np.array_equal(c.Pull([9])[1], np.full((1, 8), np.float32(0.25)))
     grp.close()
+
+
+def _dyadic(rng, shape):
+    """Gradients whose sums are exact in fp32 in any order."""
+    return (rng.integers(-64, 65, size=shape) / 256.0).astype(np.float32)
+
+
+@pytest.mark.parametrize("name,type_,conf", [c for c in OPTIM_CASES if c[0] in (
+    "sgd", "sgd_mom", "adagrad", "adam", "rmsprop_all")], ids=lambda v: v if isinstance(v, str) else None)
+@pytest.mark.parametrize("dim,n_tables,per_table", [(16, 26, 8192), (30, 3, 500), (128, 5, 70_000)])
+def test_group_push_raw_matches_dedup_sum_per_table(api, oracle, name, type_, conf, dim, n_tables, per_table):
+    """Emitter::CombinePushSparseTable (worker/emitter.cc:552-606): repeated ids of every table
+    are summed per (table, id) and each distinct row is updated once. The same id appears in
+    several tables with different gradients; the members have different row capacities and,
+    for one of them, a state column created by an earlier optimizer."""
+    rng = np.random.default_rng(dim * n_tables)
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "21"})
+    tables = [api.SparseTable(dim, gi, capacity_hint=64 << (i % 4)) for i in range(n_tables)]
+    refs = [oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=21))
+            for _ in range(n_tables)]
+    o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    # member 1 already has RMSprop's columns: its record layout differs from the others'
+    pre_ref, pre_gpu = make_optims(oracle, api, 2, {})
+    first = np.arange(10, dtype=np.uint64)
+    tables[1].Pull(first)
+    refs[1].pull(first)
+    g0 = _dyadic(rng, (10, dim))
+    assert tables[1].Push(pre_gpu, first, g0, 0.125) == 0
+    assert refs[1].push(pre_ref, first, g0, 0.125) == 0
+    grp = api.TableGroup(tables)
+    lr = 0.05
+    for step in range(3):
+        per = [zipf_ids(rng, 1.05, 100000, per_table if i != 2 or step != 1 else 0) for i in range(n_tables)]
+        off = grp._offsets([p.size for p in per])
+        ids = np.concatenate(per)
+        grads = _dyadic(rng, (ids.size, dim))
+        assert grp.CombinePull(ids, off)[0] == 0
+        for r, p in zip(refs, per):
+            r.pull(p)
+        assert grp.CombinePushRaw(o_gpu, ids, off, grads, lr) == 0
+        for r, p, a, b in zip(refs, per, off[:-1], off[1:]):
+            u, gs = oracle.dedup_sum(p, grads[a:b])
+            assert r.push(o_ref, u, gs, lr) == 0
+    for i, (t, r) in enumerate(zip(tables, refs)):
+        gid, gval, _, gsteps = t.export()
+        rid, rval, _, rsteps = r.export()
+        og, orr = np.argsort(gid), np.argsort(rid)
+        assert np.array_equal(gid[og], rid[orr])
+        assert_close(gval[og], rval[orr], "%s table %d" % (name, i), rtol=1e-5, atol=1e-7)
+        if type_ == 1:
+            assert np.array_equal(gsteps[og], rsteps[orr])    # one optimizer step per distinct id
+    grp.close()
+
+
+def test_group_push_raw_agrees_with_per_table_push_raw(api):
+    """Random gradients, Adam, identical row numbering on both sides: the combined pipeline and
+    krk_sparse_push_raw per table differ only in where tile borders fall in the sorted sequence,
+    i.e. in how the fp32 additions of one row's gradients are grouped."""
+    dim, n_tables, n = 32, 4, 30_000
+    rng = np.random.default_rng(5)
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "4"})
+    per = [zipf_ids(rng, 1.2, 50000, n) for _ in range(n_tables)]
+    grads = [(rng.standard_normal((n, dim)) * 1e-2).astype(np.float32) for _ in range(n_tables)]
+    o = api.Optim.create(api.OptimType.kAdam)
+    solo = [api.SparseTable(dim, gi) for _ in range(n_tables)]
+    grouped = [api.SparseTable(dim, gi) for _ in range(n_tables)]
+    uniq = [np.unique(p) for p in per]
+    for tabs in (solo, grouped):
+        for t, u in zip(tabs, uniq):
+            for k in range(u.size):
+                t.Pull(u[k:k + 1])                             # one id per call: rows numbered in this order
+    for a, b, u in zip(solo, grouped, uniq):
+        assert np.array_equal(a.lookup(u), b.lookup(u))
+    grp = api.TableGroup(grouped)
+    off = grp._offsets([n] * n_tables)
+    for step in range(2):
+        for t, p, g in zip(solo, per, grads):
+            assert t.PushRaw(o, p, g, 0.01) == 0
+        assert grp.CombinePushRaw(o, np.concatenate(per), off, np.concatenate(grads), 0.01) == 0
+    for i, (a, b, u) in enumerate(zip(solo, grouped, uniq)):
+        assert_close(b.Pull(u)[1], a.Pull(u)[1], "table %d" % i, rtol=1e-5, atol=1e-7)
+    grp.close()
+
+
+def test_group_push_raw_errors(api):
+    gi = api.Initializer.create(0, {"value": "1"})
+    a, b = api.SparseTable(8, gi), api.SparseTable(8, gi)
+    grp = api.TableGroup([a, b])
+    ids = np.array([1, 2, 1, 1, 5, 5], dtype=np.uint64)
+    off = [0, 4, 6]
+    assert grp.CombinePull(ids, off)[0] == 0
+    o = api.Optim.create(api.OptimType.kSGD)
+    g = np.ones((6, 8), np.float32)
+    assert grp.CombinePushRaw(o, ids, off, g, 0.5) == 0
+    assert np.array_equal(a.Pull([1, 2])[1][:, 0], np.float32([1 - 1.5, 1 - 0.5]))
+    assert np.array_equal(b.Pull([5])[1][:, 0], np.float32([0.0]))
+    bad = ids.copy()
+    bad[5] = 77                                                # b has never seen 77; 5 still gets its share
+    assert grp.CombinePushRaw(o, bad, off, g, 0.5) == 12
+    assert np.array_equal(b.Pull([5])[1][:, 0], np.float32([-0.5]))
+    assert b.lookup([77])[0] == -1
+    assert grp.CombinePushRaw(o, ids, off, np.ones((6, 4), np.float32), 0.5) == 11
+    assert grp.CombinePushRaw(o, np.zeros(0, np.uint64), [0, 0, 0], np.zeros((0, 8), np.float32), 0.5) == 0
+    assert grp.CombinePushRaw(api.Optim.create(api.OptimType.kSGD), ids, [0, 5, 4], g, 0.5) != 0
+    grp.close()

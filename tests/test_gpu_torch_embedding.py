@@ -104,3 +104,41 @@ def test_rejects_host_tensors(mods):
         emb(torch.zeros(3, dtype=torch.int64))
     with pytest.raises(TypeError):
         emb(torch.zeros(3, dtype=torch.int32).cuda())
+
+
+def test_combine_embedding_forward_backward(mods, oracle):
+    """pytorch/combine_embedding.py: tables of two widths in one request, ids repeated within a
+    table and shared between tables, one output left out of the loss."""
+    api, te = mods
+    dims = [8, 16, 8, 8]
+    seeds = [5, 6, 7, 8]
+    inits = [_init(api, oracle, s) for s in seeds]
+    o_ref, o_gpu = make_optims(oracle, api, 3, {})                      # plain SGD
+    emb = te.CombineEmbedding(dims, initializers=[g for g, _ in inits], optim=o_gpu, lr=0.5)
+    refs = [oracle.SparseTable(d, oi) for d, (_, oi) in zip(dims, inits)]
+    g = torch.Generator(device="cpu").manual_seed(2)
+    for step in range(3):
+        idx = [torch.randint(0, 200, shape, generator=g).cuda() for shape in ((32, 3), (50,), (7, 2, 2), (64,))]
+        outs = emb(idx)
+        assert [tuple(o.shape) for o in outs] == [(32, 3, 8), (50, 16), (7, 2, 2, 8), (64, 8)]
+        coefs = []
+        loss = 0.0
+        for k, (o, r, i, d) in enumerate(zip(outs, refs, idx, dims)):
+            ids = i.cpu().numpy().astype(np.uint64).ravel()
+            u, inv = oracle.dedup(ids)
+            assert np.array_equal(o.detach().cpu().numpy().reshape(-1, d), r.pull(u)[1][inv])
+            c = (torch.randint(-8, 9, o.shape, generator=g) / 16.0).cuda()
+            coefs.append(c)
+            if k != 3:                                                   # table 3 gets no gradient
+                loss = loss + (o * c).sum()
+        loss.backward()
+        for k, (r, i, d, c) in enumerate(zip(refs, idx, dims, coefs)):
+            ids = i.cpu().numpy().astype(np.uint64).ravel()
+            grad = c.cpu().numpy().reshape(-1, d) if k != 3 else np.zeros((ids.size, d), np.float32)
+            u, gs = oracle.dedup_sum(ids, grad)
+            assert r.push(o_ref, u, gs, 0.5) == 0
+    torch.cuda.synchronize()
+    for t, r in zip(emb.combine_sparse_table.tables(), refs):
+        rid, rval, _, _ = r.export()
+        assert len(t) == len(r)
+        assert np.array_equal(t.Pull(rid)[1], rval)                     # dyadic gradients, SGD: exact
