@@ -305,20 +305,26 @@ __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, con
 }
 
 // keys[cnt] ascending (entries >= empty_from are holes). LEVEL0: the value of entry j is gradient
-// row pos[j]; otherwise it is vals[j, :]. Each tile of `tile` entries writes carry slots 2t
-// (run entering from the left) and 2t+1 (run leaving to the right).
+// row pos[j]; otherwise it is vals[j, :].
 //
 // A workgroup first stages the keys (and positions) of all its tiles in LDS with coalesced loads,
 // including one neighbour on each side, so the walk itself only waits for value rows; those are
-// requested four entries ahead of where the sums are. Carry levels use short tiles: the lists
-// are short, so short tiles keep many lane groups busy (tiles of 32 with eight entries in
-// flight save one or two dependent launches but measured slower, 442 vs 432 us at 1M ids).
+// requested four entries ahead of where the sums are. A lane group walks its tile and applies
+// every run that lies wholly inside it. A run that touches a tile border leaves its partial sum
+// in LDS instead: slot 2t for the run entering tile t from the left, 2t + 1 for the one leaving
+// it to the right (a run that covers the whole tile fills both, the second with zeros). Equal
+// keys are adjacent in that list, so after a barrier the lane group that owns the first partial
+// of a run adds up the following ones (in order, from LDS) and applies the sum. Only the runs that
+// cross the workgroup's own borders go on to the next level: carry slots 2w and 2w + 1 of
+// workgroup w, which form a sorted sequence again. A level shrinks the sequence by the
+// workgroup's span over two, so two or three launches serve any request.
+//
 // Running the last, short levels in one launch of a single workgroup (barrier between levels)
 // was measured too: on one CU every level pays its dependent memory round trips one after the
 // other, 36 us against four launches of about 8 us for the tail of an 8192-id request.
 constexpr int kPrefetch = 4;
 constexpr int kPrefetchCarry = 4;
-constexpr int kCarryTile = 16;
+constexpr int kCarryTile = 4;
 
 // Weighted bags (level 0 only): the sorted payload is a position p, its gradient row is
 // vals[bag_of[p]] times weight[p]. Both null otherwise: the payload itself names the row.
@@ -337,118 +343,11 @@ struct GroupSrc {
   int use_meta;
 };
 
-// One tile: entries [t * tile, (t + 1) * tile) of the sequence, walked by the `group` lanes that
-// call this together. lds_keys[i] holds the key of entry first + i - 1 (so both neighbours of
-// the tile are there), lds_pos / lds_w the payloads and weights of entry first + i.
-template <int OPT, int VEC, bool LEVEL0, bool GROUPED>
-__device__ __forceinline__ void reduce_tile(
-    int64_t t, int64_t first, const uint32_t* lds_keys, const uint32_t* lds_pos, const float* lds_w,
-    bool weighted, const TableView& tv, const float* __restrict__ vals, int64_t cnt, int tile,
-    uint32_t empty_from, uint32_t* __restrict__ keys_out, float* __restrict__ vals_out, int dim, int elems,
-    int group, const ApplyArgs& args, const GroupSrc& gs) {
-  const int gl = threadIdx.x & (group - 1);
-  const int64_t a = t * tile;
-  if (a >= cnt) return;
-  const int64_t b = a + tile < cnt ? a + tile : cnt;
-  const int la = (int)(a - first);                          // tile's first entry, LDS-relative
-  const int lb = (int)(b - first);
-  const uint32_t left_key = lds_keys[la];                   // entry a - 1
-  const uint32_t right_key = lds_keys[lb + 1];              // entry b
-  const bool leader = gl == 0;
-  uint32_t carry_key0 = kNoRow, carry_key1 = kNoRow;        // what this tile leaves in the carry list
-
-  for (int e0 = 0; e0 < elems; e0 += group) {
-    const int e = e0 + gl;
-    const bool lane_on = e < elems;
-    const bool last_chunk = e0 + group >= elems;
-    float acc[VEC];
-#pragma unroll
-    for (int c = 0; c < VEC; ++c) acc[c] = 0.0f;
-    uint32_t run_key = lds_keys[la + 1];
-    int run_start = la;
-
-    // closes the run [run_start, end) of run_key
-    auto close_run = [&](int end) {
-      if (run_key >= empty_from) return;
-      const bool open_left = run_start == la && left_key == run_key;
-      const bool open_right = end == lb && right_key == run_key;
-      if (!open_left && !open_right) {
-        if constexpr (GROUPED) {
-          const TableDesc& d = gs.descs[run_key >> gs.row_bits];
-          TableView member = tv;
-          member.recs = d.tv.recs;
-          member.stride = d.tv.stride;
-          ApplyArgs aa = args;
-          aa.c0 = gs.st0 >= 0 ? d.col_off[gs.st0] : -1;
-          aa.c1 = gs.st1 >= 0 ? d.col_off[gs.st1] : -1;
-          aa.c2 = gs.st2 >= 0 ? d.col_off[gs.st2] : -1;
-          aa.meta_off = gs.use_meta ? d.meta_off : -1;
-          apply_row<OPT, VEC>(member, run_key & ((1u << gs.row_bits) - 1u), acc, e, lane_on, leader,
-                              last_chunk, aa);
-        } else {
-          apply_row<OPT, VEC>(tv, run_key, acc, e, lane_on, leader, last_chunk, args);
-        }
-        return;
-      }
-      const int64_t slot = open_left ? 2 * t : 2 * t + 1;
-      if (lane_on) vstore<VEC>(vals_out + slot * dim + e * VEC, acc);
-      if (open_left) carry_key0 = run_key; else carry_key1 = run_key;
-      if (open_left && open_right) {
-        // the run covers the whole tile: keep the carry list contiguous with a zero piece
-        float z[VEC];
-#pragma unroll
-        for (int c = 0; c < VEC; ++c) z[c] = 0.0f;
-        if (lane_on) vstore<VEC>(vals_out + (slot + 1) * dim + e * VEC, z);
-        carry_key1 = run_key;
-      }
-    };
-
-    constexpr int kAhead = LEVEL0 ? kPrefetch : kPrefetchCarry;
-    for (int j0 = la; j0 < lb; j0 += kAhead) {
-      float v[kAhead][VEC];
-      uint32_t k[kAhead];
-#pragma unroll
-      for (int u = 0; u < kAhead; ++u) {
-        const int j = j0 + u;
-        k[u] = j < lb ? lds_keys[j + 1] : kNoRow;
-        if (j < lb && k[u] < empty_from && lane_on) {
-          const float* src = LEVEL0 ? vals + (int64_t)lds_pos[j] * dim : vals + (first + j) * dim;
-          vload<VEC>(src + e * VEC, v[u]);
-          if (weighted) {
-            const float w = lds_w[j];
-#pragma unroll
-            for (int c = 0; c < VEC; ++c) v[u][c] = v[u][c] * w;
-          }
-        } else {
-#pragma unroll
-          for (int c = 0; c < VEC; ++c) v[u][c] = 0.0f;
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < kAhead; ++u) {
-        const int j = j0 + u;
-        if (j >= lb) break;
-        if (k[u] != run_key) {
-          close_run(j);
-          run_key = k[u];
-          run_start = j;
-        }
-        if (j == run_start) {
-          // the first addend is copied, not added to zero (worker/emitter.cc:527 clones it)
-#pragma unroll
-          for (int c = 0; c < VEC; ++c) acc[c] = v[u][c];
-        } else {
-#pragma unroll
-          for (int c = 0; c < VEC; ++c) acc[c] = acc[c] + v[u][c];
-        }
-      }
-    }
-    close_run(lb);
-  }
-  if (leader && keys_out) {
-    keys_out[2 * t] = carry_key0;
-    keys_out[2 * t + 1] = carry_key1;
-  }
+// LDS of one workgroup, in 32-bit words: partial sums [2 * per_block][group * VEC] first (vector
+// accesses, 16-byte aligned), then partial keys [2 * per_block], the two carry keys, the staged
+// keys [span + 2], payloads [span] and weights [span].
+__host__ __device__ inline size_t segreduce_lds_words(int per_block, int group, int vec, int tile) {
+  return (size_t)2 * per_block * group * vec + 2 * per_block + 2 + 3 * (size_t)per_block * tile + 2;
 }
 
 template <int OPT, int VEC, bool LEVEL0, bool GROUPED>
@@ -461,9 +360,12 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
   const int per_block = kBlock / group;
   const int span = per_block * tile;                       // entries staged by this workgroup
   const int64_t first = (int64_t)blockIdx.x * span;        // global index of lds_keys[1]
-  uint32_t* lds_keys = lds;                                // [span + 2], shifted by one
-  uint32_t* lds_pos = lds + span + 2;                      // [span]
-  float* lds_w = reinterpret_cast<float*>(lds + 2 * span + 2);   // [span], weighted bags only
+  float* part_val = reinterpret_cast<float*>(lds);         // [2 * per_block][group * VEC]
+  uint32_t* part_key = lds + 2 * per_block * group * VEC;  // [2 * per_block]
+  uint32_t* out_key = part_key + 2 * per_block;            // [2]: what this workgroup carries on
+  uint32_t* lds_keys = out_key + 2;                        // [span + 2], shifted by one
+  uint32_t* lds_pos = lds_keys + span + 2;                 // [span]
+  float* lds_w = reinterpret_cast<float*>(lds_pos + span); // [span], weighted bags only
   for (int i = threadIdx.x; i < span + 2; i += kBlock) {
     const int64_t j = first + i - 1;
     lds_keys[i] = (j >= 0 && j < cnt) ? keys[j] : kNoRow;
@@ -482,10 +384,163 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
       lds_pos[i] = p;
     }
   }
+  if (threadIdx.x < 2) out_key[threadIdx.x] = kNoRow;
   __syncthreads();
-  const int64_t t = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
-  reduce_tile<OPT, VEC, LEVEL0, GROUPED>(t, first, lds_keys, lds_pos, lds_w, weighted, tv, vals, cnt, tile,
-                                         empty_from, keys_out, vals_out, dim, elems, group, args, gs);
+
+  const int lt = threadIdx.x / group;                       // this lane group's tile in the workgroup
+  const int gl = threadIdx.x & (group - 1);
+  const int64_t a = ((int64_t)blockIdx.x * per_block + lt) * tile;
+  const bool have = a < cnt;                                // the last workgroup may have idle groups
+  const int64_t b = a + tile < cnt ? a + tile : cnt;
+  const int la = (int)(a - first);                          // tile's first entry, LDS-relative
+  const int lb = have ? (int)(b - first) : la;
+  const uint32_t left_key = have ? lds_keys[la] : kNoRow;   // entry a - 1
+  const uint32_t right_key = have ? lds_keys[lb + 1] : kNoRow;   // entry b
+  const int64_t rem_tiles = (cnt - first + tile - 1) / tile;
+  const int tiles_here = rem_tiles < per_block ? (int)rem_tiles : per_block;
+  const bool leader = gl == 0;
+  const int lane_floats = group * VEC;
+
+  // hands a finished sum to the optimizer (or stores it): once per run and chunk
+  auto apply = [&](uint32_t key, const float (&sum)[VEC], int e, bool lane_on, bool last_chunk) {
+    if constexpr (GROUPED) {
+      const TableDesc& d = gs.descs[key >> gs.row_bits];
+      TableView member = tv;
+      member.recs = d.tv.recs;
+      member.stride = d.tv.stride;
+      ApplyArgs aa = args;
+      aa.c0 = gs.st0 >= 0 ? d.col_off[gs.st0] : -1;
+      aa.c1 = gs.st1 >= 0 ? d.col_off[gs.st1] : -1;
+      aa.c2 = gs.st2 >= 0 ? d.col_off[gs.st2] : -1;
+      aa.meta_off = gs.use_meta ? d.meta_off : -1;
+      apply_row<OPT, VEC>(member, key & ((1u << gs.row_bits) - 1u), sum, e, lane_on, leader, last_chunk, aa);
+    } else {
+      apply_row<OPT, VEC>(tv, key, sum, e, lane_on, leader, last_chunk, args);
+    }
+  };
+
+  for (int e0 = 0; e0 < elems; e0 += group) {
+    const int e = e0 + gl;
+    const bool lane_on = e < elems;
+    const bool last_chunk = e0 + group >= elems;
+    uint32_t pk0 = kNoRow, pk1 = kNoRow;                    // keys of this tile's two partials
+    if (have) {
+      float acc[VEC];
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) acc[c] = 0.0f;
+      uint32_t run_key = lds_keys[la + 1];
+      int run_start = la;
+
+      // closes the run [run_start, end) of run_key
+      auto close_run = [&](int end) {
+        if (run_key >= empty_from) return;
+        const bool open_left = run_start == la && left_key == run_key;
+        const bool open_right = end == lb && right_key == run_key;
+        if (!open_left && !open_right) {
+          apply(run_key, acc, e, lane_on, last_chunk);
+          return;
+        }
+        const int slot = open_left ? 2 * lt : 2 * lt + 1;
+        vstore<VEC>(part_val + slot * lane_floats + gl * VEC, acc);
+        if (open_left) pk0 = run_key; else pk1 = run_key;
+        if (open_left && open_right) {
+          // the run covers the whole tile: keep the list contiguous with a zero piece
+          float z[VEC];
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) z[c] = 0.0f;
+          vstore<VEC>(part_val + (slot + 1) * lane_floats + gl * VEC, z);
+          pk1 = run_key;
+        }
+      };
+
+      constexpr int kAhead = LEVEL0 ? kPrefetch : kPrefetchCarry;
+      for (int j0 = la; j0 < lb; j0 += kAhead) {
+        float v[kAhead][VEC];
+        uint32_t k[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+          const int j = j0 + u;
+          k[u] = j < lb ? lds_keys[j + 1] : kNoRow;
+          if (j < lb && k[u] < empty_from && lane_on) {
+            const float* src = LEVEL0 ? vals + (int64_t)lds_pos[j] * dim : vals + (first + j) * dim;
+            vload<VEC>(src + e * VEC, v[u]);
+            if (weighted) {
+              const float w = lds_w[j];
+#pragma unroll
+              for (int c = 0; c < VEC; ++c) v[u][c] = v[u][c] * w;
+            }
+          } else {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) v[u][c] = 0.0f;
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+          const int j = j0 + u;
+          if (j >= lb) break;
+          if (k[u] != run_key) {
+            close_run(j);
+            run_key = k[u];
+            run_start = j;
+          }
+          if (j == run_start) {
+            // the first addend is copied, not added to zero (worker/emitter.cc:527 clones it)
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) acc[c] = v[u][c];
+          } else {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) acc[c] = acc[c] + v[u][c];
+          }
+        }
+      }
+      close_run(lb);
+    }
+    if (leader) {
+      part_key[2 * lt] = pk0;
+      part_key[2 * lt + 1] = pk1;
+    }
+    __syncthreads();
+
+    // the partials of one run are adjacent: the group that owns the first adds the others to it
+    if (have) {
+      const int last = 2 * tiles_here - 1;
+      for (int side = 0; side < 2; ++side) {
+        const int en = 2 * lt + side;
+        const uint32_t key = part_key[en];
+        if (key == kNoRow || (en > 0 && part_key[en - 1] == key)) continue;
+        float sum[VEC];
+        vload<VEC>(part_val + en * lane_floats + gl * VEC, sum);
+        int f = en;
+        while (f < last && part_key[f + 1] == key) {
+          ++f;
+          float nx[VEC];
+          vload<VEC>(part_val + f * lane_floats + gl * VEC, nx);
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) sum[c] = sum[c] + nx[c];
+        }
+        // slot 0 exists only for a run that enters the workgroup from the left, the last slot
+        // only for one that leaves it to the right
+        const bool open_left = en == 0;
+        const bool open_right = f == last;
+        if (!open_left && !open_right) {
+          apply(key, sum, e, lane_on, last_chunk);
+          continue;
+        }
+        const int64_t slot = 2 * (int64_t)blockIdx.x + (open_left ? 0 : 1);
+        if (lane_on) vstore<VEC>(vals_out + slot * dim + e * VEC, sum);
+        if (leader) out_key[open_left ? 0 : 1] = key;
+        if (open_left && open_right) {
+          float z[VEC];
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) z[c] = 0.0f;
+          if (lane_on) vstore<VEC>(vals_out + (slot + 1) * dim + e * VEC, z);
+          if (leader) out_key[1] = key;
+        }
+      }
+    }
+    __syncthreads();                                        // the next chunk reuses the partials
+  }
+  if (threadIdx.x < 2 && keys_out) keys_out[2 * (int64_t)blockIdx.x + threadIdx.x] = out_key[threadIdx.x];
 }
 
 // Row width and lane mapping of a reduction: a table's, or those of a stand-alone call.
@@ -503,7 +558,7 @@ static void launch_segreduce(bool level0, const TableView& tv, const uint32_t* k
   const int per_block = kBlock / t->group;
   const int64_t tiles = (cnt + tile - 1) / tile;
   const dim3 grid(grid_for(tiles, per_block)), block(kBlock);
-  const size_t lds_bytes = (size_t)(3 * per_block * tile + 2) * sizeof(uint32_t);
+  const size_t lds_bytes = segreduce_lds_words(per_block, t->group, VEC, tile) * sizeof(uint32_t);
   const PooledSrc none{nullptr, nullptr};
   if constexpr (OPT != kOptStore) {
     if (gs) {
@@ -562,10 +617,10 @@ static void dispatch_segreduce(int opt, bool level0, const TableView& tv, const 
 }
 
 static int pick_tile(int64_t cnt) {
-  // Large requests: long tiles keep the carry list small. Small ones: short tiles keep the
-  // whole GPU busy; extra reduction levels cost only a few microseconds each.
-  if (cnt >= (1 << 20)) return 32;
-  if (cnt >= (1 << 16)) return 16;
+  // The carry list has two entries per workgroup whatever the tile length, so tiles only trade
+  // lane groups in flight against per-tile work: 8 entries up to half a million ids, 16 beyond
+  // (measured 4 to 64). The carry lists themselves are short: tiles of 4 there.
+  if (cnt >= (1 << 19)) return 16;
   return 8;
 }
 
@@ -602,11 +657,12 @@ static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, Device
                                const float* d_vals, const ApplyArgs& args, const PooledSrc& ps,
                                const GroupSrc* gs, Fill fill) {
   const int tile0 = pick_tile(n);
-  const int64_t tiles0 = (n + tile0 - 1) / tile0;
+  const int per_block = kBlock / sh.group;
+  const int64_t groups0 = ((n + tile0 - 1) / tile0 + per_block - 1) / per_block;   // workgroups of level 0
   const size_t n4 = (size_t)n * sizeof(uint32_t);
   size_t sort_bytes = 0;
   KRK_HIP(sort_pairs(nullptr, sort_bytes, nullptr, nullptr, nullptr, nullptr, n, bits, stream));
-  const size_t carry_entries = (size_t)(2 * tiles0);
+  const size_t carry_entries = (size_t)(2 * groups0);
   KRK_TRY(scratch[0].reserve(4 * n4));                       // keys, payload, sorted keys, sorted payload
   KRK_TRY(scratch[1].reserve(sort_bytes));
   KRK_TRY(scratch[2].reserve(carry_entries * sizeof(uint32_t) * 2));              // carry keys A|B
@@ -631,10 +687,10 @@ static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, Device
   bool level0 = true;
   int which = 0;
   for (;;) {
-    const int64_t tiles = (cnt + tile - 1) / tile;
+    const int64_t groups = ((cnt + tile - 1) / tile + per_block - 1) / per_block;
     uint32_t* okeys = nullptr;
     float* ovals = nullptr;
-    if (tiles > 1) {
+    if (groups > 1) {
       okeys = ckeys[which];
       ovals = cvals[which];
     }
@@ -646,10 +702,10 @@ static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, Device
                             args, ps, gs, stream);
     }
     KRK_HIP(hipGetLastError());
-    if (tiles <= 1) break;
+    if (groups <= 1) break;
     in_keys = okeys;
     in_vals = ovals;
-    cnt = 2 * tiles;
+    cnt = 2 * groups;
     level0 = false;
     which ^= 1;
     tile = kCarryTile;
