@@ -630,10 +630,12 @@ static int pick_tile(int64_t cnt) {
 // million pairs on 256 CUs. For (u32, u32) pairs on this GPU the radix path with 8-bit digits
 // and the wavefront-matching rank is the faster one from about 2^16 items on; blocks of 4096
 // items serve up to two million pairs best, blocks of 8192 beyond (measured per sort of 2^20
-// pairs of 26-bit keys: 160 us merge sort, 110 us with 4096-item blocks). All paths are stable.
+// pairs of 26-bit keys: 160 us merge sort, 110 us with 4096-item blocks). Up to 8192 pairs one
+// workgroup sorts them all in a single launch (the default switches to block sort plus merge
+// passes above 2048: six launches and 26 us for 8192 pairs). All paths are stable.
 template <unsigned ItemsPerThread>
 using SortConfig = rocprim::radix_sort_config<
-    rocprim::default_config, rocprim::default_config,
+    rocprim::kernel_config<1024, 8>, rocprim::default_config,
     rocprim::radix_sort_onesweep_config<rocprim::kernel_config<256, 12>, rocprim::kernel_config<1024, ItemsPerThread>,
                                         8, rocprim::block_radix_rank_algorithm::match>,
     (size_t)1 << 16>;
