@@ -148,12 +148,13 @@ static float* g_basis_inv = nullptr;
 static int32_t ensure_basis(hipStream_t s) {
   std::lock_guard<std::mutex> lk(g_basis_mu);
   if (g_basis_fwd) return KRK_SUCCESS;
-  float* p = nullptr;
-  KRK_HIP(hipMalloc((void**)&p, 2 * sizeof(float) * kDctB * kDctB));
+  DeviceGuard guard;
+  KRK_HIP(hipMalloc(&guard.p, 2 * sizeof(float) * kDctB * kDctB));
+  float* p = reinterpret_cast<float*>(guard.p);
   hipLaunchKernelGGL(dct2_basis_kernel, dim3(kDctB * kDctB / 256), dim3(256), 0, s, p, p + kDctB * kDctB);
   KRK_HIP(hipGetLastError());
   KRK_HIP(hipStreamSynchronize(s));
-  g_basis_fwd = p;
+  g_basis_fwd = guard.release<float>();
   g_basis_inv = p + kDctB * kDctB;
   return KRK_SUCCESS;
 }

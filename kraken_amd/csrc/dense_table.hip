@@ -77,8 +77,10 @@ static unsigned dense_grid(int64_t n) {
 
 static int32_t ensure_state(krk_dense* t, int st) {
   if (t->state[st]) return KRK_SUCCESS;
-  KRK_HIP(hipMalloc((void**)&t->state[st], (size_t)t->n * sizeof(float)));
-  KRK_HIP(hipMemsetAsync(t->state[st], 0, (size_t)t->n * sizeof(float), t->stream));
+  DeviceGuard guard;
+  KRK_HIP(hipMalloc(&guard.p, (size_t)(t->n ? t->n : 1) * sizeof(float)));
+  KRK_HIP(hipMemsetAsync(guard.p, 0, (size_t)t->n * sizeof(float), t->stream));
+  t->state[st] = guard.release<float>();   // only a zeroed column counts as present
   return KRK_SUCCESS;
 }
 

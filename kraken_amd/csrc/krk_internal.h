@@ -44,6 +44,24 @@ struct DeviceBuffer {
   }
 };
 
+// Owns a fresh device allocation until it is handed over: error paths between hipMalloc and the
+// hand-over free it.
+struct DeviceGuard {
+  void* p = nullptr;
+  DeviceGuard() = default;
+  DeviceGuard(const DeviceGuard&) = delete;
+  DeviceGuard& operator=(const DeviceGuard&) = delete;
+  ~DeviceGuard() {
+    if (p) (void)hipFree(p);
+  }
+  template <typename T>
+  T* release() {
+    T* q = reinterpret_cast<T*>(p);
+    p = nullptr;
+    return q;
+  }
+};
+
 // Every API object starts with this: its own stream, the host lock that serialises
 // calls on it, and the staging buffers used when the caller hands over host pointers.
 struct ObjBase {

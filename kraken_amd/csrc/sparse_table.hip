@@ -707,15 +707,12 @@ static int32_t grow_rows(krk_sparse* t, int64_t new_cap, int64_t new_stride) {
     set_error("sparse table cannot hold more than 2^32-2 rows");
     return KRK_E_CAPACITY;
   }
-  float* nrecs = nullptr;
-  unsigned long long* nkeys = nullptr;
+  DeviceGuard recs_guard, keys_guard;
   const size_t rec_bytes = (size_t)new_cap * (size_t)new_stride * sizeof(float);
-  KRK_HIP(hipMalloc((void**)&nrecs, rec_bytes ? rec_bytes : 16));
-  hipError_t e = hipMalloc((void**)&nkeys, (size_t)(new_cap ? new_cap : 1) * sizeof(unsigned long long));
-  if (e != hipSuccess) {
-    (void)hipFree(nrecs);
-    return hip_fail(e, "hipMalloc(row_key)", __FILE__, __LINE__);
-  }
+  KRK_HIP(hipMalloc(&recs_guard.p, rec_bytes ? rec_bytes : 16));
+  KRK_HIP(hipMalloc(&keys_guard.p, (size_t)(new_cap ? new_cap : 1) * sizeof(unsigned long long)));
+  float* nrecs = reinterpret_cast<float*>(recs_guard.p);
+  unsigned long long* nkeys = reinterpret_cast<unsigned long long*>(keys_guard.p);
   const size_t used = (size_t)rows * (size_t)t->stride * sizeof(float);
   if (used) KRK_HIP(hipMemcpyAsync(nrecs, t->recs, used, hipMemcpyDeviceToDevice, t->stream));
   if (rec_bytes > used)
@@ -726,8 +723,8 @@ static int32_t grow_rows(krk_sparse* t, int64_t new_cap, int64_t new_stride) {
   KRK_HIP(hipStreamSynchronize(t->stream));
   if (t->recs) (void)hipFree(t->recs);
   if (t->row_key) (void)hipFree(t->row_key);
-  t->recs = nrecs;
-  t->row_key = nkeys;
+  t->recs = recs_guard.release<float>();
+  t->row_key = keys_guard.release<unsigned long long>();
   t->row_cap = new_cap;
   t->layout_version++;
   return KRK_SUCCESS;
@@ -736,6 +733,8 @@ static int32_t grow_rows(krk_sparse* t, int64_t new_cap, int64_t new_stride) {
 static int32_t grow_slots(krk_sparse* t, uint64_t new_cap) {
   Slot* ns = nullptr;
   KRK_TRY(alloc_slots(new_cap, &ns, t->stream));
+  DeviceGuard guard;
+  guard.p = ns;
   KRK_TRY(refresh_rows(t));
   const int64_t rows = t->size_ub;
   if (rows) {
@@ -745,7 +744,7 @@ static int32_t grow_slots(krk_sparse* t, uint64_t new_cap) {
   }
   KRK_HIP(hipStreamSynchronize(t->stream));
   if (t->slots) (void)hipFree(t->slots);
-  t->slots = ns;
+  t->slots = guard.release<Slot>();
   t->slot_cap = new_cap;
   t->layout_version++;
   return KRK_SUCCESS;
@@ -853,9 +852,10 @@ int32_t sparse_ensure_columns(krk_sparse* t, uint32_t mask) {
   const int64_t old_body = old_meta >= 0 ? old_meta : old_stride;
   KRK_TRY(refresh_rows(t));
   const int64_t rows = t->size_ub;
-  float* nrecs = nullptr;
+  DeviceGuard guard;
   const size_t rec_bytes = (size_t)t->row_cap * (size_t)stride * sizeof(float);
-  KRK_HIP(hipMalloc((void**)&nrecs, rec_bytes ? rec_bytes : 16));
+  KRK_HIP(hipMalloc(&guard.p, rec_bytes ? rec_bytes : 16));
+  float* nrecs = reinterpret_cast<float*>(guard.p);
   KRK_HIP(hipMemsetAsync(nrecs, 0, rec_bytes, t->stream));
   if (rows) {
     hipLaunchKernelGGL(restride_kernel, dim3(strided_grid(rows * old_body)), dim3(kBlock), 0,
@@ -868,7 +868,7 @@ int32_t sparse_ensure_columns(krk_sparse* t, uint32_t mask) {
   }
   KRK_HIP(hipStreamSynchronize(t->stream));
   if (t->recs) (void)hipFree(t->recs);
-  t->recs = nrecs;
+  t->recs = guard.release<float>();
   t->stride = stride;
   t->meta_off = meta_off;
   memcpy(t->col_off, col_off, sizeof(col_off));
