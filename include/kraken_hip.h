@@ -128,6 +128,12 @@ const char* krk_error_message(int32_t code);   /* ErrorCode::Msg, common/error_c
 /* Harness helpers: device buffers and timing without any other GPU library. */
 int32_t krk_malloc(void** dptr, size_t bytes);
 int32_t krk_free(void* dptr);
+/* Page-locked host memory. Host-pointer calls copy to and from the caller's buffers; when those
+ * are pageable the copies are staged through the runtime's bounce buffers (about 5 GB/s towards
+ * the host), when they come from here the GPU's copy engines reach them directly. A server
+ * that receives requests and builds replies in buffers of its own should take them from here. */
+int32_t krk_host_malloc(void** hptr, size_t bytes);
+int32_t krk_host_free(void* hptr);
 int32_t krk_memcpy_h2d(void* dst, const void* src, size_t bytes);
 int32_t krk_memcpy_d2h(void* dst, const void* src, size_t bytes);
 int32_t krk_memset(void* dptr, int value, size_t bytes);

@@ -68,6 +68,8 @@ EXPORTS = {
     "krk_memset": (C.c_int32, [C.c_void_p, C.c_int, C.c_size_t]),
     "krk_device_synchronize": (C.c_int32, []),
     "krk_mem_info": (C.c_int32, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "krk_host_malloc": (C.c_int32, [C.POINTER(C.c_void_p), C.c_size_t]),
+    "krk_host_free": (C.c_int32, [C.c_void_p]),
     "krk_stream_copy": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "krk_sparse_create": (C.c_int32, [C.c_int64, C.POINTER(krk_init), C.c_int64, C.POINTER(C.c_void_p)]),
     "krk_sparse_destroy": (C.c_int32, [C.c_void_p]),
@@ -226,6 +228,37 @@ class DeviceArray:
             self.free()
         except Exception:
             pass
+
+
+def pinned_empty(shape, dtype):
+    """A numpy array in page-locked host memory (krk_host_malloc); it is freed with the array."""
+    shape = tuple(shape) if isinstance(shape, (tuple, list)) else (int(shape),)
+    dtype = np.dtype(dtype)
+    nbytes = int(np.prod(shape)) * dtype.itemsize
+    p = C.c_void_p()
+    _check(lib().krk_host_malloc(C.byref(p), max(nbytes, 16)), "krk_host_malloc")
+
+    class _Owner:
+        def __init__(self, ptr):
+            self.ptr = ptr
+            self.__array_interface__ = {"data": (ptr, False), "shape": (max(nbytes, 1),), "typestr": "|u1",
+                                        "version": 3}
+
+        def __del__(self):
+            try:
+                lib().krk_host_free(C.c_void_p(self.ptr))
+            except Exception:
+                pass
+
+    raw = np.asarray(_Owner(p.value))
+    return raw[:nbytes].view(dtype).reshape(shape)
+
+
+def pinned_copy(a):
+    a = np.ascontiguousarray(a)
+    out = pinned_empty(a.shape, a.dtype)
+    out[...] = a
+    return out
 
 
 def synchronize():

@@ -62,12 +62,19 @@ struct DeviceGuard {
   }
 };
 
+// A host pointer that HIP knows as page-locked (hipHostMalloc, krk_host_malloc, a framework's
+// pinned tensors) can be handed to kernels as it is: they read and write it across PCIe, which
+// saves the staging copy and its launch. Returns the address kernels use, or null when the
+// memory is pageable or not aligned to `align` bytes.
+void* direct_host_pointer(const void* p, size_t align);
+
 // Every API object starts with this: its own stream, the host lock that serialises
 // calls on it, and the staging buffers used when the caller hands over host pointers.
 struct ObjBase {
   hipStream_t stream = nullptr;
   std::mutex mu;
   DeviceBuffer stage[4];
+  bool direct[4] = {false, false, false, false};   // output slot is the caller's own page-locked buffer
   int32_t open_stream();
   void close_stream();
   // Copies a host array into staging buffer `slot` (or passes a device pointer through).
@@ -75,6 +82,10 @@ struct ObjBase {
   int32_t input(const T* p, size_t count, uint32_t flags, int slot, const T** dev) {
     if (flags & KRK_DEVICE_PTRS) {
       *dev = p;
+      return KRK_SUCCESS;
+    }
+    if (void* d = direct_host_pointer(p, 16)) {
+      *dev = reinterpret_cast<const T*>(d);
       return KRK_SUCCESS;
     }
     KRK_TRY(stage[slot].reserve(count * sizeof(T) + 16));
@@ -89,13 +100,19 @@ struct ObjBase {
       *dev = p;
       return KRK_SUCCESS;
     }
+    direct[slot] = false;
+    if (void* d = direct_host_pointer(p, 16)) {
+      direct[slot] = true;
+      *dev = reinterpret_cast<T*>(d);
+      return KRK_SUCCESS;
+    }
     KRK_TRY(stage[slot].reserve(count * sizeof(T) + 16));
     *dev = stage[slot].as<T>();
     return KRK_SUCCESS;
   }
   template <typename T>
   int32_t output_back(T* p, size_t count, uint32_t flags, int slot) {
-    if ((flags & KRK_DEVICE_PTRS) || !count) return KRK_SUCCESS;
+    if ((flags & KRK_DEVICE_PTRS) || !count || direct[slot]) return KRK_SUCCESS;
     KRK_HIP(hipMemcpyAsync(p, stage[slot].ptr, count * sizeof(T), hipMemcpyDeviceToHost, stream));
     return KRK_SUCCESS;
   }

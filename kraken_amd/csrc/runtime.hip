@@ -59,6 +59,18 @@ int32_t ensure_runtime() {
   return KRK_SUCCESS;
 }
 
+void* direct_host_pointer(const void* p, size_t align) {
+  if (!p || ((uintptr_t)p & (align - 1))) return nullptr;
+  hipPointerAttribute_t attr;
+  const hipError_t e = hipPointerGetAttributes(&attr, p);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();   // pageable memory is not an error for the calls that follow
+    return nullptr;
+  }
+  if (attr.type != hipMemoryTypeHost) return nullptr;
+  return attr.devicePointer;
+}
+
 int32_t DeviceBuffer::reserve(size_t want) {
   if (want <= bytes) return KRK_SUCCESS;
   size_t grow = bytes + bytes / 2;
@@ -373,6 +385,17 @@ int32_t krk_malloc(void** dptr, size_t bytes) {
 int32_t krk_free(void* dptr) {
   if (!dptr) return KRK_SUCCESS;
   KRK_HIP(hipFree(dptr));
+  return KRK_SUCCESS;
+}
+int32_t krk_host_malloc(void** hptr, size_t bytes) {
+  if (!hptr) return KRK_E_ARGUMENT;
+  KRK_TRY(ensure_runtime());
+  KRK_HIP(hipHostMalloc(hptr, bytes ? bytes : 1, hipHostMallocDefault));
+  return KRK_SUCCESS;
+}
+int32_t krk_host_free(void* hptr) {
+  if (!hptr) return KRK_SUCCESS;
+  KRK_HIP(hipHostFree(hptr));
   return KRK_SUCCESS;
 }
 int32_t krk_memcpy_h2d(void* dst, const void* src, size_t bytes) {

@@ -1,6 +1,6 @@
 """Per-kernel timings of the table engine at the sizes of the benchmark configurations.
 
-    python -m kraken_amd.microbench [copy] [tables] [raw] [combined] [pooled] [codec] [dense] [dct2] [copy]
+    python -m kraken_amd.microbench [copy] [tables] [raw] [combined] [host] [pooled] [codec] [dense] [dct2] [copy]
 
 Every figure is the average of back-to-back launches between two HIP events recorded on the
 stream the kernels run on, with inputs resident in HBM; bandwidths are algorithmic bytes
@@ -173,6 +173,39 @@ def combined():
         t.close()
 
 
+def host():
+    print("# the same step through host pointers (blocking calls, pageable numpy arrays): what a server")
+    print("# that receives its requests in host memory pays, copies over PCIe included")
+    import time
+    n_tables, space, dim = 26, 10**6, 16
+    init = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01"})
+    rng = np.random.default_rng(0)
+    tables = [api.SparseTable(dim, init, capacity_hint=space) for _ in range(n_tables)]
+    for t in tables:
+        prefill(t, space, dim)
+    grp = api.TableGroup(tables)
+    per = [np.unique(splitmix64(zipf_ranks(rng, 1.05, space, 8192))) for _ in range(n_tables)]
+    off = grp._offsets([p.size for p in per])
+    ids = np.concatenate(per)
+    grads = (rng.standard_normal((ids.size, dim)) * 1e-2).astype(np.float32)
+    out = np.empty((ids.size, dim), np.float32)
+    o = api.Optim.create(api.OptimType.kAdagrad)
+    p_ids, p_grads, p_out = api.pinned_copy(ids), api.pinned_copy(grads), api.pinned_empty(out.shape, np.float32)
+    for name, fn in (("combined pull, pageable", lambda: grp.CombinePull(ids, off, out=out)),
+                     ("combined push, pageable", lambda: grp.CombinePush(o, ids, off, grads, 0.01)),
+                     ("combined pull, page-locked", lambda: grp.CombinePull(p_ids, off, out=p_out)),
+                     ("combined push, page-locked", lambda: grp.CombinePush(o, p_ids, off, p_grads, 0.01))):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            fn()
+        dt = (time.perf_counter() - t0) / 20
+        print("%-28s %d unique rows  %8.1f us  %.2e rows/s" % (name, ids.size, dt * 1e6, ids.size / dt), flush=True)
+    grp.close()
+    for t in tables:
+        t.close()
+
+
 def pooled():
     print("# multi-hot field of the DeepFM shape: 65536 samples x 13 fields, 1..20 ids per bag, dim 32,")
     print("# table of 1e7 rows, Zipf 1.1")
@@ -261,7 +294,7 @@ def copy():
     print("# plain copy of 1 GiB: %.1f us, %.0f GB/s read + write" % (dt * 1e6, 2 * nbytes / dt / 1e9), flush=True)
 
 
-SECTIONS = {"copy": copy, "tables": tables, "raw": raw, "combined": combined, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct}
+SECTIONS = {"copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct}
 
 
 def main(argv):

@@ -130,3 +130,62 @@ def test_requests_beyond_one_launch_are_refused_up_front(api, oracle):
     assert L.krk_sparse_lookup(t.h, p(ids), 1 << 30, p(buf), 0) == api.E_CAPACITY
     assert L.krk_sparse_pull(t.h, p(ids), -1, p(buf), 0) == api.E_ARGUMENT
     assert len(t) == 0 and t.Pull(ids)[0] == 0        # the table is untouched and usable
+
+
+def test_page_locked_host_buffers_are_used_in_place(api, oracle):
+    """Host pointers into page-locked memory are handed to the kernels as they are (no staging
+    copy); pageable ones and misaligned ones are staged. All three must give the same table and the
+    same replies, for a single table, a group and a dense table."""
+    dim, n = 16, 5000
+    rng = np.random.default_rng(3)
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "2"})
+    ids = splitmix64(np.arange(n, dtype=np.uint64))
+    g = (rng.integers(-64, 65, size=(n, dim)) / 256.0).astype(np.float32)
+    o_ref, o_gpu = make_optims(oracle, api, 0, {})
+    r = oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=2))
+    _, want0 = r.pull(ids)
+    assert r.push(o_ref, ids, g, 0.05) == 0
+    _, want1 = r.pull(ids)
+
+    def run(ids_a, g_a, out_a):
+        t = api.SparseTable(dim, gi)
+        assert t.Pull(ids_a, out=out_a)[0] == 0
+        first = np.array(out_a)
+        assert t.Push(o_gpu, ids_a, g_a, 0.05) == 0
+        assert t.Pull(ids_a, out=out_a)[0] == 0
+        return first, np.array(out_a)
+
+    pageable = run(ids, g, np.empty((n, dim), np.float32))
+    locked = run(api.pinned_copy(ids), api.pinned_copy(g), api.pinned_empty((n, dim), np.float32))
+    # page-locked but off the 16-byte grid: staged like pageable memory
+    raw_i = api.pinned_empty(n + 1, np.uint64)
+    raw_g = api.pinned_empty(n * dim + 1, np.float32)
+    raw_o = api.pinned_empty(n * dim + 1, np.float32)
+    raw_i[1:] = ids
+    raw_g[1:] = g.ravel()
+    skewed = run(raw_i[1:], raw_g[1:].reshape(n, dim), raw_o[1:].reshape(n, dim))
+    for got in (pageable, locked, skewed):
+        assert_close(got[0], want0, "first pull", rtol=1e-6)
+        assert_close(got[1], want1, "after push")
+    assert np.array_equal(pageable[0], locked[0]) and np.array_equal(pageable[1], locked[1])
+    assert np.array_equal(pageable[1], skewed[1])
+
+    # a group and a dense table through page-locked buffers
+    a, b = api.SparseTable(dim, gi), api.SparseTable(dim, gi)
+    grp = api.TableGroup([a, b])
+    off = [0, n // 2, n]
+    p_ids, p_g, p_out = api.pinned_copy(ids), api.pinned_copy(g), api.pinned_empty((n, dim), np.float32)
+    assert grp.CombinePull(p_ids, off, out=p_out)[0] == 0
+    assert np.array_equal(np.array(p_out), pageable[0])
+    assert grp.CombinePush(o_gpu, p_ids, off, p_g, 0.05) == 0
+    assert grp.CombinePull(p_ids, off, out=p_out)[0] == 0
+    assert np.array_equal(np.array(p_out), pageable[1])
+    grp.close()
+    w0 = rng.standard_normal(1000).astype(np.float32)
+    d1, d2 = api.DenseTable(w0), api.DenseTable(api.pinned_copy(w0))
+    gd = rng.standard_normal(1000).astype(np.float32)
+    adam = api.Optim.create(api.OptimType.kAdam)
+    assert d1.Push(adam, gd, 0.01) == 0 and d2.Push(adam, api.pinned_copy(gd), 0.01) == 0
+    out2 = api.pinned_empty(1000, np.float32)
+    assert d2.Pull(out=out2)[0] == 0
+    assert np.array_equal(d1.Pull()[1], np.array(out2))
