@@ -1,14 +1,15 @@
 """Table files in the reference's checkpoint layout (checkpoint/checkpoint.cc:444-509, 535-649,
 common/serialize.h).
 
-PARITY UNPINNED for the byte layout: the reference's writer cannot be built here (its Tensor
-needs Eigen) and its tests hold no table file, so the layout is checked against a second,
-independent reading of common/serialize.h written with `struct` below. What IS pinned is the
-behaviour around the file: a table that goes through a file carries on exactly like the
-oracle table that never left memory.
+The byte layout is pinned by files that the reference's own serializer wrote (tests/golden/
+ref_*.sparse, ref_*.dense, made by oracle/ref_checkpoint.cc from the reference's serialize.h and
+tensor sources compiled in place): the library loads them, and what the library writes is read
+back by the reference's own deserializer where that binary is present. The `struct` reader in
+checkpoint_format.py is a second reading of common/serialize.h, pinned against the same files.
 """
 import os
 import struct
+import subprocess
 
 import numpy as np
 import pytest
@@ -25,80 +26,7 @@ def api():
     return a
 
 
-# --- an independent reader / writer of the layout (common/serialize.h) ---------------------
-
-class Cursor:
-    def __init__(self, data):
-        self.d, self.at = data, 0
-
-    def take(self, fmt):
-        v = struct.unpack_from("<" + fmt, self.d, self.at)
-        self.at += struct.calcsize("<" + fmt)
-        return v[0] if len(v) == 1 else v
-
-    def string(self):                      # serialize.h:86-94
-        n = self.take("Q")
-        s = self.d[self.at:self.at + n].decode()
-        self.at += n
-        return s
-
-    def tensor(self):                      # serialize.h:156-176
-        assert self.take("B") == 0         # Layout::kStride
-        rank = self.take("Q")
-        dims = [self.take("q") for _ in range(rank)]
-        assert self.take("B") == 11        # DType::kFloat32
-        n = int(np.prod(dims)) if dims else 1
-        v = np.frombuffer(self.d, np.float32, n, self.at).copy()
-        self.at += 4 * n
-        return dims, v
-
-    def value(self):                       # serialize.h:296-298, 242-272
-        dims, val = self.tensor()
-        states = {}
-        for _ in range(self.take("Q")):
-            st = self.take("I")
-            states[st] = self.tensor()[1]
-        counters = {}
-        for _ in range(self.take("Q")):
-            st = self.take("I")
-            counters[st] = self.take("q")
-        return dims, val, states, counters
-
-
-def parse_sparse(path):
-    c = Cursor(open(path, "rb").read())
-    head = dict(type=c.take("B"), id=c.take("Q"), name=c.string(), dim=c.take("q"), dtype=c.take("B"),
-                init=c.take("B"))
-    head["conf"] = {c.string(): c.string() for _ in range(c.take("Q"))}
-    slots = []
-    for _ in range(c.take("Q")):
-        rows = []
-        for _ in range(c.take("Q")):
-            key = c.take("Q")
-            rows.append((key,) + c.value())
-        slots.append(rows)
-    assert c.at == len(c.d)
-    return head, slots
-
-
-def pack_tensor(v, dims=None):
-    v = np.ascontiguousarray(v, np.float32)
-    dims = list(dims) if dims is not None else [v.size]
-    return struct.pack("<BQ", 0, len(dims)) + b"".join(struct.pack("<q", d) for d in dims) + b"\x0b" + v.tobytes()
-
-
-def pack_string(s):
-    return struct.pack("<Q", len(s)) + s.encode()
-
-
-def pack_value(val, states, counters, dims=None):
-    out = pack_tensor(val, dims) + struct.pack("<Q", len(states))
-    for st, v in states.items():
-        out += struct.pack("<I", st) + pack_tensor(v, dims)
-    out += struct.pack("<Q", len(counters))
-    for st, c in counters.items():
-        out += struct.pack("<Iq", st, c)
-    return out
+from checkpoint_format import Cursor, pack_string, pack_value, parse_sparse  # noqa: E402
 
 
 def _tables(api, oracle, dim, seed):
@@ -235,3 +163,133 @@ def test_dense_file_round_trip(api, oracle, tmp_path):
             assert t2.Push(o_gpu, g, 0.01) == 0 and ref.push(o_ref, g, 0.01) == 0
         assert_close(t2.Pull()[1], ref.pull(), name + " after the file")
     assert api.DenseTable.from_file(str(tmp_path / "none.dense"))[0] == api.E_IO
+
+
+# --- files written / read by the reference's own serializer -------------------------------------
+
+from test_checkpoint_format import GOLDEN, SPARSE, expected_rows, pattern  # noqa: E402
+
+REF_TOOL = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "oracle", "_ref", "ref_checkpoint")
+
+
+@pytest.mark.parametrize("name,dim,rows,states,steps", SPARSE)
+def test_loads_sparse_files_the_reference_wrote(api, name, dim, rows, states, steps):
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01"})
+    t = api.SparseTable(dim, gi)
+    rc, taken = t.load_file(os.path.join(GOLDEN, name + ".sparse"), 7, "emb")
+    assert rc == 0 and taken == rows == len(t)
+    want = expected_rows(dim, rows, states, steps)
+    keys = np.array(list(want), np.uint64)
+    for st in range(1, 8):
+        found, vals, state, got_steps = t.fetch(keys, state_type=st)
+        assert found.all()
+        for i, k in enumerate(want):
+            w_val, w_st, w_cnt = want[k]
+            assert np.array_equal(vals[i], w_val)
+            assert np.array_equal(state[i], w_st.get(st, np.zeros(dim, np.float32)))
+            # a row with states but no counter has been updated: it must not count as new
+            assert got_steps[i] == (w_cnt[0] if w_cnt else (1 if w_st else 0))
+
+
+@pytest.mark.parametrize("name,dim,rows,states,steps", SPARSE)
+def test_writes_what_the_reference_wrote(api, tmp_path, name, dim, rows, states, steps):
+    """The same table content saved by the library: identical bytes where the layout leaves no
+    freedom (at most one state), the same parsed content otherwise (the reference emits several
+    states in its hash map's order)."""
+    golden_path = os.path.join(GOLDEN, name + ".sparse")
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"mean": "0.0", "stddev": "0.01"})
+    t = api.SparseTable(dim, gi)
+    assert t.load_file(golden_path, 7, "emb")[0] == 0
+    path = str(tmp_path / "again.sparse")
+    assert t.save(path, 7, "emb") == 0
+    got, want = open(path, "rb").read(), open(golden_path, "rb").read()
+    if len(states) <= 1:
+        # the two conf entries may come in either order (an unordered_map on the reference's side)
+        assert len(got) == len(want)
+        a, b = parse_sparse(path), parse_sparse(golden_path)
+        assert a[0] == b[0]
+
+        def after_conf(data):
+            c = Cursor(data)
+            c.take("B"), c.take("Q"), c.string(), c.take("q"), c.take("B"), c.take("B")
+            for _ in range(c.take("Q")):
+                c.string(), c.string()
+            return data[c.at:]
+
+        assert got[:len(got) - len(after_conf(got))][:21] == want[:21]     # up to the conf map
+        assert after_conf(got) == after_conf(want)
+    a, b = parse_sparse(path), parse_sparse(golden_path)
+    assert a[0] == b[0]
+    for rows_a, rows_b in zip(a[1], b[1]):
+        assert len(rows_a) == len(rows_b)
+        for ra, rb in zip(rows_a, rows_b):
+            assert ra[0] == rb[0] and ra[1] == rb[1] and np.array_equal(ra[2], rb[2])
+            assert set(ra[3]) == set(rb[3]) and all(np.array_equal(ra[3][s], rb[3][s]) for s in ra[3])
+            assert ra[4] == rb[4]
+
+
+def test_dense_file_the_reference_wrote(api, tmp_path):
+    rc, t, tid, tname, shape = api.DenseTable.from_file(os.path.join(GOLDEN, "ref_adam.dense"))
+    assert rc == 0 and tid == 3 and tname == "dense0" and shape == [6, 4]
+    assert np.array_equal(t.Pull()[1], pattern(99, 0, 24))
+    assert np.array_equal(t.state(3), pattern(99, 4, 24)) and np.array_equal(t.state(4), pattern(99, 5, 24))
+    assert t.steps == 12
+    path = str(tmp_path / "again.dense")
+    assert t.save(path, 3, "dense0", shape=[6, 4]) == 0
+    from checkpoint_format import parse_dense
+    a, b = parse_dense(path), parse_dense(os.path.join(GOLDEN, "ref_adam.dense"))
+    assert a[0] == b[0] and a[1] == b[1] and np.array_equal(a[2], b[2]) and a[4] == b[4]
+    assert set(a[3]) == set(b[3]) and all(np.array_equal(a[3][s], b[3][s]) for s in a[3])
+
+
+@pytest.mark.skipif(not os.path.exists(REF_TOOL), reason="oracle/_ref/ref_checkpoint is built only where the "
+                    "reference tree is present")
+def test_reference_reader_reads_what_the_library_writes(api, oracle, tmp_path):
+    """A table trained on the GPU, saved by the library, parsed by the reference's own
+    Deserialize (oracle/ref_checkpoint.cc dump-sparse / dump-dense): every number it prints is
+    the oracle table's."""
+    dim = 8
+    t, ref = _tables(api, oracle, dim, seed=6)
+    ids = splitmix64(np.arange(300, dtype=np.uint64))
+    t.Pull(ids)
+    ref.pull(ids)
+    o_ref, o_gpu = make_optims(oracle, api, 1, {})
+    g = (np.random.default_rng(0).integers(-64, 65, size=(150, dim)) / 4096.0).astype(np.float32)
+    for _ in range(3):
+        assert t.Push(o_gpu, ids[:150], g, 0.01) == 0 and ref.push(o_ref, ids[:150], g, 0.01) == 0
+    path = str(tmp_path / "gpu.sparse")
+    assert t.save(path, 7, "emb") == 0
+    text = subprocess.run([REF_TOOL, "dump-sparse", path], check=True, capture_output=True, text=True).stdout
+    lines = text.splitlines()
+    assert lines[0] == "type 1 id 7 name emb dim 8 dtype 11 init 2 conf mean=0.000000 stddev=0.010000"
+    assert lines[1] == "slots 8"
+    rid, rval, _, rsteps = ref.export()
+    m = ref.export(state_type=3)[2]
+    v = ref.export(state_type=4)[2]
+    by_id = {int(k): i for i, k in enumerate(rid)}
+    seen = 0
+    for ln in lines[2:]:
+        if ln.startswith("slot "):
+            continue
+        parts = ln.split(" | ")
+        head = parts[0].split()
+        assert head[0] == "id" and head[2] == "val" and head[3] == "[8]"
+        i = by_id[int(head[1])]
+        assert_close(np.array(head[4:], np.float32), rval[i], "weights the reference read")
+        fields = {p.split()[0] + " " + p.split()[1]: p.split()[2:] for p in parts[1:]}
+        if rsteps[i] > 0:
+            assert_close(np.array(fields["state 3"][1:], np.float32), m[i], "first moment")
+            assert_close(np.array(fields["state 4"][1:], np.float32), v[i], "second moment")
+            assert int(fields["int 0"][0]) == rsteps[i] == 3
+        else:
+            assert not fields
+        seen += 1
+    assert seen == 300
+
+    d = api.DenseTable(np.arange(12, dtype=np.float32))
+    assert d.Push(o_gpu, np.ones(12, np.float32), 0.5) == 0
+    dpath = str(tmp_path / "gpu.dense")
+    assert d.save(dpath, 3, "dense0", shape=[3, 4]) == 0
+    dl = subprocess.run([REF_TOOL, "dump-dense", dpath], check=True, capture_output=True, text=True).stdout.splitlines()
+    assert dl[0] == "type 0 id 3 name dense0"
+    assert dl[1].startswith("val [3x4] ") and " | state 3 [3x4] " in dl[1] and dl[1].endswith(" | int 0 1")
