@@ -212,6 +212,24 @@ int32_t krk_sparse_pull_pooled(krk_sparse* t, const uint64_t* ids, int64_t n, co
 int32_t krk_sparse_push_pooled(krk_sparse* t, const krk_optim* o, const uint64_t* ids, int64_t n,
                                const int64_t* offsets, int64_t bags, const float* weights, int32_t mode,
                                const float* bag_grads, int64_t grad_dim, float lr, uint32_t flags);
+/* The reply and the gradients of a sparse request in the reference's wire layout, so that a
+ * server can hand its send and receive buffers over as they are: std::vector<Tensor> as
+ * Serialize writes it (common/serialize.h:156-176, 214-228) = u64 count, then per row 18 header
+ * bytes {u8 layout 0, u64 rank 1, i64 dim, u8 dtype 11} and dim floats. This is the body of a
+ * PullSparseTableResponse (protocol/pull_sparse_table_prot.h:29-41) and the `grads` member of a
+ * PushSparseTableRequest (protocol/push_sparse_table_prot.h:11-30). Host buffers, 8-byte
+ * aligned, blocking; page-locked buffers are read and written in place.
+ *   krk_wire_rows_bytes   size of such a block for n rows
+ *   krk_sparse_pull_wire  krk_sparse_pull whose reply is that block (reply holds
+ *                         krk_wire_rows_bytes(n, dim) bytes)
+ *   krk_sparse_push_wire  krk_sparse_push whose gradients are that block; a count other than n, a
+ *                         header that is not a dense fp32 vector of the table's width or a short
+ *                         buffer returns 11 before any row is touched (the reference fails at
+ *                         the offending row, after updating those before it). */
+int64_t krk_wire_rows_bytes(int64_t n, int64_t dim);
+int32_t krk_sparse_pull_wire(krk_sparse* t, const uint64_t* ids, int64_t n, void* reply);
+int32_t krk_sparse_push_wire(krk_sparse* t, const krk_optim* o, const uint64_t* ids, int64_t n,
+                             const void* grads_wire, int64_t wire_bytes, float lr);
 /* id -> row lookup alone (ParallelSkipList::HitSlot + SkipList::Find,
  * common/parallel_skip_list.h:100-102, common/skip_list.h:315-324):
  * rows[i] = dense row index of ids[i], or -1 when absent. Row indices are

@@ -68,6 +68,10 @@ EXPORTS = {
     "krk_memset": (C.c_int32, [C.c_void_p, C.c_int, C.c_size_t]),
     "krk_device_synchronize": (C.c_int32, []),
     "krk_mem_info": (C.c_int32, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "krk_wire_rows_bytes": (C.c_int64, [C.c_int64, C.c_int64]),
+    "krk_sparse_pull_wire": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
+    "krk_sparse_push_wire": (C.c_int32, [C.c_void_p, C.POINTER(krk_optim), C.c_void_p, C.c_int64, C.c_void_p,
+                                         C.c_int64, C.c_float]),
     "krk_host_malloc": (C.c_int32, [C.POINTER(C.c_void_p), C.c_size_t]),
     "krk_host_free": (C.c_int32, [C.c_void_p]),
     "krk_stream_copy": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_size_t]),
@@ -413,6 +417,21 @@ class SparseTable:
         return lib().krk_sparse_push_pooled(self.h, C.byref(optim.raw), _ptr(ids), ids.size, _ptr(offsets),
                                             bags, _ptr(weights), self._POOL[mode], _ptr(bag_grads), gd, lr,
                                             _flags(ids, bag_grads, extra=ASYNC if async_ else 0))
+
+    def PullWire(self, sparse_ids, reply=None):
+        """Pull whose reply is the body of the reference's PullSparseTableResponse: -> (code, bytes)"""
+        sparse_ids = np.ascontiguousarray(sparse_ids, dtype=np.uint64)
+        nbytes = lib().krk_wire_rows_bytes(sparse_ids.size, self.dimension)
+        if reply is None:
+            reply = np.empty(nbytes // 8 + 1, np.uint64).view(np.uint8)[:nbytes]
+        rc = lib().krk_sparse_pull_wire(self.h, _ptr(sparse_ids), sparse_ids.size, _ptr(reply))
+        return rc, reply
+
+    def PushWire(self, optim, sparse_ids, grads_wire, lr):
+        """Push whose gradients are the `grads` member of the reference's PushSparseTableRequest."""
+        sparse_ids = np.ascontiguousarray(sparse_ids, dtype=np.uint64)
+        return lib().krk_sparse_push_wire(self.h, C.byref(optim.raw), _ptr(sparse_ids), sparse_ids.size,
+                                          _ptr(grads_wire), grads_wire.size, lr)
 
     def lookup(self, ids):
         if isinstance(ids, DeviceArray):

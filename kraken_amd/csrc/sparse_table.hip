@@ -661,6 +661,57 @@ __global__ __launch_bounds__(kBlock) void restride_kernel(const float* __restric
 }
 
 // ---------------------------------------------------------------------------
+// Rows in the reference's wire layout (std::vector<Tensor> as Serialize writes it,
+// common/serialize.h:156-176, 214-228): u64 count, then per row 18 header bytes {u8 layout 0,
+// u64 rank 1, i64 dim, u8 dtype 11} and dim floats. A row starts on an even offset that is not
+// always a multiple of four, so both directions move 16-bit halves.
+// ---------------------------------------------------------------------------
+constexpr int kWireHeader = 18;
+
+__device__ __forceinline__ uint32_t wire_header_byte(int b, int dim) {
+  if (b == 1) return 1u;                                   // rank, low byte
+  if (b >= 9 && b <= 16) return ((uint64_t)dim >> (8 * (b - 9))) & 0xFFu;
+  if (b == 17) return 11u;                                 // DType::kFloat32
+  return 0u;                                               // layout kStride, upper bytes
+}
+
+__global__ __launch_bounds__(kBlock) void rows_to_wire_kernel(const float* __restrict__ rows, int64_t n,
+                                                              int dim, uint16_t* __restrict__ wire) {
+  const int per_row = kWireHeader / 2 + 2 * dim;           // 16-bit halves per row
+  const int64_t total = 4 + n * per_row;
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t h = (int64_t)blockIdx.x * kBlock + threadIdx.x; h < total; h += step) {
+    uint32_t v;
+    if (h < 4) {
+      v = (uint32_t)(((uint64_t)n >> (16 * h)) & 0xFFFFu);
+    } else {
+      const int64_t r = (h - 4) / per_row;
+      const int k = (int)((h - 4) - r * per_row);
+      if (k < kWireHeader / 2) {
+        v = wire_header_byte(2 * k, dim) | (wire_header_byte(2 * k + 1, dim) << 8);
+      } else {
+        const uint32_t bits = __float_as_uint(rows[r * dim + (k - kWireHeader / 2) / 2]);
+        v = ((k - kWireHeader / 2) & 1) ? bits >> 16 : bits & 0xFFFFu;
+      }
+    }
+    wire[h] = (uint16_t)v;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void wire_to_rows_kernel(const uint16_t* __restrict__ wire, int64_t n,
+                                                              int dim, float* __restrict__ rows) {
+  const int per_row = kWireHeader / 2 + 2 * dim;
+  const int64_t total = n * dim;
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += step) {
+    const int64_t r = i / dim;
+    const int f = (int)(i - r * dim);
+    const uint16_t* p = wire + 4 + r * per_row + kWireHeader / 2 + 2 * f;
+    rows[i] = __uint_as_float((uint32_t)p[0] | ((uint32_t)p[1] << 16));
+  }
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 static inline unsigned grid_for(int64_t items, int per_block) {
@@ -1118,26 +1169,9 @@ int32_t krk_sparse_sync(krk_sparse* t) {
   return sparse_finish(t, 0);
 }
 
-int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* out, uint32_t flags) {
-  KRK_TRY(check_table(t));
-  KRK_TRY(check_flags(flags));
-  if (n < 0 || (n > 0 && (!ids || !out))) return KRK_E_ARGUMENT;
-  if ((flags & KRK_DEVICE_PTRS) && t->vec == 4 && !aligned16(out)) {
-    set_error("device output must be 16-byte aligned");
-    return KRK_E_ARGUMENT;
-  }
-  if (n > max_ids_per_launch(t->group)) {
-    set_error("at most %lld ids per call for this row width; split the request",
-              (long long)max_ids_per_launch(t->group));
-    return KRK_E_CAPACITY;
-  }
-  std::lock_guard<std::mutex> lk(t->mu);
-  if (n == 0) return sparse_finish(t, flags);
-  KRK_TRY(sparse_ensure_room(t, n));
-  const uint64_t* d_ids;
-  float* d_out;
-  KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
-  KRK_TRY(t->output(out, (size_t)n * t->dim, flags, 1, &d_out));
+// The launches of one pull of n > 0 ids into d_out [n, dim]; the caller holds the table's lock
+// and has made room for n more rows.
+static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, float* d_out) {
   KRK_TRY(sparse_next_epoch(t, n));
   const int per_block = kBlock / t->group;
   const dim3 grid(grid_for(n, per_block)), block(kBlock);
@@ -1166,6 +1200,30 @@ int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* ou
                        (int)t->dim, t->elems, t->group);
   }
   KRK_HIP(hipGetLastError());
+  return KRK_SUCCESS;
+}
+
+int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* out, uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (n < 0 || (n > 0 && (!ids || !out))) return KRK_E_ARGUMENT;
+  if ((flags & KRK_DEVICE_PTRS) && t->vec == 4 && !aligned16(out)) {
+    set_error("device output must be 16-byte aligned");
+    return KRK_E_ARGUMENT;
+  }
+  if (n > max_ids_per_launch(t->group)) {
+    set_error("at most %lld ids per call for this row width; split the request",
+              (long long)max_ids_per_launch(t->group));
+    return KRK_E_CAPACITY;
+  }
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (n == 0) return sparse_finish(t, flags);
+  KRK_TRY(sparse_ensure_room(t, n));
+  const uint64_t* d_ids;
+  float* d_out;
+  KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
+  KRK_TRY(t->output(out, (size_t)n * t->dim, flags, 1, &d_out));
+  KRK_TRY(pull_enqueue(t, d_ids, n, d_out));
   if ((flags & KRK_ASYNC) && sparse_near_full(t)) KRK_TRY(sparse_publish(&t, 1, t->stream));
   KRK_TRY(t->output_back(out, (size_t)n * t->dim, flags, 1));
   return sparse_finish(t, flags);
@@ -1269,6 +1327,95 @@ int32_t krk_sparse_push(krk_sparse* t, const krk_optim* o, const uint64_t* ids, 
   }
   KRK_HIP(hipGetLastError());
   return sparse_finish(t, flags);
+}
+
+int64_t krk_wire_rows_bytes(int64_t n, int64_t dim) {
+  if (n < 0 || dim <= 0) return -1;
+  return 8 + n * (kWireHeader + 4 * dim);
+}
+
+int32_t krk_sparse_pull_wire(krk_sparse* t, const uint64_t* ids, int64_t n, void* reply) {
+  KRK_TRY(check_table(t));
+  if (n < 0 || !reply || (n > 0 && !ids) || ((uintptr_t)reply & 7)) {
+    set_error("krk_sparse_pull_wire: reply must be an 8-byte aligned host buffer");
+    return KRK_E_ARGUMENT;
+  }
+  if (n > max_ids_per_launch(t->group)) {
+    set_error("at most %lld ids per call for this row width; split the request",
+              (long long)max_ids_per_launch(t->group));
+    return KRK_E_CAPACITY;
+  }
+  std::lock_guard<std::mutex> lk(t->mu);
+  const size_t bytes = (size_t)krk_wire_rows_bytes(n, t->dim);
+  uint8_t* d_reply;
+  KRK_TRY(t->output(reinterpret_cast<uint8_t*>(reply), bytes, 0, 1, &d_reply));
+  float* d_rows = nullptr;
+  if (n > 0) {
+    KRK_TRY(sparse_ensure_room(t, n));
+    const uint64_t* d_ids;
+    KRK_TRY(t->input(ids, (size_t)n, 0, 0, &d_ids));
+    KRK_TRY(t->stage[2].reserve((size_t)n * t->dim * sizeof(float) + 16));
+    d_rows = t->stage[2].as<float>();
+    KRK_TRY(pull_enqueue(t, d_ids, n, d_rows));
+  }
+  hipLaunchKernelGGL(rows_to_wire_kernel, dim3(strided_grid((int64_t)(bytes / 2))), dim3(kBlock), 0, t->stream,
+                     d_rows, n, (int)t->dim, reinterpret_cast<uint16_t*>(d_reply));
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(t->output_back(reinterpret_cast<uint8_t*>(reply), bytes, 0, 1));
+  return sparse_finish(t, 0);
+}
+
+int32_t krk_sparse_push_wire(krk_sparse* t, const krk_optim* o, const uint64_t* ids, int64_t n,
+                             const void* grads_wire, int64_t wire_bytes, float lr) {
+  KRK_TRY(check_table(t));
+  if (!valid_optim(o)) {
+    set_error("optimizer type is not supported");
+    return KRK_UNSUPPORTED_OPTIM;
+  }
+  if (n < 0 || !grads_wire || (n > 0 && !ids) || ((uintptr_t)grads_wire & 7)) {
+    set_error("krk_sparse_push_wire: grads_wire must be an 8-byte aligned host buffer");
+    return KRK_E_ARGUMENT;
+  }
+  if (n > max_ids_per_launch(t->group)) {
+    set_error("at most %lld ids per call for this row width; split the request",
+              (long long)max_ids_per_launch(t->group));
+    return KRK_E_CAPACITY;
+  }
+  // The request is checked before anything is applied: as many gradients as ids, each a dense
+  // fp32 vector of the table's width (ps/optim/adagrad.cc:29-32 and its siblings return 11).
+  const uint8_t* w = reinterpret_cast<const uint8_t*>(grads_wire);
+  uint64_t count = 0;
+  if (wire_bytes >= 8) memcpy(&count, w, 8);
+  uint8_t want[kWireHeader] = {0};
+  want[1] = 1;
+  const uint64_t d64 = (uint64_t)t->dim;
+  memcpy(want + 9, &d64, 8);
+  want[17] = 11;
+  const int64_t row_bytes = kWireHeader + 4 * t->dim;
+  bool ok = wire_bytes >= 8 && count == (uint64_t)n && wire_bytes >= 8 + n * row_bytes;
+  for (int64_t r = 0; ok && r < n; ++r) ok = memcmp(w + 8 + r * row_bytes, want, kWireHeader) == 0;
+  if (!ok) {
+    set_error("gradients do not match the ids or the table dimension %lld", (long long)t->dim);
+    return KRK_GRADIENT_UNCOMPATIBLE;
+  }
+  std::lock_guard<std::mutex> lk(t->mu);
+  if (n == 0) return sparse_finish(t, 0);
+  KRK_TRY(sparse_ensure_columns(t, optim_state_mask(*o)));
+  const uint64_t* d_ids;
+  const uint8_t* d_wire;
+  KRK_TRY(t->input(ids, (size_t)n, 0, 0, &d_ids));
+  KRK_TRY(t->input(w, (size_t)(8 + n * row_bytes), 0, 1, &d_wire));
+  KRK_TRY(t->stage[2].reserve((size_t)n * t->dim * sizeof(float) + 16));
+  float* d_rows = t->stage[2].as<float>();
+  hipLaunchKernelGGL(wire_to_rows_kernel, dim3(strided_grid(n * t->dim)), dim3(kBlock), 0, t->stream,
+                     reinterpret_cast<const uint16_t*>(d_wire), n, (int)t->dim, d_rows);
+  if (t->vec == 4) {
+    launch_push<4>(t, *o, d_ids, n, d_rows, lr);
+  } else {
+    launch_push<1>(t, *o, d_ids, n, d_rows, lr);
+  }
+  KRK_HIP(hipGetLastError());
+  return sparse_finish(t, 0);
 }
 
 int32_t krk_sparse_lookup(krk_sparse* t, const uint64_t* ids, int64_t n, int32_t* rows,

@@ -201,6 +201,25 @@ def host():
             fn()
         dt = (time.perf_counter() - t0) / 20
         print("%-28s %d unique rows  %8.1f us  %.2e rows/s" % (name, ids.size, dt * 1e6, ids.size / dt), flush=True)
+    # one table's request of 8192 ids, as arrays and in the reference's wire layout
+    t = tables[0]
+    one = per[0]
+    g1 = grads[:one.size]
+    rc, reply = t.PullWire(one)
+    p_reply = api.pinned_empty(reply.size, np.uint8)
+    p_one = api.pinned_copy(one)
+    for name, fn in (("pull [n, dim], pageable", lambda: t.Pull(one)),
+                     ("pull, wire layout, pageable", lambda: t.PullWire(one, reply=reply)),
+                     ("pull, wire layout, page-locked", lambda: t.PullWire(p_one, reply=p_reply)),
+                     ("push [n, dim], pageable", lambda: t.Push(o, one, g1, 0.01)),
+                     ("push, wire layout, pageable", lambda: t.PushWire(o, one, reply, 1e-6)),
+                     ("push, wire layout, page-locked", lambda: t.PushWire(o, p_one, p_reply, 1e-6))):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(50):
+            fn()
+        dt = (time.perf_counter() - t0) / 50
+        print("%-32s %d rows  %8.1f us" % (name, one.size, dt * 1e6), flush=True)
     grp.close()
     for t in tables:
         t.close()

@@ -16,6 +16,8 @@
 //   ref_checkpoint write-dense  <path> <size>
 //   ref_checkpoint dump-sparse  <path>      -> text, one row per line
 //   ref_checkpoint dump-dense   <path>
+//   ref_checkpoint write-rows   <path> <n> <dim>   -> std::vector<Tensor> as an RPC body carries it
+//   ref_checkpoint dump-rows    <path>
 //
 // Row r of a written table: id = splitmix64(r); val[j] = pattern(id, 0, j); state s:
 // pattern(id, s + 1, j); steps = 1 + id % 7. pattern is exact in fp32 (multiples of 1/64).
@@ -217,12 +219,40 @@ static int dump_dense(const char* path) {
   return 0;
 }
 
+// The body of a PullSparseTableResponse / the grads member of a PushSparseTableRequest
+// (protocol/pull_sparse_table_prot.h:29-41, push_sparse_table_prot.h:11-30): row r is
+// pattern(splitmix64(r), 0, j).
+static int write_rows(const char* path, int64_t n, int64_t dim) {
+  std::vector<Tensor> vals;
+  for (int64_t r = 0; r < n; ++r) vals.emplace_back(filled(splitmix64((uint64_t)r), 0, dim));
+  io::FileWriter writer(path);
+  if (!writer.IsOpen()) return 2;
+  Serialize serialize(&writer);
+  return (serialize << vals) ? 0 : 3;
+}
+
+static int dump_rows(const char* path) {
+  io::FileReader reader(path);
+  if (!reader.IsOpen()) return 2;
+  Deserialize deserialize(&reader);
+  std::vector<Tensor> vals;
+  if (!(deserialize >> vals)) return 3;
+  printf("rows %zu\n", vals.size());
+  for (const Tensor& t : vals) {
+    print_tensor(t);
+    printf("\n");
+  }
+  return 0;
+}
+
 int main(int argc, char** argv) {
   if (argc >= 7 && !strcmp(argv[1], "write-sparse"))
     return write_sparse(argv[2], atoll(argv[3]), atoll(argv[4]), argv[5], atoi(argv[6]));
   if (argc >= 4 && !strcmp(argv[1], "write-dense")) return write_dense(argv[2], atoll(argv[3]));
   if (argc >= 3 && !strcmp(argv[1], "dump-sparse")) return dump_sparse(argv[2]);
   if (argc >= 3 && !strcmp(argv[1], "dump-dense")) return dump_dense(argv[2]);
+  if (argc >= 5 && !strcmp(argv[1], "write-rows")) return write_rows(argv[2], atoll(argv[3]), atoll(argv[4]));
+  if (argc >= 3 && !strcmp(argv[1], "dump-rows")) return dump_rows(argv[2]);
   fprintf(stderr, "usage: see the head of oracle/ref_checkpoint.cc\n");
   return 1;
 }

@@ -87,3 +87,21 @@ def parse_dense(path):
     dims, val, states, counters = c.value()
     assert c.at == len(c.d)
     return head, dims, val, states, counters
+
+
+def pack_rows(rows):
+    """std::vector<Tensor> of 1-D fp32 rows (serialize.h:214-228): what a pull reply carries."""
+    rows = np.ascontiguousarray(rows, np.float32)
+    return struct.pack("<Q", rows.shape[0]) + b"".join(pack_tensor(r) for r in rows)
+
+
+def parse_rows(data):
+    c = Cursor(bytes(data))
+    out = []
+    for _ in range(c.take("Q")):
+        dims, v = c.tensor()
+        assert len(dims) == 1
+        out.append(v)
+    assert c.at == len(c.d)
+    return np.array(out, np.float32).reshape(len(out), -1)
+

@@ -1,4 +1,4 @@
-"""Writes tests/golden/ref_*.sparse / ref_*.dense with the reference's own serializer
+"""Writes tests/golden/ref_*.sparse / ref_*.dense / ref_rows_*.wire with the reference's own serializer
 (oracle/_ref/ref_checkpoint, built by `make -C oracle ref` from the reference's sources where they
 lie). Runs only where the reference tree is present; the files are committed as fixtures.
 
@@ -26,6 +26,9 @@ def main():
         subprocess.check_call([TOOL, "write-sparse", os.path.join(HERE, name + ".sparse"), str(dim), str(rows),
                                states, str(steps)])
     subprocess.check_call([TOOL, "write-dense", os.path.join(HERE, "ref_adam.dense"), "24"])
+    # std::vector<Tensor> as a pull reply / a push request carries it: 33 rows of 5 and of 16 floats
+    subprocess.check_call([TOOL, "write-rows", os.path.join(HERE, "ref_rows_d5.wire"), "33", "5"])
+    subprocess.check_call([TOOL, "write-rows", os.path.join(HERE, "ref_rows_d16.wire"), "33", "16"])
 
 
 if __name__ == "__main__":

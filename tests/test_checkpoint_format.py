@@ -10,7 +10,7 @@ import struct
 import numpy as np
 import pytest
 
-from checkpoint_format import pack_string, pack_value, parse_dense, parse_sparse
+from checkpoint_format import pack_rows, pack_string, pack_value, parse_dense, parse_rows, parse_sparse
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 M64 = (1 << 64) - 1
@@ -91,3 +91,14 @@ def test_dense_file_the_reference_wrote():
     assert set(states) == {3, 4}
     assert np.array_equal(states[3], pattern(99, 4, 24)) and np.array_equal(states[4], pattern(99, 5, 24))
     assert counters == {0: 12}
+
+
+@pytest.mark.parametrize("dim", [5, 16])
+def test_row_blocks_the_reference_wrote(dim):
+    """The body of a pull reply / the gradients of a push request: std::vector<Tensor>."""
+    golden = open(os.path.join(GOLDEN, "ref_rows_d%d.wire" % dim), "rb").read()
+    want = np.array([pattern(mix(r), 0, dim) for r in range(33)])
+    assert len(golden) == 8 + 33 * (18 + 4 * dim)
+    assert np.array_equal(parse_rows(golden), want)
+    assert pack_rows(want) == golden
+

@@ -293,3 +293,68 @@ def test_reference_reader_reads_what_the_library_writes(api, oracle, tmp_path):
     dl = subprocess.run([REF_TOOL, "dump-dense", dpath], check=True, capture_output=True, text=True).stdout.splitlines()
     assert dl[0] == "type 0 id 3 name dense0"
     assert dl[1].startswith("val [3x4] ") and " | state 3 [3x4] " in dl[1] and dl[1].endswith(" | int 0 1")
+
+
+# --- requests and replies in the reference's wire layout -----------------------------------------
+
+from checkpoint_format import pack_rows, parse_rows  # noqa: E402
+
+
+@pytest.mark.parametrize("dim", [5, 16])
+def test_pull_and_push_in_wire_layout(api, oracle, tmp_path, dim):
+    """krk_sparse_pull_wire writes what the reference's Serialize writes for the pulled rows
+    (checked byte for byte against a block the reference wrote, and read back by its Deserialize
+    where that binary is present); krk_sparse_push_wire applies a block the reference wrote."""
+    from test_checkpoint_format import mix
+    golden = np.frombuffer(open(os.path.join(GOLDEN, "ref_rows_d%d.wire" % dim), "rb").read(), np.uint8)
+    rows = parse_rows(golden)
+    n = rows.shape[0]
+    ids = np.array([mix(r) for r in range(n)], np.uint64)
+    gi = api.Initializer.create(api.InitializerType.kConstant, {"value": "0"})
+    t = api.SparseTable(dim, gi)
+    r = oracle.SparseTable(dim, oracle.init(oracle.INIT_CONSTANT, 0.0))
+    t.Pull(ids)
+    r.pull(ids)
+    # SGD with lr -1 on zero rows: the rows become the gradients the reference serialized
+    o_ref, o_gpu = make_optims(oracle, api, 3, {})
+    wire = np.empty(golden.size // 8 + 1, np.uint64).view(np.uint8)[:golden.size]
+    wire[:] = golden
+    assert t.PushWire(o_gpu, ids, wire, -1.0) == 0
+    assert r.push(o_ref, ids, rows, -1.0) == 0
+    assert np.array_equal(t.Pull(ids)[1], rows) and np.array_equal(r.pull(ids)[1], rows)
+    rc, reply = t.PullWire(ids)
+    assert rc == 0 and reply.tobytes() == golden.tobytes()
+    # page-locked buffers take the in-place path
+    p_reply = api.pinned_empty(golden.size, np.uint8)
+    assert t.PullWire(ids, reply=p_reply)[0] == 0 and np.array_equal(np.array(p_reply), golden)
+    p_wire = api.pinned_copy(golden)
+    assert t.PushWire(o_gpu, ids, p_wire, -1.0) == 0
+    assert np.array_equal(t.Pull(ids)[1], 2 * rows)
+    # a reply for ids in another order, with a new id, equals the struct writer's bytes
+    mixed = np.concatenate([ids[::-1][:7], np.array([12345], np.uint64)])
+    rc, reply = t.PullWire(mixed)
+    assert rc == 0 and reply.tobytes() == pack_rows(t.Pull(mixed)[1])
+    if os.path.exists(REF_TOOL):
+        path = str(tmp_path / "reply.wire")
+        open(path, "wb").write(reply.tobytes())
+        text = subprocess.run([REF_TOOL, "dump-rows", path], check=True, capture_output=True, text=True).stdout
+        lines = text.splitlines()
+        assert lines[0] == "rows 8"
+        got = np.array([ln.split()[1:] for ln in lines[1:]], np.float32)
+        assert np.array_equal(got, t.Pull(mixed)[1])
+    # malformed requests are refused whole: wrong count, wrong width, short buffer, a COO row
+    before = t.Pull(ids)[1]
+    bad = wire.copy()
+    bad[0] = n - 1
+    assert t.PushWire(o_gpu, ids, bad, 1.0) == 11
+    bad = wire.copy()
+    bad[8 + 9] = dim + 1
+    assert t.PushWire(o_gpu, ids, bad, 1.0) == 11
+    assert t.PushWire(o_gpu, ids, wire[:-4], 1.0) == 11
+    bad = wire.copy()
+    bad[8 + 3 * (18 + 4 * dim)] = 1
+    assert t.PushWire(o_gpu, ids, bad, 1.0) == 11
+    assert np.array_equal(t.Pull(ids)[1], before)
+    assert t.PushWire(o_gpu, ids[:0], np.zeros(8, np.uint8), 1.0) == 0
+    rc, empty = t.PullWire(ids[:0])
+    assert rc == 0 and empty.tobytes() == struct.pack("<Q", 0)
