@@ -7,10 +7,11 @@
 // (stable, so equal rows keep position order), then a tiled segmented reduction walks the
 // sorted sequence: every group of lanes owns a fixed-size tile, sums each run of equal rows in
 // registers and, when a run lies wholly inside the tile, applies the optimizer to that row at
-// once. Runs that touch a tile border leave a partial sum in a carry list, which is itself a
-// sorted sequence of (row, partial) and is reduced by the same kernel again until one tile is
-// left. Work per group is bounded by the tile size however skewed the ids are, and the order
-// of additions is fixed, so results do not change from run to run.
+// once. Runs that touch a tile border meet the other tiles' pieces in the workgroup's LDS; only
+// a run that crosses the workgroup's own border leaves a partial sum in a carry list, which is
+// itself a sorted sequence of (row, partial) and is reduced by the same kernel again until one
+// workgroup is left. Work per group is bounded by the tile size however skewed the ids are, and
+// the order of additions is fixed, so results do not change from run to run.
 #include <cstring>
 #include <new>
 
