@@ -27,6 +27,7 @@ struct ErrorCode {
   static constexpr int32_t kGradientUnCompatibleError = KRK_GRADIENT_UNCOMPATIBLE;
   static constexpr int32_t kSparseIdNotExistError = KRK_SPARSE_ID_NOT_EXIST;
   static constexpr int32_t kUnSupportInitializerTypeError = KRK_UNSUPPORTED_INITIALIZER;
+  static constexpr int32_t kTableNotExistError = 21;   // a combined request names a table outside the group
   static const char* Msg(int32_t code) { return krk_error_message(code); }
 };
 
@@ -203,6 +204,99 @@ class SparseTable : public Table {
   int64_t dimension_;
   std::unique_ptr<Initializer> initializer_;
   krk_sparse* h_ = nullptr;
+  int32_t create_code_ = 0;
+};
+
+// protocol/combine_push_sparse_table_prot.h:12-15
+struct CombinePushSparseTableItem {
+  std::vector<uint64_t> sparse_ids;
+  std::vector<Tensor> grads;
+};
+
+// The sparse tables of equal dimension that combined requests address together. CombinePull /
+// CombinePush have the signatures of Ps::CombinePullSparseTable / CombinePushSparseTable
+// (ps/ps_op.cc:370-387, 456-469) without the router version; where the reference loops over the
+// tables of the request, here one launch serves them all. Tables outside the request take part
+// with zero ids. Destroy the group before its tables.
+class SparseTableGroup {
+ public:
+  explicit SparseTableGroup(const std::vector<SparseTable*>& tables) : tables_(tables) {
+    std::vector<krk_sparse*> hs;
+    for (SparseTable* t : tables_) hs.push_back(t ? t->handle() : nullptr);
+    create_code_ = krk_group_create(hs.data(), (int32_t)hs.size(), &h_);
+    dimension_ = tables_.empty() || !tables_[0] ? 0 : tables_[0]->dimension();
+  }
+  ~SparseTableGroup() { krk_group_destroy(h_); }
+  SparseTableGroup(const SparseTableGroup&) = delete;
+  SparseTableGroup& operator=(const SparseTableGroup&) = delete;
+
+  int32_t create_code() const { return create_code_; }
+  krk_group* handle() const { return h_; }
+
+  int32_t CombinePull(const std::unordered_map<uint64_t, std::vector<uint64_t>>& table_sparse_ids,
+                      std::unordered_map<uint64_t, std::vector<Tensor>>* table_vals) {
+    if (!h_) return create_code_;
+    std::vector<uint64_t> ids;
+    std::vector<int64_t> offsets(tables_.size() + 1, 0);
+    size_t found = 0;
+    for (size_t m = 0; m < tables_.size(); ++m) {
+      auto it = table_sparse_ids.find(tables_[m]->id());
+      if (it != table_sparse_ids.end()) {
+        ids.insert(ids.end(), it->second.begin(), it->second.end());
+        ++found;
+      }
+      offsets[m + 1] = (int64_t)ids.size();
+    }
+    if (found != table_sparse_ids.size()) return ErrorCode::kTableNotExistError;   // ps_op.cc:348-351
+    std::vector<float> flat(ids.size() * (size_t)dimension_);
+    const int32_t rc = krk_group_pull(h_, ids.data(), offsets.data(), flat.data(), 0);
+    if (rc != ErrorCode::kSuccess) return rc;
+    for (size_t m = 0; m < tables_.size(); ++m) {
+      if (!table_sparse_ids.count(tables_[m]->id())) continue;
+      std::vector<Tensor> vals;
+      for (int64_t i = offsets[m]; i < offsets[m + 1]; ++i)
+        vals.push_back(Tensor::From(flat.data() + i * dimension_, dimension_));
+      table_vals->emplace(tables_[m]->id(), std::move(vals));
+    }
+    return ErrorCode::kSuccess;
+  }
+
+  // unique_ids = true: the request as Emitter::CombinePushSparseTable sends it (ids already
+  // deduplicated per table). false: ids may repeat within a table and their gradients are summed
+  // on the device (worker/emitter.cc:552-606 moved to the server).
+  int32_t CombinePush(Optim* optim, const std::unordered_map<uint64_t, CombinePushSparseTableItem>& table_items,
+                      float lr, bool unique_ids = true) {
+    if (!h_) return create_code_;
+    if (!optim) return ErrorCode::kUnSupportOptimTypeError;
+    std::vector<uint64_t> ids;
+    std::vector<float> flat;
+    std::vector<int64_t> offsets(tables_.size() + 1, 0);
+    size_t found = 0;
+    for (size_t m = 0; m < tables_.size(); ++m) {
+      auto it = table_items.find(tables_[m]->id());
+      if (it != table_items.end()) {
+        const CombinePushSparseTableItem& item = it->second;
+        if (item.grads.size() != item.sparse_ids.size()) return ErrorCode::kGradientUnCompatibleError;
+        for (size_t i = 0; i < item.sparse_ids.size(); ++i) {
+          const Tensor& g = item.grads[i];
+          if (g.IsCoo() || g.Size() != dimension_) return ErrorCode::kGradientUnCompatibleError;
+          ids.push_back(item.sparse_ids[i]);
+          flat.insert(flat.end(), g.Data(), g.Data() + dimension_);
+        }
+        ++found;
+      }
+      offsets[m + 1] = (int64_t)ids.size();
+    }
+    if (found != table_items.size()) return ErrorCode::kTableNotExistError;
+    return unique_ids ? krk_group_push(h_, optim->raw(), ids.data(), offsets.data(), flat.data(), dimension_, lr, 0)
+                      : krk_group_push_raw(h_, optim->raw(), ids.data(), offsets.data(), flat.data(), dimension_,
+                                           lr, 0);
+  }
+
+ private:
+  std::vector<SparseTable*> tables_;
+  int64_t dimension_ = 0;
+  krk_group* h_ = nullptr;
   int32_t create_code_ = 0;
 };
 

@@ -135,6 +135,52 @@ int main(int argc, char** argv) {
     w -= 0.1f * (gi / (std::sqrt(sum) + 1e-10f));
     EXPECT(FloatEq(vals[0][i], w));
   }
+  // emitter_test.cc:75-87, 112-158 : two tables, combined pull and combined push with SGD
+  {
+    const float c0 = 7.5f, c1 = -3.25f;
+    SparseTable t0(10, "Combine0", 100, Initializer::Create(InitializerType::kConstant, {{"value", std::to_string(c0)}}));
+    SparseTable t1(11, "Combine1", 100, Initializer::Create(InitializerType::kConstant, {{"value", std::to_string(c1)}}));
+    SparseTableGroup grp({&t0, &t1});
+    EXPECT(grp.create_code() == 0);
+    std::unordered_map<uint64_t, std::vector<Tensor>> got;
+    EXPECT(grp.CombinePull({{10, {0, 1}}, {11, {0, 1}}}, &got) == 0);
+    EXPECT(got.size() == 2 && got[10].size() == 2 && got[11].size() == 2);
+    for (int r = 0; r < 2; ++r)
+      for (int i = 0; i < 100; ++i) EXPECT(got[10][r][i] == c0 && got[11][r][i] == c1);
+    std::unordered_map<uint64_t, CombinePushSparseTableItem> items;
+    items[10] = {{0, 1}, {RandomTensor(100, rng), RandomTensor(100, rng)}};
+    items[11] = {{1}, {RandomTensor(100, rng)}};
+    lr = 0.625f;
+    EXPECT(grp.CombinePush(sgd.get(), items, lr) == 0);
+    got.clear();
+    EXPECT(grp.CombinePull({{11, {1, 0}}, {10, {1, 0}}}, &got) == 0);
+    for (int i = 0; i < 100; ++i) {
+      EXPECT(FloatEq(got[10][0][i], c0 - lr * items[10].grads[1][i]));
+      EXPECT(FloatEq(got[10][1][i], c0 - lr * items[10].grads[0][i]));
+      EXPECT(FloatEq(got[11][0][i], c1 - lr * items[11].grads[0][i]));
+      EXPECT(got[11][1][i] == c1);
+    }
+    // repeated ids: their gradients are summed before the single update (emitter.cc:584-604)
+    std::unordered_map<uint64_t, CombinePushSparseTableItem> rep;
+    Tensor ga = Tensor::Dense(100), gb = Tensor::Dense(100);
+    for (int i = 0; i < 100; ++i) {
+      ga.Data()[i] = 0.25f * (i % 7);
+      gb.Data()[i] = -0.5f * (i % 3);
+    }
+    rep[11] = {{0, 0, 0}, {ga, gb, ga}};
+    EXPECT(grp.CombinePush(sgd.get(), rep, 0.5f, /*unique_ids=*/false) == 0);
+    std::vector<Tensor> one;
+    EXPECT(t1.Pull({0}, &one) == 0);                            // a member's own call sees the group's write
+    for (int i = 0; i < 100; ++i) EXPECT(one[0][i] == c1 - 0.5f * (2 * ga[i] + gb[i]));
+    // errors: a table outside the group, an id the table has never seen, a narrow gradient
+    EXPECT(grp.CombinePull({{12, {0}}}, &got) == ErrorCode::kTableNotExistError);
+    std::unordered_map<uint64_t, CombinePushSparseTableItem> bad;
+    bad[10] = {{77}, {RandomTensor(100, rng)}};
+    EXPECT(grp.CombinePush(sgd.get(), bad, lr) == ErrorCode::kSparseIdNotExistError);
+    bad[10] = {{0}, {RandomTensor(50, rng)}};
+    EXPECT(grp.CombinePush(sgd.get(), bad, lr) == ErrorCode::kGradientUnCompatibleError);
+  }
+
   // checkpoint/checkpoint.cc:444-509, 535-649 : through *.sparse / *.dense files and on
   const char* tmp = std::getenv("TMPDIR");
   const std::string dir = tmp ? tmp : "/tmp";
