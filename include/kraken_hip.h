@@ -260,9 +260,11 @@ int32_t krk_sparse_states(krk_sparse* t, uint32_t* mask);
 /* The rest of a Value for rows brought in with krk_sparse_import (transfer-in ps/ps.cc:789-792,
  * checkpoint load checkpoint/checkpoint.cc:620-645): one optimizer state [n, dim] and / or the
  * per-row step counters [n]. Either may be NULL. An id that is not in the table returns 12 and
- * leaves the other rows written. A row whose counter is 0 counts as never updated: SGD then
- * seeds its momentum buffer from the next gradient (ps/optim/sgd.cc:46-47), so a loader gives
- * rows that carry state a counter of at least 1. */
+ * leaves the other rows written. The counter is Adam's (StateType::kSteps, ps/optim/adam.cc:60).
+ * A row that is handed a momentum buffer (state_type 1) is from then on a row that has one: SGD
+ * with momentum seeds the buffer from the gradient only on rows that have none
+ * (ps/optim/sgd.cc:46-52), so a loader hands momentum buffers over for exactly the rows whose
+ * Value holds one. */
 int32_t krk_sparse_import_state(krk_sparse* t, const uint64_t* ids, int64_t n, int32_t state_type,
                                 const float* state, const int64_t* steps, uint32_t flags);
 /* The clean-up after a cluster change (ps/ps.cc:92-109: SkipList::Remove on every row routed

@@ -156,7 +156,7 @@ int32_t krk_sparse_save_file(krk_sparse* t, const char* path, uint64_t table_id,
   std::vector<int> states;
   for (int st = 1; st < KRK_ST_COUNT; ++st)
     if (mask & (1u << st)) states.push_back(st);
-  const bool has_counter = (mask & 1u) != 0;
+  std::vector<char> row_has(states.size());
   const bool adam = (mask & (1u << KRK_ST_FIRST_MOMENT)) != 0;
   std::vector<float> vals;
   std::vector<std::vector<float>> st_vals(states.size());
@@ -182,13 +182,23 @@ int32_t krk_sparse_save_file(krk_sparse* t, const char* path, uint64_t table_id,
           set_error("the table changed while it was being written: %s", path);
           return KRK_E_IO;
         }
-        const bool touched = !has_counter || steps[(size_t)i] > 0;
-        ok = w.pod<uint64_t>(ids[(size_t)(at + i)]) && w.row(vals.data() + i * dim, dim) &&
-             w.pod<uint64_t>(touched ? states.size() : 0);
-        if (touched)
-          for (size_t s = 0; s < states.size() && ok; ++s)
-            ok = w.pod<uint32_t>((uint32_t)states[s]) && w.row(st_vals[s].data() + i * dim, dim);
+        // The reference holds a state for a row once an update has created it. Here a column
+        // exists for every row, so a row's state is written when it holds anything but zeros
+        // (an absent state and a zero state update alike), and Adam's two moments whenever the
+        // row has been counted. The counter alone does not say that a row was updated: only
+        // Adam and SGD with momentum advance it.
         const bool counter = adam && steps[(size_t)i] > 0;
+        size_t emit = 0;
+        for (size_t s = 0; s < states.size(); ++s) {
+          const float* v = st_vals[s].data() + i * dim;
+          bool any = counter && (states[s] == KRK_ST_FIRST_MOMENT || states[s] == KRK_ST_SECOND_MOMENT);
+          for (int64_t j = 0; j < dim && !any; ++j) any = v[j] != 0.0f;
+          row_has[s] = any;
+          emit += any ? 1 : 0;
+        }
+        ok = w.pod<uint64_t>(ids[(size_t)(at + i)]) && w.row(vals.data() + i * dim, dim) && w.pod<uint64_t>(emit);
+        for (size_t s = 0; s < states.size() && ok; ++s)
+          if (row_has[s]) ok = w.pod<uint32_t>((uint32_t)states[s]) && w.row(st_vals[s].data() + i * dim, dim);
         ok = ok && w.pod<uint64_t>(counter ? 1 : 0);
         if (counter) ok = ok && w.pod<uint32_t>(KRK_ST_STEPS) && w.pod<int64_t>(steps[(size_t)i]);
       }
@@ -229,6 +239,7 @@ int32_t krk_sparse_load_file(krk_sparse* t, const char* path, uint64_t table_id,
   std::vector<float> vals, tensor;
   std::vector<float> st_vals[KRK_ST_COUNT];
   std::vector<int64_t> steps;
+  std::vector<size_t> with_momentum;   // rows of the chunk whose Value holds a momentum buffer
   uint32_t chunk_states = 0;
   int64_t loaded = 0;
   auto flush = [&]() -> int32_t {
@@ -238,9 +249,22 @@ int32_t krk_sparse_load_file(krk_sparse* t, const char* path, uint64_t table_id,
     for (int st = 1; st < KRK_ST_COUNT; ++st) {
       if (!(chunk_states & (1u << st))) continue;
       st_vals[st].resize((size_t)(n * dim), 0.0f);
-      KRK_TRY(krk_sparse_import_state(t, ids.data(), n, st, st_vals[st].data(), nullptr, 0));
+      if (st == KRK_ST_MOMENTUM_BUFFER) {
+        // receiving a momentum buffer marks a row as having one (SGD's first-update test), so
+        // only the rows that carry it in the file are handed over; the others keep their zeros
+        std::vector<uint64_t> m_ids;
+        std::vector<float> m_vals;
+        for (size_t row : with_momentum) {
+          m_ids.push_back(ids[row]);
+          m_vals.insert(m_vals.end(), st_vals[st].begin() + row * dim, st_vals[st].begin() + (row + 1) * dim);
+        }
+        KRK_TRY(krk_sparse_import_state(t, m_ids.data(), (int64_t)m_ids.size(), st, m_vals.data(), nullptr, 0));
+      } else {
+        KRK_TRY(krk_sparse_import_state(t, ids.data(), n, st, st_vals[st].data(), nullptr, 0));
+      }
       st_vals[st].clear();
     }
+    with_momentum.clear();
     bool any_steps = false;
     for (int64_t s : steps) any_steps = any_steps || s != 0;
     if (any_steps) KRK_TRY(krk_sparse_import_state(t, ids.data(), n, 1, nullptr, steps.data(), 0));
@@ -276,7 +300,7 @@ int32_t krk_sparse_load_file(krk_sparse* t, const char* path, uint64_t table_id,
         chunk_states |= 1u << st;
         st_vals[st].resize(row * (size_t)dim, 0.0f);   // rows read before this state first appeared
         st_vals[st].insert(st_vals[st].end(), tensor.begin(), tensor.end());
-        if (steps[row] == 0) steps[row] = 1;
+        if (st == KRK_ST_MOMENTUM_BUFFER) with_momentum.push_back(row);
       }
       if (!r.pod(&n_counters) || n_counters > 64) return io_fail("truncated or malformed table file", path);
       for (uint64_t s = 0; s < n_counters; ++s) {

@@ -272,11 +272,16 @@ __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, con
   if (a.meta_off >= 0) {
     const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + a.meta_off);
     steps = (uint64_t)meta[0] | ((uint64_t)meta[1] << 32);
-    first = steps == 0;
-    steps += 1;
     if (OPT == KRK_ADAM) {
-      bc1 = (float)(1.0 - (double)powf(a.k.beta1, (float)steps));
-      bc2 = (float)(1.0 - (double)powf(a.k.beta2, (float)steps));
+      steps += 1;                           // the flag bit rides along untouched
+    } else {
+      first = (steps & kHasMomentumBit) == 0;
+      steps |= kHasMomentumBit;
+    }
+    if (OPT == KRK_ADAM) {
+      const float count = (float)(steps & ~kHasMomentumBit);
+      bc1 = (float)(1.0 - (double)powf(a.k.beta1, count));
+      bc2 = (float)(1.0 - (double)powf(a.k.beta2, count));
     }
   }
   if (lane_on) {

@@ -46,6 +46,12 @@ struct TableView {
 
 constexpr int kBucket = 4;   // slots per bucket: one aligned 64-byte sector
 
+// The 64-bit word a record keeps when an optimizer needs it: the low 63 bits count Adam's
+// updates of the row (ps/optim/adam.cc:60, StateType::kSteps), the top bit says that the row has a
+// momentum buffer, which is how SGD with momentum tells its first update of a row from the later
+// ones (ps/optim/sgd.cc:46-52 looks for the state in the row's map).
+constexpr unsigned long long kHasMomentumBit = 1ull << 63;
+
 __device__ __forceinline__ void unpack_slot(const uint4& raw, unsigned long long& key,
                                             unsigned long long& row_epoch) {
   key = (unsigned long long)raw.x | ((unsigned long long)raw.y << 32);

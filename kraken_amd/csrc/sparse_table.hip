@@ -131,12 +131,17 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
   if (pc.meta >= 0) {
     const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + pc.meta);
     steps = (uint64_t)meta[0] | ((uint64_t)meta[1] << 32);
-    first = steps == 0;
-    steps += 1;
+    if (OPT == KRK_ADAM) {
+      steps += 1;                           // the flag bit rides along untouched
+    } else {
+      first = (steps & kHasMomentumBit) == 0;
+      steps |= kHasMomentumBit;
+    }
     if (OPT == KRK_ADAM) {
       // ps/optim/adam.cc:61-64 : per-row step counter, float pow, double subtraction
-      bc1 = (float)(1.0 - (double)powf(k.beta1, (float)steps));
-      bc2 = (float)(1.0 - (double)powf(k.beta2, (float)steps));
+      const float count = (float)(steps & ~kHasMomentumBit);
+      bc1 = (float)(1.0 - (double)powf(k.beta1, count));
+      bc2 = (float)(1.0 - (double)powf(k.beta2, count));
     }
   }
   for (int e = gl; e < elems; e += group) {
@@ -477,7 +482,7 @@ __global__ __launch_bounds__(kBlock) void export_kernel(TableView tv, int64_t ro
         long long s = 0;
         if (meta_off >= 0) {
           const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + meta_off);
-          s = (long long)((uint64_t)meta[0] | ((uint64_t)meta[1] << 32));
+          s = (long long)(((uint64_t)meta[0] | ((uint64_t)meta[1] << 32)) & ~kHasMomentumBit);
         }
         steps[r] = s;
       }
@@ -507,7 +512,7 @@ __global__ __launch_bounds__(kBlock) void fetch_kernel(TableView tv, const uint6
       long long s = 0;
       if (hit && meta_off >= 0) {
         const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + meta_off);
-        s = (long long)((uint64_t)meta[0] | ((uint64_t)meta[1] << 32));
+        s = (long long)(((uint64_t)meta[0] | ((uint64_t)meta[1] << 32)) & ~kHasMomentumBit);
       }
       steps[i] = s;
     }
@@ -535,8 +540,9 @@ template <int VEC>
 __global__ __launch_bounds__(kBlock) void import_state_kernel(TableView tv, const uint64_t* __restrict__ ids,
                                                               int64_t n, int state_off,
                                                               const float* __restrict__ state, int meta_off,
-                                                              const long long* __restrict__ steps, int dim,
-                                                              int elems, int group) {
+                                                              const long long* __restrict__ steps,
+                                                              bool mark_momentum, int dim, int elems,
+                                                              int group) {
   const int per_block = kBlock / group;
   const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
   const int gl = threadIdx.x & (group - 1);
@@ -555,9 +561,12 @@ __global__ __launch_bounds__(kBlock) void import_state_kernel(TableView tv, cons
       vstore<VEC>(rec + state_off + e * VEC, v);
     }
   }
-  if (steps && gl == 0) {
+  if ((steps || mark_momentum) && gl == 0) {
+    // a count replaces the count, a momentum buffer sets the flag: neither disturbs the other
     uint32_t* meta = reinterpret_cast<uint32_t*>(rec + meta_off);
-    const unsigned long long s = (unsigned long long)steps[i];
+    unsigned long long s = (unsigned long long)meta[0] | ((unsigned long long)meta[1] << 32);
+    if (steps) s = (s & kHasMomentumBit) | ((unsigned long long)steps[i] & ~kHasMomentumBit);
+    if (mark_momentum) s |= kHasMomentumBit;
     meta[0] = (uint32_t)s;
     meta[1] = (uint32_t)(s >> 32);
   }
@@ -1589,7 +1598,9 @@ int32_t krk_sparse_import_state(krk_sparse* t, const uint64_t* ids, int64_t n, i
   if (n == 0 || (!state && !steps)) return sparse_finish(t, flags);
   uint32_t mask = 0;
   if (state) mask |= 1u << state_type;
-  if (steps) mask |= 1u << KRK_ST_STEPS;
+  // a row that is given a momentum buffer is marked as having one (the flag lives with the counter)
+  const bool mark_momentum = state && state_type == KRK_ST_MOMENTUM_BUFFER;
+  if (steps || mark_momentum) mask |= 1u << KRK_ST_STEPS;
   KRK_TRY(sparse_ensure_columns(t, mask));
   const uint64_t* d_ids;
   const float* d_state = nullptr;
@@ -1602,10 +1613,10 @@ int32_t krk_sparse_import_state(krk_sparse* t, const uint64_t* ids, int64_t n, i
   const int state_off = state ? t->col_off[state_type] : -1;
   if (t->vec == 4) {
     hipLaunchKernelGGL((import_state_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, state_off,
-                       d_state, t->meta_off, d_steps, (int)t->dim, t->elems, t->group);
+                       d_state, t->meta_off, d_steps, mark_momentum, (int)t->dim, t->elems, t->group);
   } else {
     hipLaunchKernelGGL((import_state_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, state_off,
-                       d_state, t->meta_off, d_steps, (int)t->dim, t->elems, t->group);
+                       d_state, t->meta_off, d_steps, mark_momentum, (int)t->dim, t->elems, t->group);
   }
   KRK_HIP(hipGetLastError());
   return sparse_finish(t, flags);

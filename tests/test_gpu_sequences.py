@@ -1,0 +1,132 @@
+"""Random sequences of table operations against the oracle table: pulls with new and old ids,
+pushes of unique ids, pushes with repeats, pooled pulls and pushes, erases, imports, a trip
+through a checkpoint file and a change of optimizer mid-way (new state columns on a populated
+table). After every operation that returns rows they are compared; at the end every row, state
+and counter. What the single-purpose tests cover one by one is covered here in combination."""
+import numpy as np
+import pytest
+
+from util import assert_close, make_optims, splitmix64
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def api():
+    from kraken_amd import api as a
+    a.lib()
+    return a
+
+
+def _dyadic(rng, shape):
+    return (rng.integers(-32, 33, size=shape) / 1024.0).astype(np.float32)
+
+
+# The optimizers a sequence switches between. SGD with momentum tells a row's first update by a
+# flag that RMSprop with momentum does not set (the reference looks for the buffer in the row's
+# state map, and a model has one optimizer, so the two never meet on a table): a sequence draws
+# from a family that holds one of them.
+FAMILIES = [[(3, {}), (0, {}), (1, {}), (2, {"momentum": 0.5})],
+            [(3, {}), (0, {}), (1, {}), (3, {"momentum": 0.9, "dampening": 0.25}), (2, {})]]
+
+
+@pytest.mark.parametrize("seed", range(120))
+def test_random_operation_sequences(api, oracle, tmp_path, seed):
+    rng = np.random.default_rng(1000 + seed)
+    dim = int(rng.choice([4, 5, 16, 32, 72]))
+    space = int(rng.choice([300, 5000, 200000]))
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.05", "seed": str(seed)})
+    oi = oracle.init(oracle.INIT_NORMAL, 0.0, 0.05, seed=seed)
+    t = api.SparseTable(dim, gi, capacity_hint=int(rng.choice([0, 64, 4096])))
+    r = oracle.SparseTable(dim, oi)
+    used = set()
+    OPTIMS = FAMILIES[seed % 2]
+    type_, conf = OPTIMS[int(rng.integers(len(OPTIMS)))]
+    o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    lr = 0.03125
+
+    def some_ids(n, known_only=False):
+        if known_only:
+            pool = np.fromiter(used, np.uint64, len(used))
+            return rng.choice(pool, size=min(n, pool.size), replace=True) if pool.size else pool
+        return splitmix64(rng.integers(0, space, size=n).astype(np.uint64))
+
+    log = []
+    for step in range(60):
+        op = rng.choice(["pull", "pull", "push", "push_raw", "pooled", "erase", "load", "file", "optim", "fetch"])
+        log.append(op)
+        n = int(rng.choice([1, 7, 300, 3000]))
+        if op == "pull":
+            ids = some_ids(n)
+            rc, got = t.Pull(ids)
+            assert rc == 0
+            assert_close(got, r.pull(ids)[1], "step %d pull" % step, rtol=1e-5, atol=1e-7)
+            used.update(ids.tolist())
+        elif op == "push" and used:
+            ids = np.unique(some_ids(n, known_only=True))
+            g = _dyadic(rng, (ids.size, dim))
+            assert t.Push(o_gpu, ids, g, lr) == 0 and r.push(o_ref, ids, g, lr) == 0
+        elif op == "push_raw" and used:
+            ids = some_ids(n, known_only=True)
+            g = _dyadic(rng, (ids.size, dim))
+            assert t.PushRaw(o_gpu, ids, g, lr) == 0
+            u, gs = oracle.dedup_sum(ids, g)
+            assert r.push(o_ref, u, gs, lr) == 0
+        elif op == "pooled" and dim <= 256:
+            bags = int(rng.choice([1, 5, 200]))
+            # bag sizes whose mean ratio is a power of two: every gradient sum stays exact, so the
+            # optimizers (Adam above all, whose step is g / |g| on a fresh row) see identical inputs
+            lengths = rng.choice([0, 1, 2, 4], size=bags)
+            off = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
+            ids = some_ids(int(off[-1]))
+            mode = str(rng.choice(["sum", "mean"]))
+            rc, got = t.PullPooled(ids, off, mode, 0.5)
+            assert rc == 0
+            u, inv = oracle.dedup(ids)
+            rows = r.pull(u)[1][inv] if ids.size else np.zeros((0, dim), np.float32)
+            assert_close(got, oracle.jagged_forward(rows, off, mode, 0.5), "step %d pooled pull" % step,
+                         rtol=1e-5, atol=1e-6)
+            used.update(ids.tolist())
+            bg = _dyadic(rng, (bags, dim))
+            assert t.PushPooled(o_gpu, ids, off, bg, lr, mode=mode) == 0
+            if ids.size:
+                u2, gs = oracle.dedup_sum(ids, oracle.jagged_backward(off, bg, mode))
+                assert r.push(o_ref, u2, gs, lr) == 0
+        elif op == "erase" and used:
+            gone = np.unique(np.concatenate([some_ids(n, known_only=True)[: max(1, n // 3)], some_ids(3)]))
+            assert t.erase(gone) == r.erase(gone)
+            used.difference_update(gone.tolist())
+        elif op == "load":
+            ids = np.unique(some_ids(min(n, 300)))
+            vals = _dyadic(rng, (ids.size, dim))
+            t.load(ids, vals)
+            r.load(ids, vals)
+            used.update(ids.tolist())
+        elif op == "file" and used:
+            path = str(tmp_path / ("t%d.sparse" % step))
+            assert t.save(path, 1, "t") == 0
+            t2 = api.SparseTable(dim, gi)
+            rc, taken = t2.load_file(path, 1, "t")
+            assert rc == 0 and taken == len(r)
+            t = t2
+        elif op == "optim":
+            type_, conf = OPTIMS[int(rng.integers(len(OPTIMS)))]
+            o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+        elif op == "fetch" and used:
+            ids = np.concatenate([some_ids(n, known_only=True), some_ids(5)])
+            found, vals, _, _ = t.fetch(ids)
+            rf, rv = r.fetch(ids)
+            assert np.array_equal(found, rf)
+            assert_close(vals[found], rv[rf], "step %d fetch" % step, rtol=1e-5, atol=1e-7)
+        assert len(t) == len(r), (step, log)
+
+    gid, gval, _, gsteps = t.export()
+    rid, rval, _, rsteps = r.export()
+    og, orr = np.argsort(gid), np.argsort(rid)
+    assert np.array_equal(gid[og], rid[orr]), log
+    assert_close(gval[og], rval[orr], "final weights after %s" % log, rtol=2e-5, atol=1e-6)
+    assert np.array_equal(gsteps[og], rsteps[orr]), log        # Adam's per-row counts
+    for st in range(1, 8):
+        gs = t.export(state_type=st)[2]
+        rs = r.export(state_type=st)[2]
+        assert_close(gs[og], rs[orr], "final state %d" % st, rtol=2e-5, atol=1e-6)
