@@ -130,3 +130,139 @@ def test_random_operation_sequences(api, oracle, tmp_path, seed):
         gs = t.export(state_type=st)[2]
         rs = r.export(state_type=st)[2]
         assert_close(gs[og], rs[orr], "final state %d" % st, rtol=2e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_sequences_on_a_group(api, oracle, seed):
+    """Combined pulls and pushes (unique ids and with repeats) interleaved with the members' own
+    calls, erases and imports, which move rows and add columns under the group's feet."""
+    rng = np.random.default_rng(7000 + seed)
+    dim = int(rng.choice([4, 6, 16, 32]))
+    n_tables = int(rng.choice([1, 2, 5, 26]))
+    space = int(rng.choice([200, 20000]))
+    tables, refs = [], []
+    for m in range(n_tables):
+        tables.append(api.SparseTable(dim, api.Initializer.create(
+            api.InitializerType.kNormal, {"stddev": "0.05", "seed": str(seed * 100 + m)}),
+            capacity_hint=int(rng.choice([0, 2048]))))
+        refs.append(oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.05, seed=seed * 100 + m)))
+    grp = api.TableGroup(tables)
+    used = [set() for _ in range(n_tables)]
+    OPTIMS = FAMILIES[seed % 2]
+    type_, conf = OPTIMS[int(rng.integers(len(OPTIMS)))]
+    o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    lr = 0.03125
+
+    def ids_for(m, n, known_only):
+        if known_only:
+            pool = np.fromiter(used[m], np.uint64, len(used[m]))
+            return rng.choice(pool, size=min(n, pool.size), replace=True) if pool.size else pool
+        return splitmix64(rng.integers(0, space, size=n).astype(np.uint64))
+
+    log = []
+    for step in range(40):
+        op = str(rng.choice(["cpull", "cpull", "cpush", "cpush_raw", "pull", "push_raw", "erase", "load", "optim"]))
+        log.append(op)
+        sizes = [int(rng.choice([0, 1, 40, 900])) for _ in range(n_tables)]
+        if op == "cpull":
+            per = [ids_for(m, sizes[m], False) for m in range(n_tables)]
+            off = grp._offsets([p.size for p in per])
+            rc, got = grp.CombinePull(np.concatenate(per), off)
+            assert rc == 0
+            want = np.concatenate([r.pull(p)[1] for r, p in zip(refs, per)])
+            assert_close(got, want, "step %d combined pull" % step, rtol=1e-5, atol=1e-7)
+            for m in range(n_tables):
+                used[m].update(per[m].tolist())
+        elif op in ("cpush", "cpush_raw"):
+            per = [ids_for(m, sizes[m], True) for m in range(n_tables)]
+            if op == "cpush":
+                per = [np.unique(p) for p in per]
+            off = grp._offsets([p.size for p in per])
+            g = _dyadic(rng, (int(off[-1]), dim))
+            ids = np.concatenate(per) if off[-1] else np.zeros(0, np.uint64)
+            assert grp.CombinePush(o_gpu, ids, off, g, lr, raw=(op == "cpush_raw")) == 0
+            for r, p, a, b in zip(refs, per, off[:-1], off[1:]):
+                if p.size:
+                    u, gs = oracle.dedup_sum(p, g[a:b])
+                    assert r.push(o_ref, u, gs, lr) == 0
+        else:
+            m = int(rng.integers(n_tables))
+            t, r = tables[m], refs[m]
+            if op == "pull":
+                ids = ids_for(m, sizes[m] + 1, False)
+                assert_close(t.Pull(ids)[1], r.pull(ids)[1], "step %d member pull" % step, rtol=1e-5, atol=1e-7)
+                used[m].update(ids.tolist())
+            elif op == "push_raw" and used[m]:
+                ids = ids_for(m, sizes[m] + 1, True)
+                g = _dyadic(rng, (ids.size, dim))
+                assert t.PushRaw(o_gpu, ids, g, lr) == 0
+                u, gs = oracle.dedup_sum(ids, g)
+                assert r.push(o_ref, u, gs, lr) == 0
+            elif op == "erase" and used[m]:
+                gone = np.unique(ids_for(m, sizes[m] // 3 + 1, True))
+                assert t.erase(gone) == r.erase(gone)
+                used[m].difference_update(gone.tolist())
+            elif op == "load":
+                ids = np.unique(ids_for(m, 50, False))
+                vals = _dyadic(rng, (ids.size, dim))
+                t.load(ids, vals)
+                r.load(ids, vals)
+                used[m].update(ids.tolist())
+            elif op == "optim":
+                type_, conf = OPTIMS[int(rng.integers(len(OPTIMS)))]
+                o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    for m, (t, r) in enumerate(zip(tables, refs)):
+        gid, gval, _, gsteps = t.export()
+        rid, rval, _, rsteps = r.export()
+        og, orr = np.argsort(gid), np.argsort(rid)
+        assert np.array_equal(gid[og], rid[orr]), (m, log)
+        assert_close(gval[og], rval[orr], "table %d after %s" % (m, log), rtol=2e-5, atol=1e-6)
+        assert np.array_equal(gsteps[og], rsteps[orr]), (m, log)
+        for st in range(1, 8):
+            assert_close(t.export(state_type=st)[2][og], r.export(state_type=st)[2][orr],
+                         "table %d state %d" % (m, st), rtol=2e-5, atol=1e-6)
+    grp.close()
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_sequences_on_a_dense_table(api, oracle, tmp_path, seed):
+    """Dense and COO gradients, optimizer changes and trips through a *.dense file, against the
+    oracle's dense table."""
+    rng = np.random.default_rng(9000 + seed)
+    n = int(rng.choice([1, 7, 256, 1000, 40000]))
+    w0 = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    t, r = api.DenseTable(w0), oracle.DenseTable(w0)
+    OPTIMS = FAMILIES[seed % 2]
+    type_, conf = OPTIMS[int(rng.integers(len(OPTIMS)))]
+    o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    for step in range(25):
+        op = str(rng.choice(["push", "push", "coo", "empty_coo", "file", "optim", "pull"]))
+        if op == "push":
+            g = _dyadic(rng, n)
+            assert t.Push(o_gpu, g, 0.0625) == 0 and r.push(o_ref, g, 0.0625) == 0
+        elif op == "coo":
+            k = int(rng.integers(1, max(2, n // 3 + 1)))
+            idx = np.sort(rng.choice(n, size=min(k, n), replace=False)).astype(np.int64)
+            val = _dyadic(rng, idx.size)
+            assert t.PushCoo(o_gpu, idx, val, 0.0625) == 0 and r.push_coo(o_ref, idx, val, 0.0625) == 0
+        elif op == "empty_coo":
+            # ps/optim/adam.cc:26-29 : success without touching state or the step counter
+            e_i, e_v = np.zeros(0, np.int64), np.zeros(0, np.float32)
+            assert t.PushCoo(o_gpu, e_i, e_v, 0.0625) == 0 and r.push_coo(o_ref, e_i, e_v, 0.0625) == 0
+        elif op == "file":
+            path = str(tmp_path / ("d%d.dense" % step))
+            assert t.save(path, 5, "d") == 0
+            rc, t, tid, name, shape = api.DenseTable.from_file(path)
+            assert rc == 0 and tid == 5 and name == "d"
+        elif op == "optim":
+            type_, conf = OPTIMS[int(rng.integers(len(OPTIMS)))]
+            o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+        assert_close(t.Pull()[1], r.pull(), "step %d %s" % (step, op), rtol=2e-5, atol=1e-6)
+        assert t.steps == r.steps
+    for st in range(1, 8):
+        want = r.state(st)
+        got = t.state(st)
+        if want is None:
+            assert got is None or not np.any(got)
+        else:
+            assert_close(got, want, "state %d" % st, rtol=2e-5, atol=1e-6)
