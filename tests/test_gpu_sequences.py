@@ -266,3 +266,72 @@ def test_random_sequences_on_a_dense_table(api, oracle, tmp_path, seed):
             assert got is None or not np.any(got)
         else:
             assert_close(got, want, "state %d" % st, rtol=2e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_sequences_enqueued_without_waiting(api, oracle, seed):
+    """The same operations through device pointers with KRK_ASYNC: nothing waits until the end,
+    tables start tiny so that they grow (records, index, new state columns) while earlier
+    launches are still queued, and every reply is checked after the final sync."""
+    rng = np.random.default_rng(12000 + seed)
+    dim = int(rng.choice([4, 16, 32]))
+    space = int(rng.choice([500, 100000]))
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.05", "seed": str(seed)})
+    t = api.SparseTable(dim, gi, capacity_hint=int(rng.choice([0, 16])))
+    r = oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.05, seed=seed))
+    OPTIMS = FAMILIES[seed % 2]
+    type_, conf = OPTIMS[int(rng.integers(len(OPTIMS)))]
+    o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    used = np.zeros(0, np.uint64)
+    pending = []          # (device output, expected rows, what)
+    keep = []             # device inputs stay alive until the sync
+    for step in range(30):
+        op = str(rng.choice(["pull", "pull", "push", "push_raw", "pooled", "optim"]))
+        n = int(rng.choice([1, 50, 2000, 20000]))
+        if op == "pull":
+            ids = splitmix64(rng.integers(0, space, size=n).astype(np.uint64))
+            d_ids = api.DeviceArray.from_host(ids)
+            rc, d_out = t.Pull(d_ids, async_=True)
+            assert rc == 0
+            pending.append((d_out, r.pull(ids)[1], "step %d pull" % step))
+            keep.append(d_ids)
+            used = np.union1d(used, ids)
+        elif op in ("push", "push_raw") and used.size:
+            ids = rng.choice(used, size=min(n, used.size), replace=(op == "push_raw"))
+            g = _dyadic(rng, (ids.size, dim))
+            d_ids, d_g = api.DeviceArray.from_host(ids), api.DeviceArray.from_host(g)
+            assert t.Push(o_gpu, d_ids, d_g, 0.03125, async_=True, raw=(op == "push_raw")) == 0
+            u, gs = oracle.dedup_sum(ids, g)
+            assert r.push(o_ref, u, gs, 0.03125) == 0
+            keep += [d_ids, d_g]
+        elif op == "pooled":
+            bags = int(rng.choice([1, 30, 3000]))
+            lengths = rng.choice([0, 1, 2, 4], size=bags)
+            off = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
+            ids = splitmix64(rng.integers(0, space, size=int(off[-1])).astype(np.uint64))
+            d_ids, d_off = api.DeviceArray.from_host(ids), api.DeviceArray.from_host(off)
+            rc, d_out = t.PullPooled(d_ids, d_off, "mean", 0.25, async_=True)
+            assert rc == 0
+            u, inv = oracle.dedup(ids)
+            rows = r.pull(u)[1][inv] if ids.size else np.zeros((0, dim), np.float32)
+            pending.append((d_out, oracle.jagged_forward(rows, off, "mean", 0.25), "step %d pooled" % step))
+            used = np.union1d(used, ids)
+            bg = _dyadic(rng, (bags, dim))
+            d_bg = api.DeviceArray.from_host(bg)
+            assert t.PushPooled(o_gpu, d_ids, d_off, d_bg, 0.03125, mode="mean", async_=True) == 0
+            if ids.size:
+                u2, gs = oracle.dedup_sum(ids, oracle.jagged_backward(off, bg, "mean"))
+                assert r.push(o_ref, u2, gs, 0.03125) == 0
+            keep += [d_ids, d_off, d_bg]
+        elif op == "optim":
+            type_, conf = OPTIMS[int(rng.integers(len(OPTIMS)))]
+            o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    assert t.sync() == 0
+    for d_out, want, what in pending:
+        assert_close(d_out.to_host(), want, what, rtol=1e-5, atol=1e-6)
+    gid, gval, _, gsteps = t.export()
+    rid, rval, _, rsteps = r.export()
+    og, orr = np.argsort(gid), np.argsort(rid)
+    assert np.array_equal(gid[og], rid[orr])
+    assert_close(gval[og], rval[orr], "final weights", rtol=2e-5, atol=1e-6)
+    assert np.array_equal(gsteps[og], rsteps[orr])
