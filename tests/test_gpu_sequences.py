@@ -335,3 +335,38 @@ def test_random_sequences_enqueued_without_waiting(api, oracle, seed):
     assert np.array_equal(gid[og], rid[orr])
     assert_close(gval[og], rval[orr], "final weights", rtol=2e-5, atol=1e-6)
     assert np.array_equal(gsteps[og], rsteps[orr])
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_sequences_of_the_threshold_codec(api, oracle, seed):
+    """Many steps of one DenseBag with awkward gradients (all zeros, all equal, a few huge values,
+    subnormals, signed zeros) and a life span that makes thresholds go stale: indices, values,
+    threshold, residual and step count equal the oracle's at every step."""
+    rng = np.random.default_rng(15000 + seed)
+    n = int(rng.choice([256, 257, 1000, 4096, 70001]))
+    life_span = int(rng.choice([1, 2, 3, 1000]))
+    eta = float(rng.choice([0.1, 0.5, 0.75, 0.99]))
+    bag, ref = api.DenseBag(n), oracle.DctState(n)
+    for step in range(10):
+        kind = str(rng.choice(["normal", "normal", "zeros", "equal", "spikes", "tiny", "negzero"]))
+        if kind == "normal":
+            g = rng.standard_normal(n).astype(np.float32)
+        elif kind == "zeros":
+            g = np.zeros(n, np.float32)
+        elif kind == "equal":
+            g = np.full(n, np.float32(rng.choice([-1.5, 0.25])))
+        elif kind == "spikes":
+            g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+            g[rng.choice(n, size=5, replace=False)] = np.float32(1e30)
+        elif kind == "tiny":
+            g = (rng.standard_normal(n) * 1e-42).astype(np.float32)       # subnormal
+        else:
+            g = np.where(rng.random(n) < 0.5, np.float32(-0.0), np.float32(0.0)).astype(np.float32)
+        idx, val = bag.MaybeToCoo(life_span, eta, g)
+        ridx, rval = ref.compress(g, life_span=life_span, eta=eta, exact_select=True)
+        assert bag.tau == ref.tau, (step, kind)
+        assert np.array_equal(idx, ridx), (step, kind)
+        assert np.array_equal(val.view(np.uint32), rval.view(np.uint32)), (step, kind)
+        assert np.array_equal(bag.residual.view(np.uint32), ref.residual.view(np.uint32)), (step, kind)
+        assert bag.step == ref.step
+        assert np.array_equal(api.coo_to_dense(idx, val, n), oracle.coo_to_dense(ridx, rval, n))
