@@ -49,7 +49,12 @@ def test_random_operation_sequences(api, oracle, tmp_path, seed):
         if known_only:
             pool = np.fromiter(used, np.uint64, len(used))
             return rng.choice(pool, size=min(n, pool.size), replace=True) if pool.size else pool
-        return splitmix64(rng.integers(0, space, size=n).astype(np.uint64))
+        ids = splitmix64(rng.integers(0, space, size=n).astype(np.uint64))
+        if n and rng.random() < 0.25:
+            ids[rng.integers(n)] = np.uint64(2**64 - 1)        # the id that equals the index's empty marker
+        if n and rng.random() < 0.25:
+            ids[rng.integers(n)] = np.uint64(0)
+        return ids
 
     log = []
     for step in range(60):
