@@ -85,17 +85,23 @@ def test_random_operation_sequences(api, oracle, tmp_path, seed):
             off = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
             ids = some_ids(int(off[-1]))
             mode = str(rng.choice(["sum", "mean"]))
-            rc, got = t.PullPooled(ids, off, mode, 0.5)
+            w = (2.0 ** rng.integers(-2, 2, size=ids.size)).astype(np.float32) if rng.random() < 0.5 else None
+            rc, got = t.PullPooled(ids, off, mode, 0.5, weights=w)
             assert rc == 0
             u, inv = oracle.dedup(ids)
             rows = r.pull(u)[1][inv] if ids.size else np.zeros((0, dim), np.float32)
+            if w is not None:
+                rows = rows * w[:, None]                       # pytorch/jagged_embedding.py:44-45
             assert_close(got, oracle.jagged_forward(rows, off, mode, 0.5), "step %d pooled pull" % step,
                          rtol=1e-5, atol=1e-6)
             used.update(ids.tolist())
             bg = _dyadic(rng, (bags, dim))
-            assert t.PushPooled(o_gpu, ids, off, bg, lr, mode=mode) == 0
+            assert t.PushPooled(o_gpu, ids, off, bg, lr, mode=mode, weights=w) == 0
             if ids.size:
-                u2, gs = oracle.dedup_sum(ids, oracle.jagged_backward(off, bg, mode))
+                vg = oracle.jagged_backward(off, bg, mode)
+                if w is not None:
+                    vg = vg * w[:, None]
+                u2, gs = oracle.dedup_sum(ids, vg)
                 assert r.push(o_ref, u2, gs, lr) == 0
         elif op == "erase" and used:
             gone = np.unique(np.concatenate([some_ids(n, known_only=True)[: max(1, n // 3)], some_ids(3)]))
