@@ -168,13 +168,88 @@ __global__ __launch_bounds__(kCodecBlock) void emit_write_kernel(
   }
 }
 
+
+// ---- densify in one pass over the output ------------------------------------------------------
+constexpr int kTileElems = 4096;                 // floats of one output tile: 16 KB of LDS
+constexpr int64_t kTiledFrom = 1 << 22;          // smaller tensors: zero + scatter, two launches are quicker
+constexpr uint32_t kNoStart = 0xFFFFFFFFu;
+
+__global__ __launch_bounds__(kCodecBlock) void coo_tiles_init_kernel(uint32_t* __restrict__ starts, int64_t tiles,
+                                                                     uint32_t* __restrict__ unordered) {
+  const int64_t i = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x;
+  if (i < tiles) starts[i] = kNoStart;
+  if (i == 0) *unordered = 0u;
+}
+
+// starts[T] = first entry whose index lies in tile T; *unordered is raised when the indices do
+// not ascend strictly or leave [0, n).
+__global__ __launch_bounds__(kCodecBlock) void coo_tiles_bounds_kernel(const long long* __restrict__ idx,
+                                                                       int64_t nnz, int64_t n,
+                                                                       uint32_t* __restrict__ starts,
+                                                                       uint32_t* __restrict__ unordered) {
+  const int64_t step = (int64_t)gridDim.x * kCodecBlock;
+  for (int64_t j = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x; j < nnz; j += step) {
+    const long long cur = idx[j];
+    const long long prev = j ? idx[j - 1] : -1;
+    if (cur <= prev || cur >= n) {
+      atomicOr(unordered, 1u);
+    } else if (prev < 0 || cur / kTileElems != prev / kTileElems) {
+      starts[cur / kTileElems] = (uint32_t)j;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kCodecBlock) void coo_tiles_write_kernel(const long long* __restrict__ idx,
+                                                                      const float* __restrict__ val, int64_t nnz,
+                                                                      float* __restrict__ dense, int64_t n,
+                                                                      const uint32_t* __restrict__ starts,
+                                                                      const uint32_t* __restrict__ unordered) {
+  if (*unordered) return;                        // the scatter launches that follow do the work
+  __shared__ float tile[kTileElems];
+  const int64_t base = (int64_t)blockIdx.x * kTileElems;
+  for (int i = threadIdx.x; i < kTileElems; i += kCodecBlock) tile[i] = 0.0f;
+  __syncthreads();
+  const uint32_t start = starts[blockIdx.x];
+  if (start != kNoStart) {
+    for (int64_t j = (int64_t)start + threadIdx.x; j < nnz; j += kCodecBlock) {
+      const long long i = idx[j];
+      if (i >= base + kTileElems) break;         // ascending: nothing further belongs to this tile
+      tile[i - base] = val[j];
+    }
+  }
+  __syncthreads();
+  const int64_t left = n - base;
+  const int cnt = left < kTileElems ? (int)left : kTileElems;
+  if (cnt == kTileElems && (((uintptr_t)dense) & 15) == 0) {
+    for (int i = threadIdx.x; i < kTileElems / 4; i += kCodecBlock)
+      reinterpret_cast<float4*>(dense + base)[i] = reinterpret_cast<const float4*>(tile)[i];
+  } else {
+    for (int i = threadIdx.x; i < cnt; i += kCodecBlock) dense[base + i] = tile[i];
+  }
+}
+
+__global__ __launch_bounds__(kCodecBlock) void coo_zero_if_kernel(float* __restrict__ dense, int64_t n,
+                                                                  const uint32_t* __restrict__ unordered) {
+  if (!*unordered) return;
+  const int64_t step = (int64_t)gridDim.x * kCodecBlock;
+  for (int64_t i = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x; i < n; i += step) dense[i] = 0.0f;
+}
+
+// dense[idx[j]] += val[j]; repeated indices add up (t/math.cc:1043). unordered null: always.
 __global__ __launch_bounds__(kCodecBlock) void coo_add_kernel(const long long* __restrict__ idx,
                                                               const float* __restrict__ val, int64_t nnz,
-                                                              float* __restrict__ dense, int64_t n) {
+                                                              float* __restrict__ dense, int64_t n,
+                                                              const uint32_t* __restrict__ unordered,
+                                                              uint32_t* __restrict__ err) {
+  if (unordered && !*unordered) return;
   const int64_t j = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x;
   if (j >= nnz) return;
   const long long i = idx[j];
-  if (i >= 0 && i < n) unsafeAtomicAdd(&dense[i], val[j]);   // hardware fp32 add, no CAS loop
+  if (i < 0 || i >= n) {
+    if (err) atomicOr(err, 1u);
+    return;
+  }
+  unsafeAtomicAdd(&dense[i], val[j]);   // hardware fp32 add, no CAS loop
 }
 
 static unsigned stream_grid(int64_t n) {
@@ -184,9 +259,48 @@ static unsigned stream_grid(int64_t n) {
   return (unsigned)blocks;
 }
 
+size_t coo_densify_work_bytes(int64_t n) {
+  return ((size_t)((n + kTileElems - 1) / kTileElems) + 4) * sizeof(uint32_t);
+}
+
+int32_t coo_densify(const long long* d_idx, const float* d_val, int64_t nnz, float* d_dense, int64_t n,
+                    void* work, uint32_t* err, hipStream_t stream) {
+  if (n <= 0) return KRK_SUCCESS;
+  const dim3 block(kCodecBlock);
+  const unsigned per_entry = (unsigned)((nnz + kCodecBlock - 1) / kCodecBlock);
+  if (n < kTiledFrom || nnz >= ((int64_t)1 << 31) || !work) {
+    KRK_HIP(hipMemsetAsync(d_dense, 0, (size_t)n * sizeof(float), stream));   // t/math.cc:1066 dense.Zero()
+    if (nnz)
+      hipLaunchKernelGGL(coo_add_kernel, dim3(per_entry), block, 0, stream, d_idx, d_val, nnz, d_dense, n,
+                         (const uint32_t*)nullptr, err);
+    KRK_HIP(hipGetLastError());
+    return KRK_SUCCESS;
+  }
+  const int64_t tiles = (n + kTileElems - 1) / kTileElems;
+  uint32_t* starts = reinterpret_cast<uint32_t*>(work);
+  uint32_t* unordered = starts + tiles;
+  hipLaunchKernelGGL(coo_tiles_init_kernel, dim3((unsigned)((tiles + kCodecBlock - 1) / kCodecBlock)), block, 0,
+                     stream, starts, tiles, unordered);
+  if (nnz)
+    hipLaunchKernelGGL(coo_tiles_bounds_kernel, dim3(stream_grid(nnz)), block, 0, stream, d_idx, nnz, n, starts,
+                       unordered);
+  hipLaunchKernelGGL(coo_tiles_write_kernel, dim3((unsigned)tiles), block, 0, stream, d_idx, d_val, nnz, d_dense,
+                     n, starts, unordered);
+  if (nnz) {
+    hipLaunchKernelGGL(coo_zero_if_kernel, dim3(stream_grid(n)), block, 0, stream, d_dense, n, unordered);
+    hipLaunchKernelGGL(coo_add_kernel, dim3(per_entry), block, 0, stream, d_idx, d_val, nnz, d_dense, n,
+                       (const uint32_t*)unordered, err);
+  }
+  KRK_HIP(hipGetLastError());
+  return KRK_SUCCESS;
+}
+
 }  // namespace krk
 
 using namespace krk;
+
+static std::mutex g_densify_mu;          // krk_coo_to_dense owns no object: one shared work buffer
+static DeviceBuffer g_densify_work;
 
 extern "C" {
 
@@ -372,11 +486,17 @@ int32_t krk_coo_to_dense(const int64_t* idx, const float* val, int64_t nnz, floa
     d_idx = si;
     d_val = sv;
   }
-  hipError_t e = hipMemsetAsync(d_dense, 0, (size_t)n * sizeof(float), st);   // t/math.cc:1066 dense.Zero()
-  if (e == hipSuccess && nnz) {
-    hipLaunchKernelGGL(coo_add_kernel, dim3((unsigned)((nnz + kCodecBlock - 1) / kCodecBlock)),
-                       dim3(kCodecBlock), 0, st, d_idx, d_val, nnz, d_dense, n);
-    e = hipGetLastError();
+  hipError_t e = hipSuccess;
+  {
+    std::lock_guard<std::mutex> lk(g_densify_mu);
+    int32_t rc = g_densify_work.reserve(coo_densify_work_bytes(n));
+    if (rc == KRK_SUCCESS) rc = coo_densify(d_idx, d_val, nnz, d_dense, n, g_densify_work.ptr, nullptr, st);
+    // the shared work buffer is free for the next caller once this call's launches are done
+    if (rc == KRK_SUCCESS && n >= kTiledFrom) e = hipStreamSynchronize(st);
+    if (rc != KRK_SUCCESS) {
+      if (tmp) (void)hipFree(tmp);
+      return rc;
+    }
   }
   if (e == hipSuccess && host) e = hipMemcpy(dense, d_dense, (size_t)n * sizeof(float), hipMemcpyDeviceToHost);
   if (e == hipSuccess && !(flags & KRK_ASYNC)) e = hipStreamSynchronize(st);

@@ -12,6 +12,7 @@ struct krk_dense : krk::ObjBase {
   float* w = nullptr;
   float* state[KRK_ST_COUNT] = {};   // created on first use, zero filled
   float* coo_grad = nullptr;         // densified COO gradient
+  krk::DeviceBuffer coo_work;        // work space of the tiled densify
   int64_t steps = 0;                 // Adam's kSteps (one counter for the whole tensor)
   bool sgd_started = false;          // momentum buffer exists (first update copies the gradient)
 };
@@ -51,21 +52,6 @@ __global__ __launch_bounds__(kDenseBlock) void dense_update_kernel(
     if (s1) s1[i] = b;
     if (s2) s2[i] = c;
   }
-}
-
-// dense[idx[j]] += val[j]; repeated indices add up (t/math.cc:1043).
-__global__ __launch_bounds__(kDenseBlock) void coo_scatter_kernel(const long long* __restrict__ idx,
-                                                                   const float* __restrict__ val,
-                                                                   int64_t nnz, float* __restrict__ dense,
-                                                                   int64_t n, uint32_t* __restrict__ err) {
-  const int64_t j = (int64_t)blockIdx.x * kDenseBlock + threadIdx.x;
-  if (j >= nnz) return;
-  const long long i = idx[j];
-  if (i < 0 || i >= n) {
-    atomicOr(err, 1u);
-    return;
-  }
-  unsafeAtomicAdd(&dense[i], val[j]);   // hardware fp32 add, no CAS loop
 }
 
 static unsigned dense_grid(int64_t n) {
@@ -182,6 +168,7 @@ int32_t krk_dense_destroy(krk_dense* t) {
   if (t->stream) (void)hipStreamSynchronize(t->stream);
   if (t->w) (void)hipFree(t->w);
   if (t->coo_grad) (void)hipFree(t->coo_grad);
+  t->coo_work.release();
   for (auto& s : t->state)
     if (s) (void)hipFree(s);
   t->close_stream();
@@ -239,12 +226,10 @@ int32_t krk_dense_push_coo(krk_dense* t, const krk_optim* o, const int64_t* idx,
   const float* d_val;
   KRK_TRY(t->input(idx, (size_t)nnz, flags, 0, &d_idx));
   KRK_TRY(t->input(val, (size_t)nnz, flags, 1, &d_val));
-  uint32_t* err = reinterpret_cast<uint32_t*>(t->coo_grad + t->n);
-  KRK_HIP(hipMemsetAsync(t->coo_grad, 0, (size_t)t->n * sizeof(float) + 16, t->stream));
-  hipLaunchKernelGGL(coo_scatter_kernel, dim3((unsigned)((nnz + kDenseBlock - 1) / kDenseBlock)),
-                     dim3(kDenseBlock), 0, t->stream, reinterpret_cast<const long long*>(d_idx), d_val,
-                     nnz, t->coo_grad, t->n, err);
-  KRK_HIP(hipGetLastError());
+  // entries whose index lies outside [0, n) are skipped
+  KRK_TRY(t->coo_work.reserve(coo_densify_work_bytes(t->n)));
+  KRK_TRY(coo_densify(reinterpret_cast<const long long*>(d_idx), d_val, nnz, t->coo_grad, t->n, t->coo_work.ptr,
+                      nullptr, t->stream));
   KRK_TRY(dense_apply(t, *o, t->coo_grad, lr));
   return dense_finish(t, flags);
 }

@@ -267,6 +267,16 @@ __device__ __forceinline__ void optim_element(const OptimK& k, float lr, float g
 
 // ---- device-wide exclusive scan of int32 (three plain launches, no spinning) ----
 // out[i] = sum(in[0..i)), total written to *total_out (device). in/out may alias.
+// CooTensorImpl::ToDense (t/coo_tensor_impl.cc:250-260, t/math.cc:1006-1096) on the device:
+// dense[0, n) = 0, then dense[idx[j]] += val[j]. Large tensors whose indices ascend strictly and
+// lie in range (what ToCoo produces) are written tile by tile in one pass over the output; any
+// other input is zeroed and scattered into, decided on the device inside the same launches.
+// work holds coo_densify_work_bytes(n); err (may be null) gets bit 0 set when an index is out
+// of range.
+size_t coo_densify_work_bytes(int64_t n);
+int32_t coo_densify(const long long* d_idx, const float* d_val, int64_t nnz, float* d_dense, int64_t n,
+                    void* work, uint32_t* err, hipStream_t stream);
+
 // scratch must hold scan_scratch_bytes(n).
 size_t scan_scratch_bytes(int64_t n);
 int32_t exclusive_scan_i32(const int32_t* in, int32_t* out, int64_t n, int32_t* total_out,

@@ -154,3 +154,54 @@ def test_codec_device_pointers_and_capacity(api, oracle):
     assert nnz == ridx.size
     assert np.array_equal(d_idx.to_host()[:nnz], ridx) and np.array_equal(d_val.to_host()[:nnz], rval)
     assert np.array_equal(bag.residual, ref.residual)
+
+
+@pytest.mark.parametrize("n", [1 << 22, (1 << 22) + 1, 5_000_003])
+def test_coo_to_dense_large_tensors(api, oracle, n):
+    """From 2^22 elements on the dense result is written tile by tile when the indices ascend
+    strictly (what ToCoo produces); anything else is zeroed and scattered into. Both against the
+    oracle: ascending with long gaps and a full last tile, every element present, nothing present,
+    shuffled, with repeats (which add up, t/math.cc:1043)."""
+    rng = np.random.default_rng(n)
+
+    def check(idx, val):
+        idx = np.ascontiguousarray(idx, np.int64)
+        val = np.ascontiguousarray(val, np.float32)
+        want = np.zeros(n, np.float32)
+        np.add.at(want, idx, val)
+        if np.unique(idx).size == idx.size:
+            assert np.array_equal(want, oracle.coo_to_dense(idx, val, n))
+        assert np.array_equal(api.coo_to_dense(idx, val, n), want)
+        d = api.coo_to_dense(api.DeviceArray.from_host(idx), api.DeviceArray.from_host(val), n)
+        assert np.array_equal(d.to_host(), want)
+
+    quarter = np.sort(rng.choice(n, size=n // 4, replace=False))
+    check(quarter, rng.standard_normal(quarter.size))
+    few = np.array([0, 5, 4095, 4096, n - 4097, n - 1])          # empty tiles in between, both ends
+    check(few, rng.standard_normal(few.size))
+    check(np.arange(n), rng.standard_normal(n))                   # every element
+    check(np.zeros(0, np.int64), np.zeros(0, np.float32))         # nothing
+    check(rng.permutation(quarter), rng.standard_normal(quarter.size))          # not ascending
+    twice = np.sort(np.concatenate([quarter[:1000], quarter[:1000], quarter[5000:6000]]))
+    check(twice, (rng.integers(-8, 9, size=twice.size) / 8.0))    # repeats add up (exact sums)
+
+
+def test_dense_push_coo_large(api, oracle):
+    n = (1 << 22) + 77
+    rng = np.random.default_rng(4)
+    w0 = rng.standard_normal(n).astype(np.float32)
+    t, r = api.DenseTable(w0), oracle.DenseTable(w0)
+    from util import make_optims
+    o_ref, o_gpu = make_optims(oracle, api, 1, {})
+    for step in range(3):
+        idx = np.sort(rng.choice(n, size=n // 5, replace=False)).astype(np.int64)
+        if step == 2:
+            idx = rng.permutation(idx)                            # the scatter path
+        val = (rng.integers(-64, 65, size=idx.size) / 1024.0).astype(np.float32)
+        assert t.PushCoo(o_gpu, idx, val, 0.01) == 0 and r.push_coo(o_ref, idx, val, 0.01) == 0
+        assert_close(t.Pull()[1], r.pull(), "step %d" % step)
+    # an entry outside [0, n) is skipped, the others are applied
+    bad = np.array([0, n], np.int64)
+    one = np.ones(2, np.float32)
+    assert t.PushCoo(o_gpu, bad, one, 0.01) == 0 and r.push_coo(o_ref, bad[:1], one[:1], 0.01) == 0
+    assert_close(t.Pull()[1], r.pull(), "after an out-of-range entry")
