@@ -357,3 +357,33 @@ def test_pull_and_push_in_wire_layout(api, oracle, tmp_path, dim):
     assert t.PushWire(o_gpu, ids[:0], np.zeros(8, np.uint8), 1.0) == 0
     rc, empty = t.PullWire(ids[:0])
     assert rc == 0 and empty.tobytes() == struct.pack("<Q", 0)
+
+
+def test_file_of_a_table_larger_than_the_writers_chunks(api, tmp_path):
+    """2.5 million rows: the writer and the loader both walk the table in chunks of 2^20 rows;
+    rows, states and counters on the far side of a chunk border must come through."""
+    dim, n = 4, 2_500_000
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.05", "seed": "8"})
+    t = api.SparseTable(dim, gi, capacity_hint=n)
+    ids = splitmix64(np.arange(n, dtype=np.uint64))
+    assert t.Pull(api.DeviceArray.from_host(ids), async_=True)[0] == 0
+    o = api.Optim.create(api.OptimType.kAdam)
+    touched = ids[::3]
+    g = (np.random.default_rng(0).integers(-64, 65, size=(touched.size, dim)) / 1024.0).astype(np.float32)
+    assert t.Push(o, touched, g, 0.01) == 0
+    path = str(tmp_path / "big.sparse")
+    assert t.save(path, 9, "big") == 0
+    t2 = api.SparseTable(dim, gi)
+    rc, taken = t2.load_file(path, 9, "big")
+    assert rc == 0 and taken == n == len(t2)
+    probe = np.concatenate([ids[:1000], ids[(1 << 20) - 500:(1 << 20) + 500], ids[-1000:], touched[-1000:]])
+    for st in (3, 4):
+        fa, va, sa, ca = t.fetch(probe, state_type=st)
+        fb, vb, sb, cb = t2.fetch(probe, state_type=st)
+        assert fa.all() and fb.all()
+        assert np.array_equal(va, vb) and np.array_equal(sa, sb) and np.array_equal(ca, cb)
+    a_id, a_val, _, a_steps = t.export()
+    b_id, b_val, _, b_steps = t2.export()
+    oa, ob = np.argsort(a_id), np.argsort(b_id)
+    assert np.array_equal(a_id[oa], b_id[ob]) and np.array_equal(a_val[oa], b_val[ob])
+    assert np.array_equal(a_steps[oa], b_steps[ob]) and int(a_steps.sum()) == touched.size
