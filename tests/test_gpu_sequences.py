@@ -32,8 +32,19 @@ FAMILIES = [[(3, {}), (0, {}), (1, {}), (2, {"momentum": 0.5})],
 
 @pytest.mark.parametrize("seed", range(120))
 def test_random_operation_sequences(api, oracle, tmp_path, seed):
+    _table_sequence(api, oracle, tmp_path, seed, [4, 5, 16, 32, 72])
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_operation_sequences_on_wide_rows(api, oracle, tmp_path, seed):
+    """Rows wider than one pass of a wavefront (more than 256 floats): every kernel walks them in
+    chunks, and a row's step counter must advance once, after its last chunk."""
+    _table_sequence(api, oracle, tmp_path, 500 + seed, [260, 1000, 1030])
+
+
+def _table_sequence(api, oracle, tmp_path, seed, dims):
     rng = np.random.default_rng(1000 + seed)
-    dim = int(rng.choice([4, 5, 16, 32, 72]))
+    dim = int(rng.choice(dims))
     space = int(rng.choice([300, 5000, 200000]))
     gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.05", "seed": str(seed)})
     oi = oracle.init(oracle.INIT_NORMAL, 0.0, 0.05, seed=seed)
