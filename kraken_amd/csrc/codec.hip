@@ -242,14 +242,15 @@ __global__ __launch_bounds__(kCodecBlock) void coo_add_kernel(const long long* _
                                                               const uint32_t* __restrict__ unordered,
                                                               uint32_t* __restrict__ err) {
   if (unordered && !*unordered) return;
-  const int64_t j = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x;
-  if (j >= nnz) return;
-  const long long i = idx[j];
-  if (i < 0 || i >= n) {
-    if (err) atomicOr(err, 1u);
-    return;
+  const int64_t step = (int64_t)gridDim.x * kCodecBlock;
+  for (int64_t j = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x; j < nnz; j += step) {
+    const long long i = idx[j];
+    if (i < 0 || i >= n) {
+      if (err) atomicOr(err, 1u);
+      continue;
+    }
+    unsafeAtomicAdd(&dense[i], val[j]);   // hardware fp32 add, no CAS loop
   }
-  unsafeAtomicAdd(&dense[i], val[j]);   // hardware fp32 add, no CAS loop
 }
 
 static unsigned stream_grid(int64_t n) {
@@ -288,7 +289,9 @@ int32_t coo_densify(const long long* d_idx, const float* d_val, int64_t nnz, flo
                      n, starts, unordered);
   if (nnz) {
     hipLaunchKernelGGL(coo_zero_if_kernel, dim3(stream_grid(n)), block, 0, stream, d_dense, n, unordered);
-    hipLaunchKernelGGL(coo_add_kernel, dim3(per_entry), block, 0, stream, d_idx, d_val, nnz, d_dense, n,
+    // a few workgroups that stride over the entries: when the tiles did the work they only look at
+    // the flag and leave
+    hipLaunchKernelGGL(coo_add_kernel, dim3(stream_grid(nnz)), block, 0, stream, d_idx, d_val, nnz, d_dense, n,
                        (const uint32_t*)unordered, err);
   }
   KRK_HIP(hipGetLastError());
