@@ -398,7 +398,10 @@ int32_t krk_dct_tau(krk_dct* s, float* tau);
 int32_t krk_dct_step(krk_dct* s, uint64_t* step);
 int32_t krk_dct_residual(krk_dct* s, float* out, uint32_t flags);
 /* CooTensorImpl::ToDense for a 1-D shape (t/math.cc:1006-1046): dense[n] is
- * zeroed, then dense[idx[j]] += val[j]. */
+ * zeroed, then dense[idx[j]] += val[j]; entries whose index lies outside [0, n) are skipped.
+ * From 2^22 elements on, strictly ascending indices (what ToCoo produces) are written in one
+ * pass over the output; such a call waits for its launches even with KRK_ASYNC, because the
+ * work space of this object-less entry point is shared between callers. */
 int32_t krk_coo_to_dense(const int64_t* idx, const float* val, int64_t nnz, float* dense,
                          int64_t n, uint32_t flags);
 
