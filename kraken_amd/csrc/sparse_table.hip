@@ -1181,10 +1181,13 @@ int32_t krk_sparse_sync(krk_sparse* t) {
 // The launches of one pull of n > 0 ids into d_out [n, dim]; the caller holds the table's lock
 // and has made room for n more rows.
 static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, float* d_out) {
+  const int64_t rows_before = t->size_ub;           // upper bound of the rows the table holds
   KRK_TRY(sparse_next_epoch(t, n));
   const int per_block = kBlock / t->group;
   const dim3 grid(grid_for(n, per_block)), block(kBlock);
-  if (n >= kTwoLaunchPull) {
+  // Two launches pay when most ids are resident; a request larger than half the table is mostly
+  // new ids (a cold start), which the fused launch inserts in one go at twice the rate.
+  if (n >= kTwoLaunchPull && rows_before >= 2 * n) {
     KRK_TRY(t->scratch[5].reserve((size_t)n * sizeof(uint32_t)));
     uint32_t* todo = t->scratch[5].as<uint32_t>();
     const int parity = t->pull_parity;
