@@ -93,6 +93,52 @@ class Embedding(torch.nn.Module):
         return EmbeddingFunction.apply(self.sparse_table, indices)
 
 
+class JaggedTensor:
+    """pytorch/jagged_tensor.py: tensors that agree in all but their first dimension, kept as one
+    `values` tensor and the `offsets` of the pieces (offsets[0] = 0, offsets[-1] = len(values)),
+    with optional per-row `weights`. Offsets that live on the GPU are not read back to be checked
+    (that would wait for the device); the pooling kernels clamp them to the values' range."""
+
+    def __init__(self, values, offsets, weights=None):
+        if not offsets.is_cuda:
+            o = offsets.tolist()
+            if not o or o[0] != 0 or o[-1] != values.shape[0] or any(b < a for a, b in zip(o, o[1:])):
+                raise ValueError("JaggedTensor's offsets is invalid:%s, values shape:%s" % (o, tuple(values.shape)))
+        if weights is not None and weights.shape != values.shape:
+            raise ValueError("JaggedTensor need values and weights has same shape but got weights shape:%s, "
+                             "values shape:%s." % (tuple(weights.shape), tuple(values.shape)))
+        self._values, self._offsets, self._weights = values, offsets, weights
+
+    def values(self):
+        return self._values
+
+    def offsets(self):
+        return self._offsets
+
+    def weights(self):
+        return self._weights
+
+    def to(self, device):
+        return JaggedTensor(self._values.to(device), self._offsets.to(device),
+                            None if self._weights is None else self._weights.to(device))
+
+    @staticmethod
+    def from_list_tensors(list_values, list_weights=None):
+        """pytorch/jagged_tensor.py:56-84"""
+        assert len(list_values) > 0
+        tail = list_values[0].shape[1:]
+        offsets = [0]
+        for v in list_values:
+            if v.shape[1:] != tail:
+                raise ValueError("JaggedTensor need values has tha same dimension except the first rank.")
+            offsets.append(offsets[-1] + v.shape[0])
+        weights = None
+        if list_weights:
+            assert len(list_values) == len(list_weights)
+            weights = torch.cat(list_weights, dim=0)
+        return JaggedTensor(torch.cat(list_values, dim=0), torch.as_tensor(offsets), weights)
+
+
 class JaggedEmbeddingFunction(torch.autograd.Function):
     """pytorch/jagged_embedding_funcs.py over pytorch/py/jagged_ops.cc, fused with the table."""
 
@@ -140,7 +186,11 @@ class JaggedEmbedding(torch.nn.Module):
         self._mode = 0 if mode == "sum" else 1
         self._patch_value = float(patch_value)
 
-    def forward(self, values, offsets, weights=None):
+    def forward(self, values, offsets=None, weights=None):
+        """forward(JaggedTensor), as the reference's module is called, or forward(values, offsets,
+        weights) with the three tensors themselves."""
+        if isinstance(values, JaggedTensor):
+            values, offsets, weights = values.values(), values.offsets(), values.weights()
         return JaggedEmbeddingFunction.apply(self.sparse_table, values, offsets, weights, self._mode,
                                              self._patch_value)
 

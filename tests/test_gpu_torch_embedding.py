@@ -142,3 +142,35 @@ def test_combine_embedding_forward_backward(mods, oracle):
         rid, rval, _, _ = r.export()
         assert len(t) == len(r)
         assert np.array_equal(t.Pull(rid)[1], rval)                     # dyadic gradients, SGD: exact
+
+
+def test_jagged_tensor(mods, oracle):
+    """test/pytorch/jagged_tensor_test.py: values and offsets of from_list_tensors, also for
+    pieces of more than one dimension; then the module called with a JaggedTensor."""
+    api, te = mods
+    g = torch.Generator(device="cpu").manual_seed(0)
+    for tail in ((), (2, 3)):
+        pieces = [torch.rand((int(n),) + tail, generator=g) for n in torch.randint(1, 11, (5,), generator=g)]
+        jt = te.JaggedTensor.from_list_tensors(pieces)
+        assert torch.equal(jt.values(), torch.cat(pieces, 0))
+        want, at = [0], 0
+        for p in pieces:
+            at += p.shape[0]
+            want.append(at)
+        assert jt.offsets().tolist() == want and jt.weights() is None
+    with pytest.raises(ValueError):
+        te.JaggedTensor(torch.zeros(5), torch.tensor([0, 3, 2, 5]))
+    with pytest.raises(ValueError):
+        te.JaggedTensor(torch.zeros(5), torch.tensor([0, 6]))
+    with pytest.raises(ValueError):
+        te.JaggedTensor.from_list_tensors([torch.zeros(2, 3), torch.zeros(2, 4)])
+    bags = [torch.randint(0, 50, (int(n),), generator=g) for n in (3, 0, 5, 1)]
+    jt = te.JaggedTensor.from_list_tensors(bags).to("cuda")
+    gi, oi = _init(api, oracle, 4)
+    emb = te.JaggedEmbedding(8, initializer=gi, mode="sum", patch_value=0.5)
+    out = emb(jt)
+    ref = oracle.SparseTable(8, oi)
+    ids = torch.cat(bags).numpy().astype(np.uint64)
+    u, inv = oracle.dedup(ids)
+    want = oracle.jagged_forward(ref.pull(u)[1][inv], np.array([0, 3, 3, 8, 9], np.int64), "sum", 0.5)
+    assert np.array_equal(out.detach().cpu().numpy(), want)
