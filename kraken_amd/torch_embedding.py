@@ -16,6 +16,7 @@ import ctypes as C
 import torch
 
 from . import api
+from .configs import as_initializer, as_optim
 
 
 def _stream_ptr():
@@ -32,14 +33,16 @@ def _ids_ptr(indices):
 
 class GpuSparseTable(torch.nn.Parameter):
     """pytorch/sparse_table.py: a Parameter that stands for the table so that autograd calls the
-    Function's backward. The rows are not in this tensor but in the engine's table."""
+    Function's backward. The rows are not in this tensor but in the engine's table.
+    `initializer` and `optim` are the engine's (api.Initializer / api.Optim) or the reference's
+    descriptions of them (configs.NormalInitializer(...), configs.Adagrad(...))."""
 
     def __new__(cls, dimension, initializer=None, optim=None, lr=0.01, capacity_hint=0):
         self = super().__new__(cls, torch.empty(0), requires_grad=True)
         self._dimension = int(dimension)
-        self._table = api.SparseTable(dimension, initializer or api.Initializer.create(
+        self._table = api.SparseTable(dimension, as_initializer(initializer) or api.Initializer.create(
             api.InitializerType.kNormal, {}), capacity_hint=capacity_hint)
-        self._optim = optim or api.Optim.create(api.OptimType.kSGD)
+        self._optim = as_optim(optim) or api.Optim.create(api.OptimType.kSGD)
         self.lr = float(lr)
         return self
 
@@ -206,14 +209,14 @@ class GpuCombineSparseTable(torch.nn.Parameter):
             raise ValueError("dimensions and initializers must have the same length")
         self._dimensions = [int(d) for d in dimensions]
         self._tables = [
-            api.SparseTable(d, (initializers[i] if initializers else None) or api.Initializer.create(
+            api.SparseTable(d, as_initializer(initializers[i] if initializers else None) or api.Initializer.create(
                 api.InitializerType.kNormal, {}), capacity_hint=capacity_hint)
             for i, d in enumerate(self._dimensions)]
         self._members = {}                        # dimension -> positions of its tables in the request
         for i, d in enumerate(self._dimensions):
             self._members.setdefault(d, []).append(i)
         self._groups = {d: api.TableGroup([self._tables[i] for i in idx]) for d, idx in self._members.items()}
-        self._optim = optim or api.Optim.create(api.OptimType.kSGD)
+        self._optim = as_optim(optim) or api.Optim.create(api.OptimType.kSGD)
         self.lr = float(lr)
         return self
 
@@ -293,3 +296,84 @@ class CombineEmbedding(torch.nn.Module):
         if len(indices) != len(self.combine_sparse_table.dimensions()):
             raise ValueError("one index tensor per table")
         return list(CombineEmbeddingFunction.apply(self.combine_sparse_table, *indices))
+
+
+class CombineJaggedEmbeddingFunction(torch.autograd.Function):
+    """The pooling of pytorch/combine_jagged_embedding.py:47-80 fused with the tables: per table
+    one pooled pull forward and one pooled push backward, so the [n, dim] rows that the
+    reference pulls, scales and then pools (JaggedEmbeddingSum/MeanFunction over
+    pytorch/py/jagged_ops.cc) never exist in memory."""
+
+    @staticmethod
+    def forward(ctx, table, modes, patch_values, n_tables, *tensors):
+        values = tensors[:n_tables]
+        offsets = tensors[n_tables:2 * n_tables]
+        weights = tensors[2 * n_tables:]
+        outs, saved, ws = [], [], []
+        for dim in table._members:                  # members run on their group's stream
+            table._on_current_stream(dim)
+        for i, t in enumerate(table.tables()):
+            ids, p_ids = _ids_ptr(values[i])
+            off = offsets[i]
+            if off.dtype != torch.int64 or not off.is_cuda:
+                raise TypeError("offsets must be an int64 CUDA tensor")
+            off = off.contiguous()
+            w = weights[i].contiguous().to(torch.float32) if weights[i] is not None else None
+            bags = off.numel() - 1
+            out = torch.empty((bags, table.dimensions()[i]), dtype=torch.float32, device=ids.device)
+            api._check(api.lib().krk_sparse_pull_pooled(
+                t.h, p_ids, ids.numel(), C.c_void_p(off.data_ptr()), bags,
+                C.c_void_p(w.data_ptr()) if w is not None else None, modes[i], patch_values[i],
+                C.c_void_p(out.data_ptr()), api.DEVICE_PTRS | api.ASYNC), "krk_sparse_pull_pooled")
+            outs.append(out)
+            saved += [ids, off]
+            ws.append(w)
+        ctx.table, ctx.modes, ctx.weights = table, modes, ws
+        ctx.save_for_backward(*saved)
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        table = ctx.table
+        for dim in table._members:
+            table._on_current_stream(dim)
+        for i, t in enumerate(table.tables()):
+            if grads[i] is None:                    # an output the loss never used: nothing to push
+                continue
+            ids, off = ctx.saved_tensors[2 * i], ctx.saved_tensors[2 * i + 1]
+            w = ctx.weights[i]
+            g = grads[i].contiguous().to(torch.float32)
+            api._check(api.lib().krk_sparse_push_pooled(
+                t.h, C.byref(table._optim.raw), C.c_void_p(ids.data_ptr()), ids.numel(), C.c_void_p(off.data_ptr()),
+                off.numel() - 1, C.c_void_p(w.data_ptr()) if w is not None else None, ctx.modes[i],
+                C.c_void_p(g.data_ptr()), table.dimensions()[i], table.lr, api.DEVICE_PTRS | api.ASYNC),
+                "krk_sparse_push_pooled")
+        return (None,) * (4 + 3 * len(table.tables()))
+
+
+class CombineJaggedEmbedding(torch.nn.Module):
+    """pytorch/combine_jagged_embedding.py:11-80: one JaggedTensor per table, pooled per table
+    with its own mode and patch value. Per-row weights scale the rows before the pooling, as
+    the reference's `embeddings *= weights.unsqueeze(-1)` means to (its `if weights:` raises for
+    a tensor of more than one element, so there only a batch without weights gets through)."""
+
+    def __init__(self, dimensions, initializers=None, modes=None, patch_values=None, optim=None, lr=0.01,
+                 capacity_hint=0):
+        super().__init__()
+        if modes:
+            assert len(dimensions) == len(modes)
+            for mode in modes:
+                if mode not in ("sum", "mean"):
+                    raise ValueError("CombineJaggedEmbedding's mode only support sum/mean.")
+        if patch_values:
+            assert len(dimensions) == len(patch_values)
+        self.combine_sparse_table = GpuCombineSparseTable(dimensions, initializers, optim, lr, capacity_hint)
+        self._modes = [0 if m == "sum" else 1 for m in (modes or ["sum"] * len(dimensions))]
+        self._patch_values = [float(p) for p in (patch_values or [0.0] * len(dimensions))]
+
+    def forward(self, inputs):
+        assert len(self._modes) == len(inputs)
+        n = len(inputs)
+        tensors = ([x.values() for x in inputs] + [x.offsets() for x in inputs] + [x.weights() for x in inputs])
+        return list(CombineJaggedEmbeddingFunction.apply(self.combine_sparse_table, self._modes,
+                                                         self._patch_values, n, *tensors))

@@ -174,3 +174,81 @@ def test_jagged_tensor(mods, oracle):
     u, inv = oracle.dedup(ids)
     want = oracle.jagged_forward(ref.pull(u)[1][inv], np.array([0, 3, 3, 8, 9], np.int64), "sum", 0.5)
     assert np.array_equal(out.detach().cpu().numpy(), want)
+
+
+def test_combine_jagged_embedding(mods, oracle):
+    """pytorch/combine_jagged_embedding.py: a JaggedTensor per table, each table with its own
+    mode and patch value; forward and the rows after backward against the oracle."""
+    api, te = mods
+    dims, modes, patches = [8, 8, 4], ["sum", "mean", "sum"], [0.0, 0.25, -1.0]
+    inits = [_init(api, oracle, 20 + i) for i in range(3)]
+    o_ref, o_gpu = make_optims(oracle, api, 3, {})
+    emb = te.CombineJaggedEmbedding(dims, initializers=[g for g, _ in inits], modes=modes, patch_values=patches,
+                                    optim=o_gpu, lr=0.5)
+    refs = [oracle.SparseTable(d, oi) for d, (_, oi) in zip(dims, inits)]
+    rng = np.random.default_rng(3)
+    for step in range(2):
+        batch, inputs = [], []
+        for i in range(3):
+            lengths = rng.choice([0, 1, 2, 4], size=120)
+            off = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int64)
+            ids = rng.integers(0, 200, size=int(off[-1])).astype(np.uint64)
+            w = (2.0 ** rng.integers(-1, 2, size=ids.size)).astype(np.float32) if i == 2 else None
+            batch.append((off, ids, w))
+            inputs.append(te.JaggedTensor(torch.from_numpy(ids.astype(np.int64)).cuda(), torch.from_numpy(off).cuda(),
+                                          torch.from_numpy(w).cuda() if w is not None else None))
+        outs = emb(inputs)
+        assert len(outs) == 3
+        loss, coefs = 0, []
+        for i, (off, ids, w) in enumerate(batch):
+            u, inv = oracle.dedup(ids)
+            rows = refs[i].pull(u)[1][inv]
+            if w is not None:
+                rows = rows * w[:, None]
+            want = oracle.jagged_forward(rows, off, modes[i], patches[i])
+            assert outs[i].shape == (off.size - 1, dims[i])
+            assert_close(outs[i].detach().cpu().numpy(), want, "pooled forward of table %d" % i, rtol=1e-5, atol=1e-6)
+            coef = (rng.integers(-8, 9, size=(off.size - 1, dims[i])) / 16.0).astype(np.float32)
+            coefs.append(coef)
+            if i != 1 or step == 0:                 # table 1's output stays out of the second loss
+                loss = loss + (outs[i] * torch.from_numpy(coef).cuda()).sum()
+        loss.backward()
+        for i, (off, ids, w) in enumerate(batch):
+            if i == 1 and step == 1:
+                continue
+            vg = oracle.jagged_backward(off, coefs[i], modes[i])
+            if w is not None:
+                vg = vg * w[:, None]
+            u2, gs = oracle.dedup_sum(ids, vg)
+            assert refs[i].push(o_ref, u2, gs, 0.5) == 0
+    torch.cuda.synchronize()
+    for i in range(3):
+        rid, rval, _, _ = refs[i].export()
+        assert_close(emb.combine_sparse_table.tables()[i].Pull(rid)[1], rval, "rows of table %d" % i,
+                     rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        te.CombineJaggedEmbedding([4], modes=["max"])
+
+
+def test_modules_take_the_reference_descriptions(mods, oracle):
+    """Initializers and optimizers given as the reference's Python classes
+    (pytorch/initializer.py, pytorch/optim.py) reach the engine with the same meaning."""
+    api, te = mods
+    from kraken_amd import configs
+    dim = 4
+    emb = te.Embedding(dim, initializer=configs.ConstantInitializer(0.5),
+                       optim=configs.Adagrad(eps=1e-6), lr=0.25)
+    ref = oracle.SparseTable(dim, oracle.init(oracle.INIT_CONSTANT, 0.5, 0.0))
+    o_ref, _ = make_optims(oracle, api, 0, {"eps": 1e-6})
+    ids = np.array([5, 9, 5, 2], np.uint64)
+    out = emb(torch.from_numpy(ids.astype(np.int64)).cuda())
+    assert np.array_equal(out.detach().cpu().numpy(), np.full((4, dim), 0.5, np.float32))
+    coef = np.arange(16, dtype=np.float32).reshape(4, dim) / 8
+    (out * torch.from_numpy(coef).cuda()).sum().backward()
+    torch.cuda.synchronize()
+    u, inv = oracle.dedup(ids)
+    assert np.array_equal(ref.pull(u)[1], np.full((3, dim), 0.5, np.float32))
+    u2, gs = oracle.dedup_sum(ids, coef)
+    assert ref.push(o_ref, u2, gs, 0.25) == 0
+    rid, rval, _, _ = ref.export()
+    assert_close(emb.sparse_table.table().Pull(rid)[1], rval, "rows after an Adagrad step", rtol=1e-5, atol=1e-6)
