@@ -20,8 +20,11 @@
  *     call (t/math.cc:455-464, 486-495), so no reproducible output exists.
  *     The oracle defines a counter-based generator instead (kro_init_row) and
  *     only its distribution moments can be compared with the reference.
- *   Adam AMSGrad branch (bias-corrected max, unlike torch)  parity unpinned
- *     beyond hand-computed steps.
+ *   Adam AMSGrad branch (bias-corrected max, unlike torch)  pinned by closed
+ *     forms: an impulse gradient (the maximum keeps the first, exact value;
+ *     weights follow sum 1/(2^t - 1)), doubling gradients (the maximum is
+ *     always the newest value: plain Adam, which torch pins), a constant
+ *     gradient and a single step (both reduce to torch's AMSGrad).
  */
 #ifndef KRAKEN_ORACLE_H_
 #define KRAKEN_ORACLE_H_

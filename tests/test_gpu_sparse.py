@@ -260,3 +260,38 @@ def test_config1_plumbing(api, oracle):
     og = np.argsort(gid)                                      # rows of one request are numbered in no particular order
     assert np.array_equal(gid[og], ids0)
     assert_close(gval[og], rval[np.argsort(rid)], "final table", rtol=1e-5, atol=1e-7)
+
+
+def test_adam_amsgrad_impulse_closed_form(api, oracle):
+    """ps/optim/adam.cc:66-75 on the device against what the mathematics fixes, not against the
+    oracle: one gradient s*a, zeros afterwards, beta1 = beta2 = 1/2, eps = 1. The corrected second
+    moment peaks at the first step with exactly a^2, so the running maximum stays a^2 and
+    W_T = W_0 - lr * s*a/(a + 1) * sum_{t<=T} 1/(2^t - 1). Rows are pushed from different steps
+    on, so each carries its own count."""
+    from fractions import Fraction
+    dim = 8
+    a = np.array([1.0, 2.0, 4.0, 0.5, 8.0, 0.25, 1.0, 16.0], np.float32)
+    sgn = np.array([1, -1, 1, -1, -1, 1, -1, 1], np.float32)
+    gi, _ = _const_init(api, oracle, 0.0)
+    t = api.SparseTable(dim, gi)
+    ids = np.array([3, 2**50 + 1, 17], np.uint64)
+    w0 = np.arange(ids.size * dim, dtype=np.float32).reshape(ids.size, dim) / 16
+    t.load(ids, w0)
+    o = api.Optim.create(api.OptimType.kAdam, {"amsgrad": "true", "beta1": "0.5", "beta2": "0.5", "eps": "1.0"})
+    lr = 0.125
+    start = [0, 1, 3]                             # the step at which each row gets its impulse
+    for step in range(6):
+        live = [k for k in range(ids.size) if step >= start[k]]
+        g = np.stack([(sgn * a) if step == start[k] else np.zeros(dim, np.float32) for k in live])
+        assert t.Push(o, ids[live], g, lr) == 0
+    rc, got = t.Pull(ids)
+    assert rc == 0
+    for k in range(ids.size):
+        T = 6 - start[k]
+        series = float(sum(Fraction(1, 2 ** n - 1) for n in range(1, T + 1)))
+        want = w0[k].astype(np.float64) - lr * (sgn * a / (a + 1.0)).astype(np.float64) * series
+        assert_close(got[k], want, "row %d after %d steps" % (k, T), rtol=1e-6, atol=1e-6)
+    gid, _, vmax, steps = t.export(state_type=5)
+    order = np.argsort(gid)
+    assert np.array_equal(vmax[order], np.tile(a * a, (3, 1)))
+    assert sorted(steps.tolist()) == [3, 5, 6]

@@ -331,6 +331,54 @@ def test_adam_amsgrad_special_cases(oracle):
     np.testing.assert_allclose(v.state(oracle.ST_SECOND_MOMENT_MAX), vmax, rtol=1e-5)
 
 
+def test_adam_amsgrad_closed_forms(oracle):
+    """What the mathematics fixes for the branch of ps/optim/adam.cc:66-75, without restating it.
+
+    Impulse: g_1 = s*a, zero afterwards, beta1 = beta2 = 1/2, eps = 1. Then m_t = s*a/2^t and
+    v_t = a^2/2^t, the corrected moments are s*a/(2^t - 1) and a^2/(2^t - 1), so the corrected
+    second moment peaks at t = 1 with exactly a^2 and the running maximum stays there: every step
+    divides by sqrt(a^2) + 1, and
+
+        W_T = W_0 - lr * s*a/(a + 1) * sum_{t=1..T} 1/(2^t - 1).
+
+    The partial sums are 1, 4/3, 31/21, 54/35, ... A maximum taken
+    over the uncorrected moment (torch's order), no maximum at all, eps inside the root or a
+    missing correction of m each give a different W_2 already.
+
+    Growth: |g_t| doubling makes the corrected second moment grow at every step, so the maximum
+    is always the newest value and the result is plain Adam's, which torch pins."""
+    a = np.array([1.0, 2.0, 4.0, 0.5, 8.0, 0.25], np.float32)
+    sgn = np.array([1, -1, 1, -1, -1, 1], np.float32)
+    w0 = np.array([0.5, -1.0, 2.0, 0.0, -0.25, 3.0], np.float32)
+    lr = 0.125
+    o = oracle.optim(oracle.ADAM, amsgrad=True, beta1=0.5, beta2=0.5, eps=1.0)
+    from fractions import Fraction
+    exact = [sum(Fraction(1, 2 ** t - 1) for t in range(1, T + 1)) for T in range(1, 6)]
+    assert exact[:4] == [Fraction(1), Fraction(4, 3), Fraction(31, 21), Fraction(54, 35)]
+    v = oracle.Value(w0)
+    zero = np.zeros_like(w0)
+    for T in range(1, 6):
+        assert v.update(o, (sgn * a) if T == 1 else zero, lr) == 0
+        want = w0.astype(np.float64) - lr * (sgn * a / (a + 1.0)).astype(np.float64) * float(exact[T - 1])
+        np.testing.assert_allclose(v.val, want, rtol=1e-6, atol=1e-7)
+        np.testing.assert_array_equal(v.state(oracle.ST_SECOND_MOMENT_MAX), a * a)
+    assert v.steps == 5
+
+    w0, _ = _inputs(seed=6)
+    rng = np.random.default_rng(7)
+    base = (rng.choice([-1.0, 1.0], size=w0.size) * rng.uniform(0.5, 1.0, size=w0.size)).astype(np.float32)
+    grads = [base * np.float32(2.0 ** t) for t in range(6)]
+    for conf in ({"beta1": 0.5, "beta2": 0.5}, {}):
+        o = oracle.optim(oracle.ADAM, amsgrad=True, **conf)
+        v = _oracle_run(oracle, o, w0, grads, 1e-2)
+        w, st = _torch_run(lambda t, ps, lr: t.optim.Adam(
+            ps, lr=lr, betas=(conf.get("beta1", 0.9), conf.get("beta2", 0.999))), w0, grads, 1e-2)
+        np.testing.assert_allclose(v.val, w, rtol=1e-5, atol=1e-6)
+        # the maximum is the newest corrected second moment
+        bc2 = 1.0 - conf.get("beta2", 0.999) ** 6
+        np.testing.assert_allclose(v.state(oracle.ST_SECOND_MOMENT_MAX), st["exp_avg_sq"].numpy() / bc2, rtol=1e-5)
+
+
 @pytest.mark.parametrize("conf", [
     {}, {"alpha": 0.9}, {"centered": True}, {"momentum": 0.7}, {"momentum": 0.7, "centered": True},
     {"weight_decay": 0.03, "alpha": 0.9, "eps": 1e-6},
