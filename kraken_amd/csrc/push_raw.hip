@@ -844,9 +844,11 @@ static int32_t dedup_layout(int64_t n, size_t extra_bytes, DedupWork* w) {
 }
 
 // unique ids in first-occurrence order into d_uids, every position's slot into w.slot_of (the
-// slot then holds the id's index in the unique list); *u = number of unique ids
-static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, uint64_t* d_uids, hipStream_t s,
-                          int32_t* u) {
+// slot then holds the id's index in the unique list), every position's index in the unique list
+// into d_inv (when not null); *u = number of unique ids. The count is read back last, so the
+// call waits for the device once.
+static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, uint64_t* d_uids,
+                          long long* d_inv, hipStream_t s, int32_t* u) {
   KRK_HIP(hipMemsetAsync(w.slots, 0xFF, (w.cap + 1) * sizeof(DSlot), s));
   const dim3 grid(grid_for(n, kBlock)), block(kBlock);
   hipLaunchKernelGGL(dedup_claim_kernel, dim3(grid_for(n, kDedupBlock)), dim3(kDedupBlock), 0, s, w.slots,
@@ -855,6 +857,7 @@ static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, 
   KRK_HIP(hipGetLastError());
   KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
   hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids);
+  if (d_inv) hipLaunchKernelGGL(dedup_inv_kernel, grid, block, 0, s, w.slots, w.slot_of, n, d_inv);
   KRK_HIP(hipGetLastError());
   KRK_HIP(hipMemcpy(u, w.d_total, sizeof(*u), hipMemcpyDeviceToHost));
   return KRK_SUCCESS;
@@ -889,12 +892,7 @@ int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, 
   }
   hipStream_t s = nullptr;
   int32_t u = 0;
-  KRK_TRY(dedup_core(w, d_ids, n, d_uids, s, &u));
-  if (inv) {
-    hipLaunchKernelGGL(dedup_inv_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, w.slots, w.slot_of, n,
-                       d_inv);
-    KRK_HIP(hipGetLastError());
-  }
+  KRK_TRY(dedup_core(w, d_ids, n, d_uids, inv ? d_inv : nullptr, s, &u));
   *n_unique = u;
   if (host) {
     KRK_HIP(hipMemcpy(uids, d_uids, (size_t)u * 8, hipMemcpyDeviceToHost));
@@ -950,12 +948,7 @@ int32_t krk_dedup_sum(const uint64_t* ids, int64_t n, const float* grads, int64_
   }
   hipStream_t s = nullptr;
   int32_t u = 0;
-  KRK_TRY(dedup_core(w, d_ids, n, d_uids, s, &u));
-  if (inv) {
-    hipLaunchKernelGGL(dedup_inv_kernel, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, w.slots, w.slot_of, n,
-                       d_inv);
-    KRK_HIP(hipGetLastError());
-  }
+  KRK_TRY(dedup_core(w, d_ids, n, d_uids, inv ? d_inv : nullptr, s, &u));
   // positions sorted by unique index (stable: position order inside a run, as
   // worker/emitter.cc:527-529 adds them), every run summed and stored as row `index` of sums
   uint32_t miss_key = 1;
