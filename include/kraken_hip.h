@@ -268,12 +268,25 @@ int32_t krk_sparse_states(krk_sparse* t, uint32_t* mask);
 int32_t krk_sparse_import_state(krk_sparse* t, const uint64_t* ids, int64_t n, int32_t state_type,
                                 const float* state, const int64_t* steps, uint32_t flags);
 /* The clean-up after a cluster change (ps/ps.cc:92-109: SkipList::Remove on every row routed
- * elsewhere). The routing decision stays on the host: it reads the ids (krk_sparse_export),
- * picks those that go and hands them here. Ids that are not present are ignored; *erased (may
- * be NULL) receives how many rows went. Rows stay densely numbered, so the row numbers
+ * elsewhere). The caller names the rows that go: krk_sparse_select_routed picks them by the
+ * reference's routing rule on the device, or the host decides from krk_sparse_export's ids.
+ * Ids that are not present are ignored; *erased (may be NULL) receives how many rows went. Rows stay densely numbered, so the row numbers
  * krk_sparse_lookup reports change. Costs a pass over the whole index; blocking. */
 int32_t krk_sparse_erase(krk_sparse* t, const uint64_t* ids, int64_t n, int64_t* erased,
                          uint32_t flags);
+/* The ids of the rows that Router::Hit(utils::Hash(table_id, sparse_id)) (common/router.cc:262-277,
+ * common/utils.h:30-48) gives to node_id (owned != 0: the transfer-out walk, ps/ps.cc:289-321,
+ * with the target's id) or to any other node (owned == 0: the clean-up, ps/ps.cc:92-109, with
+ * this server's id), in row order (krk_sparse_export's), decided on the device from the table's
+ * own keys. The ring is Router::vnodes() as two HOST arrays whatever the flags say: hash_v in
+ * ascending order and the node id of each virtual node; an empty ring owns nothing. ids holds
+ * `capacity` entries; *count receives how many were selected; KRK_E_CAPACITY (nothing written,
+ * *count = the room needed) when capacity is too small. Feed the ids to krk_sparse_fetch /
+ * krk_sparse_erase. Blocking. */
+int32_t krk_sparse_select_routed(krk_sparse* t, uint64_t table_id, const uint64_t* ring_hash,
+                                 const uint64_t* ring_node, int64_t ring_n, uint64_t node_id,
+                                 int32_t owned, uint64_t* ids, int64_t capacity, int64_t* count,
+                                 uint32_t flags);
 
 /* ---- table files ------------------------------------------------------------- */
 /* Checkpoint::SaveSparseTable (checkpoint/checkpoint.cc:465-509): the table as a *.sparse file in

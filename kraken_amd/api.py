@@ -112,6 +112,9 @@ EXPORTS = {
     "krk_dense_load_file": (C.c_int32, [C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_uint64), C.c_char_p,
                                         C.c_size_t, C.POINTER(C.c_int64), C.POINTER(C.c_int32)]),
     "krk_sparse_erase": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.POINTER(C.c_int64), C.c_uint32]),
+    "krk_sparse_select_routed": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p, C.c_int64,
+                                             C.c_uint64, C.c_int32, C.c_void_p, C.c_int64,
+                                             C.POINTER(C.c_int64), C.c_uint32]),
     "krk_dedup": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64),
                               C.c_uint32]),
     "krk_dedup_sum": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
@@ -498,6 +501,25 @@ class SparseTable:
         gone = C.c_int64()
         _check(lib().krk_sparse_erase(self.h, _ptr(ids), ids.size, C.byref(gone), 0), "krk_sparse_erase")
         return gone.value
+
+    def select_routed(self, table_id, ring, node_id, owned=True):
+        """The ids of the rows that the reference's router (common/router.cc:262-277 over
+        utils::Hash(table_id, id)) gives to node_id (owned) or to other nodes (not owned), in
+        row order (export's). ring = [(hash_v, node_id), ...] in ascending hash order."""
+        rh = np.ascontiguousarray([h for h, _ in ring], dtype=np.uint64)
+        rn = np.ascontiguousarray([n for _, n in ring], dtype=np.uint64)
+        count = C.c_int64()
+        rc = lib().krk_sparse_select_routed(self.h, int(table_id), _ptr(rh), _ptr(rn), len(ring), int(node_id),
+                                            1 if owned else 0, None, 0, C.byref(count), 0)
+        if rc == SUCCESS:
+            return np.empty(0, np.uint64)
+        if rc != E_CAPACITY:
+            _check(rc, "krk_sparse_select_routed")
+        ids = np.empty(count.value, np.uint64)
+        _check(lib().krk_sparse_select_routed(self.h, int(table_id), _ptr(rh), _ptr(rn), len(ring), int(node_id),
+                                              1 if owned else 0, _ptr(ids), ids.size, C.byref(count), 0),
+               "krk_sparse_select_routed")
+        return ids[:count.value]
 
     def export(self, state_type=None):
         """-> ids[rows], vals[rows, dim], state[rows, dim] or None, steps[rows] (insertion order)"""

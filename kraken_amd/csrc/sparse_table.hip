@@ -572,6 +572,53 @@ __global__ __launch_bounds__(kBlock) void import_state_kernel(TableView tv, cons
   }
 }
 
+// ---- which rows a node of the cluster owns ------------------------------------------------------
+// common/utils.h:30-44: the mixer behind utils::Hash, which routes rows to servers.
+__host__ __device__ inline unsigned long long route_hash64(unsigned long long v) {
+  v = v * 3935559000370003845ull + 2691343689449507681ull;
+  v ^= v >> 21;
+  v ^= v << 37;
+  v ^= v >> 4;
+  v *= 4768777513237032717ull;
+  v ^= v << 20;
+  v ^= v >> 41;
+  v ^= v << 5;
+  return v;
+}
+
+// flag[r] = 1 where Router::Hit(utils::Hash(table_id, id of row r)) (common/router.cc:262-277,
+// common/utils.h:46-48) is node_id (want_owned) or another node (!want_owned). The ring is the
+// virtual nodes in ascending hash order: a hash belongs to the first one at or above it, or to
+// the first of the ring when it lies above them all; an empty ring owns nothing.
+__global__ __launch_bounds__(kBlock) void route_flag_kernel(const unsigned long long* __restrict__ row_key,
+                                                            int64_t rows, unsigned long long table_hash,
+                                                            const unsigned long long* __restrict__ ring_hash,
+                                                            const unsigned long long* __restrict__ ring_node,
+                                                            int m, unsigned long long node_id, bool want_owned,
+                                                            int32_t* __restrict__ flag) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r >= rows) return;
+  const unsigned long long hv = table_hash ^ route_hash64(row_key[r]);
+  unsigned long long owner = ~0ull;
+  if (m > 0) {
+    int lo = 0, hi = m;
+    while (lo < hi) {
+      const int mid = lo + ((hi - lo) >> 1);
+      if (ring_hash[mid] < hv) lo = mid + 1; else hi = mid;
+    }
+    owner = ring_node[lo == m ? 0 : lo];
+  }
+  flag[r] = ((owner == node_id) == want_owned) ? 1 : 0;
+}
+
+__global__ __launch_bounds__(kBlock) void route_emit_kernel(const unsigned long long* __restrict__ row_key,
+                                                            int64_t rows, const int32_t* __restrict__ flag,
+                                                            const int32_t* __restrict__ rank,
+                                                            unsigned long long* __restrict__ ids) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r < rows && flag[r]) ids[rank[r]] = row_key[r];
+}
+
 // ---- erase -------------------------------------------------------------------
 // Rows are kept dense: the rows that go leave holes, and the live rows at the tail move into
 // the holes below the new row count. Sources lie at or above that count, destinations below
@@ -1694,6 +1741,68 @@ int32_t krk_sparse_erase(krk_sparse* t, const uint64_t* ids, int64_t n, int64_t*
   KRK_HIP(hipStreamSynchronize(t->stream));
   t->size_ub = keep;
   t->layout_version++;
+  return KRK_SUCCESS;
+}
+
+int32_t krk_sparse_select_routed(krk_sparse* t, uint64_t table_id, const uint64_t* ring_hash,
+                                 const uint64_t* ring_node, int64_t ring_n, uint64_t node_id, int32_t owned,
+                                 uint64_t* ids, int64_t capacity, int64_t* count, uint32_t flags) {
+  KRK_TRY(check_table(t));
+  KRK_TRY(check_flags(flags));
+  if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;   // the count comes back by value
+  if (!count || ring_n < 0 || ring_n > (1 << 24) || (ring_n > 0 && (!ring_hash || !ring_node)) || capacity < 0 ||
+      (capacity > 0 && !ids))
+    return KRK_E_ARGUMENT;
+  for (int64_t i = 1; i < ring_n; ++i) {
+    if (ring_hash[i - 1] > ring_hash[i]) {
+      set_error("krk_sparse_select_routed: the ring must be in ascending hash order");
+      return KRK_E_ARGUMENT;
+    }
+  }
+  *count = 0;
+  std::lock_guard<std::mutex> lk(t->mu);
+  KRK_TRY(sparse_finish(t, 0));
+  KRK_TRY(refresh_rows(t));
+  const int64_t rows = t->size_ub;
+  if (rows == 0) return KRK_SUCCESS;
+  // work space: flag[rows] | rank[rows] | scan scratch | total | ring hashes | ring nodes
+  const size_t r4 = ((size_t)rows * 4 + 255) & ~(size_t)255;
+  const size_t scan_b = (scan_scratch_bytes(rows) + 255) & ~(size_t)255;
+  const size_t ring_b = ((size_t)ring_n * 8 + 255) & ~(size_t)255;
+  KRK_TRY(t->scratch[5].reserve(2 * r4 + scan_b + 256 + 2 * ring_b + 16));
+  char* base = t->scratch[5].as<char>();
+  int32_t* flag = reinterpret_cast<int32_t*>(base);
+  int32_t* rank = reinterpret_cast<int32_t*>(base + r4);
+  void* scan_tmp = base + 2 * r4;
+  int32_t* d_total = reinterpret_cast<int32_t*>(base + 2 * r4 + scan_b);
+  unsigned long long* d_ring_hash = reinterpret_cast<unsigned long long*>(base + 2 * r4 + scan_b + 256);
+  unsigned long long* d_ring_node = reinterpret_cast<unsigned long long*>(base + 2 * r4 + scan_b + 256 + ring_b);
+  if (ring_n) {
+    // pageable sources: these copies return once the bytes are staged
+    KRK_HIP(hipMemcpyAsync(d_ring_hash, ring_hash, (size_t)ring_n * 8, hipMemcpyHostToDevice, t->stream));
+    KRK_HIP(hipMemcpyAsync(d_ring_node, ring_node, (size_t)ring_n * 8, hipMemcpyHostToDevice, t->stream));
+  }
+  hipLaunchKernelGGL(route_flag_kernel, dim3(grid_for(rows, kBlock)), dim3(kBlock), 0, t->stream, t->row_key, rows,
+                     route_hash64(table_id), d_ring_hash, d_ring_node, (int)ring_n, (unsigned long long)node_id,
+                     owned != 0, flag);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(exclusive_scan_i32(flag, rank, rows, d_total, scan_tmp, t->stream));
+  int32_t total = 0;
+  KRK_HIP(hipMemcpyAsync(&total, d_total, sizeof(total), hipMemcpyDeviceToHost, t->stream));
+  KRK_HIP(hipStreamSynchronize(t->stream));
+  *count = total;
+  if (total > capacity) {
+    set_error("krk_sparse_select_routed: %lld ids selected, room for %lld", (long long)total, (long long)capacity);
+    return KRK_E_CAPACITY;
+  }
+  if (total == 0) return KRK_SUCCESS;
+  unsigned long long* d_ids;
+  KRK_TRY(t->output(reinterpret_cast<unsigned long long*>(ids), (size_t)total, flags, 0, &d_ids));
+  hipLaunchKernelGGL(route_emit_kernel, dim3(grid_for(rows, kBlock)), dim3(kBlock), 0, t->stream, t->row_key, rows,
+                     flag, rank, d_ids);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(t->output_back(reinterpret_cast<unsigned long long*>(ids), (size_t)total, flags, 0));
+  KRK_HIP(hipStreamSynchronize(t->stream));
   return KRK_SUCCESS;
 }
 

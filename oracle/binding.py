@@ -71,6 +71,8 @@ def lib():
     sig = {
         "kro_hash64": (u64, [u64]),
         "kro_hash64_pair": (u64, [u64, u64]),
+        "kro_ring_hit": (u64, [pu, pu, i64, u64]),
+        "kro_route_owner": (u64, [pu, pu, i64, u64, u64]),
         "kro_hit_slot": (u64, [u64]),
         "kro_splitmix64": (u64, [u64]),
         "kro_optim_defaults": (None, [i32, C.POINTER(Optim)]),
@@ -192,6 +194,16 @@ def optim(type_, **conf):
         else:
             raise KeyError(k)
     return o
+
+
+def route_owners(ring, table_id, ids):
+    """common/router.cc:262-277 over utils::Hash(table_id, id): the owner of every id.
+    ring = [(hash_v, node_id), ...] in ascending hash order."""
+    rh = np.ascontiguousarray([h for h, _ in ring], dtype=np.uint64)
+    rn = np.ascontiguousarray([n for _, n in ring], dtype=np.uint64)
+    L = lib()
+    return np.array([L.kro_route_owner(_p(rh, C.c_uint64), _p(rn, C.c_uint64), len(ring), int(table_id), int(i))
+                     for i in np.asarray(ids, dtype=np.uint64)], dtype=np.uint64)
 
 
 def init(type_, a=0.0, b=0.0, seed=0):

@@ -37,6 +37,25 @@ uint64_t kro_hash64_pair(uint64_t a, uint64_t b) {
   return kro_hash64(a) ^ kro_hash64(b);
 }
 
+/* common/router.cc:262-277 (Router::Hit): the ring is the virtual nodes in ascending hash
+ * order; a hash belongs to the first virtual node at or above it, or to the first of the ring
+ * when it lies above them all. An empty ring owns nothing (uint64 -1). */
+uint64_t kro_ring_hit(const uint64_t* ring_hash, const uint64_t* ring_node, int64_t m, uint64_t hv) {
+  if (m <= 0) return UINT64_MAX;
+  int64_t lo = 0, hi = m;                        /* std::lower_bound */
+  while (lo < hi) {
+    int64_t mid = lo + (hi - lo) / 2;
+    if (ring_hash[mid] < hv) lo = mid + 1; else hi = mid;
+  }
+  return ring_node[lo == m ? 0 : lo];
+}
+
+/* ps/ps.cc:100, 306: who owns row `id` of table `table_id` */
+uint64_t kro_route_owner(const uint64_t* ring_hash, const uint64_t* ring_node, int64_t m,
+                         uint64_t table_id, uint64_t id) {
+  return kro_ring_hit(ring_hash, ring_node, m, kro_hash64_pair(table_id, id));
+}
+
 /* common/parallel_skip_list.h:12-21 (identity hash, 8 slots), :100-102 */
 #define KRO_SLOTS 8
 uint64_t kro_hit_slot(uint64_t id) { return id % KRO_SLOTS; }

@@ -13,8 +13,8 @@
  * temporary per elementwise operation in the optimizer chains.
  *
  * Parity status of each group (what pins it is in the tests that load this):
- *   hash, skip list, dedup, codec KATs, optimizers (closed forms + library
- *   optimizers), COO densify ............................ pinned
+ *   hash, skip list, routing ring, dedup, codec KATs, optimizers (closed
+ *   forms + library optimizers), COO densify ............ pinned
  *   Normal/Uniform/Xavier row initialisers ............... parity unpinned:
  *     the reference seeds a fresh mt19937 from std::random_device on every
  *     call (t/math.cc:455-464, 486-495), so no reproducible output exists.
@@ -97,6 +97,11 @@ typedef struct kro_init {
 /* ---- integer helpers ---------------------------------------------------- */
 uint64_t kro_hash64(uint64_t v);                 /* common/utils.h:30-44 */
 uint64_t kro_hash64_pair(uint64_t a, uint64_t b);/* common/utils.h:46-48 */
+/* common/router.cc:262-277; ring_hash ascending, m virtual nodes */
+uint64_t kro_ring_hit(const uint64_t* ring_hash, const uint64_t* ring_node, int64_t m, uint64_t hv);
+/* ps/ps.cc:100, 306 : Router::Hit(utils::Hash(table_id, sparse_id)) */
+uint64_t kro_route_owner(const uint64_t* ring_hash, const uint64_t* ring_node, int64_t m,
+                         uint64_t table_id, uint64_t id);
 uint64_t kro_hit_slot(uint64_t id);              /* common/parallel_skip_list.h:12-21,100-102 */
 uint64_t kro_splitmix64(uint64_t x);             /* harness generator, no reference counterpart */
 

@@ -138,3 +138,56 @@ def test_values_move_between_tables_with_their_state(api, oracle, name, type_, c
     rc, want = ref.pull(ids)
     assert_close(dst.Pull(moved)[1], want[::2], name + " moved half")
     assert_close(src.Pull(rest)[1], want[1::2], name + " staying half")
+
+
+def test_select_routed_follows_the_references_ring(api, oracle):
+    """The clean-up (ps/ps.cc:92-109) and the transfer-out walk (ps/ps.cc:289-321) decide by
+    Router::Hit(utils::Hash(table_id, sparse_id)). Rings built by the reference's own router
+    (tests/golden/ref_router.json); the owner of every row by the oracle, itself pinned on the
+    same file."""
+    import json
+    import os
+    cases = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "ref_router.json")))
+    dim = 4
+    for case in cases:
+        ring = [(int(h), int(n)) for h, n in case["ring"]]
+        table_id = case["table_id"]
+        t, _ = _tables(api, oracle, dim, seed=3)
+        # the ids the reference answered for, and many more
+        ids = np.concatenate([np.array([int(i) for i, _ in case["ids"]], np.uint64),
+                              splitmix64(np.arange(1000, 41000, dtype=np.uint64))])
+        ids = ids[np.sort(np.unique(ids, return_index=True)[1])]
+        assert t.Pull(ids)[0] == 0
+        golden = {int(i): int(o) for i, o in case["ids"]}
+        for i, o in zip(ids[:len(golden)].tolist(), oracle.route_owners(ring, table_id, ids[:len(golden)]).tolist()):
+            assert golden[i] == o
+        ids = t.export()[0]                                   # row order: what a selection follows
+        owners = oracle.route_owners(ring, table_id, ids)
+        nodes = sorted(set(n for _, n in ring))
+        total = 0
+        for node in nodes + [max(nodes) + 1]:                 # the last one owns nothing
+            mine = t.select_routed(table_id, ring, node, owned=True)
+            assert np.array_equal(mine, ids[owners == node])  # row order
+            others = t.select_routed(table_id, ring, node, owned=False)
+            assert np.array_equal(others, ids[owners != node])
+            total += mine.size
+        assert total == ids.size
+        # another table id routes the same ids differently
+        if len(nodes) > 1:
+            assert not np.array_equal(oracle.route_owners(ring, table_id + 1, ids), owners)
+            assert np.array_equal(t.select_routed(table_id + 1, ring, nodes[0]),
+                                  ids[oracle.route_owners(ring, table_id + 1, ids) == nodes[0]])
+        # the clean-up itself: drop what belongs to the others, keep the rest
+        keep = ids[owners == nodes[0]]
+        gone = t.erase(t.select_routed(table_id, ring, nodes[0], owned=False))
+        assert gone == ids.size - keep.size and len(t) == keep.size
+        assert np.array_equal(np.sort(t.export()[0]), np.sort(keep))
+        assert t.select_routed(table_id, ring, nodes[0], owned=False).size == 0
+    # an empty ring owns nothing; an empty table selects nothing; an unsorted ring is refused
+    t, _ = _tables(api, oracle, dim, seed=4)
+    assert t.select_routed(1, [(5, 0)], 0).size == 0
+    assert t.Pull(np.arange(10, dtype=np.uint64))[0] == 0
+    assert t.select_routed(1, [], 0).size == 0 and t.select_routed(1, [], 0, owned=False).size == 10
+    assert t.select_routed(1, [(5, 0)], 0).size == 10          # one virtual node owns the whole ring
+    with pytest.raises(api.KrakenHipError):
+        t.select_routed(1, [(9, 0), (5, 1)], 0)

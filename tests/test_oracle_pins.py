@@ -10,6 +10,7 @@ Sources of truth used here, none of which is the oracle's own formula retyped:
     rmsprop.h:10-11);
   * brute force and invariants on small inputs.
 """
+import ctypes as C
 import json
 import os
 
@@ -30,6 +31,44 @@ def test_hash64_matches_reference_vectors(oracle):
         assert L.kro_hash64(int(k)) == int(h)
     for a, b, h in g["hash64_pair"]:
         assert L.kro_hash64_pair(int(a), int(b)) == int(h)
+
+
+def test_routing_ring_matches_reference_vectors(oracle):
+    """Router::Hit(utils::Hash(table, id)) as ps/ps.cc:100, 306 call it, against rings the
+    reference's own router built and answered (tests/golden/make_ref_router_vectors.py)."""
+    L = oracle.lib()
+    for case in json.load(open(os.path.join(GOLDEN, "ref_router.json"))):
+        ring = [(int(h), int(n)) for h, n in case["ring"]]
+        assert ring == sorted(ring) and len(ring) == 3 * len(case["nodes"])      # router.cc:12, 153-157
+        rh = np.array([h for h, _ in ring], np.uint64)
+        rn = np.array([n for _, n in ring], np.uint64)
+        ph, pn = rh.ctypes.data_as(C.POINTER(C.c_uint64)), rn.ctypes.data_as(C.POINTER(C.c_uint64))
+        for hv, owner in case["hits"]:
+            assert L.kro_ring_hit(ph, pn, len(ring), int(hv)) == int(owner)
+        ids = [int(i) for i, _ in case["ids"]]
+        want = np.array([int(o) for _, o in case["ids"]], np.uint64)
+        assert np.array_equal(oracle.route_owners(ring, case["table_id"], ids), want)
+        if len(case["nodes"]) > 1:
+            assert len(set(want.tolist())) > 1
+    assert L.kro_ring_hit(None, None, 0, 5) == 2**64 - 1                          # router.cc:263-265
+
+
+def test_routing_ring_matches_reference_live(oracle):
+    """The same against the reference's router compiled in place, where that binary exists."""
+    tool = os.path.join(os.path.dirname(__file__), "..", "oracle", "_ref", "ref_router")
+    if not os.path.exists(tool):
+        pytest.skip("oracle/_ref/ref_router is not built (no reference tree here)")
+    import subprocess
+    text = subprocess.check_output([tool, "99", "500", "n0", "n1", "n2", "n3"], text=True)
+    ring, ids = [], []
+    for line in text.splitlines():
+        kind, a, b = line.split()
+        if kind == "vnode":
+            ring.append((int(a), int(b)))
+        elif kind == "id":
+            ids.append((int(a), int(b)))
+    got = oracle.route_owners(ring, 99, [i for i, _ in ids])
+    assert np.array_equal(got, np.array([o for _, o in ids], np.uint64))
 
 
 def test_container_matches_reference_vectors(oracle):
