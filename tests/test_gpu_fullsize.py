@@ -172,6 +172,18 @@ def test_config3_deepfm_full(api, oracle):
     gid, _, _, gsteps = None, None, None, None
     rows = t.lookup(u[sample][:1000])
     assert (rows >= 0).all() and len(t) == space
+    # who owns which of the 1e8 rows under a ring of five nodes (the walks of ps/ps.cc:92-109 and
+    # :289-321 at full size): the nodes' shares partition the table, and a sample of every share
+    # is what the oracle's router says
+    ring = sorted((int(splitmix64(np.array([7000 + k], np.uint64))[0]), k % 5) for k in range(15))
+    total = 0
+    for node in range(5):
+        mine = t.select_routed(42, ring, node)
+        total += mine.size
+        assert mine.size > space // 50
+        probe = mine[rng.choice(mine.size, size=2000, replace=False)]
+        assert (oracle.route_owners(ring, 42, probe) == node).all()
+    assert total == space
 
 
 def test_config5_codec_full(api, oracle):
