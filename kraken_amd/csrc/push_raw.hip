@@ -259,12 +259,21 @@ constexpr int kOptStore = 4;
 
 template <int OPT, int VEC>
 __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, const float (&gsum)[VEC],
-                                          int e, bool lane_on, bool leader, bool last_chunk,
+                                          int e, bool lane_on, int gl, bool last_chunk, int dim,
                                           const ApplyArgs& a) {
   float* rec = tv.recs + (int64_t)row * tv.stride;
   if constexpr (OPT == kOptStore) {
     if (lane_on) vstore<VEC>(rec + e * VEC, gsum);
     return;
+  }
+  // the lane's slice of the record is requested before the 64-bit word is looked at: the bias
+  // corrections (two powf) then overlap with the loads instead of preceding them
+  float w[VEC], s0[VEC], s1[VEC], s2[VEC];
+  if (lane_on) {
+    vload<VEC>(rec + e * VEC, w);
+    if (a.c0 >= 0) vload<VEC>(rec + a.c0 + e * VEC, s0);
+    if (a.c1 >= 0) vload<VEC>(rec + a.c1 + e * VEC, s1);
+    if (a.c2 >= 0) vload<VEC>(rec + a.c2 + e * VEC, s2);
   }
   bool first = false;
   float bc1 = 1.0f, bc2 = 1.0f;
@@ -285,11 +294,6 @@ __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, con
     }
   }
   if (lane_on) {
-    float w[VEC], s0[VEC], s1[VEC], s2[VEC];
-    vload<VEC>(rec + e * VEC, w);
-    if (a.c0 >= 0) vload<VEC>(rec + a.c0 + e * VEC, s0);
-    if (a.c1 >= 0) vload<VEC>(rec + a.c1 + e * VEC, s1);
-    if (a.c2 >= 0) vload<VEC>(rec + a.c2 + e * VEC, s2);
 #pragma unroll
     for (int c = 0; c < VEC; ++c) {
       if (a.c0 < 0) s0[c] = 0.0f;
@@ -302,12 +306,8 @@ __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, con
     if (a.c1 >= 0) vstore<VEC>(rec + a.c1 + e * VEC, s1);
     if (a.c2 >= 0) vstore<VEC>(rec + a.c2 + e * VEC, s2);
   }
-  // The counter is read by every chunk of the row before the last chunk's leader advances it.
-  if (a.meta_off >= 0 && leader && last_chunk) {
-    uint32_t* meta = reinterpret_cast<uint32_t*>(rec + a.meta_off);
-    meta[0] = (uint32_t)steps;
-    meta[1] = (uint32_t)(steps >> 32);
-  }
+  // The counter is read by every chunk of the row before the last chunk advances it.
+  if (a.meta_off >= 0 && last_chunk) store_row_word<VEC>(rec + a.meta_off, steps, gl, dim);
 }
 
 // keys[cnt] ascending (entries >= empty_from are holes). LEVEL0: the value of entry j is gradient
@@ -419,9 +419,9 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
       aa.c1 = gs.st1 >= 0 ? d.col_off[gs.st1] : -1;
       aa.c2 = gs.st2 >= 0 ? d.col_off[gs.st2] : -1;
       aa.meta_off = gs.use_meta ? d.meta_off : -1;
-      apply_row<OPT, VEC>(member, key & ((1u << gs.row_bits) - 1u), sum, e, lane_on, leader, last_chunk, aa);
+      apply_row<OPT, VEC>(member, key & ((1u << gs.row_bits) - 1u), sum, e, lane_on, gl, last_chunk, dim, aa);
     } else {
-      apply_row<OPT, VEC>(tv, key, sum, e, lane_on, leader, last_chunk, args);
+      apply_row<OPT, VEC>(tv, key, sum, e, lane_on, gl, last_chunk, dim, args);
     }
   };
 

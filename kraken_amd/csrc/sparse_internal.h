@@ -7,7 +7,9 @@
 //                                   extra last slot belongs to the one id whose value is all-ones.
 //                                   epoch = number of the launch that created the row.
 //   recs    [row_cap] x stride      one record per row, rows numbered in insertion order:
-//                                   [ weight D | state columns D each, in creation order | steps ]
+//                                   [ weight D | state columns D each, in creation order | word ]
+//                                   (word: 64 bits of counter and flag, see kHasMomentumBit;
+//                                   a 64-byte sector of its own where dim is a multiple of 16)
 //                                   so a push touches one contiguous record instead of one line
 //                                   per state array.
 //   row_key [row_cap] x 8 B         id of each row (export and re-indexing walk rows, not slots)
@@ -51,6 +53,35 @@ constexpr int kBucket = 4;   // slots per bucket: one aligned 64-byte sector
 // momentum buffer, which is how SGD with momentum tells its first update of a row from the later
 // ones (ps/optim/sgd.cc:46-52 looks for the state in the row's map).
 constexpr unsigned long long kHasMomentumBit = 1ull << 63;
+
+// Room of that word in a record, in floats. A row whose arrays are whole 64-byte sectors
+// (dim a multiple of 16) gives the word a sector of its own and the hot kernels write that sector
+// whole: an 8-byte store into a sector is a read-modify-write for the memory, which was measured
+// to cost a push of one million rows more than a whole extra state array does (70-86 us against
+// 55 us at dim 32). Narrow rows keep the word packed behind the arrays.
+__host__ __device__ inline int row_word_floats(int dim, int vec) {
+  return (dim & 15) == 0 ? 16 : (vec == 4 ? 4 : 2);
+}
+
+// Writes the word of a record from inside a kernel whose lane groups have at least four lanes
+// (gl = lane within the group; every lane of the group calls this).
+template <int VEC>
+__device__ __forceinline__ void store_row_word(float* word, unsigned long long value, int gl, int dim) {
+  if (VEC == 4 && (dim & 15) == 0) {
+    if (gl < 4) {
+      uint4 v = {0u, 0u, 0u, 0u};
+      if (gl == 0) {
+        v.x = (uint32_t)value;
+        v.y = (uint32_t)(value >> 32);
+      }
+      reinterpret_cast<uint4*>(word)[gl] = v;   // four lanes: the sector is written whole
+    }
+  } else if (gl == 0) {
+    uint32_t* meta = reinterpret_cast<uint32_t*>(word);
+    meta[0] = (uint32_t)value;
+    meta[1] = (uint32_t)(value >> 32);
+  }
+}
 
 __device__ __forceinline__ void unpack_slot(const uint4& raw, unsigned long long& key,
                                             unsigned long long& row_epoch) {

@@ -125,6 +125,15 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
   }
   float* rec = tv.recs + (int64_t)row * tv.stride;
 
+  // The lane's first slice of the record is requested before the 64-bit word is looked at: the
+  // bias corrections (two powf) then overlap with the loads instead of preceding them.
+  float w[VEC], s0[VEC], s1[VEC], s2[VEC];
+  if (gl < elems) {
+    vload<VEC>(rec + gl * VEC, w);
+    if (pc.c0 >= 0) vload<VEC>(rec + pc.c0 + gl * VEC, s0);
+    if (pc.c1 >= 0) vload<VEC>(rec + pc.c1 + gl * VEC, s1);
+    if (pc.c2 >= 0) vload<VEC>(rec + pc.c2 + gl * VEC, s2);
+  }
   bool first = false;
   float bc1 = 1.0f, bc2 = 1.0f;
   uint64_t steps = 0;
@@ -145,17 +154,17 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
     }
   }
   for (int e = gl; e < elems; e += group) {
-    float gv[VEC], w[VEC], s0[VEC], s1[VEC], s2[VEC];
+    float gv[VEC];
     if (e == gl) {
 #pragma unroll
       for (int c = 0; c < VEC; ++c) gv[c] = g_first[c];
     } else {
       vload<VEC>(g + e * VEC, gv);
+      vload<VEC>(rec + e * VEC, w);
+      if (pc.c0 >= 0) vload<VEC>(rec + pc.c0 + e * VEC, s0);
+      if (pc.c1 >= 0) vload<VEC>(rec + pc.c1 + e * VEC, s1);
+      if (pc.c2 >= 0) vload<VEC>(rec + pc.c2 + e * VEC, s2);
     }
-    vload<VEC>(rec + e * VEC, w);
-    if (pc.c0 >= 0) vload<VEC>(rec + pc.c0 + e * VEC, s0);
-    if (pc.c1 >= 0) vload<VEC>(rec + pc.c1 + e * VEC, s1);
-    if (pc.c2 >= 0) vload<VEC>(rec + pc.c2 + e * VEC, s2);
 #pragma unroll
     for (int c = 0; c < VEC; ++c) {
       if (pc.c0 < 0) s0[c] = 0.0f;
@@ -168,11 +177,7 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
     if (pc.c1 >= 0) vstore<VEC>(rec + pc.c1 + e * VEC, s1);
     if (pc.c2 >= 0) vstore<VEC>(rec + pc.c2 + e * VEC, s2);
   }
-  if (pc.meta >= 0 && gl == 0) {
-    uint32_t* meta = reinterpret_cast<uint32_t*>(rec + pc.meta);
-    meta[0] = (uint32_t)steps;
-    meta[1] = (uint32_t)(steps >> 32);
-  }
+  if (pc.meta >= 0) store_row_word<VEC>(rec + pc.meta, steps, gl, dim);
 }
 
 // ---- single-table launches ---------------------------------------------------
@@ -952,6 +957,7 @@ int32_t sparse_ensure_columns(krk_sparse* t, uint32_t mask) {
   if (want_meta && t->meta_off < 0) change = true;
   if (!change) return KRK_SUCCESS;
   const int32_t meta_off = want_meta ? (int32_t)body : -1;
+  // with a sector-wide word the stride stays a multiple of the sector too (dim is one)
   const int64_t stride = body + (want_meta ? t->meta_floats : 0);
 
   const int64_t old_stride = t->stride;
@@ -1137,7 +1143,7 @@ int32_t krk_sparse_create(int64_t dim, const krk_init* init, int64_t capacity_hi
   t->init = *init;
   t->initk = make_init_k(*init, dim);
   t->stride = dim;
-  t->meta_floats = t->vec == 4 ? 4 : 2;
+  t->meta_floats = row_word_floats((int)dim, t->vec);
   for (auto& c : t->col_off) c = -1;
   int32_t rc = t->open_stream();
   t->own_stream = t->stream;
