@@ -307,7 +307,7 @@ __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, con
     if (a.c2 >= 0) vstore<VEC>(rec + a.c2 + e * VEC, s2);
   }
   // The counter is read by every chunk of the row before the last chunk advances it.
-  if (a.meta_off >= 0 && last_chunk) store_row_word<VEC>(rec + a.meta_off, steps, gl, dim);
+  if (a.meta_off >= 0 && last_chunk) store_row_word<VEC>(rec + a.meta_off, steps, gl, dim, (int)tv.stride - a.meta_off);
 }
 
 // keys[cnt] ascending (entries >= empty_from are holes). LEVEL0: the value of entry j is gradient

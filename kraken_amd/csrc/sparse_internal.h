@@ -55,26 +55,31 @@ constexpr int kBucket = 4;   // slots per bucket: one aligned 64-byte sector
 constexpr unsigned long long kHasMomentumBit = 1ull << 63;
 
 // Room of that word in a record, in floats. A row whose arrays are whole 64-byte sectors
-// (dim a multiple of 16) gives the word a sector of its own and the hot kernels write that sector
-// whole: an 8-byte store into a sector is a read-modify-write for the memory, which was measured
-// to cost a push of one million rows more than a whole extra state array does (70-86 us against
-// 55 us at dim 32). Narrow rows keep the word packed behind the arrays.
+// (dim a multiple of 16) gives the word a sector of its own, pads the record to a whole 128-byte
+// line, and the push kernels write everything behind the arrays whole: a line written in part
+// costs the memory a read as well, and a packed word (records of 208 or 400 bytes) shifts every
+// array off its sectors. Measured per million rows at dim 32: Adam push 299 -> 266 us, pull
+// 102 -> 84 us. Narrow rows keep the word packed behind the arrays.
 __host__ __device__ inline int row_word_floats(int dim, int vec) {
   return (dim & 15) == 0 ? 16 : (vec == 4 ? 4 : 2);
 }
 
 // Writes the word of a record from inside a kernel whose lane groups have at least four lanes
-// (gl = lane within the group; every lane of the group calls this).
+// (gl = lane within the group; every lane of the group calls this). room = floats from the
+// word to the end of the record: 16, or 32 when the padding sector follows.
 template <int VEC>
-__device__ __forceinline__ void store_row_word(float* word, unsigned long long value, int gl, int dim) {
+__device__ __forceinline__ void store_row_word(float* word, unsigned long long value, int gl, int dim,
+                                               int room) {
   if (VEC == 4 && (dim & 15) == 0) {
     if (gl < 4) {
       uint4 v = {0u, 0u, 0u, 0u};
+      const uint4 zero = {0u, 0u, 0u, 0u};
       if (gl == 0) {
         v.x = (uint32_t)value;
         v.y = (uint32_t)(value >> 32);
       }
       reinterpret_cast<uint4*>(word)[gl] = v;   // four lanes: the sector is written whole
+      if (room >= 32) reinterpret_cast<uint4*>(word)[gl + 4] = zero;   // and the rest of its line
     }
   } else if (gl == 0) {
     uint32_t* meta = reinterpret_cast<uint32_t*>(word);

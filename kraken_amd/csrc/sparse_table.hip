@@ -177,7 +177,7 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
     if (pc.c1 >= 0) vstore<VEC>(rec + pc.c1 + e * VEC, s1);
     if (pc.c2 >= 0) vstore<VEC>(rec + pc.c2 + e * VEC, s2);
   }
-  if (pc.meta >= 0) store_row_word<VEC>(rec + pc.meta, steps, gl, dim);
+  if (pc.meta >= 0) store_row_word<VEC>(rec + pc.meta, steps, gl, dim, (int)tv.stride - pc.meta);
 }
 
 // ---- single-table launches ---------------------------------------------------
@@ -957,8 +957,11 @@ int32_t sparse_ensure_columns(krk_sparse* t, uint32_t mask) {
   if (want_meta && t->meta_off < 0) change = true;
   if (!change) return KRK_SUCCESS;
   const int32_t meta_off = want_meta ? (int32_t)body : -1;
-  // with a sector-wide word the stride stays a multiple of the sector too (dim is one)
-  const int64_t stride = body + (want_meta ? t->meta_floats : 0);
+  // A record that carries the word ends on a 128-byte line where its arrays are whole sectors:
+  // the push kernels then write the word's sector and the padding behind it, so no line of the
+  // record is written in part (see store_row_word).
+  int64_t stride = body + (want_meta ? t->meta_floats : 0);
+  if (want_meta && t->dim % 16 == 0) stride = (stride + 31) & ~(int64_t)31;
 
   const int64_t old_stride = t->stride;
   const int32_t old_meta = t->meta_off;
