@@ -69,7 +69,8 @@ def _table_sequence(api, oracle, tmp_path, seed, dims):
 
     log = []
     for step in range(60):
-        op = rng.choice(["pull", "pull", "push", "push_raw", "pooled", "erase", "load", "file", "optim", "fetch"])
+        op = rng.choice(["pull", "pull", "push", "push_raw", "pooled", "erase", "load", "file", "optim", "fetch",
+                         "route"])
         log.append(op)
         n = int(rng.choice([1, 7, 300, 3000]))
         if op == "pull":
@@ -118,6 +119,21 @@ def _table_sequence(api, oracle, tmp_path, seed, dims):
             gone = np.unique(np.concatenate([some_ids(n, known_only=True)[: max(1, n // 3)], some_ids(3)]))
             assert t.erase(gone) == r.erase(gone)
             used.difference_update(gone.tolist())
+        elif op == "route" and used:
+            # a cluster change (ps/ps.cc:92-109): a ring of a few nodes, this server keeps its share
+            nodes = int(rng.integers(1, 5))
+            ring = sorted((int(h), int(k) % nodes) for k, h in enumerate(
+                rng.integers(0, 2**63, size=3 * nodes, dtype=np.int64).astype(np.uint64) * np.uint64(2)))
+            table_id, me = int(rng.integers(0, 1000)), int(rng.integers(0, nodes))
+            live = r.export()[0]
+            owners = oracle.route_owners(ring, table_id, live)
+            mine = t.select_routed(table_id, ring, me)
+            assert np.array_equal(np.sort(mine), np.sort(live[owners == me]))
+            gone = t.select_routed(table_id, ring, me, owned=False)
+            assert np.array_equal(np.sort(gone), np.sort(live[owners != me]))
+            if rng.random() < 0.5:
+                assert t.erase(gone) == r.erase(gone) == gone.size
+                used.difference_update(gone.tolist())
         elif op == "load":
             ids = np.unique(some_ids(min(n, 300)))
             vals = _dyadic(rng, (ids.size, dim))
