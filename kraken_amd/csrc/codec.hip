@@ -62,28 +62,50 @@ __global__ __launch_bounds__(kCodecBlock) void select_hist_kernel(const float* _
   }
 }
 
-// Walks the histogram from the top bin down until k elements are covered; extends the prefix by
-// that bin and leaves the rank still to be found inside it. One workgroup; clears the histogram.
+// Finds the bin that holds the k-th largest element, counting from the top bin down; extends the
+// prefix by that bin and leaves the rank still to be found inside it. One workgroup; clears the
+// histogram. Every thread owns kBins / kCodecBlock consecutive bins: the bins above a thread's
+// own are summed with a scan over the threads' totals, and the one thread whose bins straddle k
+// walks them. Bin 0 takes whatever no higher bin covers (k larger than the histogram's total).
 __global__ __launch_bounds__(kCodecBlock) void select_pick_kernel(uint32_t* __restrict__ hist, int bits,
                                                                   uint32_t* __restrict__ sel, int last) {
+  constexpr int kPer = kBins / kCodecBlock;
   __shared__ uint32_t lh[kBins];
+  __shared__ uint32_t above[kCodecBlock];      // inclusive suffix sums of the threads' totals
   const int nb = 1 << bits;
+  const uint32_t k = sel[1];                   // read by all before the barriers, written by one after
   for (int i = threadIdx.x; i < kBins; i += kCodecBlock) {
     lh[i] = i < nb ? hist[i] : 0;
     hist[i] = 0;
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    uint32_t k = sel[1];
-    int b = nb - 1;
-    for (; b > 0; --b) {
+  const int t = threadIdx.x;
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) mine += lh[t * kPer + j];
+  above[t] = mine;
+  __syncthreads();
+  for (int d = 1; d < kCodecBlock; d <<= 1) {
+    const uint32_t add = t + d < kCodecBlock ? above[t + d] : 0u;
+    __syncthreads();
+    above[t] += add;
+    __syncthreads();
+  }
+  const uint32_t higher = above[t] - mine;     // elements in the bins of the threads above this one
+  const bool owner = t == 0 ? higher < k : (higher < k && k <= higher + mine);
+  if (owner) {
+    uint32_t rem = k - higher;                 // rank inside this thread's bins, from the top
+    int b = t * kPer + kPer - 1;
+    for (; b > t * kPer; --b) {
       const uint32_t c = lh[b];
-      if (c >= k) break;
-      k -= c;
+      if (c >= rem) break;
+      rem -= c;
     }
+    // b stopped on the bin, or on the thread's lowest bin: for thread 0 that is bin 0, the
+    // catch-all; for the others the rank is known to lie inside it
     const uint32_t prefix = (sel[0] << bits) | (uint32_t)b;
     sel[0] = prefix;
-    sel[1] = k;
+    sel[1] = rem;
     if (last) sel[2] = prefix;   // the full bit pattern of tau
   }
 }
