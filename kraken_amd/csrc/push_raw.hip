@@ -15,6 +15,7 @@
 #include <cstring>
 #include <new>
 
+#include <rocprim/block/block_radix_sort.hpp>
 #include <rocprim/device/device_radix_sort.hpp>
 
 #include "sparse_internal.h"
@@ -666,6 +667,46 @@ static hipError_t sort_pairs(void* tmp, size_t& tmp_bytes, uint32_t* keys, uint3
   return sort_pairs_with<8>(tmp, tmp_bytes, keys, keys_out, vals, vals_out, n, bits, stream);
 }
 
+// Combined requests whose members each bring at most 8192 ids: one workgroup per member sorts
+// that member's pairs in LDS, all members in one launch (26 tables of 8192 ids: 30 us, against
+// 45 us for histogram, scan and three digit passes over the whole request; for a single table
+// of 8192 ids the library's one-workgroup sort is the faster one, 21 us). Inside a member's
+// segment the member number is constant, so only the row bits are sorted; a missing id's key
+// has those bits zero and lands at the front of its segment, which is as good as anywhere: the
+// reduction needs equal keys adjacent, and skips keys at or above the missing-id key wherever
+// they stand. Entries past the segment's end are all-ones and stay behind it (the sort is stable).
+constexpr int kSegSortBlock = 1024;
+constexpr int kSegSortItems = 8;
+constexpr int64_t kSegSortMax = kSegSortBlock * kSegSortItems;
+
+__global__ __launch_bounds__(kSegSortBlock) void segment_sort_kernel(GroupCall call,
+                                                                     const uint32_t* __restrict__ keys,
+                                                                     const uint32_t* __restrict__ pos,
+                                                                     uint32_t* __restrict__ skeys,
+                                                                     uint32_t* __restrict__ spos, int row_bits) {
+  using Sort = rocprim::block_radix_sort<uint32_t, kSegSortBlock, kSegSortItems, uint32_t, 1, 1, 7>;
+  __shared__ typename Sort::storage_type storage;
+  const int64_t a = call.row_start[blockIdx.x];
+  const int len = (int)(call.row_start[blockIdx.x + 1] - a);
+  if (len <= 0) return;                          // uniform for the workgroup
+  uint32_t k[kSegSortItems], v[kSegSortItems];
+#pragma unroll
+  for (int i = 0; i < kSegSortItems; ++i) {
+    const int j = threadIdx.x * kSegSortItems + i;
+    k[i] = j < len ? keys[a + j] : 0xFFFFFFFFu;
+    v[i] = j < len ? pos[a + j] : 0u;
+  }
+  Sort().sort(k, v, storage, 0, (unsigned)row_bits);
+#pragma unroll
+  for (int i = 0; i < kSegSortItems; ++i) {
+    const int j = threadIdx.x * kSegSortItems + i;
+    if (j < len) {
+      skeys[a + j] = k[i];
+      spos[a + j] = v[i];
+    }
+  }
+}
+
 // Stable sort of (key, payload) by key, then the tiled segmented reduction: every run of equal
 // keys is summed in payload order and handed to apply_row<opt> once. `fill(keys, payload)`
 // enqueues the kernel that writes the n unsorted pairs; keys >= miss_key are skipped. d_vals
@@ -674,7 +715,7 @@ template <typename Fill>
 static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, DeviceBuffer* scratch,
                                const TableView& tv, int opt, int64_t n, uint32_t miss_key, int bits,
                                const float* d_vals, const ApplyArgs& args, const PooledSrc& ps,
-                               const GroupSrc* gs, Fill fill) {
+                               const GroupSrc* gs, Fill fill, const GroupCall* segments = nullptr) {
   const int tile0 = pick_tile(n);
   const int per_block = kBlock / sh.group;
   const int64_t groups0 = ((n + tile0 - 1) / tile0 + per_block - 1) / per_block;   // workgroups of level 0
@@ -694,7 +735,13 @@ static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, Device
 
   fill(keys, pos);
   KRK_HIP(hipGetLastError());
-  KRK_HIP(sort_pairs(scratch[1].ptr, sort_bytes, keys, skeys, pos, spos, n, bits, stream));
+  if (segments) {
+    hipLaunchKernelGGL(segment_sort_kernel, dim3((unsigned)segments->n_tables), dim3(kSegSortBlock), 0, stream,
+                       *segments, keys, pos, skeys, spos, gs->row_bits);
+    KRK_HIP(hipGetLastError());
+  } else {
+    KRK_HIP(sort_pairs(scratch[1].ptr, sort_bytes, keys, skeys, pos, spos, n, bits, stream));
+  }
 
   // level 0 reads value rows through the sorted payloads; later levels read the carry list
   uint32_t* ckeys[2] = {scratch[2].as<uint32_t>(), scratch[2].as<uint32_t>() + carry_entries};
@@ -1105,6 +1152,9 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
     return KRK_E_CAPACITY;
   }
   const uint32_t miss_key = (uint32_t)n_tables << row_bits;
+  // members of at most 8192 ids each are sorted one workgroup a member (segment_sort_kernel)
+  bool by_member = n_tables > 1;
+  for (int m = 0; m < n_tables; ++m) by_member = by_member && offsets[m + 1] - offsets[m] <= kSegSortMax;
   const uint64_t* d_ids;
   const float* d_g;
   KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
@@ -1124,7 +1174,7 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
                                                dim3(grid_for(total, kBlock / kBucket)), dim3(kBlock), 0,
                                                g->stream, g->d_descs, call, d_ids, total, row_bits, miss_key,
                                                keys, pos);
-                          }));
+                          }, by_member ? &call : nullptr));
   return group_finish(g, flags);
 }
 
