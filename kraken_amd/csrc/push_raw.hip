@@ -196,11 +196,14 @@ __global__ __launch_bounds__(kBlock) void group_rows_of_ids_kernel(const TableDe
                                                                    int row_bits, uint32_t miss_key,
                                                                    uint32_t* __restrict__ keys,
                                                                    uint32_t* __restrict__ pos) {
-  const int64_t p = (int64_t)blockIdx.x * (kBlock / kBucket) + threadIdx.x / kBucket;
-  const int gl = threadIdx.x & (kBucket - 1);
-  const bool active = p < n;
+  // a workgroup serves one member (call.block_start counts workgroups of kBlock / kBucket
+  // positions here), so the member's layout comes in through scalar loads
   int m = 0;
-  while (active && m + 1 < call.n_tables && p >= call.row_start[m + 1]) ++m;
+  while (m + 1 < call.n_tables && blockIdx.x >= call.block_start[m + 1]) ++m;
+  const int64_t p = call.row_start[m] + (int64_t)(blockIdx.x - call.block_start[m]) * (kBlock / kBucket) +
+                    threadIdx.x / kBucket;
+  const int gl = threadIdx.x & (kBucket - 1);
+  const bool active = p < call.row_start[m + 1];
   const TableView tv = descs[m].tv;
   uint32_t r = probe_find(tv, active ? ids[p] : 0, active, gl, kBucket);
   if (!active || gl != 0) return;
@@ -1155,6 +1158,14 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
   // members of at most 8192 ids each are sorted one workgroup a member (segment_sort_kernel)
   bool by_member = n_tables > 1;
   for (int m = 0; m < n_tables; ++m) by_member = by_member && offsets[m + 1] - offsets[m] <= kSegSortMax;
+  // the launch that turns ids into rows gives every member whole workgroups of its own
+  GroupCall rows_call = call;
+  uint32_t blocks = 0;
+  for (int m = 0; m < n_tables; ++m) {
+    rows_call.block_start[m] = blocks;
+    blocks += grid_for(offsets[m + 1] - offsets[m], kBlock / kBucket);
+  }
+  rows_call.block_start[n_tables] = blocks;
   const uint64_t* d_ids;
   const float* d_g;
   KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
@@ -1170,10 +1181,9 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
   const ReduceShape sh{g->dim, g->vec, g->elems, g->group};
   KRK_TRY(sort_and_reduce(sh, g->stream, g->scratch, none, o->type, total, miss_key, row_bits + member_bits,
                           d_g, args, PooledSrc{nullptr, nullptr}, &gs, [&](uint32_t* keys, uint32_t* pos) {
-                            hipLaunchKernelGGL(group_rows_of_ids_kernel,
-                                               dim3(grid_for(total, kBlock / kBucket)), dim3(kBlock), 0,
-                                               g->stream, g->d_descs, call, d_ids, total, row_bits, miss_key,
-                                               keys, pos);
+                            hipLaunchKernelGGL(group_rows_of_ids_kernel, dim3(rows_call.block_start[n_tables]),
+                                               dim3(kBlock), 0, g->stream, g->d_descs, rows_call, d_ids, total,
+                                               row_bits, miss_key, keys, pos);
                           }, by_member ? &call : nullptr));
   return group_finish(g, flags);
 }
