@@ -671,9 +671,8 @@ static hipError_t sort_pairs(void* tmp, size_t& tmp_bytes, uint32_t* keys, uint3
 }
 
 // Combined requests whose members each bring at most 8192 ids: one workgroup per member sorts
-// that member's pairs in LDS, all members in one launch (26 tables of 8192 ids: 30 us, against
-// 45 us for histogram, scan and three digit passes over the whole request; for a single table
-// of 8192 ids the library's one-workgroup sort is the faster one, 21 us). Inside a member's
+// that member's pairs in LDS, all members in one launch (26 tables of 8192 ids: 23 us, against
+// 45 us for histogram, scan and three digit passes over the whole request). Inside a member's
 // segment the member number is constant, so only the row bits are sorted; a missing id's key
 // has those bits zero and lands at the front of its segment, which is as good as anywhere: the
 // reduction needs equal keys adjacent, and skips keys at or above the missing-id key wherever
@@ -687,22 +686,26 @@ __global__ __launch_bounds__(kSegSortBlock) void segment_sort_kernel(GroupCall c
                                                                      const uint32_t* __restrict__ pos,
                                                                      uint32_t* __restrict__ skeys,
                                                                      uint32_t* __restrict__ spos, int row_bits) {
-  using Sort = rocprim::block_radix_sort<uint32_t, kSegSortBlock, kSegSortItems, uint32_t, 1, 1, 7>;
+  using Sort = rocprim::block_radix_sort<uint32_t, kSegSortBlock, kSegSortItems, uint32_t>;
   __shared__ typename Sort::storage_type storage;
   const int64_t a = call.row_start[blockIdx.x];
   const int len = (int)(call.row_start[blockIdx.x + 1] - a);
   if (len <= 0) return;                          // uniform for the workgroup
+  // in: every wavefront holds 64 * kSegSortItems consecutive pairs, item i of lane l being pair
+  // i * 64 + l of them; out: item i of thread t is pair i * kSegSortBlock + t of the sorted
+  // segment. Both ways a load or store instruction covers consecutive addresses.
   uint32_t k[kSegSortItems], v[kSegSortItems];
+  const int wave_base = (threadIdx.x / 64) * (64 * kSegSortItems) + (threadIdx.x & 63);
 #pragma unroll
   for (int i = 0; i < kSegSortItems; ++i) {
-    const int j = threadIdx.x * kSegSortItems + i;
+    const int j = wave_base + i * 64;
     k[i] = j < len ? keys[a + j] : 0xFFFFFFFFu;
     v[i] = j < len ? pos[a + j] : 0u;
   }
-  Sort().sort(k, v, storage, 0, (unsigned)row_bits);
+  Sort().sort_warp_striped_to_striped(k, v, storage, 0, (unsigned)row_bits);
 #pragma unroll
   for (int i = 0; i < kSegSortItems; ++i) {
-    const int j = threadIdx.x * kSegSortItems + i;
+    const int j = i * kSegSortBlock + threadIdx.x;
     if (j < len) {
       skeys[a + j] = k[i];
       spos[a + j] = v[i];
