@@ -218,3 +218,32 @@ def test_group_push_raw_errors(api):
     assert grp.CombinePushRaw(o, np.zeros(0, np.uint64), [0, 0, 0], np.zeros((0, 8), np.float32), 0.5) == 0
     assert grp.CombinePushRaw(api.Optim.create(api.OptimType.kSGD), ids, [0, 5, 4], g, 0.5) != 0
     grp.close()
+
+
+@pytest.mark.parametrize("filler", [5, 9000])
+def test_group_push_raw_adds_repeats_in_position_order(api, filler):
+    """worker/emitter.cc:563-606 adds the gradients of a repeated (table, id) in the order the
+    request lists them. 1e8 + 1 - 1e8 is 0 in that order and 1 in the other two, so the sort
+    has to be stable: members of few ids take the one-workgroup-a-member sort, a member above
+    8192 ids the radix sort over the whole request."""
+    dim = 4
+    gi = api.Initializer.create(api.InitializerType.kConstant, {"value": "0.5"})
+    a, b = api.SparseTable(dim, gi), api.SparseTable(dim, gi)
+    first = np.array([7], np.uint64)
+    a.Pull(first)                                   # row 0 of member 0: its key sorts first
+    b.Pull(first)
+    rest = np.arange(100, 100 + filler, dtype=np.uint64)
+    a.Pull(rest)
+    b.Pull(rest)
+    grp = api.TableGroup([a, b])
+    ids = np.concatenate([[7], rest[: filler // 2], [7], rest[filler // 2:], [7], [7, 7, 7]]).astype(np.uint64)
+    off = grp._offsets([ids.size - 3, 3])
+    g = np.zeros((ids.size, dim), np.float32)
+    at = [0, 1 + filler // 2, ids.size - 4]         # the three positions of id 7 in member 0
+    g[at[0]], g[at[1]], g[at[2]] = 1e8, 1.0, -1e8
+    g[-3], g[-2], g[-1] = -1e8, 1e8, 1.0            # member 1: (-1e8 + 1e8) + 1 = 1
+    sgd = api.Optim.create(api.OptimType.kSGD)
+    assert grp.CombinePushRaw(sgd, ids, off, g, 1.0) == 0
+    assert np.array_equal(a.Pull(first)[1], np.full((1, dim), 0.5, np.float32))     # 0.5 - 0
+    assert np.array_equal(b.Pull(first)[1], np.full((1, dim), -0.5, np.float32))    # 0.5 - 1
+    grp.close()
