@@ -161,9 +161,13 @@ int32_t krk_sparse_reserve(krk_sparse* t, int64_t rows);
 int32_t krk_sparse_sync(krk_sparse* t);
 /* Makes the table enqueue its work on the caller's HIP stream (a hipStream_t) instead of its
  * own, so that KRK_ASYNC calls are ordered with the caller's other work on that stream: a
- * training framework passes the stream its tensors are produced and consumed on. NULL returns
- * to the table's own stream. Work already enqueued is waited for first. The stream must outlive
- * its use by the table; tables that belong to a group cannot switch. No reference counterpart. */
+ * training framework passes the stream its tensors are produced and consumed on. NULL is a
+ * stream like any other: HIP's default (null) stream, which is what a framework's "current
+ * stream" handle is until the user switches streams. KRK_OWN_STREAM returns to the stream
+ * created with the table (which does not wait for the null stream, nor the null stream for it).
+ * Work already enqueued is waited for first. The stream must outlive its use by the table;
+ * tables that belong to a group cannot switch. No reference counterpart. */
+#define KRK_OWN_STREAM ((void*)(intptr_t)-1)
 int32_t krk_sparse_set_stream(krk_sparse* t, void* stream);
 
 /* SparseTable::Pull (ps/sparse_table.cc:33-75): out[i,:] = row of ids[i];
@@ -364,7 +368,9 @@ int32_t krk_dense_create(const float* val, int64_t n, uint32_t flags, krk_dense*
 int32_t krk_dense_destroy(krk_dense* t);
 int32_t krk_dense_sync(krk_dense* t);
 int32_t krk_dense_pull(krk_dense* t, float* out, uint32_t flags);      /* ps/dense_table.cc:31-37 */
-/* DenseTable::Push (ps/dense_table.cc:39-43); n != table size returns 11. */
+/* DenseTable::Push (ps/dense_table.cc:39-43); n != table size returns 11. A device gradient
+ * must be 16-byte aligned (KRK_E_ARGUMENT otherwise), as every device row buffer of the sparse
+ * calls must. */
 int32_t krk_dense_push(krk_dense* t, const krk_optim* o, const float* grad, int64_t n, float lr,
                        uint32_t flags);
 /* COO gradient (values + int64 flat indices, as ToCoo emits them): densified

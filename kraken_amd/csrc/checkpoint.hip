@@ -69,14 +69,27 @@ class FileWriter {   // checkpoint/file_writer.cc: a truncating binary stream
 
 class FileReader {
  public:
-  explicit FileReader(const char* path) : fs_(path, std::ios::in | std::ios::binary) {}
+  explicit FileReader(const char* path) : fs_(path, std::ios::in | std::ios::binary) {
+    if (fs_.is_open()) {
+      fs_.seekg(0, std::ios::end);
+      size_ = (uint64_t)std::max<std::streamoff>(0, fs_.tellg());
+      fs_.seekg(0, std::ios::beg);
+    }
+  }
   bool is_open() const { return fs_.is_open(); }
-  bool bytes(void* p, size_t n) { return (bool)fs_.read(static_cast<char*>(p), (std::streamsize)n); }
+  bool bytes(void* p, size_t n) {
+    if (!fs_.read(static_cast<char*>(p), (std::streamsize)n)) return false;
+    at_ += n;
+    return true;
+  }
+  // What is left of the file: no field may claim more than that, so a corrupt length can
+  // neither overflow nor make this process allocate more than the file could fill.
+  uint64_t left() const { return size_ - at_; }
   template <typename T>
   bool pod(T* v) { return bytes(v, sizeof(T)); }
   bool str(std::string* s) {
     uint64_t n;
-    if (!pod(&n) || n > (1ull << 32)) return false;
+    if (!pod(&n) || n > left()) return false;
     s->resize((size_t)n);
     return n == 0 || bytes(&(*s)[0], (size_t)n);
   }
@@ -85,21 +98,24 @@ class FileReader {
     uint8_t layout, dtype;
     uint64_t rank;
     if (!pod(&layout) || layout != kLayoutStride || !pod(&rank) || rank > 16) return false;
-    int64_t size = 1;
+    uint64_t size = 1;
     if (shape) shape->clear();
     for (uint64_t i = 0; i < rank; ++i) {
       int64_t d;
       if (!pod(&d) || d < 0) return false;
-      size *= d;
+      if (d != 0 && size > left() / (uint64_t)d) return false;   // more elements than bytes left
+      size *= (uint64_t)d;
       if (shape) shape->push_back(d);
     }
-    if (!pod(&dtype) || dtype != kDTypeFloat32 || size > ((int64_t)1 << 40)) return false;
+    if (!pod(&dtype) || dtype != kDTypeFloat32 || size > left() / sizeof(float)) return false;
     out->resize((size_t)size);
     return size == 0 || bytes(out->data(), sizeof(float) * (size_t)size);
   }
 
  private:
   std::ifstream fs_;
+  uint64_t size_ = 0;
+  uint64_t at_ = 0;
 };
 
 // The conf map Initializer::conf() returns (ps/initializer/*_initializer.cc:11-13), values
@@ -172,7 +188,8 @@ int32_t krk_sparse_save_file(krk_sparse* t, const char* path, uint64_t table_id,
       vals.resize((size_t)(n * dim));
       steps.resize((size_t)n);
       found.resize((size_t)n);
-      KRK_TRY(krk_sparse_fetch(t, ids.data() + at, n, found.data(), vals.data(), 1, nullptr, steps.data(), 0));
+      KRK_TRY(krk_sparse_fetch(t, ids.data() + at, n, found.data(), vals.data(), 1, nullptr, nullptr, 0));
+      KRK_TRY(sparse_fetch_words(t, ids.data() + at, n, steps.data()));
       for (size_t s = 0; s < states.size(); ++s) {
         st_vals[s].resize((size_t)(n * dim));
         KRK_TRY(krk_sparse_fetch(t, ids.data() + at, n, nullptr, nullptr, states[s], st_vals[s].data(), nullptr, 0));
@@ -187,11 +204,16 @@ int32_t krk_sparse_save_file(krk_sparse* t, const char* path, uint64_t table_id,
         // (an absent state and a zero state update alike), and Adam's two moments whenever the
         // row has been counted. The counter alone does not say that a row was updated: only
         // Adam and SGD with momentum advance it.
+        const bool has_momentum = ((uint64_t)steps[(size_t)i] & kHasMomentumBit) != 0;
+        steps[(size_t)i] = (int64_t)((uint64_t)steps[(size_t)i] & ~kHasMomentumBit);
         const bool counter = adam && steps[(size_t)i] > 0;
         size_t emit = 0;
         for (size_t s = 0; s < states.size(); ++s) {
           const float* v = st_vals[s].data() + i * dim;
-          bool any = counter && (states[s] == KRK_ST_FIRST_MOMENT || states[s] == KRK_ST_SECOND_MOMENT);
+          // a row that SGD with momentum has updated holds a buffer even when it is all zeros:
+          // its next update continues the buffer instead of seeding it (ps/optim/sgd.cc:46-52)
+          bool any = (counter && (states[s] == KRK_ST_FIRST_MOMENT || states[s] == KRK_ST_SECOND_MOMENT)) ||
+                     (has_momentum && states[s] == KRK_ST_MOMENTUM_BUFFER);
           for (int64_t j = 0; j < dim && !any; ++j) any = v[j] != 0.0f;
           row_has[s] = any;
           emit += any ? 1 : 0;
@@ -210,8 +232,24 @@ int32_t krk_sparse_save_file(krk_sparse* t, const char* path, uint64_t table_id,
   return w.close() ? KRK_SUCCESS : io_fail("write failed", path);
 }
 
+static int32_t sparse_load_file(krk_sparse* t, const char* path, uint64_t table_id, const char* name,
+                                krk_keep_fn keep, void* keep_ctx, int64_t* rows_loaded);
+
 int32_t krk_sparse_load_file(krk_sparse* t, const char* path, uint64_t table_id, const char* name,
                              krk_keep_fn keep, void* keep_ctx, int64_t* rows_loaded) {
+  // nothing may throw across the C boundary: a file this process cannot hold is a file error
+  try {
+    return sparse_load_file(t, path, table_id, name, keep, keep_ctx, rows_loaded);
+  } catch (const std::exception& e) {
+    set_error("loading %s failed: %s", path ? path : "(null)", e.what());
+    return KRK_E_IO;
+  } catch (...) {
+    return io_fail("loading failed", path);
+  }
+}
+
+static int32_t sparse_load_file(krk_sparse* t, const char* path, uint64_t table_id, const char* name,
+                                krk_keep_fn keep, void* keep_ctx, int64_t* rows_loaded) {
   if (!t || !path || !name) return KRK_E_ARGUMENT;
   if (rows_loaded) *rows_loaded = 0;
   int64_t dim = 0;
@@ -243,10 +281,44 @@ int32_t krk_sparse_load_file(krk_sparse* t, const char* path, uint64_t table_id,
   uint32_t chunk_states = 0;
   int64_t loaded = 0;
   auto flush = [&]() -> int32_t {
-    const int64_t n = (int64_t)ids.size();
+    int64_t n = (int64_t)ids.size();
     if (n == 0) return KRK_SUCCESS;
-    KRK_TRY(krk_sparse_import(t, ids.data(), n, vals.data(), 0));
-    for (int st = 1; st < KRK_ST_COUNT; ++st) {
+    loaded += n;
+    // checkpoint/checkpoint.cc:640 inserts whole Values with SkipList::Insert, which leaves an id
+    // that is already present untouched (common/skip_list.h:240-242): weights, states and
+    // counter alike. So only the ids the table does not hold yet are handed on.
+    std::vector<int32_t> where((size_t)n);
+    KRK_TRY(krk_sparse_lookup(t, ids.data(), n, where.data(), 0));
+    size_t keep_n = 0;
+    std::vector<size_t> new_index((size_t)n, (size_t)-1);
+    for (size_t i = 0; i < (size_t)n; ++i) {
+      if (where[i] >= 0) continue;
+      new_index[i] = keep_n;
+      if (keep_n != i) {
+        ids[keep_n] = ids[i];
+        steps[keep_n] = steps[i];
+        std::copy(vals.begin() + i * dim, vals.begin() + (i + 1) * dim, vals.begin() + keep_n * dim);
+        for (int st = 1; st < KRK_ST_COUNT; ++st)
+          if (chunk_states & (1u << st))
+            std::copy(st_vals[st].begin() + i * dim, st_vals[st].begin() + (i + 1) * dim,
+                      st_vals[st].begin() + keep_n * dim);
+      }
+      ++keep_n;
+    }
+    if (keep_n != (size_t)n) {
+      std::vector<size_t> moved;
+      for (size_t row : with_momentum)
+        if (new_index[row] != (size_t)-1) moved.push_back(new_index[row]);
+      with_momentum.swap(moved);
+      n = (int64_t)keep_n;
+      ids.resize(keep_n);
+      steps.resize(keep_n);
+      vals.resize(keep_n * (size_t)dim);
+      for (int st = 1; st < KRK_ST_COUNT; ++st)
+        if (chunk_states & (1u << st)) st_vals[st].resize(keep_n * (size_t)dim);
+    }
+    if (n > 0) KRK_TRY(krk_sparse_import(t, ids.data(), n, vals.data(), 0));
+    for (int st = 1; st < KRK_ST_COUNT && n > 0; ++st) {
       if (!(chunk_states & (1u << st))) continue;
       st_vals[st].resize((size_t)(n * dim), 0.0f);
       if (st == KRK_ST_MOMENTUM_BUFFER) {
@@ -267,8 +339,8 @@ int32_t krk_sparse_load_file(krk_sparse* t, const char* path, uint64_t table_id,
     with_momentum.clear();
     bool any_steps = false;
     for (int64_t s : steps) any_steps = any_steps || s != 0;
-    if (any_steps) KRK_TRY(krk_sparse_import_state(t, ids.data(), n, 1, nullptr, steps.data(), 0));
-    loaded += n;
+    if (any_steps && n > 0) KRK_TRY(krk_sparse_import_state(t, ids.data(), n, 1, nullptr, steps.data(), 0));
+    for (int st = 1; st < KRK_ST_COUNT; ++st) st_vals[st].clear();
     ids.clear();
     vals.clear();
     steps.clear();
@@ -359,8 +431,23 @@ int32_t krk_dense_save_file(krk_dense* t, const char* path, uint64_t table_id, c
   return ok && w.close() ? KRK_SUCCESS : io_fail("write failed", path);
 }
 
+static int32_t dense_load_file(const char* path, krk_dense** out, uint64_t* table_id, char* name, size_t name_cap,
+                               int64_t* shape, int32_t* rank);
+
 int32_t krk_dense_load_file(const char* path, krk_dense** out, uint64_t* table_id, char* name, size_t name_cap,
                             int64_t* shape, int32_t* rank) {
+  try {
+    return dense_load_file(path, out, table_id, name, name_cap, shape, rank);
+  } catch (const std::exception& e) {
+    set_error("loading %s failed: %s", path ? path : "(null)", e.what());
+    return KRK_E_IO;
+  } catch (...) {
+    return io_fail("loading failed", path);
+  }
+}
+
+static int32_t dense_load_file(const char* path, krk_dense** out, uint64_t* table_id, char* name, size_t name_cap,
+                               int64_t* shape, int32_t* rank) {
   if (!path || !out) return KRK_E_ARGUMENT;
   *out = nullptr;
   FileReader r(path);

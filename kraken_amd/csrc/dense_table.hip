@@ -200,6 +200,10 @@ int32_t krk_dense_push(krk_dense* t, const krk_optim* o, const float* grad, int6
   KRK_TRY(check_flags(flags));
   if (!o || o->type < KRK_ADAGRAD || o->type > KRK_SGD) return KRK_UNSUPPORTED_OPTIM;
   if (n < 0 || (n > 0 && !grad)) return KRK_E_ARGUMENT;
+  if ((flags & KRK_DEVICE_PTRS) && ((uintptr_t)grad & 15)) {   // the update moves 16 bytes per lane
+    set_error("device gradient must be 16-byte aligned");
+    return KRK_E_ARGUMENT;
+  }
   std::lock_guard<std::mutex> lk(t->mu);
   if (n != t->n) {   // ps/optim/sgd.cc:36-39
     set_error("gradient has %lld elements, table has %lld", (long long)n, (long long)t->n);

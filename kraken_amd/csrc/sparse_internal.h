@@ -416,6 +416,8 @@ int32_t sparse_next_epoch(krk_sparse* t, int64_t n);
 bool sparse_near_full(const krk_sparse* t);
 // Enqueues the kernel that publishes {rows used, launch number} of each table to the host.
 int32_t sparse_publish(krk_sparse* const* tables, int n, hipStream_t stream);
+// Host ids -> each row's stored 64-bit word (counter and momentum flag), blocking.
+int32_t sparse_fetch_words(krk_sparse* t, const uint64_t* ids, int64_t n, int64_t* words);
 // Column offsets an optimizer's three state slots map to (-1 = unused).
 void sparse_optim_columns(const krk_sparse* t, const krk_optim& o, int32_t cols[3]);
 // The three state types an optimizer's slots s0/s1/s2 hold (-1 = unused).

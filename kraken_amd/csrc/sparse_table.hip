@@ -501,8 +501,8 @@ __global__ __launch_bounds__(kBlock) void fetch_kernel(TableView tv, const uint6
                                                        int64_t n, unsigned char* __restrict__ found,
                                                        float* __restrict__ vals, int state_off,
                                                        float* __restrict__ state, int meta_off,
-                                                       long long* __restrict__ steps, int dim, int elems,
-                                                       int group) {
+                                                       long long* __restrict__ steps, bool raw_word,
+                                                       int dim, int elems, int group) {
   const int per_block = kBlock / group;
   const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
   const int gl = threadIdx.x & (group - 1);
@@ -517,7 +517,8 @@ __global__ __launch_bounds__(kBlock) void fetch_kernel(TableView tv, const uint6
       long long s = 0;
       if (hit && meta_off >= 0) {
         const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + meta_off);
-        s = (long long)(((uint64_t)meta[0] | ((uint64_t)meta[1] << 32)) & ~kHasMomentumBit);
+        const uint64_t word = (uint64_t)meta[0] | ((uint64_t)meta[1] << 32);
+        s = (long long)(raw_word ? word : word & ~kHasMomentumBit);
       }
       steps[i] = s;
     }
@@ -1176,7 +1177,7 @@ int32_t krk_sparse_destroy(krk_sparse* t) {
     set_error("destroy the group before its tables");
     return KRK_E_ARGUMENT;
   }
-  if (t->stream) (void)hipStreamSynchronize(t->stream);
+  (void)hipStreamSynchronize(t->stream);   // also when the table runs on the null stream
   if (t->slots) (void)hipFree(t->slots);
   if (t->recs) (void)hipFree(t->recs);
   if (t->row_key) (void)hipFree(t->row_key);
@@ -1197,7 +1198,7 @@ int32_t krk_sparse_set_stream(krk_sparse* t, void* stream) {
     set_error("a group member runs on its group's stream");
     return KRK_E_ARGUMENT;
   }
-  hipStream_t next = stream ? reinterpret_cast<hipStream_t>(stream) : t->own_stream;
+  hipStream_t next = stream == KRK_OWN_STREAM ? t->own_stream : reinterpret_cast<hipStream_t>(stream);
   if (next == t->stream) return KRK_SUCCESS;
   // what is enqueued on the old stream must be complete before work on the new one may follow
   KRK_TRY(sparse_finish(t, 0));
@@ -1593,8 +1594,16 @@ int32_t krk_sparse_states(krk_sparse* t, uint32_t* mask) {
   return KRK_SUCCESS;
 }
 
+static int32_t fetch_impl(krk_sparse* t, const uint64_t* ids, int64_t n, uint8_t* found, float* vals,
+                          int32_t state_type, float* state, int64_t* steps, uint32_t flags, bool raw_word);
+
 int32_t krk_sparse_fetch(krk_sparse* t, const uint64_t* ids, int64_t n, uint8_t* found, float* vals,
                          int32_t state_type, float* state, int64_t* steps, uint32_t flags) {
+  return fetch_impl(t, ids, n, found, vals, state_type, state, steps, flags, false);
+}
+
+static int32_t fetch_impl(krk_sparse* t, const uint64_t* ids, int64_t n, uint8_t* found, float* vals,
+                          int32_t state_type, float* state, int64_t* steps, uint32_t flags, bool raw_word) {
   KRK_TRY(check_table(t));
   KRK_TRY(check_flags(flags));
   if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;
@@ -1630,10 +1639,10 @@ int32_t krk_sparse_fetch(krk_sparse* t, const uint64_t* ids, int64_t n, uint8_t*
   const int state_off = state ? t->col_off[state_type] : -1;
   if (t->vec == 4) {
     hipLaunchKernelGGL((fetch_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_found, d_vals,
-                       state_off, d_state, t->meta_off, d_steps, (int)t->dim, t->elems, t->group);
+                       state_off, d_state, t->meta_off, d_steps, raw_word, (int)t->dim, t->elems, t->group);
   } else {
     hipLaunchKernelGGL((fetch_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, d_found, d_vals,
-                       state_off, d_state, t->meta_off, d_steps, (int)t->dim, t->elems, t->group);
+                       state_off, d_state, t->meta_off, d_steps, raw_word, (int)t->dim, t->elems, t->group);
   }
   KRK_HIP(hipGetLastError());
   if (vals) KRK_TRY(t->output_back(vals, cells, flags, 1));
@@ -1869,7 +1878,7 @@ int32_t krk_group_create(krk_sparse** tables, int32_t n, krk_group** out) {
 
 int32_t krk_group_destroy(krk_group* g) {
   if (!g) return KRK_SUCCESS;
-  if (g->stream) (void)hipStreamSynchronize(g->stream);
+  (void)hipStreamSynchronize(g->stream);   // also when the group runs on the null stream
   for (krk_sparse* t : g->tables) {
     std::lock_guard<std::mutex> lk(t->mu);
     t->stream = t->own_stream;
@@ -1888,7 +1897,7 @@ int32_t krk_group_set_stream(krk_group* g, void* stream) {
   if (!g) return KRK_E_ARGUMENT;
   KRK_TRY(ensure_runtime());
   GroupLock lk(g);
-  hipStream_t next = stream ? reinterpret_cast<hipStream_t>(stream) : g->own_stream;
+  hipStream_t next = stream == KRK_OWN_STREAM ? g->own_stream : reinterpret_cast<hipStream_t>(stream);
   if (next == g->stream) return KRK_SUCCESS;
   // what is enqueued on the old stream must be complete before work on the new one may follow
   KRK_TRY(group_finish(g, 0));
@@ -1898,6 +1907,12 @@ int32_t krk_group_set_stream(krk_group* g, void* stream) {
 }
 
 }  // extern "C"
+
+// The 64-bit word of each row as it is stored (counter and "has a momentum buffer" flag), zero
+// for ids that are absent: what the table-file writer needs besides krk_sparse_fetch.
+int32_t krk::sparse_fetch_words(krk_sparse* t, const uint64_t* ids, int64_t n, int64_t* words) {
+  return fetch_impl(t, ids, n, nullptr, nullptr, 1, nullptr, words, 0, true);
+}
 
 // Uploads the layouts of tables that moved since the last call.
 int32_t krk::group_refresh(krk_group* g) {

@@ -102,3 +102,28 @@ def test_row_blocks_the_reference_wrote(dim):
     assert np.array_equal(parse_rows(golden), want)
     assert pack_rows(want) == golden
 
+
+
+def test_malformed_dense_files_are_errors_before_any_gpu_work(tmp_path):
+    """krk_dense_load_file reads the Value before it creates the table, so a file whose lengths
+    no file could back is refused here, without a GPU: error code, no exception, no huge
+    allocation."""
+    import ctypes as C
+    from kraken_amd import api
+    L = api.lib()
+    cases = {
+        "huge tensor": struct.pack("<BQ", 0, 5) + pack_string("d") + struct.pack("<BQqB", 0, 1, 1 << 40, 11),
+        "overflowing dims": struct.pack("<BQ", 0, 5) + pack_string("d") + struct.pack("<BQ", 0, 3) +
+                            struct.pack("<qqq", 1 << 31, 1 << 31, 1 << 31) + b"\x0b",
+        "huge name": struct.pack("<BQ", 0, 5) + struct.pack("<Q", 1 << 40) + b"d",
+        "negative dim": struct.pack("<BQ", 0, 5) + pack_string("d") + struct.pack("<BQqB", 0, 1, -4, 11),
+        "rank 17": struct.pack("<BQ", 0, 5) + pack_string("d") + struct.pack("<BQ", 0, 17),
+        "cut": struct.pack("<BQ", 0, 5),
+    }
+    for what, body in cases.items():
+        path = str(tmp_path / "bad.dense")
+        open(path, "wb").write(body)
+        out = C.c_void_p()
+        rc = L.krk_dense_load_file(os.fsencode(path), C.byref(out), None, None, 0, None, None)
+        assert rc == api.E_IO, what
+        assert not out.value

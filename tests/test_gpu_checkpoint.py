@@ -387,3 +387,99 @@ def test_file_of_a_table_larger_than_the_writers_chunks(api, tmp_path):
     oa, ob = np.argsort(a_id), np.argsort(b_id)
     assert np.array_equal(a_id[oa], b_id[ob]) and np.array_equal(a_val[oa], b_val[ob])
     assert np.array_equal(a_steps[oa], b_steps[ob]) and int(a_steps.sum()) == touched.size
+
+
+def test_load_leaves_rows_that_exist_untouched(api, oracle, tmp_path):
+    """checkpoint/checkpoint.cc:640 inserts each Value with SkipList::Insert, which does nothing
+    for an id that is present (common/skip_list.h:240-242): a row the table already holds keeps
+    its weights, its optimizer state and its counter, all three; only absent ids come in."""
+    dim = 8
+    t, ref = _tables(api, oracle, dim, seed=5)
+    ids = splitmix64(np.arange(3000, dtype=np.uint64))
+    o_ref, o_gpu = make_optims(oracle, api, 1, {})                      # Adam: two states and a counter
+    assert t.Pull(ids)[0] == 0 and ref.pull(ids)[0] == 0
+    g = (np.random.default_rng(1).integers(-64, 65, size=(ids.size, dim)) / 4096.0).astype(np.float32)
+    assert t.Push(o_gpu, ids, g, 0.01) == 0 and ref.push(o_ref, ids, g, 0.01) == 0
+    path = str(tmp_path / "a.sparse")
+    assert t.save(path, 3, "a") == 0
+
+    # the receiving table holds every third id already, trained differently (three updates)
+    t2, ref2 = _tables(api, oracle, dim, seed=9)
+    mine = ids[::3]
+    assert t2.Pull(mine)[0] == 0 and ref2.pull(mine)[0] == 0
+    for step in range(3):
+        g2 = (np.random.default_rng(10 + step).integers(-64, 65, size=(mine.size, dim)) / 4096.0).astype(np.float32)
+        assert t2.Push(o_gpu, mine, g2, 0.02) == 0 and ref2.push(o_ref, mine, g2, 0.02) == 0
+    rc, taken = t2.load_file(path, 3, "a")
+    assert rc == 0 and taken == ids.size and len(t2) == ids.size
+    other = np.setdiff1d(ids, mine)
+    for st in (3, 4):
+        found, vals, state, steps = t2.fetch(mine, state_type=st)
+        assert found.all() and (steps == 3).all()                        # its own counter, not the file's 1
+        assert_close(vals, ref2.pull(mine)[1], "weights of rows that were present")
+        assert_close(state, _oracle_state(ref2, mine, st), "state %d of rows that were present" % st)
+        found, vals, state, steps = t2.fetch(other, state_type=st)
+        assert found.all() and (steps == 1).all()
+        assert_close(vals, ref.pull(other)[1], "weights of rows from the file")
+        assert_close(state, _oracle_state(ref, other, st), "state %d of rows from the file" % st)
+    # and both kinds keep training like the oracle's rows
+    g3 = (np.random.default_rng(77).integers(-64, 65, size=(ids.size, dim)) / 4096.0).astype(np.float32)
+    assert t2.Push(o_gpu, ids, g3, 0.01) == 0
+    pos = {int(k): i for i, k in enumerate(ids.tolist())}
+    sel_m = np.array([pos[int(k)] for k in mine]); sel_o = np.array([pos[int(k)] for k in other])
+    assert ref2.push(o_ref, mine, g3[sel_m], 0.01) == 0 and ref.push(o_ref, other, g3[sel_o], 0.01) == 0
+    assert_close(t2.Pull(mine)[1], ref2.pull(mine)[1], "present rows after one more step")
+    assert_close(t2.Pull(other)[1], ref.pull(other)[1], "loaded rows after one more step")
+
+
+def _oracle_state(ref, ids, st):
+    rid, _, state, _ = ref.export(state_type=st)
+    where = {int(k): i for i, k in enumerate(rid.tolist())}
+    return state[[where[int(k)] for k in ids.tolist()]]
+
+
+def test_zero_momentum_buffer_survives_the_file(api, oracle, tmp_path):
+    """A row whose first SGD-with-momentum update had an all-zero gradient holds a momentum buffer
+    of zeros. It is a buffer all the same: the row's next update continues it,
+    buf = momentum * buf + (1 - dampening) * g (ps/optim/sgd.cc:46-52), where a row without a buffer
+    would take buf = g. With dampening != 0 the two differ, so the file must carry the buffer."""
+    dim = 8
+    t, ref = _tables(api, oracle, dim, seed=6)
+    ids = splitmix64(np.arange(500, dtype=np.uint64))
+    o_ref, o_gpu = make_optims(oracle, api, 3, {"momentum": 0.8, "dampening": 0.3})
+    assert t.Pull(ids)[0] == 0 and ref.pull(ids)[0] == 0
+    g0 = np.zeros((ids.size, dim), np.float32)
+    g0[::2] = 0.125                                                    # every second row: a zero first gradient
+    assert t.Push(o_gpu, ids, g0, 0.1) == 0 and ref.push(o_ref, ids, g0, 0.1) == 0
+    path = str(tmp_path / "m.sparse")
+    assert t.save(path, 4, "m") == 0
+    _, slots = parse_sparse(path)
+    assert all(1 in r[3] for rows in slots for r in rows)              # every row carries its buffer
+    t2, _ = _tables(api, oracle, dim, seed=6)
+    assert t2.load_file(path, 4, "m") == (0, ids.size)
+    g1 = np.full((ids.size, dim), 0.25, np.float32)
+    assert t2.Push(o_gpu, ids, g1, 0.1) == 0 and ref.push(o_ref, ids, g1, 0.1) == 0
+    assert_close(t2.Pull(ids)[1], ref.pull(ids)[1], "update after the file continues the zero buffer")
+
+
+def test_malformed_sparse_files_are_errors(api, tmp_path):
+    """Lengths that no file could back (a tensor of 2^40 elements, a string of 2^31 bytes, dims whose
+    product overflows) are refused before anything is allocated for them."""
+    dim = 4
+    gi = api.Initializer.create(api.InitializerType.kConstant, {"value": "0.25"})
+    head = struct.pack("<BQ", 1, 21) + pack_string("t") + struct.pack("<qBB", dim, 11, 0)
+    head += struct.pack("<Q", 1) + pack_string("value") + pack_string("0.250000") + struct.pack("<Q", 1)
+    cases = {
+        "huge tensor": head + struct.pack("<Q", 1) + struct.pack("<Q", 5) + struct.pack("<BQqB", 0, 1, 1 << 40, 11),
+        "overflowing dims": head + struct.pack("<Q", 1) + struct.pack("<Q", 5) +
+                            struct.pack("<BQ", 0, 3) + struct.pack("<qqq", 1 << 31, 1 << 31, 1 << 31) + b"\x0b",
+        "huge name": struct.pack("<BQ", 1, 21) + struct.pack("<Q", 1 << 31) + b"t",
+        "huge conf value": struct.pack("<BQ", 1, 21) + pack_string("t") + struct.pack("<qBB", dim, 11, 0) +
+                           struct.pack("<Q", 1) + pack_string("value") + struct.pack("<Q", 1 << 33),
+    }
+    for what, body in cases.items():
+        path = str(tmp_path / "bad.sparse")
+        open(path, "wb").write(body)
+        t = api.SparseTable(dim, gi)
+        assert t.load_file(path, 21, "t")[0] == api.E_IO, what
+        assert len(t) == 0

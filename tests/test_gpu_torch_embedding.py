@@ -252,3 +252,56 @@ def test_modules_take_the_reference_descriptions(mods, oracle):
     assert ref.push(o_ref, u2, gs, 0.25) == 0
     rid, rval, _, _ = ref.export()
     assert_close(emb.sparse_table.table().Pull(rid)[1], rval, "rows after an Adagrad step", rtol=1e-5, atol=1e-6)
+
+
+def _ordered_with_torch(api, te, oracle, seed):
+    """The pull must see indices that torch's stream produces behind a long kernel, and torch's
+    next kernel must see the rows the pull wrote: both only hold when the table's launches are
+    enqueued on the very stream torch is using."""
+    dim = 16
+    gi, oi = _init(api, oracle, seed)
+    o_ref, o_gpu = make_optims(oracle, api, 0, {})
+    emb = te.Embedding(dim, initializer=gi, optim=o_gpu, lr=0.05)
+    ref = oracle.SparseTable(dim, oi)
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    a = torch.randn(4096, 4096, device="cuda")
+    for step in range(3):
+        want = torch.randint(0, 5000, (4096,), generator=g)
+        staged = want.cuda()
+        idx = torch.full((4096,), 10**9 + step, dtype=torch.int64, device="cuda")   # stale ids
+        torch.cuda.synchronize()
+        b = a
+        for _ in range(6):                       # some milliseconds of work ahead of the copy
+            b = b @ a
+            b = b / b.abs().max()
+        idx.copy_(staged)                        # the real ids arrive behind it, on torch's stream
+        out = emb(idx)
+        total = out.sum(dim=0)                   # torch reads the rows right behind the pull
+        out.backward(torch.ones_like(out) * 0.01)
+        ids = want.numpy().astype(np.uint64)
+        u, inv = oracle.dedup(ids)
+        rc, rows = ref.pull(u)
+        assert_close(out.detach().cpu().numpy(), rows[inv], "ordered pull %d" % step, rtol=1e-6)
+        assert_close(total.detach().cpu().numpy(), rows[inv].astype(np.float64).sum(axis=0).astype(np.float32),
+                     "torch op behind the pull %d" % step, rtol=1e-4, atol=1e-6)
+        u2, gs = oracle.dedup_sum(ids, np.full((ids.size, dim), 0.01, np.float32))
+        assert ref.push(o_ref, u2, gs, 0.05) == 0
+    torch.cuda.synchronize()
+    rid, rval, _, _ = ref.export()
+    t = emb.sparse_table.table()
+    assert len(t) == len(ref)                    # no stale id was ever inserted
+    assert_close(t.Pull(rid)[1], rval, "rows after ordered steps", rtol=1e-4, atol=1e-6)
+
+
+def test_embedding_is_ordered_on_torchs_default_stream(mods, oracle):
+    api, te = mods
+    assert torch.cuda.current_stream().cuda_stream == 0      # the handle a NULL stream stands for
+    _ordered_with_torch(api, te, oracle, 21)
+
+
+def test_embedding_is_ordered_on_a_side_stream(mods, oracle):
+    api, te = mods
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        _ordered_with_torch(api, te, oracle, 22)
+    side.synchronize()
