@@ -349,6 +349,19 @@ int32_t krk_group_set_stream(krk_group* g, void* stream);
 int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv,
                   int64_t* n_unique, uint32_t flags);
 
+/* krk_dedup for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Every pointer
+ * is a device pointer, n_unique included (one int64, written on the device); the launches are
+ * enqueued on `stream` (a hipStream_t, NULL = the null stream) and the call returns without
+ * waiting. The work space (request-local index, per-position arrays, scan sums) is a fixed array
+ * of about 11.5 MB inside the library image, held by each GPU the library runs on until the
+ * process ends; more than KRK_DEDUP_NOALLOC_MAX ids return KRK_E_CAPACITY. The array is shared by
+ * all calls on a GPU: calls that overlap there (two streams, two threads) race. Results are
+ * those of krk_dedup. inv may be NULL. */
+#define KRK_DEDUP_NOALLOC_MAX (1 << 18)
+int32_t krk_dedup_noalloc(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv,
+                          int64_t* n_unique, void* stream);
+
 /* Emitter::PushSparseTable's dedup + sum as a call of its own (worker/emitter.cc:510-531), for a
  * worker whose server is elsewhere: uids as krk_dedup, sums[u, :] = the gradient rows of unique
  * id u added in position order starting from a copy of the first. grads is [n, dim]; sums needs

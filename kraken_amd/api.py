@@ -117,6 +117,7 @@ EXPORTS = {
                                              C.POINTER(C.c_int64), C.c_uint32]),
     "krk_dedup": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64),
                               C.c_uint32]),
+    "krk_dedup_noalloc": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "krk_dedup_sum": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
                                   C.c_void_p, C.POINTER(C.c_int64), C.c_uint32]),
     "krk_expand_rows": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p,
@@ -691,6 +692,18 @@ def dedup(ids):
     if isinstance(ids, DeviceArray):
         return uids, inv, u.value
     return uids[:u.value].copy(), inv
+
+
+DEDUP_NOALLOC_MAX = 1 << 18
+
+
+def dedup_noalloc(ids, uids, inv, n_unique, n=None, stream=None):
+    """krk_dedup for callers that cannot allocate: every argument is a DeviceArray the caller
+    owns (n_unique: one int64), the launches go to `stream` (None = the null stream) and nothing
+    is waited for. Returns the call's code."""
+    n = ids.size if n is None else n
+    return lib().krk_dedup_noalloc(_ptr(ids), n, _ptr(uids), _ptr(inv), _ptr(n_unique),
+                                   C.c_void_p(stream) if stream else None)
 
 
 def dedup_sum(ids, grads):

@@ -900,6 +900,25 @@ static int32_t dedup_layout(int64_t n, size_t extra_bytes, DedupWork* w) {
 // slot then holds the id's index in the unique list), every position's index in the unique list
 // into d_inv (when not null); *u = number of unique ids. The count is read back last, so the
 // call waits for the device once.
+// The launches alone, nothing read back. The index is cleared by a fill kernel rather than a
+// memset node so that a caller may record these launches into a graph.
+static int32_t dedup_enqueue(const DedupWork& w, const uint64_t* d_ids, int64_t n, uint64_t* d_uids,
+                             long long* d_inv, hipStream_t s) {
+  const int64_t words = (int64_t)(w.cap + 1) * (int64_t)(sizeof(DSlot) / 4);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(words, kBlock)), dim3(kBlock), 0, s,
+                     reinterpret_cast<uint32_t*>(w.slots), words, 0xFFFFFFFFu);
+  const dim3 grid(grid_for(n, kBlock)), block(kBlock);
+  hipLaunchKernelGGL(dedup_claim_kernel, dim3(grid_for(n, kDedupBlock)), dim3(kDedupBlock), 0, s, w.slots,
+                     w.cap - 1, d_ids, n, w.slot_of);
+  hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, w.slots, w.slot_of, n, w.flag);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
+  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids);
+  if (d_inv) hipLaunchKernelGGL(dedup_inv_kernel, grid, block, 0, s, w.slots, w.slot_of, n, d_inv);
+  KRK_HIP(hipGetLastError());
+  return KRK_SUCCESS;
+}
+
 static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, uint64_t* d_uids,
                           long long* d_inv, hipStream_t s, int32_t* u) {
   KRK_HIP(hipMemsetAsync(w.slots, 0xFF, (w.cap + 1) * sizeof(DSlot), s));
@@ -952,6 +971,90 @@ int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, 
     if (inv) KRK_HIP(hipMemcpy(inv, d_inv, (size_t)n * 8, hipMemcpyDeviceToHost));
   }
   KRK_HIP(hipStreamSynchronize(s));
+  return KRK_SUCCESS;
+}
+
+// ---- krk_dedup for callers that cannot allocate ---------------------------------------------
+// Same launches as krk_dedup, with the request-local index, the per-position arrays and the scan's
+// partial sums in one fixed array of device memory that belongs to the library image instead of
+// a pool that grows. The array is shared by every call on the device and keeps the last call's
+// contents: the index is cleared by the first launch, everything else is written before it is
+// read. Calls that overlap on one device race.
+constexpr int64_t kNoAllocCap = (int64_t)KRK_DEDUP_NOALLOC_MAX * 2;   // index slots: at most half full
+constexpr size_t kNoAllocSlotsBytes = (((size_t)kNoAllocCap + 1) * sizeof(DSlot) + 255) & ~(size_t)255;
+constexpr size_t kNoAllocN4 = (size_t)KRK_DEDUP_NOALLOC_MAX * 4;
+constexpr size_t kNoAllocScanBytes = 4096;   // one partial sum per 2048 positions: 512 bytes at the maximum
+constexpr size_t kNoAllocBytes = kNoAllocSlotsBytes + 3 * kNoAllocN4 + kNoAllocScanBytes + 256;
+
+static __device__ __align__(256) unsigned char scratch[kNoAllocBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_noalloc_mu;
+static unsigned char* g_noalloc_ptr[kMaxDevices] = {};   // the array's address on each device
+
+namespace krk {
+__global__ void widen_total_kernel(const int32_t* __restrict__ total, long long* __restrict__ out) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) *out = (long long)*total;
+}
+}  // namespace krk
+
+// The address of `scratch` on the current device (each device holds its own copy of the array
+// at its own address), resolved once per device.
+static int32_t noalloc_scratch(unsigned char** out) {
+  const int dev = current_device();
+  if (dev < 0 || dev >= kMaxDevices) {
+    set_error("device %d out of range for krk_dedup_noalloc", dev);
+    return KRK_E_ARGUMENT;
+  }
+  std::lock_guard<std::mutex> lk(g_noalloc_mu);
+  if (!g_noalloc_ptr[dev]) {
+    void* p = nullptr;
+    KRK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) {
+      set_error("hipGetSymbolAddress returned no address for the dedup work space");
+      return KRK_E_DEVICE;
+    }
+    g_noalloc_ptr[dev] = reinterpret_cast<unsigned char*>(p);
+  }
+  *out = g_noalloc_ptr[dev];
+  return KRK_SUCCESS;
+}
+
+int32_t krk_dedup_noalloc(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv,
+                          int64_t* n_unique, void* stream) {
+  if (n < 0 || !n_unique || (n > 0 && (!ids || !uids))) return KRK_E_ARGUMENT;
+  if (n > (int64_t)KRK_DEDUP_NOALLOC_MAX) {
+    set_error("krk_dedup_noalloc handles at most %d ids per call (%lld given); use krk_dedup",
+              (int)KRK_DEDUP_NOALLOC_MAX, (long long)n);
+    return KRK_E_CAPACITY;
+  }
+  KRK_TRY(ensure_runtime());
+  unsigned char* base = nullptr;
+  KRK_TRY(noalloc_scratch(&base));
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  DedupWork w;
+  uint64_t cap = 1024;
+  while (cap < (uint64_t)n * 2) cap <<= 1;
+  unsigned char* cur = base;
+  w.slots = reinterpret_cast<DSlot*>(cur); cur += kNoAllocSlotsBytes;
+  w.cap = cap;
+  w.slot_of = reinterpret_cast<uint32_t*>(cur); cur += kNoAllocN4;
+  w.flag = reinterpret_cast<int32_t*>(cur); cur += kNoAllocN4;
+  w.rank = reinterpret_cast<int32_t*>(cur); cur += kNoAllocN4;
+  w.scan_tmp = cur; cur += kNoAllocScanBytes;
+  w.d_total = reinterpret_cast<int32_t*>(cur);
+  w.extra = nullptr;
+  if (n == 0) {
+    // the count still has to arrive in the caller's memory, in stream order
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(kBlock), 0, s, reinterpret_cast<uint32_t*>(n_unique),
+                       (int64_t)2, 0u);
+    KRK_HIP(hipGetLastError());
+    return KRK_SUCCESS;
+  }
+  KRK_TRY(dedup_enqueue(w, ids, n, uids, reinterpret_cast<long long*>(inv), s));
+  hipLaunchKernelGGL(widen_total_kernel, dim3(1), dim3(64), 0, s, w.d_total,
+                     reinterpret_cast<long long*>(n_unique));
+  KRK_HIP(hipGetLastError());
   return KRK_SUCCESS;
 }
 
