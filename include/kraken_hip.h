@@ -143,6 +143,19 @@ int32_t krk_mem_info(size_t* free_bytes, size_t* total_bytes);
  * measured bandwidth ceiling, and the known-size kernel byte counters are calibrated against.
  * Pointers and size must be multiples of 16. */
 int32_t krk_stream_copy(void* dst, const void* src, size_t bytes);
+/* The measured ceilings the table kernels are compared with (no reference counterpart; null
+ * stream, not synchronised; time them with events on the null stream).
+ * krk_hbm_probe: one streaming pass over `bytes` bytes: kind 0 reads src, 1 fills dst, 2 copies
+ * src to dst; unroll = independent 16-byte accesses in flight per lane (1, 2, 4, 8);
+ * nontemporal != 0 gives them the streaming hint; blocks = workgroups of 256 lanes. dst is
+ * needed by every kind (the read-only kind never writes it). Pointers and size multiples of 16.
+ * krk_hbm_probe_lines: n random, independent 128-byte lines inside base[0, region_bytes) (the
+ * largest power-of-two number of lines that fits), eight lanes a line, read only (rmw == 0) or
+ * read, changed and written back (rmw != 0): what a table kernel does per row, without the
+ * index. salt picks the lines. base must be 128-byte aligned. */
+int32_t krk_hbm_probe(int32_t kind, int32_t unroll, int32_t nontemporal, int32_t blocks, void* dst,
+                      const void* src, size_t bytes);
+int32_t krk_hbm_probe_lines(int32_t rmw, void* base, size_t region_bytes, int64_t n, uint64_t salt);
 
 /* ---- sparse table --------------------------------------------------------- */
 typedef struct krk_sparse krk_sparse;

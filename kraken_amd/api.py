@@ -115,6 +115,8 @@ EXPORTS = {
     "krk_sparse_select_routed": (C.c_int32, [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p, C.c_int64,
                                              C.c_uint64, C.c_int32, C.c_void_p, C.c_int64,
                                              C.POINTER(C.c_int64), C.c_uint32]),
+    "krk_hbm_probe": (C.c_int32, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "krk_hbm_probe_lines": (C.c_int32, [C.c_int32, C.c_void_p, C.c_size_t, C.c_int64, C.c_uint64]),
     "krk_dedup": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64),
                               C.c_uint32]),
     "krk_dedup_noalloc": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),

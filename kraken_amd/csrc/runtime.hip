@@ -510,3 +510,148 @@ extern "C" int32_t krk_stream_copy(void* dst, const void* src, size_t bytes) {
   KRK_HIP(hipGetLastError());
   return KRK_SUCCESS;
 }
+
+// ---------------------------------------------------------------------------
+// Bandwidth ceilings of this GPU, measured rather than quoted: streaming read / fill / copy
+// kernels with 1-8 independent 16-byte accesses in flight per lane, with and without the
+// non-temporal hint, over a caller-chosen number of workgroups; and random 128-byte lines (read
+// only, or read-modify-write), the access pattern of the table kernels. The harness sweeps the
+// variants and keeps the best of each kind.
+// ---------------------------------------------------------------------------
+namespace krk {
+
+template <bool NT>
+__device__ __forceinline__ uint4 probe_load(const uint4* p) {
+  if (NT) {
+    const unsigned long long* q = reinterpret_cast<const unsigned long long*>(p);
+    const unsigned long long a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1);
+    return uint4{(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
+  }
+  return *p;
+}
+template <bool NT>
+__device__ __forceinline__ void probe_store(uint4* p, const uint4& v) {
+  if (NT) {
+    unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
+    __builtin_nontemporal_store((unsigned long long)v.x | ((unsigned long long)v.y << 32), q);
+    __builtin_nontemporal_store((unsigned long long)v.z | ((unsigned long long)v.w << 32), q + 1);
+  } else {
+    *p = v;
+  }
+}
+
+// kind 0: read src (one value per workgroup survives), 1: fill dst, 2: copy src -> dst
+template <int KIND, int U, bool NT>
+__global__ __launch_bounds__(256) void hbm_stream_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                         int64_t n16, uint4* __restrict__ sink) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  uint4 acc = {0u, 0u, 0u, 0u};
+  const uint4 fill = {7u, 7u, 7u, 7u};
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + (U - 1) * stride < n16; i += U * stride) {
+    uint4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = KIND == 1 ? fill : probe_load<NT>(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (KIND == 0) {
+        acc.x ^= v[u].x; acc.y ^= v[u].y; acc.z ^= v[u].z; acc.w ^= v[u].w;
+      } else {
+        probe_store<NT>(dst + i + u * stride, v[u]);
+      }
+    }
+  }
+  for (; i < n16; i += stride) {
+    const uint4 v = KIND == 1 ? fill : src[i];
+    if (KIND == 0) {
+      acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
+    } else {
+      dst[i] = v;
+    }
+  }
+  // never true for the harness's buffers; keeps the loads of the read-only kind alive
+  if (KIND == 0 && (acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[blockIdx.x & 63] = acc;
+}
+
+template <int KIND, int U>
+static void launch_stream_nt(bool nt, unsigned blocks, const uint4* src, uint4* dst, int64_t n16, uint4* sink) {
+  if (nt) {
+    hipLaunchKernelGGL((hbm_stream_kernel<KIND, U, true>), dim3(blocks), dim3(256), 0, nullptr, src, dst, n16, sink);
+  } else {
+    hipLaunchKernelGGL((hbm_stream_kernel<KIND, U, false>), dim3(blocks), dim3(256), 0, nullptr, src, dst, n16, sink);
+  }
+}
+template <int KIND>
+static bool launch_stream(int unroll, bool nt, unsigned blocks, const uint4* src, uint4* dst, int64_t n16,
+                          uint4* sink) {
+  switch (unroll) {
+    case 1: launch_stream_nt<KIND, 1>(nt, blocks, src, dst, n16, sink); return true;
+    case 2: launch_stream_nt<KIND, 2>(nt, blocks, src, dst, n16, sink); return true;
+    case 4: launch_stream_nt<KIND, 4>(nt, blocks, src, dst, n16, sink); return true;
+    case 8: launch_stream_nt<KIND, 8>(nt, blocks, src, dst, n16, sink); return true;
+    default: return false;
+  }
+}
+
+// n random 128-byte lines of `base` (line number = mix64(i ^ salt) & line_mask), eight lanes a
+// line. RMW = false: read only; true: one word of the line is changed and the line written back.
+template <bool RMW>
+__global__ __launch_bounds__(256) void hbm_lines_kernel(uint4* __restrict__ base, uint64_t line_mask, int64_t n,
+                                                        uint64_t salt, uint4* __restrict__ sink) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
+  const int part = threadIdx.x & 7;
+  if (i >= n) return;
+  uint4* p = base + (mix64((uint64_t)i ^ salt) & line_mask) * 8 + part;
+  uint4 v = *p;
+  if (RMW) {
+    v.x += 1u;
+    *p = v;
+  } else if ((v.x ^ v.w) == 0x9e3779b9u && v.y == 0x85ebca6bu) {
+    sink[part] = v;
+  }
+}
+
+}  // namespace krk
+
+extern "C" int32_t krk_hbm_probe(int32_t kind, int32_t unroll, int32_t nontemporal, int32_t blocks, void* dst,
+                                 const void* src, size_t bytes) {
+  KRK_TRY(ensure_runtime());
+  if (kind < 0 || kind > 2 || blocks <= 0 || blocks > (1 << 20) || (bytes & 15) || bytes < 1024 ||
+      ((uintptr_t)dst & 15) || ((uintptr_t)src & 15) || !dst || (kind != 1 && !src)) {
+    set_error("krk_hbm_probe: bad argument");
+    return KRK_E_ARGUMENT;
+  }
+  const int64_t n16 = (int64_t)(bytes / 16);
+  const uint4* s = reinterpret_cast<const uint4*>(src);
+  uint4* d = reinterpret_cast<uint4*>(dst);
+  bool ok;
+  // the read-only kind uses the first 1 KiB of dst as the place its impossible store would go
+  if (kind == 0) ok = launch_stream<0>(unroll, nontemporal != 0, (unsigned)blocks, s, d, n16, d);
+  else if (kind == 1) ok = launch_stream<1>(unroll, nontemporal != 0, (unsigned)blocks, s, d, n16, d);
+  else ok = launch_stream<2>(unroll, nontemporal != 0, (unsigned)blocks, s, d, n16, d);
+  if (!ok) {
+    set_error("krk_hbm_probe: unroll must be 1, 2, 4 or 8");
+    return KRK_E_ARGUMENT;
+  }
+  KRK_HIP(hipGetLastError());
+  return KRK_SUCCESS;
+}
+
+extern "C" int32_t krk_hbm_probe_lines(int32_t rmw, void* base, size_t region_bytes, int64_t n, uint64_t salt) {
+  KRK_TRY(ensure_runtime());
+  if (!base || ((uintptr_t)base & 127) || region_bytes < 4096 || n <= 0 || n > ((int64_t)1 << 27)) {
+    set_error("krk_hbm_probe_lines: bad argument");
+    return KRK_E_ARGUMENT;
+  }
+  uint64_t lines = 1;
+  while (lines * 2 * 128 <= region_bytes) lines *= 2;   // the largest power of two that fits
+  uint4* b = reinterpret_cast<uint4*>(base);
+  const dim3 grid((unsigned)((n * 8 + 255) / 256)), block(256);
+  if (rmw) {
+    hipLaunchKernelGGL(krk::hbm_lines_kernel<true>, grid, block, 0, nullptr, b, lines - 1, n, salt, b);
+  } else {
+    hipLaunchKernelGGL(krk::hbm_lines_kernel<false>, grid, block, 0, nullptr, b, lines - 1, n, salt, b);
+  }
+  KRK_HIP(hipGetLastError());
+  return KRK_SUCCESS;
+}

@@ -365,6 +365,10 @@ struct TableDesc {
 // in workgroups of the one-launch kernels (block_start) and in positions (row_start).
 struct GroupCall {
   int32_t n_tables;
+  // > 0: every member owns exactly this many workgroups (block_start[t] = t * even_blocks), so a
+  // workgroup finds its member by one division instead of walking block_start. The host lays a
+  // request out like this whenever that costs at most a quarter more workgroups.
+  uint32_t even_blocks;
   uint32_t epoch[kMaxGroupTables];
   uint32_t block_start[kMaxGroupTables + 1];
   int64_t row_start[kMaxGroupTables + 1];

@@ -375,6 +375,7 @@ __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64
 // Table t owns workgroups [block_start[t], block_start[t+1]) and the positions
 // [row_start[t], row_start[t+1]) of the concatenated ids / rows.
 __device__ __forceinline__ int find_table(const GroupCall& c) {
+  if (c.even_blocks) return (int)(blockIdx.x / c.even_blocks);
   int t = 0;
   while (t + 1 < c.n_tables && blockIdx.x >= c.block_start[t + 1]) ++t;
   return t;
@@ -1941,7 +1942,8 @@ int32_t krk::group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, i
   const int n = (int)g->tables.size();
   const int per_block = kBlock / g->group;
   call->n_tables = n;
-  uint64_t blocks = 0;
+  call->even_blocks = 0;
+  uint64_t blocks = 0, widest = 0;
   if (offsets[0] != 0) return KRK_E_ARGUMENT;
   for (int i = 0; i < n; ++i) {
     const int64_t cnt = offsets[i + 1] - offsets[i];
@@ -1951,7 +1953,16 @@ int32_t krk::group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, i
     }
     call->block_start[i] = (uint32_t)blocks;
     call->row_start[i] = offsets[i];
-    blocks += (uint64_t)((cnt + per_block - 1) / per_block);
+    const uint64_t mine = (uint64_t)((cnt + per_block - 1) / per_block);
+    blocks += mine;
+    if (mine > widest) widest = mine;
+  }
+  // Members of similar size (the usual combined request): give each the same number of
+  // workgroups. The surplus workgroups find no position of theirs and leave at once.
+  if (widest > 0 && widest * (uint64_t)n <= blocks + blocks / 4 + (uint64_t)n) {
+    call->even_blocks = (uint32_t)widest;
+    for (int i = 0; i < n; ++i) call->block_start[i] = (uint32_t)(widest * (uint64_t)i);
+    blocks = widest * (uint64_t)n;
   }
   if (blocks * (uint64_t)kBlock >= 0x7FFFFFFFull) {
     set_error("combined request too large for one launch; split it");
