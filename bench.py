@@ -34,7 +34,8 @@ HBM_PEAK_GBS = 8000.0
 # each scaled by what it reads for the plain 1 GiB copy kernel); the runs and their commands are
 # summarised in profiles/wide_deep_adagrad_d16_hbm_counters.md. Counters cannot be read from
 # inside this script, so the figure is carried here for the workload it was measured on.
-COUNTER_TRAFFIC_BYTES = {"wide_deep": 45.3e6}
+COUNTER_FIGURES = {"wide_deep": {"traffic": 45.3e6, "tcc_hit_rate": None,
+                                 "source": "profiles/wide_deep_adagrad_d16_hbm_counters.md"}}
 
 WORKLOADS = {
     # name: tables, id space, zipf s, dim, ids per table per step, optimizer, dense params
@@ -85,11 +86,20 @@ def table_ids(cfg, t, lo, hi):
     return splitmix64(np.arange(lo, hi, dtype=np.uint64) + np.uint64(t) * np.uint64(cfg["space"]))
 
 
-def run_gpu(cfg, steps, warmup, n_batches=32):
+def _percentiles(xs):
+    xs = np.sort(np.asarray(xs, np.float64))
+    return float(np.median(xs)), float(xs[int(0.1 * (xs.size - 1))]), float(xs[int(np.ceil(0.9 * (xs.size - 1)))])
+
+
+def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32):
+    """Builds the workload's tables, fills their key space, and times `blocks` blocks of `steps`
+    steps each (a synchronisation on both sides of every block). -> dict of figures."""
+    import ctypes as C
     from kraken_amd import api
-    rc = api.lib().krk_runtime_init(0)
+    L = api.lib()
+    rc = L.krk_runtime_init(0)
     if rc != 0:
-        raise RuntimeError("no usable GPU: " + api.lib().krk_last_error_string().decode())
+        raise RuntimeError("no usable GPU: " + L.krk_last_error_string().decode())
     dim = cfg["dim"]
     batches = make_batches(cfg, n_batches, seed=1)
     init = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "0"})
@@ -114,35 +124,6 @@ def run_gpu(cfg, steps, warmup, n_batches=32):
         dev.append((api.DeviceArray.from_host(ids), api.DeviceArray.from_host(g),
                     api.DeviceArray((ids.size, dim), np.float32), off, ids.size))
 
-    # several tables: one combined request per step (one launch each way); a single table
-    # is called directly, as a server with one sparse table would
-    def pull(d_ids, off, d_out):
-        if single:
-            tables[0].Pull(d_ids, out=d_out, async_=True)
-        else:
-            group.CombinePull(d_ids, off, out=d_out, async_=True)
-
-    def push(d_ids, off, d_g):
-        if single:
-            tables[0].Push(optim, d_ids, d_g, lr, async_=True)
-        else:
-            group.CombinePush(optim, d_ids, off, d_g, lr, async_=True)
-
-    def step(i):
-        d_ids, d_g, d_out, off, _ = dev[i % n_batches]
-        pull(d_ids, off, d_out)
-        push(d_ids, off, d_g)
-        if dense is not None:
-            dense.Push(dense_opt, d_dense_g[i % n_batches], 1e-3, async_=True)
-
-    def sync_all():
-        rc = owner.sync()
-        if rc != 0:
-            raise RuntimeError("sparse tables reported error %d" % rc)
-        if dense is not None:
-            dense.sync()
-        api.synchronize()
-
     # steady state: every id of the key space is resident before timing, so a step's rows come
     # from HBM-sized tables (the hot head of the Zipf draw stays in cache, the tail does not)
     chunk = 1 << 22
@@ -160,58 +141,119 @@ def run_gpu(cfg, steps, warmup, n_batches=32):
     single = len(tables) == 1
     group = None if single else api.TableGroup(tables)
     owner = tables[0] if single else group          # whose stream the step's launches run on
+
+    # The step's three calls through the C ABI, arguments converted once: a C++ server thread
+    # pays no argument marshalling either. several tables: one combined request per step (one
+    # launch each way); a single table is called directly.
+    flags = api.DEVICE_PTRS | api.ASYNC
+    o_raw = C.byref(optim.raw)
+    calls = []
+    for i in range(n_batches):
+        d_ids, d_g, d_out, off, n = dev[i]
+        p_ids, p_g, p_out = C.c_void_p(d_ids.ptr), C.c_void_p(d_g.ptr), C.c_void_p(d_out.ptr)
+        if single:
+            pull = (L.krk_sparse_pull, (tables[0].h, p_ids, n, p_out, flags))
+            push = (L.krk_sparse_push, (tables[0].h, o_raw, p_ids, n, p_g, dim, lr, flags))
+        else:
+            p_off = off.ctypes.data_as(C.c_void_p)
+            pull = (L.krk_group_pull, (group.h, p_ids, p_off, p_out, flags))
+            push = (L.krk_group_push, (group.h, o_raw, p_ids, p_off, p_g, dim, lr, flags))
+        dpush = None
+        if dense is not None:
+            dpush = (L.krk_dense_push, (dense.h, C.byref(dense_opt.raw), C.c_void_p(d_dense_g[i].ptr),
+                                        cfg["dense"], 1e-3, flags))
+        calls.append((pull, push, dpush))
+
+    def step(i):
+        pull, push, dpush = calls[i % n_batches]
+        rc = pull[0](*pull[1]) | push[0](*push[1])
+        if dpush is not None:
+            rc |= dpush[0](*dpush[1])
+        if rc:
+            raise RuntimeError("step failed: " + L.krk_last_error_string().decode())
+
+    def sync_all():
+        rc = owner.sync()
+        if rc != 0:
+            raise RuntimeError("sparse tables reported error %d" % rc)
+        if dense is not None:
+            dense.sync()
+        api.synchronize()
+
     for i in range(n_batches):
         step(i)
     sync_all()
     for i in range(warmup):
         step(i)
     sync_all()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        step(i)
-    t_enq = time.perf_counter() - t0
-    sync_all()
-    dt = time.perf_counter() - t0
-    print("host enqueue %.1f us/step, drained %.1f us/step" % (t_enq / steps * 1e6, dt / steps * 1e6),
-          file=sys.stderr)
-    rows = sum(dev[i % n_batches][4] for i in range(steps))
+    per_step, enq = [], []
+    rows_per_step = float(np.mean([dev[i % n_batches][4] for i in range(steps)]))
+    for b in range(blocks):
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(i)
+        t1 = time.perf_counter()
+        sync_all()
+        t2 = time.perf_counter()
+        per_step.append((t2 - t0) / steps)
+        enq.append((t1 - t0) / steps)
+    med, p10, p90 = _percentiles(per_step)
+    print("dim %d: host enqueue %.1f us/step, drained %.1f us/step (median of %d blocks of %d steps)" % (
+        dim, np.median(enq) * 1e6, med * 1e6, blocks, steps), file=sys.stderr)
 
-    # dominant kernel: the fused push over all tables of the request. M back-to-back launches
-    # on the group's stream, bracketed by HIP events recorded on that stream.
+    # the two kernels of the step: M back-to-back launches on the owner's stream, bracketed by
+    # HIP events recorded on that stream
     S = state_arrays(cfg["optim"])
     e0, e1 = api.Event(), api.Event()
     reps = 50 if cfg["batch"] < 10**6 else 10
-    for kind in ("push", "pull"):
-        for timed in (False, True):
-            if timed:
-                e0.record(owner)
+    timed = {}
+    for kind in (1, 0):
+        samples = []
+        for trial in range(6):
+            e0.record(owner)
             for j in range(reps):
-                d_ids, d_g, d_out, off, _ = dev[j % n_batches]
-                if kind == "push":
-                    push(d_ids, off, d_g)
-                else:
-                    pull(d_ids, off, d_out)
-            if timed:
-                e1.record(owner)
+                c = calls[j % n_batches][kind]
+                c[0](*c[1])
+            e1.record(owner)
             owner.sync()
-        ms = e0.elapsed_ms(e1) / reps
-        u = float(np.mean([dev[j % n_batches][4] for j in range(reps)]))
-        if kind == "push":
-            push_ms, push_u = ms, u
-        else:
-            pull_ms, pull_u = ms, u
+            if trial:
+                samples.append(e0.elapsed_ms(e1) / reps)
+        timed[kind] = float(np.median(samples))
+    push_ms, pull_ms = timed[1], timed[0]
+    u = float(np.mean([dev[j % n_batches][4] for j in range(reps)]))
     extra = 16 if cfg["optim"] == "adam" else 0
-    push_bytes = push_u * (8 + 4 * dim + 8 * dim * (1 + S) + extra)
-    pull_bytes = pull_u * (8 + 8 * dim)
+    push_bytes = u * (8 + 4 * dim + 8 * dim * (1 + S) + extra)
+    pull_bytes = u * (8 + 8 * dim)
     roofline = {
         "bound": "hbm", "kernel": "%spush_kernel<%s,4>" % ("" if single else "group_", cfg["optim"]),
         "achieved": push_bytes / (push_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": push_bytes / (push_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
         "bytes_per_launch": push_bytes, "us_per_launch": push_ms * 1e3,
         "pull_kernel": {"achieved": pull_bytes / (pull_ms * 1e-3) / 1e9, "us_per_launch": pull_ms * 1e3,
-                        "bytes_per_launch": pull_bytes},
+                        "bytes_per_launch": pull_bytes,
+                        "frac": pull_bytes / (pull_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
-    return dt, rows, roofline, batches
+    per_row = 16 + 4 * dim * (2 + 1 + 2 * (1 + S)) + extra
+    res = {
+        "value": rows_per_step / med, "ms_per_step": med * 1e3, "ms_per_step_p10": p10 * 1e3,
+        "ms_per_step_p90": p90 * 1e3, "blocks": blocks, "rows_per_step": rows_per_step,
+        "host_enqueue_us_per_step": float(np.median(enq) * 1e6),
+        "algorithmic_bytes_per_row": per_row,
+        "achieved_gbs_whole_step": rows_per_step / med * per_row / 1e9,
+        "frac_whole_step": rows_per_step / med * per_row / 1e9 / HBM_PEAK_GBS,
+        "roofline": roofline, "batches": batches,
+    }
+    # give the memory back before the next configuration is built
+    if group is not None:
+        group.close()
+    for t in tables:
+        t.close()
+    if dense is not None:
+        dense.close()
+    for d in dev:
+        for a in d[:3]:
+            a.free()
+    return res
 
 
 def run_cpu(cfg, batches, budget_s=20.0, threads=1, n_tables=4, prefill_cap=2 * 10**6):
@@ -272,7 +314,7 @@ def run_cpu(cfg, batches, budget_s=20.0, threads=1, n_tables=4, prefill_cap=2 * 
 
 
 def copy_calibration(nbytes=1 << 30, reps=20):
-    """A plain device-to-device copy of known size: the measured bandwidth ceiling."""
+    """The plain 1 GiB device-to-device copy kernel that hardware byte counters are scaled by."""
     from kraken_amd import api
     L = api.lib()
     if L.krk_runtime_init(0) != 0:
@@ -288,8 +330,98 @@ def copy_calibration(nbytes=1 << 30, reps=20):
         L.krk_stream_copy(api._ptr(b), api._ptr(a), nbytes)
     api.synchronize()
     dt = (time.perf_counter() - t0) / reps
+    a.free()
+    b.free()
     return {"kernel": "stream_copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes,
             "us_per_launch": dt * 1e6, "copy_gbs_read_plus_write": 2 * nbytes / dt / 1e9}
+
+
+def hbm_ceilings(nbytes=1 << 31, verbose=False):
+    """What this GPU's memory delivers to the simplest kernels, measured now: streaming read, fill
+    and copy (best over unroll x non-temporal x workgroup count, HIP events on the null stream
+    around 5 launches), and random independent 128-byte lines over a 16 GiB region, read only and
+    read-modify-write (the table kernels' access pattern without their index). GB/s."""
+    from kraken_amd import api
+    L = api.lib()
+    if L.krk_runtime_init(0) != 0:
+        raise RuntimeError("no usable GPU: " + L.krk_last_error_string().decode())
+    a = api.DeviceArray(nbytes // 4, np.float32)
+    b = api.DeviceArray(nbytes // 4, np.float32)
+    L.krk_memset(api._ptr(a), 1, nbytes)
+    L.krk_memset(api._ptr(b), 2, nbytes)
+    e0, e1 = api.Event(), api.Event()
+
+    def timed(fn, reps=5):
+        fn()
+        e0.record(None)
+        for _ in range(reps):
+            fn()
+        e1.record(None)
+        return e0.elapsed_ms(e1) / reps * 1e-3
+
+    best = {}
+    table = []
+    for kind, name, moved in ((0, "read", nbytes), (1, "write", nbytes), (2, "copy", 2 * nbytes)):
+        for unroll in (1, 2, 4, 8):
+            for nt in (0, 1):
+                for blocks in (256, 512, 1024, 4096):
+                    def run():
+                        rc = L.krk_hbm_probe(kind, unroll, nt, blocks, api._ptr(b), api._ptr(a), nbytes)
+                        if rc:
+                            raise RuntimeError(L.krk_last_error_string().decode())
+                    gbs = moved / timed(run) / 1e9
+                    table.append((name, unroll, nt, blocks, gbs))
+                    if gbs > best.get(name, (0,))[0]:
+                        best[name] = (gbs, {"unroll": unroll, "nontemporal": nt, "workgroups": blocks})
+    a.free()
+    b.free()
+    region = 1 << 34
+    big = api.DeviceArray(region // 4, np.float32)
+    L.krk_memset(api._ptr(big), 1, region)
+    lines = {}
+    for n in (98600, 1 << 20, 1 << 22):
+        for rmw, name in ((0, "random_line_read"), (1, "random_line_rmw")):
+            salt = [1]
+
+            def run():
+                salt[0] += 1
+                rc = L.krk_hbm_probe_lines(rmw, api._ptr(big), region, n, salt[0] * 0x9E3779B97F4A7C15 % (1 << 64))
+                if rc:
+                    raise RuntimeError(L.krk_last_error_string().decode())
+            sec = timed(run, reps=10)
+            lines["%s_%d" % (name, n)] = {"us_per_launch": sec * 1e6, "lines_per_s": n / sec,
+                                          "gbs": n * 128 * (2 if rmw else 1) / sec / 1e9}
+    big.free()
+    out = {
+        "read_ceiling": best["read"][0], "read_variant": best["read"][1],
+        "write_ceiling": best["write"][0], "write_variant": best["write"][1],
+        "copy_ceiling": best["copy"][0], "copy_variant": best["copy"][1],
+        "random_line_read_ceiling": lines["random_line_read_%d" % (1 << 22)]["gbs"],
+        "random_line_rmw_ceiling": lines["random_line_rmw_%d" % (1 << 22)]["gbs"],
+        "random_lines": lines, "unit": "GB/s",
+    }
+    if verbose:
+        out["stream_table"] = [dict(kind=k, unroll=u, nontemporal=nt, workgroups=bl, gbs=g)
+                               for k, u, nt, bl, g in table]
+    return out
+
+
+def host_description():
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        affinity = len(os.sched_getaffinity(0))
+    except AttributeError:
+        affinity = os.cpu_count()
+    return {"nproc": os.cpu_count(), "usable_cpus": affinity, "cpu_model": model,
+            "pinning": "none (threads float over the usable cpus)"}
 
 
 def main():
@@ -297,58 +429,84 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--blocks", type=int, default=30,
+                    help="timed blocks of --steps steps each; the line carries their median, p10 and p90")
     ap.add_argument("--workload", default="wide_deep", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-dims", action="store_true", help="skip the dim 32 / dim 64 legs of the default workload")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain 1 GiB streaming-copy kernel (hardware byte counters are "
                          "scaled by what they read for it) and print its bandwidth")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="only measure the streaming and random-line ceilings (every variant listed)")
     args = ap.parse_args()
     if args.copy_calibration:
         print(json.dumps(copy_calibration()))
+        return
+    if args.ceilings:
+        print(json.dumps(hbm_ceilings(verbose=True)))
         return
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
     cfg = WORKLOADS[args.workload]
-    dt, rows, roofline, batches = run_gpu(cfg, args.steps, args.warmup)
-    # the same achieved figure against what a plain copy kernel moves on this very box
-    ceiling = copy_calibration(nbytes=1 << 30, reps=10)["copy_gbs_read_plus_write"]
-    roofline["copy_ceiling"] = ceiling
-    roofline["frac_of_copy_ceiling"] = roofline["achieved"] / ceiling
-    value = rows / dt
+    r = run_gpu(cfg, args.steps, args.warmup, blocks=args.blocks)
+    batches = r.pop("batches")
+    roofline = r.pop("roofline")
+    ceil = hbm_ceilings()
+    roofline["ceilings"] = ceil
+    # the push reads and writes random lines: its honest ceiling is the random-line one
+    roofline["frac_of_random_line_rmw_ceiling"] = roofline["achieved"] / ceil["random_line_rmw_ceiling"]
+    roofline["copy_ceiling"] = ceil["copy_ceiling"]
+    roofline["frac_of_copy_ceiling"] = roofline["achieved"] / ceil["copy_ceiling"]
+    carried = COUNTER_FIGURES.get(args.workload)
+    if carried:
+        roofline["traffic"] = carried["traffic"]
+        roofline["traffic_source"] = carried["source"] + " (carried: hardware counters cannot be read from inside this process)"
+        roofline["tcc_hit_rate"] = carried["tcc_hit_rate"]
     dim = cfg["dim"]
-    S = state_arrays(cfg["optim"])
-    per_row = 16 + 4 * dim * (2 + 1 + 2 * (1 + S)) + (16 if cfg["optim"] == "adam" else 0)
-    roofline["traffic"] = COUNTER_TRAFFIC_BYTES.get(args.workload)
     line = {
         "metric": "sparse pull+push unique-rows/sec (%s, dim %d fp32)" % (cfg["optim"], dim),
-        "value": value, "unit": "unique-rows/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
+        "value": r["value"], "unit": "unique-rows/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "ms_per_step_p10": r["ms_per_step_p10"],
+        "ms_per_step_p90": r["ms_per_step_p90"], "timed_blocks": r["blocks"],
+        "host_enqueue_us_per_step": r["host_enqueue_us_per_step"],
+        "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": args.workload, "tables": cfg["tables"], "dim": dim,
                    "ids_per_table_per_step": cfg["batch"], "id_space": cfg["space"],
                    "zipf_s": cfg["s"], "optimizer": cfg["optim"], "dense_params": cfg["dense"],
+                   "unique_rows_per_step": r["rows_per_step"],
                    "boundary": "unique ids (server boundary), inputs resident in HBM"},
-        "algorithmic_bytes_per_row": per_row,
-        "achieved_gbs_whole_step": value * per_row / 1e9,
+        "algorithmic_bytes_per_row": r["algorithmic_bytes_per_row"],
+        "achieved_gbs_whole_step": r["achieved_gbs_whole_step"],
+        "frac_whole_step": r["frac_whole_step"],
         "roofline": roofline,
     }
+    if args.workload == "wide_deep" and not args.no_dims:
+        by_dim = {}
+        for d in (32, 64):
+            c2 = dict(cfg, dim=d)
+            r2 = run_gpu(c2, args.steps, args.warmup, blocks=args.blocks)
+            r2.pop("batches")
+            by_dim[str(d)] = r2
+        line["by_dim"] = by_dim
     if not args.no_cpu:
-        ncpu = min(16, os.cpu_count() or 1)
+        host = host_description()
+        ncpu = min(16, host["usable_cpus"] or 1)
         # three points: one caller thread, the reference server's default of two
         # (ps_server_main.cc:6), and eight (its eight slot locks bound the concurrency)
         v1, s1 = run_cpu(cfg, batches, budget_s=8.0, threads=1)
         v2, s2 = run_cpu(cfg, batches, budget_s=8.0, threads=min(2, ncpu))
         threads = min(8, ncpu)
         v8, s8 = run_cpu(cfg, batches, budget_s=8.0, threads=threads)
-        best, cores = max(((v1, 1), (v2, min(2, ncpu)), (v8, threads)))
         line["cpu_baseline"] = {
-            "value": best, "unit": "unique-rows/s", "cores": cores, "kind": "port",
-            "sample": "first 4 tables of the workload with their key space resident, %d steps "
-                      "(same ids, gradients, optimizer) through the CPU oracle in process; "
-                      "1 thread: %.3g rows/s, 2 threads: %.3g rows/s, %d threads: %.3g rows/s"
-                      % (s1 + s2 + s8, v1, v2, threads, v8),
+            "value": v2, "unit": "unique-rows/s", "cores": min(2, ncpu), "kind": "port",
+            "threads_1": v1, "threads_2": v2, "threads_%d" % threads: v8, "host": host,
+            "sample": "first 4 of the workload's %d tables with their key space resident, %d steps in all "
+                      "(same ids, gradients, optimizer) through the CPU oracle in process; value = the "
+                      "reference server's default of 2 caller threads" % (cfg["tables"], s1 + s2 + s8),
         }
     print(json.dumps(line))
 
