@@ -184,7 +184,7 @@ __global__ __launch_bounds__(kBlock) void rows_of_ids_kernel(TableView tv, const
     r = miss_key;
   }
   keys[p] = r;
-  pos[p] = payload_is_bag ? bag : (uint32_t)p;
+  if (pos) pos[p] = payload_is_bag ? bag : (uint32_t)p;
 }
 
 // The same for a combined request: position p belongs to the member whose [row_start, row_start
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(kBlock) void group_rows_of_ids_kernel(const TableDe
     r |= (uint32_t)m << row_bits;
   }
   keys[p] = r;
-  pos[p] = (uint32_t)p;
+  if (pos) pos[p] = (uint32_t)p;
 }
 
 // ---- pooled pushes: from bag offsets to per-position bag numbers ----------------
@@ -261,23 +261,36 @@ struct ApplyArgs {
 // just store it as row `row` of the output.
 constexpr int kOptStore = 4;
 
+// A lane's slice of a record: weight and the optimizer's state columns.
+template <int VEC>
+struct RowRegs {
+  float w[VEC], s0[VEC], s1[VEC], s2[VEC];
+};
+
+// Requests the lane's slice of row `row`. Kept apart from the update so that a caller can have
+// the record on its way while it is still adding up the row's gradient.
 template <int OPT, int VEC>
-__device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, const float (&gsum)[VEC],
-                                          int e, bool lane_on, int gl, bool last_chunk, int dim,
-                                          const ApplyArgs& a) {
+__device__ __forceinline__ void load_row(const TableView& tv, uint32_t row, int e, bool lane_on, const ApplyArgs& a,
+                                         RowRegs<VEC>& r) {
+  if constexpr (OPT == kOptStore) return;
+  const float* rec = tv.recs + (int64_t)row * tv.stride;
+  if (lane_on) {
+    vload<VEC>(rec + e * VEC, r.w);
+    if (a.c0 >= 0) vload<VEC>(rec + a.c0 + e * VEC, r.s0);
+    if (a.c1 >= 0) vload<VEC>(rec + a.c1 + e * VEC, r.s1);
+    if (a.c2 >= 0) vload<VEC>(rec + a.c2 + e * VEC, r.s2);
+  }
+}
+
+// The update of row `row` with the summed gradient, on the slice load_row requested.
+template <int OPT, int VEC>
+__device__ __forceinline__ void finish_row(const TableView& tv, uint32_t row, const float (&gsum)[VEC], int e,
+                                           bool lane_on, int gl, bool last_chunk, int dim, const ApplyArgs& a,
+                                           RowRegs<VEC>& r) {
   float* rec = tv.recs + (int64_t)row * tv.stride;
   if constexpr (OPT == kOptStore) {
     if (lane_on) vstore<VEC>(rec + e * VEC, gsum);
     return;
-  }
-  // the lane's slice of the record is requested before the 64-bit word is looked at: the bias
-  // corrections (two powf) then overlap with the loads instead of preceding them
-  float w[VEC], s0[VEC], s1[VEC], s2[VEC];
-  if (lane_on) {
-    vload<VEC>(rec + e * VEC, w);
-    if (a.c0 >= 0) vload<VEC>(rec + a.c0 + e * VEC, s0);
-    if (a.c1 >= 0) vload<VEC>(rec + a.c1 + e * VEC, s1);
-    if (a.c2 >= 0) vload<VEC>(rec + a.c2 + e * VEC, s2);
   }
   bool first = false;
   float bc1 = 1.0f, bc2 = 1.0f;
@@ -300,18 +313,29 @@ __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, con
   if (lane_on) {
 #pragma unroll
     for (int c = 0; c < VEC; ++c) {
-      if (a.c0 < 0) s0[c] = 0.0f;
-      if (a.c1 < 0) s1[c] = 0.0f;
-      if (a.c2 < 0) s2[c] = 0.0f;
-      optim_element<OPT>(a.k, a.lr, gsum[c], w[c], s0[c], s1[c], s2[c], first, bc1, bc2);
+      if (a.c0 < 0) r.s0[c] = 0.0f;
+      if (a.c1 < 0) r.s1[c] = 0.0f;
+      if (a.c2 < 0) r.s2[c] = 0.0f;
+      optim_element<OPT>(a.k, a.lr, gsum[c], r.w[c], r.s0[c], r.s1[c], r.s2[c], first, bc1, bc2);
     }
-    vstore<VEC>(rec + e * VEC, w);
-    if (a.c0 >= 0) vstore<VEC>(rec + a.c0 + e * VEC, s0);
-    if (a.c1 >= 0) vstore<VEC>(rec + a.c1 + e * VEC, s1);
-    if (a.c2 >= 0) vstore<VEC>(rec + a.c2 + e * VEC, s2);
+    vstore<VEC>(rec + e * VEC, r.w);
+    if (a.c0 >= 0) vstore<VEC>(rec + a.c0 + e * VEC, r.s0);
+    if (a.c1 >= 0) vstore<VEC>(rec + a.c1 + e * VEC, r.s1);
+    if (a.c2 >= 0) vstore<VEC>(rec + a.c2 + e * VEC, r.s2);
   }
   // The counter is read by every chunk of the row before the last chunk advances it.
   if (a.meta_off >= 0 && last_chunk) store_row_word<VEC>(rec + a.meta_off, steps, gl, dim, (int)tv.stride - a.meta_off);
+}
+
+// The lane's slice of the record is requested before the 64-bit word is looked at: the bias
+// corrections (two powf) then overlap with the loads instead of preceding them.
+template <int OPT, int VEC>
+__device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, const float (&gsum)[VEC],
+                                          int e, bool lane_on, int gl, bool last_chunk, int dim,
+                                          const ApplyArgs& a) {
+  RowRegs<VEC> r;
+  load_row<OPT, VEC>(tv, row, e, lane_on, a, r);
+  finish_row<OPT, VEC>(tv, row, gsum, e, lane_on, gl, last_chunk, dim, a, r);
 }
 
 // keys[cnt] ascending (entries >= empty_from are holes). LEVEL0: the value of entry j is gradient
@@ -670,47 +694,372 @@ static hipError_t sort_pairs(void* tmp, size_t& tmp_bytes, uint32_t* keys, uint3
   return sort_pairs_with<8>(tmp, tmp_bytes, keys, keys_out, vals, vals_out, n, bits, stream);
 }
 
-// Combined requests whose members each bring at most 8192 ids: one workgroup per member sorts
-// that member's pairs in LDS, all members in one launch (26 tables of 8192 ids: 23 us, against
-// 45 us for histogram, scan and three digit passes over the whole request). Inside a member's
-// segment the member number is constant, so only the row bits are sorted; a missing id's key
-// has those bits zero and lands at the front of its segment, which is as good as anywhere: the
-// reduction needs equal keys adjacent, and skips keys at or above the missing-id key wherever
-// they stand. Entries past the segment's end are all-ones and stay behind it (the sort is stable).
-constexpr int kSegSortBlock = 1024;
-constexpr int kSegSortItems = 8;
-constexpr int64_t kSegSortMax = kSegSortBlock * kSegSortItems;
+// ---------------------------------------------------------------------------
+// Requests of at most 8192 ids per table: two launches, no carry levels, no library sort.
+//   1. ids -> rows for every position, over the whole chip (rows_of_ids / group_rows_of_ids).
+//   2. bucket_push_kernel, one workgroup of 1024 lanes for each of a table's 8 to 32 buckets
+//      (bucket = row mod the number of buckets; as many as keep the request at about one
+//      workgroup per compute unit), so that both one table and 26 tables use much of the chip:
+//      a. the workgroup reads its table's row numbers and keeps the positions of its bucket, in
+//         position order (one scan over the workgroup);
+//      b. the (row, position) pairs are sorted by row in LDS with a stable radix sort, nine bits
+//         a pass (two passes for tables of up to two million rows). Every wavefront ranks its own
+//         elements with wave-wide votes (lanes holding the same digit find each other through
+//         nine ballots), a per-wavefront histogram in LDS turns into offsets by one scan over
+//         (digit, wavefront), and the pairs are scattered through LDS;
+//      c. the sorted list is cut into one tile per lane group; a group adds the gradient rows of
+//         each run of equal rows in position order (worker/emitter.cc:527-529; eight rows are
+//         requested ahead of the sums) and applies every run that lies inside its tile. Runs
+//         that cross tile borders (hot ids) leave partial sums in LDS, and after a barrier the
+//         group that owns a run's first partial adds the others in order and applies the sum.
+//      Nothing but the row numbers passes through global memory between the stages.
+// Measured on the way here, 8192 Zipf ids, dim 16: the whole push in one workgroup per table
+// 88 us (one compute unit keeps too few random reads in flight for index, gradients and
+// records); sorting a table's 8192 pairs in one workgroup 20-30 us whoever wrote the sort (a
+// pass is a chain of LDS round trips and barriers, and a wavefront instruction holds its SIMD
+// for four cycles), 19 us even for a bucket's 1024 pairs when the pairs arrive unordered and
+// position has to be sorted as well (five passes).
+// ---------------------------------------------------------------------------
+constexpr int kSortBlock = 1024;
+constexpr int kSortItems = 8;
+constexpr int kSortMax = kSortBlock * kSortItems;      // ids per table
+constexpr int kSortWaves = kSortBlock / kWave;
+constexpr int kMaxBucketBits = 5;                      // up to 32 buckets a table
+constexpr int kDigitBits = 9;
+constexpr int kDigits = 1 << kDigitBits;
+constexpr int kRunAhead = 8;                           // gradient rows requested ahead of the sums
+constexpr int kLongRun = 64;                           // runs longer than this are shared out over the workgroup
+constexpr int kShortMaxDim = 64;
+static_assert(kSortWaves * kDigits <= kSortMax + 1, "the histogram fits the work space");
 
-__global__ __launch_bounds__(kSegSortBlock) void segment_sort_kernel(GroupCall call,
-                                                                     const uint32_t* __restrict__ keys,
-                                                                     const uint32_t* __restrict__ pos,
-                                                                     uint32_t* __restrict__ skeys,
-                                                                     uint32_t* __restrict__ spos, int row_bits) {
-  using Sort = rocprim::block_radix_sort<uint32_t, kSegSortBlock, kSegSortItems, uint32_t>;
-  __shared__ typename Sort::storage_type storage;
-  const int64_t a = call.row_start[blockIdx.x];
-  const int len = (int)(call.row_start[blockIdx.x + 1] - a);
-  if (len <= 0) return;                          // uniform for the workgroup
-  // in: every wavefront holds 64 * kSegSortItems consecutive pairs, item i of lane l being pair
-  // i * 64 + l of them; out: item i of thread t is pair i * kSegSortBlock + t of the sorted
-  // segment. Both ways a load or store instruction covers consecutive addresses.
-  uint32_t k[kSegSortItems], v[kSegSortItems];
-  const int wave_base = (threadIdx.x / 64) * (64 * kSegSortItems) + (threadIdx.x & 63);
+struct SortCall {
+  int32_t n_tables;
+  int32_t bucket_bits;                                 // a table's rows are dealt to 2^bucket_bits workgroups
+  int32_t row_bits;                                    // bits of a row number
+  uint32_t row_mask;                                   // a key's row (member bits above it)
+  uint32_t miss_key;                                   // keys at or above it stand for missing ids
+  int64_t row_start[kMaxGroupTables + 1];
+};
+
+// lanes of this wavefront (bit mask) whose `digit` equals this lane's
+__device__ __forceinline__ unsigned long long match_digit(uint32_t digit) {
+  unsigned long long same = ~0ull;
 #pragma unroll
-  for (int i = 0; i < kSegSortItems; ++i) {
-    const int j = wave_base + i * 64;
-    k[i] = j < len ? keys[a + j] : 0xFFFFFFFFu;
-    v[i] = j < len ? pos[a + j] : 0u;
+  for (int b = 0; b < kDigitBits; ++b) {
+    const bool bit = (digit >> b) & 1u;
+    const unsigned long long votes = __ballot(bit);
+    same &= bit ? votes : ~votes;
   }
-  Sort().sort_warp_striped_to_striped(k, v, storage, 0, (unsigned)row_bits);
+  return same;
+}
+
+// exclusive prefix sum of one value per lane over the workgroup (1024 lanes); total to all
+__device__ __forceinline__ uint32_t sort_block_scan(uint32_t v, uint32_t* wave_total, uint32_t& total) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  uint32_t incl = v;
 #pragma unroll
-  for (int i = 0; i < kSegSortItems; ++i) {
-    const int j = i * kSegSortBlock + threadIdx.x;
-    if (j < len) {
-      skeys[a + j] = k[i];
-      spos[a + j] = v[i];
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t y = __shfl_up(incl, d);
+    if (lane >= d) incl += y;
+  }
+  __syncthreads();                                     // wave_total may still be read from a previous scan
+  if (lane == kWave - 1) wave_total[wave] = incl;
+  __syncthreads();
+  uint32_t offset = incl - v;
+  uint32_t sum = 0;
+  for (int w = 0; w < kSortWaves; ++w) {
+    const uint32_t x = wave_total[w];
+    if (w < wave) offset += x;
+    sum += x;
+  }
+  total = sum;
+  return offset;
+}
+
+// grid: one workgroup per bucket (n_tables << bucket_bits)
+template <int OPT, int VEC, bool GROUPED>
+__global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc* __restrict__ descs, TableView tv,
+                                                                 SortCall call, const uint32_t* __restrict__ keys,
+                                                                 const float* __restrict__ grads, int dim,
+                                                                 int elems, int group, ApplyArgs args, GroupSrc gs) {
+  __shared__ uint32_t skey[kSortMax];                  // row >> bucket_bits
+  __shared__ uint16_t spos[kSortMax];
+  // histogram [wave][digit] while sorting; partial sums and their keys while reducing
+  // histogram [wave][digit] while sorting; then run starts, the list of long runs, and the
+  // wavefronts' partial sums of a long run
+  __shared__ uint32_t work[kSortMax + 1 + kSortMax / kLongRun + 1 + kSortWaves * kWave * 4];
+  __shared__ uint32_t wave_total[kSortWaves];
+  const int mb = blockIdx.x;
+  const int bucket_bits = call.bucket_bits;
+  const uint32_t n_buckets = 1u << bucket_bits;
+  const int m = mb >> bucket_bits;
+  const uint32_t bucket = (uint32_t)mb & (n_buckets - 1);
+  const int t = threadIdx.x;
+  const int64_t a = call.row_start[m];
+  const int all = (int)(call.row_start[m + 1] - a);    // positions of the table's request
+  if (all <= 0) return;                                // uniform for the workgroup
+  if constexpr (GROUPED) {
+    const TableDesc& d = descs[m];
+    tv = d.tv;
+    args.c0 = gs.st0 >= 0 ? d.col_off[gs.st0] : -1;
+    args.c1 = gs.st1 >= 0 ? d.col_off[gs.st1] : -1;
+    args.c2 = gs.st2 >= 0 ? d.col_off[gs.st2] : -1;
+    args.meta_off = gs.use_meta ? d.meta_off : -1;
+  }
+  const int lane = t & (kWave - 1);
+  const int wave = t / kWave;
+
+  // ---- a. the bucket's positions, in position order -------------------------------------------
+  const int own = (all + kSortBlock - 1) / kSortBlock;  // positions a lane looks at, 1..8
+  for (int j = t; j < all; j += kSortBlock) skey[j] = keys[a + j];   // coalesced; re-read by ownership below
+  __syncthreads();
+  uint32_t mine[kSortItems];
+  uint32_t take = 0;
+#pragma unroll
+  for (int i = 0; i < kSortItems; ++i) {
+    const int j = t * own + i;
+    if (i < own && j < all) {
+      mine[i] = skey[j];
+      if (mine[i] < call.miss_key && ((mine[i] & call.row_mask) & (n_buckets - 1)) == bucket) take |= 1u << i;
     }
   }
+  uint32_t total;
+  uint32_t at = sort_block_scan((uint32_t)__popc(take), wave_total, total);   // its barriers follow the reads
+#pragma unroll
+  for (int i = 0; i < kSortItems; ++i) {
+    if (take & (1u << i)) {
+      skey[at] = (mine[i] & call.row_mask) >> bucket_bits;
+      spos[at] = (uint16_t)(t * own + i);
+      ++at;
+    }
+  }
+  const int len = (int)total;
+  if (len == 0) return;                                // uniform
+  const int per_lane = (len + kSortBlock - 1) / kSortBlock;   // 1..8
+  const int padded = per_lane * kSortBlock;
+  __syncthreads();
+  for (int j = len + t; j < padded; j += kSortBlock) {
+    skey[j] = 0xFFFFFFFFu;                             // padding sorts behind everything
+    spos[j] = 0;
+  }
+  __syncthreads();
+
+  // ---- b. stable radix sort by row -----------------------------------------------------------
+  // element i of lane l in wavefront w is pair w * 64 * per_lane + i * 64 + l: a wavefront's
+  // elements are consecutive, and taking i in ascending order visits them in list order
+  {
+    uint32_t* hist = work;                             // [kSortWaves][kDigits]
+    const int wbase = wave * kWave * per_lane + lane;
+    const int bits = call.row_bits > bucket_bits ? call.row_bits - bucket_bits : 1;
+    const int passes = (bits + kDigitBits - 1) / kDigitBits;
+    const int width = (bits + passes - 1) / passes;    // bits per pass, at most kDigitBits
+    const uint32_t digit_mask = (1u << width) - 1u;
+    for (int pass = 0; pass < passes; ++pass) {
+      const int shift = pass * width;
+      uint32_t key[kSortItems], rank[kSortItems];
+      uint16_t pos[kSortItems];
+#pragma unroll
+      for (int i = 0; i < kSortItems; ++i) {
+        if (i < per_lane) {
+          key[i] = skey[wbase + i * kWave];
+          pos[i] = spos[wbase + i * kWave];
+        }
+      }
+      for (int i = t; i < kSortWaves * kDigits; i += kSortBlock) hist[i] = 0u;
+      __syncthreads();                                 // everyone holds its pairs; the histogram is clear
+#pragma unroll
+      for (int i = 0; i < kSortItems; ++i) {
+        if (i < per_lane) {                            // uniform
+          // the last pass also sees the padding's upper bits: they stay the largest digit
+          const uint32_t digit = (key[i] >> shift) & digit_mask;
+          const unsigned long long same = match_digit(digit);
+          const uint32_t before = (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
+          uint32_t* cell = &hist[wave * kDigits + digit];
+          const uint32_t old = *cell;                  // read by all lanes of the digit ...
+          if (before == 0) *cell = old + (uint32_t)__popcll(same);   // ... then advanced by their first
+          rank[i] = old + before;
+        }
+      }
+      __syncthreads();
+      // exclusive scan over (digit, wavefront): lane t owns digit t / 2, wavefronts 8 (t % 2) .. + 7
+      {
+        const int digit = t >> 1;
+        const int w0 = (t & 1) * 8;
+        uint32_t c[8], sum = 0, whole;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          c[k] = hist[(w0 + k) * kDigits + digit];
+          sum += c[k];
+        }
+        uint32_t offset = sort_block_scan(sum, wave_total, whole);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          hist[(w0 + k) * kDigits + digit] = offset;
+          offset += c[k];
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < kSortItems; ++i) {
+        if (i < per_lane) {
+          const uint32_t dest = hist[wave * kDigits + ((key[i] >> shift) & digit_mask)] + rank[i];
+          skey[dest] = key[i];
+          spos[dest] = pos[i];
+        }
+      }
+      __syncthreads();
+    }
+  }
+
+  // ---- c. runs of equal rows: sums in position order, one update per row -----------------------
+  uint32_t* run_start = work;                          // [runs + 1]; the histogram is done with
+  uint32_t* long_run = work + kSortMax + 1;            // [<= kSortMax / kLongRun] runs longer than kLongRun
+  __shared__ uint32_t n_long;
+  uint32_t runs;
+  {
+    // lane t looks at entries [t * per_lane, (t + 1) * per_lane): where does a new row begin?
+    const int j0 = t * per_lane;
+    uint32_t heads = 0;
+#pragma unroll
+    for (int i = 0; i < kSortItems; ++i) {
+      const int j = j0 + i;
+      if (i < per_lane && j < len && (j == 0 || skey[j - 1] != skey[j])) heads |= 1u << i;
+    }
+    if (t == 0) n_long = 0u;
+    uint32_t r = sort_block_scan((uint32_t)__popc(heads), wave_total, runs);
+#pragma unroll
+    for (int i = 0; i < kSortItems; ++i)
+      if (heads & (1u << i)) run_start[r++] = (uint32_t)(j0 + i);
+    if (t == 0) run_start[runs] = (uint32_t)len;
+    __syncthreads();
+  }
+  const int per_block = kSortBlock / group;
+  const int lt = t / group;
+  const int gl = t & (group - 1);
+  const bool lane_on = gl < elems;
+  const float* g_base = grads + a * (int64_t)dim;
+
+  // adds entries [lo, hi) of the sorted list in list order; the first addend is copied, not added
+  // to zero (worker/emitter.cc:527 clones it)
+  auto sum_entries = [&](int lo, int hi, float (&acc)[VEC]) {
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) acc[c] = 0.0f;
+    for (int j0 = lo; j0 < hi; j0 += kRunAhead) {
+      float v[kRunAhead][VEC];
+#pragma unroll
+      for (int u = 0; u < kRunAhead; ++u) {
+        if (j0 + u < hi && lane_on) {
+          vload<VEC>(g_base + (int64_t)spos[j0 + u] * dim + gl * VEC, v[u]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) v[u][c] = 0.0f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kRunAhead; ++u) {
+        if (j0 + u >= hi) break;
+        if (j0 + u == lo) {
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) acc[c] = v[u][c];
+        } else {
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) acc[c] = acc[c] + v[u][c];
+        }
+      }
+    }
+  };
+
+  // runs of at most kLongRun entries: one lane group each, exactly the reference's order
+  for (uint32_t q = (uint32_t)lt; q < runs; q += (uint32_t)per_block) {
+    const int start = (int)run_start[q], end = (int)run_start[q + 1];
+    if (end - start > kLongRun) {
+      if (gl == 0) long_run[atomicAdd(&n_long, 1u)] = q;
+      continue;
+    }
+    const uint32_t row = (skey[start] << bucket_bits) | bucket;
+    RowRegs<VEC> rec;
+    load_row<OPT, VEC>(tv, row, gl, lane_on, args, rec);   // on its way while the gradients are added
+    float acc[VEC];
+    sum_entries(start, end, acc);
+    finish_row<OPT, VEC>(tv, row, acc, gl, lane_on, gl, true, dim, args, rec);
+  }
+  __syncthreads();
+  // hot ids: every lane group adds a stretch of the run; the stretches' sums are added in order,
+  // first inside each wavefront (neighbouring lane groups, by doubling), then across wavefronts
+  float* part = reinterpret_cast<float*>(work + kSortMax + 1 + kSortMax / kLongRun + 1);   // [kSortWaves][group * VEC]
+  const uint32_t longs = n_long;
+  const int lane_floats = group * VEC;
+  for (uint32_t k = 0; k < longs; ++k) {
+    const uint32_t q = long_run[k];                    // in any order: the runs are different rows
+    const int start = (int)run_start[q], count = (int)run_start[q + 1] - start;
+    const int stretch = (count + per_block - 1) / per_block;
+    const int lo = start + lt * stretch < start + count ? start + lt * stretch : start + count;
+    const int hi = lo + stretch < start + count ? lo + stretch : start + count;
+    float acc[VEC];
+    sum_entries(lo, hi, acc);
+    // inside the wavefront: lane group i takes in group i + 1, then i + 2, i + 4, ...
+    for (int d = group; d < kWave; d <<= 1) {
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) {
+        const float other = __shfl_down(acc[c], d);
+        if (((lane / group) & ((2 * d / group) - 1)) == 0) acc[c] = acc[c] + other;
+      }
+    }
+    if (lane < group) vstore<VEC>(part + wave * lane_floats + gl * VEC, acc);
+    __syncthreads();
+    if (lt == 0) {
+      float w[kSortWaves][VEC];
+#pragma unroll
+      for (int f = 1; f < kSortWaves; ++f) vload<VEC>(part + f * lane_floats + gl * VEC, w[f]);
+#pragma unroll
+      for (int f = 1; f < kSortWaves; ++f) {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) acc[c] = acc[c] + w[f][c];
+      }
+      apply_row<OPT, VEC>(tv, (skey[start] << bucket_bits) | bucket, acc, gl, lane_on, gl, true, dim, args);
+    }
+    __syncthreads();
+  }
+}
+
+template <int VEC, bool GROUPED>
+static void launch_bucket_push(int opt, unsigned buckets, hipStream_t stream, const TableDesc* descs,
+                               const TableView& tv, const SortCall& call, const uint32_t* keys, const float* grads,
+                               int dim, int elems, int group, const ApplyArgs& args, const GroupSrc& gs) {
+  const dim3 grid(buckets), block(kSortBlock);
+  switch (opt) {
+    case KRK_SGD:
+      hipLaunchKernelGGL((bucket_push_kernel<KRK_SGD, VEC, GROUPED>), grid, block, 0, stream, descs, tv, call, keys,
+                         grads, dim, elems, group, args, gs);
+      break;
+    case KRK_ADAGRAD:
+      hipLaunchKernelGGL((bucket_push_kernel<KRK_ADAGRAD, VEC, GROUPED>), grid, block, 0, stream, descs, tv, call,
+                         keys, grads, dim, elems, group, args, gs);
+      break;
+    case KRK_ADAM:
+      hipLaunchKernelGGL((bucket_push_kernel<KRK_ADAM, VEC, GROUPED>), grid, block, 0, stream, descs, tv, call, keys,
+                         grads, dim, elems, group, args, gs);
+      break;
+    default:
+      hipLaunchKernelGGL((bucket_push_kernel<KRK_RMSPROP, VEC, GROUPED>), grid, block, 0, stream, descs, tv, call,
+                         keys, grads, dim, elems, group, args, gs);
+      break;
+  }
+}
+
+// Workgroups per table: as many as keep the request within about one workgroup per compute unit
+// (a workgroup's LDS leaves room for one per unit), between 8 and 32.
+static int short_bucket_bits(int n_tables) {
+  int bits = kMaxBucketBits;
+  while (bits > 3 && (n_tables << bits) > 256) --bits;
+  return bits;
+}
+
+// Whether a request whose longest table brings `longest` ids takes the two-launch path: a lane
+// group must own a whole row, and a bucket's gradients pass through one compute unit.
+static bool short_push_fits(int64_t longest, int64_t dim, int elems, int group) {
+  return longest <= kSortMax && dim <= kShortMaxDim && elems <= group;
 }
 
 // Stable sort of (key, payload) by key, then the tiled segmented reduction: every run of equal
@@ -721,7 +1070,7 @@ template <typename Fill>
 static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, DeviceBuffer* scratch,
                                const TableView& tv, int opt, int64_t n, uint32_t miss_key, int bits,
                                const float* d_vals, const ApplyArgs& args, const PooledSrc& ps,
-                               const GroupSrc* gs, Fill fill, const GroupCall* segments = nullptr) {
+                               const GroupSrc* gs, Fill fill) {
   const int tile0 = pick_tile(n);
   const int per_block = kBlock / sh.group;
   const int64_t groups0 = ((n + tile0 - 1) / tile0 + per_block - 1) / per_block;   // workgroups of level 0
@@ -741,13 +1090,7 @@ static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, Device
 
   fill(keys, pos);
   KRK_HIP(hipGetLastError());
-  if (segments) {
-    hipLaunchKernelGGL(segment_sort_kernel, dim3((unsigned)segments->n_tables), dim3(kSegSortBlock), 0, stream,
-                       *segments, keys, pos, skeys, spos, gs->row_bits);
-    KRK_HIP(hipGetLastError());
-  } else {
-    KRK_HIP(sort_pairs(scratch[1].ptr, sort_bytes, keys, skeys, pos, spos, n, bits, stream));
-  }
+  KRK_HIP(sort_pairs(scratch[1].ptr, sort_bytes, keys, skeys, pos, spos, n, bits, stream));
 
   // level 0 reads value rows through the sorted payloads; later levels read the carry list
   uint32_t* ckeys[2] = {scratch[2].as<uint32_t>(), scratch[2].as<uint32_t>() + carry_entries};
@@ -1217,6 +1560,42 @@ int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* i
   KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
   KRK_TRY(t->input(grads, (size_t)n * t->dim, flags, 1, &d_g));
 
+  if (short_push_fits(n, t->dim, t->elems, t->group)) {
+    // a short request: see bucket_push_kernel
+    SortCall sc;
+    sc.n_tables = 1;
+    sc.bucket_bits = short_bucket_bits(1);
+    sc.row_bits = 1;
+    while (((int64_t)1 << sc.row_bits) < t->row_cap) ++sc.row_bits;
+    sc.row_mask = 0xFFFFFFFFu;
+    sc.miss_key = kNoRow;
+    sc.row_start[0] = 0;
+    sc.row_start[1] = n;
+    ApplyArgs args;
+    args.lr = lr;
+    args.k = make_optim_k(*o);
+    int32_t cols[3];
+    sparse_optim_columns(t, *o, cols);
+    args.c0 = cols[0];
+    args.c1 = cols[1];
+    args.c2 = cols[2];
+    args.meta_off = ((optim_state_mask(*o) >> KRK_ST_STEPS) & 1u) ? t->meta_off : -1;
+    KRK_TRY(t->scratch[0].reserve((size_t)n * sizeof(uint32_t)));
+    uint32_t* keys = t->scratch[0].as<uint32_t>();
+    const TableView tv = t->view();
+    hipLaunchKernelGGL(rows_of_ids_kernel, dim3(grid_for(n, kBlock / kBucket)), dim3(kBlock), 0, t->stream, tv,
+                       d_ids, n, kNoRow, (const uint32_t*)nullptr, false, keys, (uint32_t*)nullptr);
+    const GroupSrc none{nullptr, 0, -1, -1, -1, 0};
+    if (t->vec == 4) {
+      launch_bucket_push<4, false>(o->type, 1u << sc.bucket_bits, t->stream, nullptr, tv, sc, keys, d_g, (int)t->dim, t->elems,
+                                   t->group, args, none);
+    } else {
+      launch_bucket_push<1, false>(o->type, 1u << sc.bucket_bits, t->stream, nullptr, tv, sc, keys, d_g, (int)t->dim, t->elems,
+                                   t->group, args, none);
+    }
+    KRK_HIP(hipGetLastError());
+    return sparse_finish(t, flags);
+  }
   KRK_TRY(push_sorted(t, o, d_ids, n, d_g, lr, nullptr, false, PooledSrc{nullptr, nullptr}));
   return sparse_finish(t, flags);
 }
@@ -1261,9 +1640,13 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
     return KRK_E_CAPACITY;
   }
   const uint32_t miss_key = (uint32_t)n_tables << row_bits;
-  // members of at most 8192 ids each are sorted one workgroup a member (segment_sort_kernel)
-  bool by_member = n_tables > 1;
-  for (int m = 0; m < n_tables; ++m) by_member = by_member && offsets[m + 1] - offsets[m] <= kSegSortMax;
+  // members of at most 8192 ids each are sorted one workgroup a member
+  bool by_member = true;
+  int64_t longest = 0;
+  for (int m = 0; m < n_tables; ++m) {
+    by_member = by_member && offsets[m + 1] - offsets[m] <= kSortMax;
+    longest = std::max(longest, offsets[m + 1] - offsets[m]);
+  }
   // the launch that turns ids into rows gives every member whole workgroups of its own
   GroupCall rows_call = call;
   uint32_t blocks = 0;
@@ -1283,6 +1666,29 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
   int32_t st[3];
   optim_state_slots(*o, st);
   const GroupSrc gs{g->d_descs, row_bits, st[0], st[1], st[2], (int)((mask >> KRK_ST_STEPS) & 1u)};
+  if (by_member && short_push_fits(longest, g->dim, g->elems, g->group)) {
+    // short members: see bucket_push_kernel
+    SortCall sc;
+    sc.n_tables = n_tables;
+    sc.bucket_bits = short_bucket_bits(n_tables);
+    sc.row_bits = row_bits;
+    sc.row_mask = row_bits >= 32 ? 0xFFFFFFFFu : ((1u << row_bits) - 1u);
+    sc.miss_key = miss_key;
+    for (int m = 0; m <= n_tables; ++m) sc.row_start[m] = offsets[m];
+    KRK_TRY(g->scratch[0].reserve((size_t)total * sizeof(uint32_t)));
+    uint32_t* keys = g->scratch[0].as<uint32_t>();
+    hipLaunchKernelGGL(group_rows_of_ids_kernel, dim3(rows_call.block_start[n_tables]), dim3(kBlock), 0, g->stream,
+                       g->d_descs, rows_call, d_ids, total, row_bits, miss_key, keys, (uint32_t*)nullptr);
+    if (g->vec == 4) {
+      launch_bucket_push<4, true>(o->type, (unsigned)n_tables << sc.bucket_bits, g->stream, g->d_descs, TableView{}, sc,
+                                  keys, d_g, (int)g->dim, g->elems, g->group, args, gs);
+    } else {
+      launch_bucket_push<1, true>(o->type, (unsigned)n_tables << sc.bucket_bits, g->stream, g->d_descs, TableView{}, sc,
+                                  keys, d_g, (int)g->dim, g->elems, g->group, args, gs);
+    }
+    KRK_HIP(hipGetLastError());
+    return group_finish(g, flags);
+  }
   TableView none{};
   const ReduceShape sh{g->dim, g->vec, g->elems, g->group};
   KRK_TRY(sort_and_reduce(sh, g->stream, g->scratch, none, o->type, total, miss_key, row_bits + member_bits,
@@ -1290,7 +1696,7 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
                             hipLaunchKernelGGL(group_rows_of_ids_kernel, dim3(rows_call.block_start[n_tables]),
                                                dim3(kBlock), 0, g->stream, g->d_descs, rows_call, d_ids, total,
                                                row_bits, miss_key, keys, pos);
-                          }, by_member ? &call : nullptr));
+                          }));
   return group_finish(g, flags);
 }
 

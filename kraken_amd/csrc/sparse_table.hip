@@ -285,27 +285,6 @@ __global__ __launch_bounds__(kBlock) void pooled_probe_kernel(TableView tv, Init
 
 constexpr int kPoolAhead = 4;   // records of one bag requested together
 
-// One lane looking an id up by itself (no votes): the rare second look of pooled_sum_kernel.
-__device__ inline uint32_t probe_find_alone(const TableView& tv, uint64_t id) {
-  if (id == kEmptyKey) {
-    const Slot* s = &tv.slots[tv.mask + 1];
-    return __atomic_load_n(&s->key, __ATOMIC_RELAXED) != kEmptyKey
-               ? (uint32_t)__atomic_load_n(&s->row_epoch, __ATOMIC_RELAXED) : kEmptyRow;
-  }
-  const uint64_t nb_mask = tv.mask >> 2;
-  uint64_t b = mix64(id) & nb_mask;
-  for (uint64_t tried = 0; tried <= nb_mask; ++tried) {
-    for (int i = 0; i < kBucket; ++i) {
-      const Slot* s = &tv.slots[b * kBucket + i];
-      const unsigned long long key = __atomic_load_n(&s->key, __ATOMIC_RELAXED);
-      if (key == id) return (uint32_t)__atomic_load_n(&s->row_epoch, __ATOMIC_RELAXED);
-      if (key == kEmptyKey) return kEmptyRow;
-    }
-    b = (b + 1) & nb_mask;
-  }
-  return kEmptyRow;
-}
-
 template <int VEC>
 __global__ __launch_bounds__(kBlock) void pooled_sum_kernel(TableView tv, const uint32_t* __restrict__ rows,
                                                             const uint64_t* __restrict__ ids,
