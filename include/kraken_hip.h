@@ -305,6 +305,24 @@ int32_t krk_sparse_select_routed(krk_sparse* t, uint64_t table_id, const uint64_
                                  int32_t owned, uint64_t* ids, int64_t capacity, int64_t* count,
                                  uint32_t flags);
 
+/* The worker's routing of a request (Emitter::PullSparseTableImpl, worker/emitter.cc:139-149; push
+ * :516-531; combined :221-233, 595-606): every id goes to the server that
+ * Router::Hit(utils::Hash(table_id, sparse_id)) names (common/router.cc:262-277,
+ * common/utils.h:30-48), and each server's request lists its ids in the order the worker met them.
+ * Call it on the unique ids krk_dedup returns, as the reference routes after its dedup, so that a
+ * hot id is routed once. The ring is Router::vnodes() as two HOST arrays whatever the flags say
+ * (hash_v ascending, node id of each virtual node; at most 256 distinct nodes).
+ *   node_ids[k], counts[k]  (host, node_capacity entries) the ring's nodes in ascending id order
+ *                           and how many of the ids each owns; *n_nodes = how many nodes
+ *   owner[p]                (may be NULL) the node id that owns ids[p]
+ *   perm[n]                 the positions grouped by owner in node_ids order, position order kept
+ *                           inside a group (a stable partition): node k's request is ids[perm[j]]
+ *                           for j in [counts[0] + .. + counts[k-1], .. + counts[k])
+ * Blocking. KRK_E_CAPACITY when node_capacity is too small (*n_nodes = the room needed). */
+int32_t krk_route_ids(uint64_t table_id, const uint64_t* ring_hash, const uint64_t* ring_node, int64_t ring_n,
+                      const uint64_t* ids, int64_t n, uint64_t* owner, int64_t* perm, uint64_t* node_ids,
+                      int64_t* counts, int64_t node_capacity, int64_t* n_nodes, uint32_t flags);
+
 /* ---- table files ------------------------------------------------------------- */
 /* Checkpoint::SaveSparseTable (checkpoint/checkpoint.cc:465-509): the table as a *.sparse file in
  * the reference's byte layout (common/serialize.h), rows grouped by id % 8 and ascending inside

@@ -117,6 +117,9 @@ EXPORTS = {
                                              C.POINTER(C.c_int64), C.c_uint32]),
     "krk_hbm_probe": (C.c_int32, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t]),
     "krk_hbm_probe_lines": (C.c_int32, [C.c_int32, C.c_void_p, C.c_size_t, C.c_int64, C.c_uint64]),
+    "krk_route_ids": (C.c_int32, [C.c_uint64, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64,
+                                  C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                  C.POINTER(C.c_int64), C.c_uint32]),
     "krk_dedup": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64),
                               C.c_uint32]),
     "krk_dedup_noalloc": (C.c_int32, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
@@ -694,6 +697,28 @@ def dedup(ids):
     if isinstance(ids, DeviceArray):
         return uids, inv, u.value
     return uids[:u.value].copy(), inv
+
+
+def route_ids(table_id, ring, ids):
+    """The worker's routing of a request's (unique) ids (worker/emitter.cc:139-149).
+    ring = [(hash_v, node_id), ...] in ascending hash order.
+    -> (node_ids[m], counts[m], owner[n], perm[n]); device ids give device owner / perm."""
+    rh = np.ascontiguousarray([h for h, _ in ring], dtype=np.uint64)
+    rn = np.ascontiguousarray([n for _, n in ring], dtype=np.uint64)
+    dev = isinstance(ids, DeviceArray)
+    if not dev:
+        ids = np.ascontiguousarray(ids, dtype=np.uint64)
+    n = ids.size
+    owner = DeviceArray(max(n, 1), np.uint64) if dev else np.empty(n, np.uint64)
+    perm = DeviceArray(max(n, 1), np.int64) if dev else np.empty(n, np.int64)
+    cap = max(len(set(int(x) for x in rn)), 1)
+    node_ids = np.empty(cap, np.uint64)
+    counts = np.empty(cap, np.int64)
+    m = C.c_int64()
+    _check(lib().krk_route_ids(int(table_id), _ptr(rh), _ptr(rn), len(ring), _ptr(ids), n, _ptr(owner),
+                               _ptr(perm), _ptr(node_ids), _ptr(counts), cap, C.byref(m),
+                               DEVICE_PTRS if dev else 0), "krk_route_ids")
+    return node_ids[:m.value], counts[:m.value], owner, perm
 
 
 DEDUP_NOALLOC_MAX = 1 << 18

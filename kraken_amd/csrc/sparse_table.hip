@@ -605,6 +605,73 @@ __global__ __launch_bounds__(kBlock) void route_emit_kernel(const unsigned long 
   if (r < rows && flag[r]) ids[rank[r]] = row_key[r];
 }
 
+// ---- a request's ids by owning node (worker/emitter.cc:139-149) ---------------------------------
+// rank8[p] = index (in ascending node-id order) of the node that owns ids[p]; owner[p] = that
+// node's id; block_counts[k * blocks + block] = ids of this workgroup owned by node k.
+constexpr int kRouteMaxNodes = 256;
+
+__global__ __launch_bounds__(kBlock) void route_rank_kernel(const uint64_t* __restrict__ ids, int64_t n,
+                                                            unsigned long long table_hash,
+                                                            const unsigned long long* __restrict__ ring_hash,
+                                                            const uint32_t* __restrict__ ring_rank, int m,
+                                                            const unsigned long long* __restrict__ node_of_rank,
+                                                            int nodes, unsigned long long* __restrict__ owner,
+                                                            uint8_t* __restrict__ rank8,
+                                                            int32_t* __restrict__ block_counts,
+                                                            int32_t* __restrict__ node_count) {
+  __shared__ int32_t hist[kRouteMaxNodes];
+  if ((int)threadIdx.x < nodes) hist[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (p < n) {
+    const unsigned long long hv = table_hash ^ route_hash64(ids[p]);
+    int lo = 0, hi = m;
+    while (lo < hi) {
+      const int mid = lo + ((hi - lo) >> 1);
+      if (ring_hash[mid] < hv) lo = mid + 1; else hi = mid;
+    }
+    const uint32_t k = ring_rank[lo == m ? 0 : lo];
+    rank8[p] = (uint8_t)k;
+    if (owner) owner[p] = node_of_rank[k];
+    atomicAdd(&hist[k], 1);
+  }
+  __syncthreads();
+  if ((int)threadIdx.x < nodes) {
+    const int32_t c = hist[threadIdx.x];
+    block_counts[(int64_t)threadIdx.x * gridDim.x + blockIdx.x] = c;
+    if (c) atomicAdd(&node_count[threadIdx.x], c);
+  }
+}
+
+// perm[where node k's ids begin + ids of node k in earlier workgroups + earlier in this one] = p:
+// a stable partition of the positions by owner.
+__global__ __launch_bounds__(kBlock) void route_scatter_kernel(const uint8_t* __restrict__ rank8, int64_t n,
+                                                               const int32_t* __restrict__ block_base,
+                                                               long long* __restrict__ perm) {
+  __shared__ int32_t wave_count[kBlock / kWave][kRouteMaxNodes];
+  for (int i = threadIdx.x; i < (kBlock / kWave) * kRouteMaxNodes; i += kBlock) (&wave_count[0][0])[i] = 0;
+  __syncthreads();
+  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const bool on = p < n;
+  const uint32_t k = on ? rank8[p] : 0u;
+  const int lane = wave_lane();
+  const int wave = threadIdx.x / kWave;
+  unsigned long long same = __ballot(on);
+#pragma unroll
+  for (int b = 0; b < 8; ++b) {
+    const bool bit = (k >> b) & 1u;
+    const unsigned long long votes = __ballot(bit);
+    same &= bit ? votes : ~votes;
+  }
+  const int before = __popcll(same & ((1ull << lane) - 1ull));
+  if (on && before == 0) wave_count[wave][k] = __popcll(same);
+  __syncthreads();
+  if (!on) return;
+  int offset = before;
+  for (int w = 0; w < wave; ++w) offset += wave_count[w][k];
+  perm[block_base[(int64_t)k * gridDim.x + blockIdx.x] + offset] = p;
+}
+
 // ---- erase -------------------------------------------------------------------
 // Rows are kept dense: the rows that go leave holes, and the live rows at the tail move into
 // the holes below the new row count. Sources lie at or above that count, destinations below
@@ -1803,6 +1870,110 @@ int32_t krk_sparse_select_routed(krk_sparse* t, uint64_t table_id, const uint64_
   KRK_HIP(hipGetLastError());
   KRK_TRY(t->output_back(reinterpret_cast<unsigned long long*>(ids), (size_t)total, flags, 0));
   KRK_HIP(hipStreamSynchronize(t->stream));
+  return KRK_SUCCESS;
+}
+
+// The routing call owns no table: its work space is kept between calls under one lock, and it
+// runs on the null stream.
+static std::mutex g_route_mu;
+static DeviceBuffer g_route_pool;
+
+int32_t krk_route_ids(uint64_t table_id, const uint64_t* ring_hash, const uint64_t* ring_node, int64_t ring_n,
+                      const uint64_t* ids, int64_t n, uint64_t* owner, int64_t* perm, uint64_t* node_ids,
+                      int64_t* counts, int64_t node_capacity, int64_t* n_nodes, uint32_t flags) {
+  KRK_TRY(check_flags(flags));
+  if (flags & KRK_ASYNC) return KRK_E_ARGUMENT;   // the counts come back by value
+  if (!n_nodes || ring_n < 0 || ring_n > (1 << 24) || (ring_n > 0 && (!ring_hash || !ring_node)) || n < 0 ||
+      (n > 0 && (!ids || !perm)) || node_capacity < 0 || (node_capacity > 0 && (!node_ids || !counts)))
+    return KRK_E_ARGUMENT;
+  if (n > ((int64_t)1 << 30)) {
+    set_error("krk_route_ids handles at most 2^30 ids per call");
+    return KRK_E_CAPACITY;
+  }
+  for (int64_t i = 1; i < ring_n; ++i) {
+    if (ring_hash[i - 1] > ring_hash[i]) {
+      set_error("krk_route_ids: the ring must be in ascending hash order");
+      return KRK_E_ARGUMENT;
+    }
+  }
+  KRK_TRY(ensure_runtime());
+  // the nodes of the ring in ascending id order, and each virtual node's index among them
+  std::vector<unsigned long long> nodes(ring_node, ring_node + ring_n);
+  std::sort(nodes.begin(), nodes.end());
+  nodes.erase(std::unique(nodes.begin(), nodes.end()), nodes.end());
+  const int64_t m = (int64_t)nodes.size();
+  *n_nodes = m;
+  if (m > node_capacity) {
+    set_error("krk_route_ids: the ring has %lld nodes, room for %lld", (long long)m, (long long)node_capacity);
+    return KRK_E_CAPACITY;
+  }
+  if (m > kRouteMaxNodes) {
+    set_error("krk_route_ids handles rings of at most %d nodes", kRouteMaxNodes);
+    return KRK_E_CAPACITY;
+  }
+  for (int64_t k = 0; k < m; ++k) {
+    node_ids[k] = nodes[(size_t)k];
+    counts[k] = 0;
+  }
+  if (n == 0) return KRK_SUCCESS;
+  if (m == 0) {
+    set_error("krk_route_ids: an empty ring owns nothing");   // Router::Hit on an empty ring has no answer
+    return KRK_E_ARGUMENT;
+  }
+  std::vector<uint32_t> ring_rank((size_t)ring_n);
+  for (int64_t i = 0; i < ring_n; ++i)
+    ring_rank[(size_t)i] = (uint32_t)(std::lower_bound(nodes.begin(), nodes.end(), ring_node[i]) - nodes.begin());
+
+  const bool host = !(flags & KRK_DEVICE_PTRS);
+  const int64_t blocks = (n + kBlock - 1) / kBlock;
+  const auto r256 = [](size_t b) { return (b + 255) & ~(size_t)255; };
+  const size_t ring_hash_b = r256((size_t)ring_n * 8), ring_rank_b = r256((size_t)ring_n * 4);
+  const size_t nodes_b = r256((size_t)m * 8), count_b = r256((size_t)m * 4);
+  const size_t rank8_b = r256((size_t)n), bc_b = r256((size_t)m * (size_t)blocks * 4);
+  const size_t scan_b = r256(scan_scratch_bytes(m * blocks));
+  const size_t n8 = r256((size_t)n * 8);
+  std::lock_guard<std::mutex> pool_lock(g_route_mu);
+  KRK_TRY(g_route_pool.reserve(ring_hash_b + ring_rank_b + nodes_b + count_b + rank8_b + bc_b + scan_b + 256 +
+                               (host ? 3 * n8 : 0)));
+  char* cur = g_route_pool.as<char>();
+  unsigned long long* d_ring_hash = reinterpret_cast<unsigned long long*>(cur); cur += ring_hash_b;
+  uint32_t* d_ring_rank = reinterpret_cast<uint32_t*>(cur); cur += ring_rank_b;
+  unsigned long long* d_nodes = reinterpret_cast<unsigned long long*>(cur); cur += nodes_b;
+  int32_t* d_count = reinterpret_cast<int32_t*>(cur); cur += count_b;
+  uint8_t* d_rank8 = reinterpret_cast<uint8_t*>(cur); cur += rank8_b;
+  int32_t* d_bc = reinterpret_cast<int32_t*>(cur); cur += bc_b;
+  void* d_scan = cur; cur += scan_b;
+  int32_t* d_total = reinterpret_cast<int32_t*>(cur); cur += 256;
+  const uint64_t* d_ids = ids;
+  unsigned long long* d_owner = reinterpret_cast<unsigned long long*>(owner);
+  long long* d_perm = reinterpret_cast<long long*>(perm);
+  hipStream_t st = nullptr;
+  if (host) {
+    uint64_t* s_ids = reinterpret_cast<uint64_t*>(cur);
+    d_owner = owner ? reinterpret_cast<unsigned long long*>(cur + n8) : nullptr;
+    d_perm = reinterpret_cast<long long*>(cur + 2 * n8);
+    KRK_HIP(hipMemcpy(s_ids, ids, (size_t)n * 8, hipMemcpyHostToDevice));
+    d_ids = s_ids;
+  }
+  KRK_HIP(hipMemcpy(d_ring_hash, ring_hash, (size_t)ring_n * 8, hipMemcpyHostToDevice));
+  KRK_HIP(hipMemcpy(d_ring_rank, ring_rank.data(), (size_t)ring_n * 4, hipMemcpyHostToDevice));
+  KRK_HIP(hipMemcpy(d_nodes, nodes.data(), (size_t)m * 8, hipMemcpyHostToDevice));
+  KRK_HIP(hipMemsetAsync(d_count, 0, (size_t)m * 4, st));
+  hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, st, d_ids, n,
+                     (unsigned long long)route_hash64(table_id), d_ring_hash, d_ring_rank, (int)ring_n, d_nodes,
+                     (int)m, d_owner, d_rank8, d_bc, d_count);
+  KRK_HIP(hipGetLastError());
+  KRK_TRY(exclusive_scan_i32(d_bc, d_bc, m * blocks, d_total, d_scan, st));
+  hipLaunchKernelGGL(route_scatter_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, st, d_rank8, n, d_bc, d_perm);
+  KRK_HIP(hipGetLastError());
+  std::vector<int32_t> h_count((size_t)m);
+  KRK_HIP(hipMemcpy(h_count.data(), d_count, (size_t)m * 4, hipMemcpyDeviceToHost));
+  for (int64_t k = 0; k < m; ++k) counts[k] = h_count[(size_t)k];
+  if (host) {
+    if (owner) KRK_HIP(hipMemcpy(owner, d_owner, (size_t)n * 8, hipMemcpyDeviceToHost));
+    KRK_HIP(hipMemcpy(perm, d_perm, (size_t)n * 8, hipMemcpyDeviceToHost));
+  }
+  KRK_HIP(hipStreamSynchronize(st));
   return KRK_SUCCESS;
 }
 

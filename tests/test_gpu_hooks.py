@@ -3,6 +3,8 @@ fetch without insert (ps/ps.cc:914-935), erase after a cluster change (ps/ps.cc:
 and moving whole Values (weights + optimizer state + step counter) from one table into
 another (transfer ps/ps.cc:289-321 / 789-792, checkpoint load checkpoint/checkpoint.cc:620-645).
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -191,3 +193,50 @@ def test_select_routed_follows_the_references_ring(api, oracle):
     assert t.select_routed(1, [(5, 0)], 0).size == 10          # one virtual node owns the whole ring
     with pytest.raises(api.KrakenHipError):
         t.select_routed(1, [(9, 0), (5, 1)], 0)
+
+
+def test_route_ids_partitions_a_request_like_the_worker(api, oracle):
+    """Emitter::PullSparseTableImpl (worker/emitter.cc:139-149) sends every distinct id to
+    router_.Hit(utils::Hash(table_id, sparse_id)) and lists each server's ids in the order it met
+    them. Owners against every id the reference's own router answered for
+    (tests/golden/ref_router.json) and, for a million more, against the oracle (pinned on the same
+    file); the grouping against a plain stable partition."""
+    import json
+    import os
+    cases = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "ref_router.json")))
+    for ci, case in enumerate(cases):
+        ring = [(int(h), int(n)) for h, n in case["ring"]]
+        table_id = int(case["table_id"])
+        golden_ids = np.array([int(i) for i, _ in case["ids"]], np.uint64)
+        golden_owner = np.array([int(o) for _, o in case["ids"]], np.uint64)
+        node_ids, counts, owner, perm = api.route_ids(table_id, ring, golden_ids)
+        assert np.array_equal(owner, golden_owner)
+        assert node_ids.tolist() == sorted(set(n for _, n in ring))
+        n_more = 1_000_000 if ci == 0 else 50_000
+        ids = np.concatenate([golden_ids, splitmix64(np.arange(7, 7 + n_more, dtype=np.uint64))])
+        want_owner = oracle.route_owners(ring, table_id, ids)
+        # host pointers and device pointers give the same answer
+        node_ids, counts, owner, perm = api.route_ids(table_id, ring, ids)
+        d_nodes, d_counts, d_owner, d_perm = api.route_ids(table_id, ring, api.DeviceArray.from_host(ids))
+        assert np.array_equal(owner, want_owner) and np.array_equal(d_owner.to_host()[:ids.size], want_owner)
+        rank = np.searchsorted(node_ids, want_owner)
+        want_perm = np.argsort(rank, kind="stable")
+        assert np.array_equal(perm, want_perm) and np.array_equal(d_perm.to_host()[:ids.size], want_perm)
+        assert counts.tolist() == np.bincount(rank, minlength=node_ids.size).tolist() == d_counts.tolist()
+        assert counts.sum() == ids.size
+    # errors: an unsorted ring, too little room for the nodes, an empty ring with ids to route
+    ring = [(int(h), int(n)) for h, n in cases[0]["ring"]]
+    with pytest.raises(api.KrakenHipError):
+        api.route_ids(1, [(9, 0), (5, 1)], np.arange(4, dtype=np.uint64))
+    with pytest.raises(api.KrakenHipError):
+        api.route_ids(1, [], np.arange(4, dtype=np.uint64))
+    node_ids, counts, owner, perm = api.route_ids(1, ring, np.zeros(0, np.uint64))
+    assert counts.tolist() == [0] * node_ids.size and perm.size == 0
+    m = C.c_int64()
+    rh = np.array([h for h, _ in ring], np.uint64)
+    rn = np.array([n for _, n in ring], np.uint64)
+    one = np.zeros(1, np.uint64)
+    rc = api.lib().krk_route_ids(1, api._ptr(rh), api._ptr(rn), len(ring), api._ptr(one), 1, None,
+                                 api._ptr(np.zeros(1, np.int64)), api._ptr(one), api._ptr(np.zeros(1, np.int64)), 1,
+                                 C.byref(m), 0)
+    assert rc == api.E_CAPACITY and m.value == len(set(n for _, n in ring))
