@@ -1,8 +1,9 @@
 """Blockwise DCT-II on the matrix cores. The reference has no cosine transform (its "DCT"
 emitter is the threshold codec), so there is no reference output to match: the transform is
 pinned by the library definition scipy.fft.dct(type=2, norm="ortho") on blocks of 256, by the
-orthonormality of the basis (Parseval) and by the round trip. Tolerance: fp32 accumulation of
-256 products, 2e-5 relative to the block's norm."""
+orthonormality of the basis (Parseval) and by the round trip. Tolerance: 1e-5 relative to the
+block's norm (a coefficient is a sum of 256 fp32 products; relative to a single coefficient no
+bound exists, since coefficients pass through zero)."""
 import numpy as np
 import pytest
 
@@ -29,8 +30,8 @@ def test_forward_matches_scipy(dct2, blocks, keep):
     got = dct2.forward(x, keep)
     want = _ref(x, keep)
     scale = np.linalg.norm(x.reshape(-1, 256), axis=1, keepdims=True)
-    assert np.abs(got - want).max() <= 2e-5 * scale.max()
-    assert (np.abs(got - want) <= 2e-5 * scale + 1e-7).all()
+    assert np.abs(got - want).max() <= 1e-5 * scale.max()
+    assert (np.abs(got - want) <= 1e-5 * scale + 1e-7).all()
 
 
 def test_known_vectors(dct2):
@@ -53,7 +54,7 @@ def test_round_trip_and_parseval(dct2):
     y = dct2.forward(x, 256)
     assert abs(np.sum(y.astype(np.float64) ** 2) / np.sum(x.astype(np.float64) ** 2) - 1.0) < 1e-5
     back = dct2.inverse(y, n, 256)
-    assert np.abs(back - x).max() < 2e-5 * 16
+    assert np.abs(back - x).max() < 1e-5 * 16
     # truncated: inverse(keep) equals the inverse of the zero-padded coefficients
     y64 = dct2.forward(x, 64)
     assert np.array_equal(y64, y[:, :64])
@@ -62,7 +63,7 @@ def test_round_trip_and_parseval(dct2):
     pad[:, :64] = y64
     want = fft.idct(pad, type=2, norm="ortho", axis=1).ravel()
     got = dct2.inverse(y64, n, 64)
-    assert np.abs(got - want).max() < 2e-5 * 16
+    assert np.abs(got - want).max() < 1e-5 * 16
 
 
 def test_device_pointers_and_arguments(dct2):
@@ -76,3 +77,37 @@ def test_device_pointers_and_arguments(dct2):
         dct2.forward(x[:100], 64)
     with pytest.raises(api.KrakenHipError):
         dct2.forward(x, 50)
+
+
+@pytest.mark.parametrize("keep", [64, 256])
+def test_config_size_tensor(dct2, keep):
+    """The configuration's own shape, fp32 [4096, 16384] of N(0, 1) = 262144 blocks: scipy on a
+    random 1 % of the blocks at 1e-5 of the block norm, Parseval over the whole tensor (keep 256;
+    for keep 64 the kept energy can only be smaller, and equals scipy's on the sample), and the
+    round trip through the inverse."""
+    fft = pytest.importorskip("scipy.fft")
+    rng = np.random.default_rng(keep)
+    n = 4096 * 16384
+    x = rng.standard_normal(n, dtype=np.float32)
+    y = dct2.forward(x, keep)
+    assert y.shape == (n // 256, keep)
+    blocks = rng.choice(n // 256, size=n // 256 // 100, replace=False)
+    xb = x.reshape(-1, 256)[blocks]
+    want = fft.dct(xb.astype(np.float64), type=2, norm="ortho", axis=1)[:, :keep]
+    scale = np.linalg.norm(xb.astype(np.float64), axis=1, keepdims=True)
+    err = np.abs(y[blocks] - want) / scale
+    assert err.max() <= 1e-5, err.max()
+    energy_x = float(np.sum(x.astype(np.float64) ** 2))
+    energy_y = float(np.sum(y.astype(np.float64) ** 2))
+    if keep == 256:
+        assert abs(energy_y / energy_x - 1.0) < 1e-5
+        back = dct2.inverse(y, n, keep)
+        assert np.abs(back - x).max() <= 1e-5 * np.linalg.norm(xb, axis=1).max()
+    else:
+        assert energy_y < energy_x
+        assert abs(np.sum(y[blocks].astype(np.float64) ** 2) / np.sum(want ** 2) - 1.0) < 1e-5
+        pad = np.zeros((blocks.size, 256))
+        pad[:, :keep] = want
+        back = dct2.inverse(y, n, keep).reshape(-1, 256)[blocks]
+        assert np.abs(back - fft.idct(pad, type=2, norm="ortho", axis=1)).max() <= 1e-5 * scale.max()
+    print("keep %d: worst coefficient error %.2e of the block norm" % (keep, err.max()))
