@@ -1,0 +1,167 @@
+// The drop-in itself: kraken::Table subclasses over the C ABI (include/kraken_hip.h), written
+// against the REFERENCE's own headers (kraken/ps/table.h, ps/optim/optim.h,
+// ps/initializer/initializer.h, t/tensor.h), which must be on the include path. This is the file a
+// Kraken maintainer adds to the tree; kraken_gpu_tables.h is the same code over a minimal Tensor
+// for builds that have no Kraken tree.
+//
+// Nothing here throws, whatever the device does: the reference's server threads catch nothing
+// (common/exception.h:13-31 is only thrown by tensor misuse), so every failure is an ErrorCode.
+#pragma once
+
+#include <cstring>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "common/error_code.h"
+#include "kraken_hip.h"
+#include "ps/initializer/initializer.h"
+#include "ps/optim/optim.h"
+#include "ps/table.h"
+#include "t/element_type.h"
+#include "t/shape.h"
+#include "t/storage.h"
+#include "t/tensor.h"
+
+namespace kraken {
+
+// [integration:begin]
+// The model's optimizer for GPU tables (created where Ps::CreateModel calls Optim::Create,
+// ps/ps.cc:604-633): the reference's Adagrad / Adam / RMSprop / SGD keep their hyper-parameters
+// private, so the same conf map is parsed into the C ABI's krk_optim (krk_optim_set follows
+// ps/optim/optim.cc:23-101 key by key). A GPU table never calls Update: the update runs on the
+// device, fused with the row access.
+class GpuOptim : public Optim {
+  krk_optim raw_;
+
+ public:
+  GpuOptim(OptimType optim_type, const krk_optim& raw) : Optim(optim_type), raw_(raw) {}
+  int32_t Update(const Tensor&, float, Value*) const override { return ErrorCode::kInterfaceUnImplementError; }
+  const krk_optim* raw() const { return &raw_; }
+
+  static std::unique_ptr<Optim> Create(OptimType optim_type,
+                                       const std::unordered_map<std::string, std::string>& optim_conf) {
+    std::unique_ptr<Optim> optim;
+    krk_optim raw;
+    if (krk_optim_defaults((int32_t)optim_type, &raw) != KRK_SUCCESS) return optim;   // as Optim::Create: null
+    for (const auto& kv : optim_conf) krk_optim_set(&raw, kv.first.c_str(), kv.second.c_str());
+    optim.reset(new GpuOptim(optim_type, raw));
+    return optim;
+  }
+};
+
+// null when `optim` is one of the reference's CPU optimizers: the table then answers 6
+inline const krk_optim* ToKrkOptim(Optim* optim) {
+  const GpuOptim* g = dynamic_cast<const GpuOptim*>(optim);
+  return g ? g->raw() : nullptr;
+}
+
+class GpuSparseTable : public Table {
+  int64_t dimension_;
+  ElementType element_type_;
+  std::unique_ptr<Initializer> initializer_;   // kept for conf() / checkpoint metadata
+  krk_sparse* h_ = nullptr;
+  int32_t create_rc_ = ErrorCode::kSuccess;
+
+ public:
+  GpuSparseTable(uint64_t id, const std::string& name, int64_t dimension, ElementType element_type,
+                 std::unique_ptr<Initializer>&& initializer)
+      : Table(TableType::kSparse, id, name),
+        dimension_(dimension),
+        element_type_(element_type),
+        initializer_(std::move(initializer)) {
+    krk_init ki;
+    create_rc_ = krk_init_defaults((int32_t)initializer_->type(), &ki);
+    if (create_rc_ != KRK_SUCCESS) return;
+    for (const auto& kv : initializer_->conf()) krk_init_set(&ki, kv.first.c_str(), kv.second.c_str());
+    // the engine holds fp32 rows; another element type is refused at the first call
+    create_rc_ = element_type_.Is<float>() ? krk_sparse_create(dimension, &ki, /*capacity_hint=*/0, &h_)
+                                           : ErrorCode::kSparseTableUnCompatibleError;
+  }
+  ~GpuSparseTable() override { krk_sparse_destroy(h_); }
+
+  int64_t dimension() const { return dimension_; }
+  ElementType element_type() const { return element_type_; }
+  Initializer* initializer() const { return initializer_.get(); }
+  krk_sparse* handle() const { return h_; }   // for the users of SparseTable::mutable_vals()
+
+  int32_t Pull(const std::vector<uint64_t>& sparse_ids, std::vector<Tensor>* vals) override {
+    if (!h_) return create_rc_;
+    // one contiguous [n, dimension] buffer; each returned Tensor is a row view of it
+    // (Tensor::Dense(shape, storage, byte offset, etype), t/tensor.h:58-59), so the serializer
+    // sees the same vector<Tensor> as before without an allocation and a copy per row
+    const size_t row_bytes = (size_t)dimension_ * sizeof(float);
+    std::shared_ptr<Storage> storage = Storage::Create(sparse_ids.size() * row_bytes + sizeof(float));
+    const int32_t rc = krk_sparse_pull(h_, sparse_ids.data(), (int64_t)sparse_ids.size(),
+                                       static_cast<float*>(storage->ptr()), 0);
+    if (rc != ErrorCode::kSuccess) return rc;
+    vals->clear();
+    vals->reserve(sparse_ids.size());
+    const Shape row_shape(std::vector<int64_t>{dimension_});
+    for (size_t i = 0; i < sparse_ids.size(); ++i)
+      vals->emplace_back(Tensor::Dense(row_shape, storage, i * row_bytes, element_type_));
+    return ErrorCode::kSuccess;
+  }
+
+  int32_t Push(Optim* optim, const std::vector<uint64_t>& sparse_ids, const std::vector<Tensor>& grads,
+               float lr) override {
+    if (!h_) return create_rc_;
+    const krk_optim* o = ToKrkOptim(optim);
+    if (!o) return ErrorCode::kUnSupportOptimTypeError;
+    if (grads.size() != sparse_ids.size()) return ErrorCode::kGradientUnCompatibleError;
+    std::vector<float> flat(sparse_ids.size() * (size_t)dimension_);
+    for (size_t i = 0; i < sparse_ids.size(); ++i) {
+      // ps/optim/adagrad.cc:29-32 and its siblings: a dense gradient of the row's size and type
+      if (!grads[i].IsDense() || grads[i].Size() != dimension_ || grads[i].element_type() != element_type_)
+        return ErrorCode::kGradientUnCompatibleError;
+      std::memcpy(&flat[i * (size_t)dimension_], grads[i].Ptr(), (size_t)dimension_ * sizeof(float));
+    }
+    return krk_sparse_push(h_, o, sparse_ids.data(), (int64_t)sparse_ids.size(), flat.data(), dimension_, lr, 0);
+  }
+};
+
+class GpuDenseTable : public Table {
+  Shape shape_;
+  ElementType element_type_;
+  krk_dense* h_ = nullptr;
+  int32_t create_rc_ = ErrorCode::kSuccess;
+
+ public:
+  // ps/dense_table.cc:10-13: the table starts as the given value
+  GpuDenseTable(uint64_t id, const std::string& name, const Tensor& val)
+      : Table(TableType::kDense, id, name), shape_(val.shape()), element_type_(val.element_type()) {
+    create_rc_ = element_type_.Is<float>() && val.IsDense()
+                     ? krk_dense_create(val.Data<float>(), val.Size(), 0, &h_)
+                     : ErrorCode::kDenseTableUnCompatibleError;
+  }
+  ~GpuDenseTable() override { krk_dense_destroy(h_); }
+  krk_dense* handle() const { return h_; }
+
+  int32_t Pull(Tensor* val) override {   // ps/dense_table.cc:31-37: a copy
+    if (!h_) return create_rc_;
+    Tensor out = Tensor::Dense(shape_, element_type_);
+    const int32_t rc = krk_dense_pull(h_, out.Data<float>(), 0);
+    if (rc == ErrorCode::kSuccess) *val = out;
+    return rc;
+  }
+
+  int32_t Push(Optim* optim, const Tensor& grad, float lr) override {   // ps/dense_table.cc:39-43
+    if (!h_) return create_rc_;
+    const krk_optim* o = ToKrkOptim(optim);
+    if (!o) return ErrorCode::kUnSupportOptimTypeError;
+    if (grad.IsCoo()) {
+      // densified on the device like CooTensorImpl::ToDense (t/coo_tensor_impl.cc:250-260)
+      const Tensor& idx = grad.indices();
+      const Tensor& v = grad.values();
+      if (grad.Size() != shape_.Size() || !v.element_type().Is<float>() || !idx.element_type().Is<int64_t>())
+        return ErrorCode::kGradientUnCompatibleError;
+      return krk_dense_push_coo(h_, o, idx.Data<int64_t>(), v.Data<float>(), v.Size(), lr, 0);
+    }
+    if (grad.element_type() != element_type_) return ErrorCode::kGradientUnCompatibleError;
+    return krk_dense_push(h_, o, grad.Data<float>(), grad.Size(), lr, 0);
+  }
+};
+// [integration:end]
+
+}  // namespace kraken
