@@ -34,6 +34,18 @@ __device__ __forceinline__ void vload(const float* p, float (&v)[VEC]) {
     v[0] = *p;
   }
 }
+// A row that is read exactly once (the gradient rows a reduction gathers): non-temporal, so the
+// half gigabyte that passes through does not push the table's records out of the caches.
+typedef float vfloat4_t __attribute__((ext_vector_type(4)));
+template <int VEC>
+__device__ __forceinline__ void vload_once(const float* p, float (&v)[VEC]) {
+  if constexpr (VEC == 4) {
+    const vfloat4_t x = __builtin_nontemporal_load(reinterpret_cast<const vfloat4_t*>(p));
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  } else {
+    v[0] = __builtin_nontemporal_load(p);
+  }
+}
 template <int VEC>
 __device__ __forceinline__ void vstore(float* p, const float (&v)[VEC]) {
   if constexpr (VEC == 4) {
@@ -435,22 +447,46 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
   const bool leader = gl == 0;
   const int lane_floats = group * VEC;
 
-  // hands a finished sum to the optimizer (or stores it): once per run and chunk
-  auto apply = [&](uint32_t key, const float (&sum)[VEC], int e, bool lane_on, bool last_chunk) {
+  // whose record a key names: the table's, or in a combined push the member's
+  auto resolve = [&](uint32_t key, TableView& member, ApplyArgs& aa) -> uint32_t {
     if constexpr (GROUPED) {
       const TableDesc& d = gs.descs[key >> gs.row_bits];
-      TableView member = tv;
       member.recs = d.tv.recs;
       member.stride = d.tv.stride;
-      ApplyArgs aa = args;
       aa.c0 = gs.st0 >= 0 ? d.col_off[gs.st0] : -1;
       aa.c1 = gs.st1 >= 0 ? d.col_off[gs.st1] : -1;
       aa.c2 = gs.st2 >= 0 ? d.col_off[gs.st2] : -1;
       aa.meta_off = gs.use_meta ? d.meta_off : -1;
-      apply_row<OPT, VEC>(member, key & ((1u << gs.row_bits) - 1u), sum, e, lane_on, gl, last_chunk, dim, aa);
+      return key & ((1u << gs.row_bits) - 1u);
     } else {
-      apply_row<OPT, VEC>(tv, key, sum, e, lane_on, gl, last_chunk, dim, args);
+      return key;
     }
+  };
+
+  // A finished sum goes to the optimizer (or is stored) once per run and chunk, in two steps: the
+  // record is requested when the run closes, and updated when the lane group closes its next run
+  // or has walked its tile. In between it goes on requesting and adding gradient rows, so the
+  // record's round trip is not waited for on its own.
+  RowRegs<VEC> pend_regs;
+  float pend_sum[VEC];
+  uint32_t pend_key = kNoRow;
+  auto finish_pending = [&](int e, bool lane_on, bool last_chunk) {
+    if (pend_key == kNoRow) return;
+    TableView member = tv;
+    ApplyArgs aa = args;
+    const uint32_t row = resolve(pend_key, member, aa);
+    finish_row<OPT, VEC>(member, row, pend_sum, e, lane_on, gl, last_chunk, dim, aa, pend_regs);
+    pend_key = kNoRow;
+  };
+  auto apply = [&](uint32_t key, const float (&sum)[VEC], int e, bool lane_on, bool last_chunk) {
+    finish_pending(e, lane_on, last_chunk);
+    TableView member = tv;
+    ApplyArgs aa = args;
+    const uint32_t row = resolve(key, member, aa);
+    load_row<OPT, VEC>(member, row, e, lane_on, aa, pend_regs);
+    pend_key = key;
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) pend_sum[c] = sum[c];
   };
 
   for (int e0 = 0; e0 < elems; e0 += group) {
@@ -497,7 +533,7 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
           k[u] = j < lb ? lds_keys[j + 1] : kNoRow;
           if (j < lb && k[u] < empty_from && lane_on) {
             const float* src = LEVEL0 ? vals + (int64_t)lds_pos[j] * dim : vals + (first + j) * dim;
-            vload<VEC>(src + e * VEC, v[u]);
+            if constexpr (LEVEL0) vload_once<VEC>(src + e * VEC, v[u]); else vload<VEC>(src + e * VEC, v[u]);
             if (weighted) {
               const float w = lds_w[j];
 #pragma unroll
@@ -572,6 +608,7 @@ __global__ __launch_bounds__(kBlock) void segreduce_kernel(
         }
       }
     }
+    finish_pending(e, lane_on, last_chunk);
     __syncthreads();                                        // the next chunk reuses the partials
   }
   if (threadIdx.x < 2 && keys_out) keys_out[2 * (int64_t)blockIdx.x + threadIdx.x] = out_key[threadIdx.x];
