@@ -47,6 +47,27 @@ __device__ __forceinline__ void vload(const float* p, float (&v)[VEC]) {
     v[0] = *p;
   }
 }
+// Streams that pass once (gradient rows in, pulled rows out): non-temporal, so they leave the
+// caches to the index and the records.
+typedef float vfloat4_t __attribute__((ext_vector_type(4)));
+template <int VEC>
+__device__ __forceinline__ void vload_once(const float* p, float (&v)[VEC]) {
+  if constexpr (VEC == 4) {
+    const vfloat4_t x = __builtin_nontemporal_load(reinterpret_cast<const vfloat4_t*>(p));
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  } else {
+    v[0] = __builtin_nontemporal_load(p);
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void vstore_once(float* p, const float (&v)[VEC]) {
+  if constexpr (VEC == 4) {
+    const vfloat4_t x = {v[0], v[1], v[2], v[3]};
+    __builtin_nontemporal_store(x, reinterpret_cast<vfloat4_t*>(p));
+  } else {
+    __builtin_nontemporal_store(v[0], p);
+  }
+}
 template <int VEC>
 __device__ __forceinline__ void vstore(float* p, const float (&v)[VEC]) {
   if constexpr (VEC == 4) {
@@ -94,7 +115,7 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
     } else {
       vload<VEC>(rec + e * VEC, v);
     }
-    vstore<VEC>(dst + e * VEC, v);
+    vstore_once<VEC>(dst + e * VEC, v);
   }
 }
 
@@ -116,7 +137,7 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
   float g_first[VEC];
 #pragma unroll
   for (int c = 0; c < VEC; ++c) g_first[c] = 0.0f;
-  if (active && gl < elems) vload<VEC>(g + gl * VEC, g_first);
+  if (active && gl < elems) vload_once<VEC>(g + gl * VEC, g_first);
   const uint32_t row = probe_find(tv, active ? ids[i] : 0, active, gl, group);
   if (!active) return;
   if (row == kEmptyRow) {
@@ -159,7 +180,7 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
 #pragma unroll
       for (int c = 0; c < VEC; ++c) gv[c] = g_first[c];
     } else {
-      vload<VEC>(g + e * VEC, gv);
+      vload_once<VEC>(g + e * VEC, gv);
       vload<VEC>(rec + e * VEC, w);
       if (pc.c0 >= 0) vload<VEC>(rec + pc.c0 + e * VEC, s0);
       if (pc.c1 >= 0) vload<VEC>(rec + pc.c1 + e * VEC, s1);
@@ -226,7 +247,7 @@ __global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, con
   for (int e = gl; e < elems; e += group) {
     float v[VEC];
     vload<VEC>(rec + e * VEC, v);
-    vstore<VEC>(dst + e * VEC, v);
+    vstore_once<VEC>(dst + e * VEC, v);
   }
 }
 
