@@ -47,6 +47,15 @@ __device__ __forceinline__ void vload_once(const float* p, float (&v)[VEC]) {
   }
 }
 template <int VEC>
+__device__ __forceinline__ void vstore_once(float* p, const float (&v)[VEC]) {
+  if constexpr (VEC == 4) {
+    const vfloat4_t x = {v[0], v[1], v[2], v[3]};
+    __builtin_nontemporal_store(x, reinterpret_cast<vfloat4_t*>(p));
+  } else {
+    __builtin_nontemporal_store(v[0], p);
+  }
+}
+template <int VEC>
 __device__ __forceinline__ void vstore(float* p, const float (&v)[VEC]) {
   if constexpr (VEC == 4) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
@@ -330,10 +339,12 @@ __device__ __forceinline__ void finish_row(const TableView& tv, uint32_t row, co
       if (a.c2 < 0) r.s2[c] = 0.0f;
       optim_element<OPT>(a.k, a.lr, gsum[c], r.w[c], r.s0[c], r.s1[c], r.s2[c], first, bc1, bc2);
     }
-    vstore<VEC>(rec + e * VEC, r.w);
-    if (a.c0 >= 0) vstore<VEC>(rec + a.c0 + e * VEC, r.s0);
-    if (a.c1 >= 0) vstore<VEC>(rec + a.c1 + e * VEC, r.s1);
-    if (a.c2 >= 0) vstore<VEC>(rec + a.c2 + e * VEC, r.s2);
+    // a record is written once per request: past the caches, so the kernel ends with no dirty
+    // lines to write back
+    vstore_once<VEC>(rec + e * VEC, r.w);
+    if (a.c0 >= 0) vstore_once<VEC>(rec + a.c0 + e * VEC, r.s0);
+    if (a.c1 >= 0) vstore_once<VEC>(rec + a.c1 + e * VEC, r.s1);
+    if (a.c2 >= 0) vstore_once<VEC>(rec + a.c2 + e * VEC, r.s2);
   }
   // The counter is read by every chunk of the row before the last chunk advances it.
   if (a.meta_off >= 0 && last_chunk) store_row_word<VEC>(rec + a.meta_off, steps, gl, dim, (int)tv.stride - a.meta_off);

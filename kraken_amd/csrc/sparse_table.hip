@@ -193,10 +193,12 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
       if (pc.c2 < 0) s2[c] = 0.0f;
       optim_element<OPT>(k, lr, gv[c], w[c], s0[c], s1[c], s2[c], first, bc1, bc2);
     }
-    vstore<VEC>(rec + e * VEC, w);
-    if (pc.c0 >= 0) vstore<VEC>(rec + pc.c0 + e * VEC, s0);
-    if (pc.c1 >= 0) vstore<VEC>(rec + pc.c1 + e * VEC, s1);
-    if (pc.c2 >= 0) vstore<VEC>(rec + pc.c2 + e * VEC, s2);
+    // written once per launch and not read again by it: past the caches, so that the end of the
+    // kernel has no dirty lines left to write back
+    vstore_once<VEC>(rec + e * VEC, w);
+    if (pc.c0 >= 0) vstore_once<VEC>(rec + pc.c0 + e * VEC, s0);
+    if (pc.c1 >= 0) vstore_once<VEC>(rec + pc.c1 + e * VEC, s1);
+    if (pc.c2 >= 0) vstore_once<VEC>(rec + pc.c2 + e * VEC, s2);
   }
   if (pc.meta >= 0) store_row_word<VEC>(rec + pc.meta, steps, gl, dim, (int)tv.stride - pc.meta);
 }
@@ -358,7 +360,7 @@ __global__ __launch_bounds__(kBlock) void pooled_sum_kernel(TableView tv, const 
 #pragma unroll
     for (int c = 0; c < VEC; ++c) acc[c] = acc[c] * ratio;
   }
-  vstore<VEC>(out + bag * (int64_t)dim + gl * VEC, acc);
+  vstore_once<VEC>(out + bag * (int64_t)dim + gl * VEC, acc);
 }
 
 template <int OPT, int VEC>
