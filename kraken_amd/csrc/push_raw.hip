@@ -766,7 +766,11 @@ static hipError_t sort_pairs(void* tmp, size_t& tmp_bytes, uint32_t* keys, uint3
 // records); sorting a table's 8192 pairs in one workgroup 20-30 us whoever wrote the sort (a
 // pass is a chain of LDS round trips and barriers, and a wavefront instruction holds its SIMD
 // for four cycles), 19 us even for a bucket's 1024 pairs when the pairs arrive unordered and
-// position has to be sorted as well (five passes).
+// position has to be sorted as well (five passes); the whole request in one launch (buckets by a
+// hash of the id, the look-up inside the bucket's workgroup, gradient rows staged through LDS a
+// chunk at a time) 38 us, 57 us for 26 tables: the workgroup that draws the hottest id holds five
+// times the entries of the others, and the sixteen wavefronts of a workgroup share four SIMDs,
+// so every instruction of a wavefront costs sixteen cycles there.
 // ---------------------------------------------------------------------------
 constexpr int kSortBlock = 1024;
 constexpr int kSortItems = 8;
@@ -1044,6 +1048,9 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
     const int stretch = (count + per_block - 1) / per_block;
     const int lo = start + lt * stretch < start + count ? start + lt * stretch : start + count;
     const int hi = lo + stretch < start + count ? lo + stretch : start + count;
+    const uint32_t row = (skey[start] << bucket_bits) | bucket;
+    RowRegs<VEC> rec;
+    if (lt == 0) load_row<OPT, VEC>(tv, row, gl, lane_on, args, rec);   // on its way while the stretches are added
     float acc[VEC];
     sum_entries(lo, hi, acc);
     // inside the wavefront: lane group i takes in group i + 1, then i + 2, i + 4, ...
@@ -1054,20 +1061,22 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
         if (((lane / group) & ((2 * d / group) - 1)) == 0) acc[c] = acc[c] + other;
       }
     }
-    if (lane < group) vstore<VEC>(part + wave * lane_floats + gl * VEC, acc);
+    // two sets of partial sums in turn: one barrier a run, the next run's stretches are requested
+    // while the first lane group still updates this run's row
+    float* mine = part + (k & 1u) * kSortWaves * lane_floats;
+    if (lane < group) vstore<VEC>(mine + wave * lane_floats + gl * VEC, acc);
     __syncthreads();
     if (lt == 0) {
       float w[kSortWaves][VEC];
 #pragma unroll
-      for (int f = 1; f < kSortWaves; ++f) vload<VEC>(part + f * lane_floats + gl * VEC, w[f]);
+      for (int f = 1; f < kSortWaves; ++f) vload<VEC>(mine + f * lane_floats + gl * VEC, w[f]);
 #pragma unroll
       for (int f = 1; f < kSortWaves; ++f) {
 #pragma unroll
         for (int c = 0; c < VEC; ++c) acc[c] = acc[c] + w[f][c];
       }
-      apply_row<OPT, VEC>(tv, (skey[start] << bucket_bits) | bucket, acc, gl, lane_on, gl, true, dim, args);
+      finish_row<OPT, VEC>(tv, row, acc, gl, lane_on, gl, true, dim, args, rec);
     }
-    __syncthreads();
   }
 }
 
