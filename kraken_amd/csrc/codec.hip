@@ -283,8 +283,8 @@ __global__ __launch_bounds__(kCodecBlock) void emit_write_kernel(
     const int64_t out0 = tile_offsets[tile];
     const int64_t tile_base = tile * kCodecTile;
     for (int i = threadIdx.x; i < count; i += kCodecBlock) {
-      idx[out0 + i] = tile_base + kept_at[i];
-      val[out0 + i] = kept_val[i];
+      __builtin_nontemporal_store((long long)(tile_base + kept_at[i]), idx + out0 + i);
+      __builtin_nontemporal_store(kept_val[i], val + out0 + i);
     }
     __syncthreads();                               // the next tile reuses the LDS arrays
   }
@@ -303,48 +303,70 @@ __global__ __launch_bounds__(kCodecBlock) void coo_tiles_init_kernel(uint32_t* _
   if (i == 0) *unordered = 0u;
 }
 
-// starts[T] = first entry whose index lies in tile T; *unordered is raised when the indices do
-// not ascend strictly or leave [0, n).
+// starts[T] / ends[T] = the entries whose index lies in tile T (ends is only read where starts is
+// set); *unordered is raised when the indices do not ascend strictly or leave [0, n).
 __global__ __launch_bounds__(kCodecBlock) void coo_tiles_bounds_kernel(const long long* __restrict__ idx,
                                                                        int64_t nnz, int64_t n,
                                                                        uint32_t* __restrict__ starts,
+                                                                       uint32_t* __restrict__ ends,
                                                                        uint32_t* __restrict__ unordered) {
   const int64_t step = (int64_t)gridDim.x * kCodecBlock;
   for (int64_t j = (int64_t)blockIdx.x * kCodecBlock + threadIdx.x; j < nnz; j += step) {
-    const long long cur = idx[j];
+    const long long cur = __builtin_nontemporal_load(idx + j);
     const long long prev = j ? idx[j - 1] : -1;
     if (cur <= prev || cur >= n) {
       atomicOr(unordered, 1u);
-    } else if (prev < 0 || cur / kTileElems != prev / kTileElems) {
-      starts[cur / kTileElems] = (uint32_t)j;
+    } else {
+      if (prev < 0 || cur / kTileElems != prev / kTileElems) {
+        starts[cur / kTileElems] = (uint32_t)j;
+        if (prev >= 0) ends[prev / kTileElems] = (uint32_t)j;
+      }
+      if (j == nnz - 1) ends[cur / kTileElems] = (uint32_t)nnz;
     }
   }
 }
 
+// One workgroup per output tile: the tile is put together in LDS (zeros, then the tile's entries,
+// whose range is known, so their loads do not wait for one another) and leaves in whole lines,
+// past the caches.
 __global__ __launch_bounds__(kCodecBlock) void coo_tiles_write_kernel(const long long* __restrict__ idx,
                                                                       const float* __restrict__ val, int64_t nnz,
                                                                       float* __restrict__ dense, int64_t n,
                                                                       const uint32_t* __restrict__ starts,
+                                                                      const uint32_t* __restrict__ ends,
                                                                       const uint32_t* __restrict__ unordered) {
   if (*unordered) return;                        // the scatter launches that follow do the work
-  __shared__ float tile[kTileElems];
+  __shared__ __align__(16) float tile[kTileElems];
   const int64_t base = (int64_t)blockIdx.x * kTileElems;
-  for (int i = threadIdx.x; i < kTileElems; i += kCodecBlock) tile[i] = 0.0f;
-  __syncthreads();
   const uint32_t start = starts[blockIdx.x];
+  const uint32_t end = start != kNoStart ? ends[blockIdx.x] : 0u;
+  for (int i = threadIdx.x; i < kTileElems / 4; i += kCodecBlock)
+    reinterpret_cast<float4*>(tile)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  __syncthreads();
   if (start != kNoStart) {
-    for (int64_t j = (int64_t)start + threadIdx.x; j < nnz; j += kCodecBlock) {
-      const long long i = idx[j];
-      if (i >= base + kTileElems) break;         // ascending: nothing further belongs to this tile
-      tile[i - base] = val[j];
+    for (int64_t j0 = (int64_t)start + threadIdx.x; j0 < (int64_t)end; j0 += 4 * kCodecBlock) {
+      long long at[4];
+      float v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t j = j0 + u * kCodecBlock;
+        if (j < (int64_t)end) {
+          at[u] = __builtin_nontemporal_load(idx + j);
+          v[u] = __builtin_nontemporal_load(val + j);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (j0 + u * kCodecBlock < (int64_t)end) tile[at[u] - base] = v[u];
     }
   }
   __syncthreads();
   const int64_t left = n - base;
   const int cnt = left < kTileElems ? (int)left : kTileElems;
   if (cnt == kTileElems && (((uintptr_t)dense) & 15) == 0) {
+    typedef float tile4 __attribute__((ext_vector_type(4)));
     for (int i = threadIdx.x; i < kTileElems / 4; i += kCodecBlock)
-      reinterpret_cast<float4*>(dense + base)[i] = reinterpret_cast<const float4*>(tile)[i];
+      __builtin_nontemporal_store(reinterpret_cast<const tile4*>(tile)[i], reinterpret_cast<tile4*>(dense + base) + i);
   } else {
     for (int i = threadIdx.x; i < cnt; i += kCodecBlock) dense[base + i] = tile[i];
   }
@@ -383,7 +405,7 @@ static unsigned stream_grid(int64_t n) {
 }
 
 size_t coo_densify_work_bytes(int64_t n) {
-  return ((size_t)((n + kTileElems - 1) / kTileElems) + 4) * sizeof(uint32_t);
+  return (2 * (size_t)((n + kTileElems - 1) / kTileElems) + 4) * sizeof(uint32_t);
 }
 
 int32_t coo_densify(const long long* d_idx, const float* d_val, int64_t nnz, float* d_dense, int64_t n,
@@ -401,14 +423,15 @@ int32_t coo_densify(const long long* d_idx, const float* d_val, int64_t nnz, flo
   }
   const int64_t tiles = (n + kTileElems - 1) / kTileElems;
   uint32_t* starts = reinterpret_cast<uint32_t*>(work);
-  uint32_t* unordered = starts + tiles;
+  uint32_t* ends = starts + tiles;
+  uint32_t* unordered = ends + tiles;
   hipLaunchKernelGGL(coo_tiles_init_kernel, dim3((unsigned)((tiles + kCodecBlock - 1) / kCodecBlock)), block, 0,
                      stream, starts, tiles, unordered);
   if (nnz)
     hipLaunchKernelGGL(coo_tiles_bounds_kernel, dim3(stream_grid(nnz)), block, 0, stream, d_idx, nnz, n, starts,
-                       unordered);
+                       ends, unordered);
   hipLaunchKernelGGL(coo_tiles_write_kernel, dim3((unsigned)tiles), block, 0, stream, d_idx, d_val, nnz, d_dense,
-                     n, starts, unordered);
+                     n, starts, ends, unordered);
   if (nnz) {
     hipLaunchKernelGGL(coo_zero_if_kernel, dim3(stream_grid(n)), block, 0, stream, d_dense, n, unordered);
     // a few workgroups that stride over the entries: when the tiles did the work they only look at
