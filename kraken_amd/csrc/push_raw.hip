@@ -177,6 +177,96 @@ __global__ __launch_bounds__(kBlock) void dedup_inv_kernel(const DSlot* __restri
   inv[p] = (long long)slots[slot_of[p]].uidx;
 }
 
+// Requests of at most kDedupSmall ids: the whole dedup in one launch of one workgroup. The ids
+// sit in LDS; an open-addressing table of positions (a slot holds the smallest position of the
+// id that owns it, and the id itself is looked up through that position) replaces the index in
+// global memory; a lane owns eight consecutive positions, so one scan over the workgroup gives
+// every first occurrence its place in the unique list.
+constexpr int kDedupSmall = 8192;
+constexpr int kDedupSmallSlots = 2 * kDedupSmall;
+constexpr int kDedupSmallOwn = kDedupSmall / kDedupBlock;
+constexpr uint32_t kNoPos = 0xFFFFFFFFu;
+
+__global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t* __restrict__ ids, int n,
+                                                                  uint64_t* __restrict__ uids,
+                                                                  long long* __restrict__ inv,
+                                                                  int32_t* __restrict__ total) {
+  __shared__ unsigned long long sid[kDedupSmall];
+  __shared__ uint32_t tab[kDedupSmallSlots];           // position of the id's first occurrence, then its unique index
+  __shared__ uint32_t wave_total[kDedupBlock / kWave];
+  const int t = threadIdx.x;
+  // table size by request size: a small request clears and probes a small table
+  int bits = 5;
+  while ((1 << bits) < 2 * n) ++bits;
+  const uint32_t mask = (1u << bits) - 1u;
+  for (int i = t; i <= (int)mask; i += kDedupBlock) tab[i] = kNoPos;
+  for (int i = t; i < n; i += kDedupBlock) sid[i] = ids[i];
+  __syncthreads();
+  uint32_t slot[kDedupSmallOwn];
+#pragma unroll
+  for (int i = 0; i < kDedupSmallOwn; ++i) {
+    const int p = t * kDedupSmallOwn + i;
+    if (p < n) {
+      const unsigned long long id = sid[p];
+      uint32_t h = (uint32_t)(mix64(id) >> 32) & mask;
+      for (;;) {
+        uint32_t q = tab[h];
+        if (q == kNoPos) {
+          q = atomicCAS(&tab[h], kNoPos, (uint32_t)p);
+          if (q == kNoPos) break;                      // the slot is this id's now
+        }
+        if (sid[q] == id) {                            // whoever holds it, it is the same id
+          atomicMin(&tab[h], (uint32_t)p);
+          break;
+        }
+        h = (h + 1) & mask;
+      }
+      slot[i] = h;
+    }
+  }
+  __syncthreads();
+  uint32_t first = 0;                                  // bit i: my position i is its id's first
+#pragma unroll
+  for (int i = 0; i < kDedupSmallOwn; ++i) {
+    const int p = t * kDedupSmallOwn + i;
+    if (p < n && tab[slot[i]] == (uint32_t)p) first |= 1u << i;
+  }
+  // exclusive scan of the counts over the workgroup
+  const int lane = t & (kWave - 1), wave = t / kWave;
+  const uint32_t mine = (uint32_t)__popc(first);
+  uint32_t incl = mine;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const uint32_t y = __shfl_up(incl, d);
+    if (lane >= d) incl += y;
+  }
+  if (lane == kWave - 1) wave_total[wave] = incl;
+  __syncthreads();                                     // also: every first occurrence has been read from the table
+  uint32_t rank = incl - mine, all = 0;
+  for (int w = 0; w < kDedupBlock / kWave; ++w) {
+    const uint32_t x = wave_total[w];
+    if (w < wave) rank += x;
+    all += x;
+  }
+#pragma unroll
+  for (int i = 0; i < kDedupSmallOwn; ++i) {
+    if (first & (1u << i)) {
+      const int p = t * kDedupSmallOwn + i;
+      uids[rank] = sid[p];
+      tab[slot[i]] = rank;                             // the table now answers with the unique index
+      ++rank;
+    }
+  }
+  if (t == 0) *total = (int32_t)all;
+  if (!inv) return;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < kDedupSmallOwn; ++i) {
+    const int p = t * kDedupSmallOwn + i;
+    if (p < n) inv[p] = (long long)tab[slot[i]];
+  }
+}
+
 // ---------------------------------------------------------------------------
 // push_raw stage 1: position -> row number (the sort key), positions as payload
 // ---------------------------------------------------------------------------
@@ -1319,6 +1409,24 @@ static int32_t dedup_enqueue(const DedupWork& w, const uint64_t* d_ids, int64_t 
   return KRK_SUCCESS;
 }
 
+// Where a blocking dedup's count lands: page-locked host memory the last kernel's total is copied
+// into in stream order, so the host waits for the stream once and reads it (no blocking copy).
+static int32_t* g_dedup_count = nullptr;
+
+static int32_t dedup_count_buffer() {
+  if (g_dedup_count) return KRK_SUCCESS;
+  KRK_HIP(hipHostMalloc((void**)&g_dedup_count, 64, hipHostMallocDefault));
+  return KRK_SUCCESS;
+}
+
+static int32_t dedup_read_count(const int32_t* d_total, hipStream_t s, int32_t* u) {
+  KRK_TRY(dedup_count_buffer());
+  KRK_HIP(hipMemcpyAsync(g_dedup_count, d_total, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  KRK_HIP(hipStreamSynchronize(s));
+  *u = *g_dedup_count;
+  return KRK_SUCCESS;
+}
+
 static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, uint64_t* d_uids,
                           long long* d_inv, hipStream_t s, int32_t* u) {
   KRK_HIP(hipMemsetAsync(w.slots, 0xFF, (w.cap + 1) * sizeof(DSlot), s));
@@ -1331,8 +1439,7 @@ static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, 
   hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids);
   if (d_inv) hipLaunchKernelGGL(dedup_inv_kernel, grid, block, 0, s, w.slots, w.slot_of, n, d_inv);
   KRK_HIP(hipGetLastError());
-  KRK_HIP(hipMemcpy(u, w.d_total, sizeof(*u), hipMemcpyDeviceToHost));
-  return KRK_SUCCESS;
+  return dedup_read_count(w.d_total, s, u);
 }
 
 int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, int64_t* n_unique,
@@ -1364,7 +1471,14 @@ int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, 
   }
   hipStream_t s = nullptr;
   int32_t u = 0;
-  KRK_TRY(dedup_core(w, d_ids, n, d_uids, inv ? d_inv : nullptr, s, &u));
+  if (n <= kDedupSmall) {
+    hipLaunchKernelGGL(dedup_small_kernel, dim3(1), dim3(kDedupBlock), 0, s, d_ids, (int)n, d_uids,
+                       inv ? d_inv : nullptr, w.d_total);
+    KRK_HIP(hipGetLastError());
+    KRK_TRY(dedup_read_count(w.d_total, s, &u));
+  } else {
+    KRK_TRY(dedup_core(w, d_ids, n, d_uids, inv ? d_inv : nullptr, s, &u));
+  }
   *n_unique = u;
   if (host) {
     KRK_HIP(hipMemcpy(uids, d_uids, (size_t)u * 8, hipMemcpyDeviceToHost));
