@@ -310,7 +310,11 @@ __global__ __launch_bounds__(kBlock) void group_rows_of_ids_kernel(const TableDe
   // a workgroup serves one member (call.block_start counts workgroups of kBlock / kBucket
   // positions here), so the member's layout comes in through scalar loads
   int m = 0;
-  while (m + 1 < call.n_tables && blockIdx.x >= call.block_start[m + 1]) ++m;
+  if (call.even_blocks) {
+    m = (int)(blockIdx.x / call.even_blocks);          // members of equal length: no walk
+  } else {
+    while (m + 1 < call.n_tables && blockIdx.x >= call.block_start[m + 1]) ++m;
+  }
   const int64_t p = call.row_start[m] + (int64_t)(blockIdx.x - call.block_start[m]) * (kBlock / kBucket) +
                     threadIdx.x / kBucket;
   const int gl = threadIdx.x & (kBucket - 1);
@@ -1821,11 +1825,15 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
   // the launch that turns ids into rows gives every member whole workgroups of its own
   GroupCall rows_call = call;
   uint32_t blocks = 0;
+  bool even = true;
   for (int m = 0; m < n_tables; ++m) {
     rows_call.block_start[m] = blocks;
-    blocks += grid_for(offsets[m + 1] - offsets[m], kBlock / kBucket);
+    const uint32_t mine = grid_for(offsets[m + 1] - offsets[m], kBlock / kBucket);
+    even = even && mine == grid_for(offsets[1] - offsets[0], kBlock / kBucket);
+    blocks += mine;
   }
   rows_call.block_start[n_tables] = blocks;
+  rows_call.even_blocks = even && blocks > 0 ? blocks / (uint32_t)n_tables : 0u;
   const uint64_t* d_ids;
   const float* d_g;
   KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
