@@ -31,6 +31,31 @@ def test_dedup_small(api, oracle, ids):
     assert np.array_equal(u, ru) and np.array_equal(inv, rinv)
 
 
+@pytest.mark.parametrize("n", [1, 63, 1024, 8191, 8192, 8193])
+@pytest.mark.parametrize("kind", ["distinct", "same", "pairs", "sentinels"])
+def test_dedup_single_launch_boundaries(api, oracle, n, kind):
+    """Requests of at most 8192 ids are deduplicated by one workgroup; 8193 ids take the path of
+    large requests. Both must give the oracle's unique list (first-occurrence order) and inverse,
+    for all-distinct ids (the table at its fullest), one id throughout, every id twice, and the
+    two ids an index might mistake for markers (0 and all ones)."""
+    rng = np.random.default_rng(n)
+    if kind == "distinct":
+        ids = rng.permutation(n).astype(np.uint64) * np.uint64(0x9E3779B97F4A7C15)
+    elif kind == "same":
+        ids = np.full(n, 77, np.uint64)
+    elif kind == "pairs":
+        ids = np.repeat(rng.permutation((n + 1) // 2).astype(np.uint64) + np.uint64(10), 2)[:n]
+        rng.shuffle(ids)
+    else:
+        ids = rng.choice(np.array([0, 2**64 - 1, 5], np.uint64), size=n)
+    u, inv = api.dedup(ids)
+    ru, rinv = oracle.dedup(ids)
+    assert np.array_equal(u, ru) and np.array_equal(inv, rinv)
+    du, dinv, cnt = api.dedup(api.DeviceArray.from_host(ids))
+    assert cnt == ru.size
+    assert np.array_equal(du.to_host()[:cnt], ru) and np.array_equal(dinv.to_host(), rinv)
+
+
 def test_dedup_empty(api):
     u, inv = api.dedup(np.zeros(0, np.uint64))
     assert u.size == 0 and inv.size == 0
