@@ -17,6 +17,7 @@ the same machine on a bounded sample of the same workload.
 """
 import argparse
 import concurrent.futures
+import gc
 import json
 import os
 import sys
@@ -188,15 +189,23 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32):
     sync_all()
     per_step, enq = [], []
     rows_per_step = float(np.mean([dev[i % n_batches][4] for i in range(steps)]))
-    for b in range(blocks):
-        t0 = time.perf_counter()
-        for i in range(steps):
-            step(i)
-        t1 = time.perf_counter()
-        sync_all()
-        t2 = time.perf_counter()
-        per_step.append((t2 - t0) / steps)
-        enq.append((t1 - t0) / steps)
+    # the interpreter's garbage is collected between blocks, not inside one: a collection stalls
+    # the host for longer than several steps take on the device
+    gc.collect()
+    gc.disable()
+    try:
+        for b in range(blocks):
+            t0 = time.perf_counter()
+            for i in range(steps):
+                step(i)
+            t1 = time.perf_counter()
+            sync_all()
+            t2 = time.perf_counter()
+            per_step.append((t2 - t0) / steps)
+            enq.append((t1 - t0) / steps)
+            gc.collect()
+    finally:
+        gc.enable()
     med, p10, p90 = _percentiles(per_step)
     print("dim %d: host enqueue %.1f us/step, drained %.1f us/step (median of %d blocks of %d steps)" % (
         dim, np.median(enq) * 1e6, med * 1e6, blocks, steps), file=sys.stderr)

@@ -7,6 +7,7 @@ stream the kernels run on, with inputs resident in HBM; bandwidths are algorithm
 (stated per line) over that time. With no argument all sections run (about a minute). This is
 the program the rocprofv3 summaries of the individual kernels are taken from.
 """
+import gc
 import sys
 
 import numpy as np
@@ -34,12 +35,21 @@ def timed(owner, fn, reps=10, sync=None):
     sync = sync or (owner.sync if owner is not None else api.synchronize)
     fn()
     sync()
-    e0, e1 = api.Event(), api.Event()
-    e0.record(owner)
-    for _ in range(reps):
-        fn()
-    e1.record(owner)
-    sync()
+    # a collection of the interpreter's garbage in the middle of ten calls stalls the host for
+    # longer than the calls take on the device, and the stream runs dry: collect before, not during
+    gc.collect()
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        e0, e1 = api.Event(), api.Event()
+        e0.record(owner)
+        for _ in range(reps):
+            fn()
+        e1.record(owner)
+        sync()
+    finally:
+        if was_enabled:
+            gc.enable()
     return e0.elapsed_ms(e1) / reps * 1e-3
 
 
