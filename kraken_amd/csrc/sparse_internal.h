@@ -425,7 +425,8 @@ struct GroupLock {
   GroupLock& operator=(const GroupLock&) = delete;
 };
 // Checks the offsets of a combined request and lays its members out over the grid.
-int32_t group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, int64_t* total);
+// per_block: positions a workgroup of the launch takes (0: kBlock / the group's lanes per row)
+int32_t group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, int64_t* total, int per_block = 0);
 // Uploads the layouts of members that moved since the last call.
 int32_t group_refresh(krk_group* g);
 // Blocking calls: waits for the group's stream and reports the first member's error.

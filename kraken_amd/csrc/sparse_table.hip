@@ -373,6 +373,117 @@ __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64
   push_body<OPT, VEC>(tv, ids, i, i < n, threadIdx.x & (group - 1), grads, dim, elems, group, lr, k, pc);
 }
 
+// ---- pulls of rows 32 to 128 floats wide -------------------------------------------------------
+// With one lane group of dim / 4 lanes per id from the search on, a wavefront of a wide table
+// looks up only two to eight ids at a time, and a pull is then bound by how few index buckets
+// are on their way. Here the search and the copy use different lane mappings: a wavefront takes
+// sixteen ids, four lanes search for each (all sixteen buckets requested at once), and then its
+// lane groups of dim / 4 lanes copy the sixteen rows, several at a time, taking each row's number
+// from the lanes that found it. INSERT: missing ids are inserted and initialised as in pull_body;
+// otherwise they are queued for pull_missing_kernel as in pull_resident_kernel.
+constexpr int kWideIds = kWave / kBucket;        // ids a wavefront takes: 16
+
+template <int VEC, bool INSERT>
+__device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init,
+                                          const uint64_t* __restrict__ ids, int64_t first, int64_t end,
+                                          float* __restrict__ out, int dim, int elems, int group,
+                                          uint32_t* __restrict__ todo, int parity) {
+  const int lane = wave_lane();
+  const int gl4 = lane & (kBucket - 1);
+  const int64_t i = first + (lane >> 2);
+  const bool active = i < end;
+  const uint64_t id = active ? ids[i] : 0;
+  const FindResult f = probe_find_slot(tv, id, active, gl4, kBucket);
+  ProbeResult pr;
+  pr.row = (uint32_t)f.row_epoch;
+  pr.owner = false;
+  pr.fresh = pr.row == kEmptyRow || (uint32_t)(f.row_epoch >> 32) == tv.epoch;
+  const bool miss = active && !f.found;
+  bool copy = active;
+  if constexpr (INSERT) {
+    if (__any(miss)) {
+      const ProbeResult q = probe_insert(tv, id, miss, gl4, kBucket);
+      if (miss) pr = q;
+    }
+  } else {
+    // one atomic per wavefront reserves queue entries for all of its missing ids
+    const bool queue = miss && gl4 == 0;
+    const unsigned long long votes = __ballot(queue);
+    if (votes) {
+      const int leader = __ffsll(votes) - 1;
+      uint32_t base = 0;
+      if (lane == leader) base = atomicAdd(&tv.counters[2 + parity], (uint32_t)__popcll(votes));
+      base = __shfl(base, leader);
+      if (queue) todo[base + (uint32_t)__popcll(votes & ((1ull << lane) - 1ull))] = (uint32_t)i;
+    }
+    copy = active && f.found;
+    pr.fresh = false;                              // nothing is created here: what was found is read
+  }
+  // the copy: lane group `sub` of the wavefront takes ids sub, sub + rows_per_step, ...
+  const int rows_per_step = kWave / group;       // 8, 4 or 2
+  const int steps = kWideIds / rows_per_step;    // 2, 4 or 8
+  const int sub = lane / group;
+  const int gl = lane & (group - 1);
+  const uint32_t id_lo = (uint32_t)id, id_hi = (uint32_t)(id >> 32);
+  float v[8][VEC];
+  uint32_t live = 0;                             // bit s: this lane has a slice of step s to store
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    if (s < steps) {                             // uniform
+      const int src = kBucket * (s * rows_per_step + sub);
+      const uint32_t row = __shfl(pr.row, src);
+      const int fresh = __shfl((int)pr.fresh, src);
+      const int owner = __shfl((int)pr.owner, src);
+      const int on = __shfl((int)copy, src);
+      const uint64_t its_id = (uint64_t)__shfl(id_lo, src) | ((uint64_t)__shfl(id_hi, src) << 32);
+      if (on && gl < elems) {
+        float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
+        if (fresh) {
+          // the value of a new row is a pure function of (seed, id, element): every group that
+          // meets it computes the same numbers, only the creator stores them
+          init_vec<VEC>(init, its_id, (int64_t)gl * VEC, v[s]);
+          if (owner) vstore<VEC>(rec + gl * VEC, v[s]);
+        } else {
+          vload<VEC>(rec + gl * VEC, v[s]);
+        }
+        live |= 1u << s;
+      }
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    if (live & (1u << s))
+      vstore_once<VEC>(out + (first + s * rows_per_step + sub) * (int64_t)dim + gl * VEC, v[s]);
+  }
+}
+
+// whether a table's rows take the wide pull: lane groups of 8 to 32 lanes that hold a whole row
+__host__ __device__ inline bool pull_is_wide(int group, int elems) {
+  return group >= 8 && group <= 32 && elems <= group;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pull_wide_kernel(TableView tv, InitK init,
+                                                           const uint64_t* __restrict__ ids, int64_t n,
+                                                           float* __restrict__ out, int dim, int elems,
+                                                           int group) {
+  const int64_t first = ((int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds;
+  if (first >= n) return;                        // the whole wavefront
+  pull_wide<VEC, true>(tv, init, ids, first, n, out, dim, elems, group, nullptr, 0);
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pull_resident_wide_kernel(TableView tv,
+                                                                    const uint64_t* __restrict__ ids,
+                                                                    int64_t n, float* __restrict__ out,
+                                                                    uint32_t* __restrict__ todo, int parity,
+                                                                    int dim, int elems, int group) {
+  const int64_t first = ((int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds;
+  if (first >= n) return;
+  InitK none{};
+  pull_wide<VEC, false>(tv, none, ids, first, n, out, dim, elems, group, todo, parity);
+}
+
 // ---- one launch over several tables of equal row width ------------------------
 // Table t owns workgroups [block_start[t], block_start[t+1]) and the positions
 // [row_start[t], row_start[t+1]) of the concatenated ids / rows.
@@ -398,6 +509,24 @@ __global__ __launch_bounds__(kBlock) void group_pull_kernel(const TableDesc* __r
   const int64_t i = call.row_start[t] + local;
   pull_body<VEC>(tv, init, ids, i, i < call.row_start[t + 1], threadIdx.x & (group - 1), out, dim,
                  elems, group);
+}
+
+// the same for rows 32 to 128 floats wide: a workgroup takes 64 positions of its table
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void group_pull_wide_kernel(const TableDesc* __restrict__ descs,
+                                                                 GroupCall call,
+                                                                 const uint64_t* __restrict__ ids,
+                                                                 float* __restrict__ out, int dim,
+                                                                 int elems, int group) {
+  const int t = find_table(call);
+  TableView tv = descs[t].tv;
+  tv.epoch = call.epoch[t];
+  const InitK init = descs[t].init;
+  const int64_t local = ((int64_t)(blockIdx.x - call.block_start[t]) * (kBlock / kWave) + threadIdx.x / kWave) *
+                        kWideIds;
+  const int64_t first = call.row_start[t] + local;
+  if (first >= call.row_start[t + 1]) return;    // the whole wavefront
+  pull_wide<VEC, true>(tv, init, ids, first, call.row_start[t + 1], out, dim, elems, group, nullptr, 0);
 }
 
 template <int OPT, int VEC>
@@ -1310,7 +1439,8 @@ int32_t krk_sparse_sync(krk_sparse* t) {
 static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, float* d_out) {
   const int64_t rows_before = t->size_ub;           // upper bound of the rows the table holds
   KRK_TRY(sparse_next_epoch(t, n));
-  const int per_block = kBlock / t->group;
+  const bool wide = t->vec == 4 && pull_is_wide(t->group, t->elems);
+  const int per_block = wide ? (kBlock / kWave) * kWideIds : kBlock / t->group;
   const dim3 grid(grid_for(n, per_block)), block(kBlock);
   // Two launches pay when most ids are resident; a request larger than the table is mostly new
   // ids (a cold start), which the fused launch inserts in one go at twice the rate. A request
@@ -1323,8 +1453,13 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
     t->pull_parity ^= 1;
     const dim3 small(kMissingGrid);
     if (t->vec == 4) {
-      hipLaunchKernelGGL((pull_resident_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
-                         parity, (int)t->dim, t->elems, t->group);
+      if (wide) {
+        hipLaunchKernelGGL((pull_resident_wide_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
+                           todo, parity, (int)t->dim, t->elems, t->group);
+      } else {
+        hipLaunchKernelGGL((pull_resident_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
+                           parity, (int)t->dim, t->elems, t->group);
+      }
       hipLaunchKernelGGL((pull_missing_kernel<4>), small, block, 0, t->stream, t->view(), t->initk, d_ids, d_out,
                          todo, parity, (int)t->dim, t->elems, t->group);
     } else {
@@ -1333,6 +1468,9 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
       hipLaunchKernelGGL((pull_missing_kernel<1>), small, block, 0, t->stream, t->view(), t->initk, d_ids, d_out,
                          todo, parity, (int)t->dim, t->elems, t->group);
     }
+  } else if (t->vec == 4 && wide) {
+    hipLaunchKernelGGL((pull_wide_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
+                       (int)t->dim, t->elems, t->group);
   } else if (t->vec == 4) {
     hipLaunchKernelGGL((pull_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
                        (int)t->dim, t->elems, t->group);
@@ -2111,9 +2249,9 @@ int32_t krk::group_refresh(krk_group* g) {
   return KRK_SUCCESS;
 }
 
-int32_t krk::group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, int64_t* total) {
+int32_t krk::group_plan(krk_group* g, const int64_t* offsets, GroupCall* call, int64_t* total, int per_block) {
   const int n = (int)g->tables.size();
-  const int per_block = kBlock / g->group;
+  if (per_block <= 0) per_block = kBlock / g->group;
   call->n_tables = n;
   call->even_blocks = 0;
   uint64_t blocks = 0, widest = 0;
@@ -2178,7 +2316,8 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
   GroupLock lk(g);
   GroupCall call;
   int64_t total = 0;
-  KRK_TRY(group_plan(g, offsets, &call, &total));
+  const bool wide = g->vec == 4 && pull_is_wide(g->group, g->elems);
+  KRK_TRY(group_plan(g, offsets, &call, &total, wide ? (kBlock / kWave) * kWideIds : 0));
   if (total == 0) return group_finish(g, flags);
   if (!ids || !out) return KRK_E_ARGUMENT;
   if ((flags & KRK_DEVICE_PTRS) && g->vec == 4 && !aligned16(out)) return KRK_E_ARGUMENT;
@@ -2199,7 +2338,10 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
   KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
   KRK_TRY(g->output(out, (size_t)total * g->dim, flags, 1, &d_out));
   const dim3 grid(call.block_start[call.n_tables]), block(kBlock);
-  if (g->vec == 4) {
+  if (wide) {
+    hipLaunchKernelGGL((group_pull_wide_kernel<4>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
+                       (int)g->dim, g->elems, g->group);
+  } else if (g->vec == 4) {
     hipLaunchKernelGGL((group_pull_kernel<4>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
                        (int)g->dim, g->elems, g->group);
   } else {
