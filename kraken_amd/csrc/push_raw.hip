@@ -957,21 +957,24 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
   const int wave = t / kWave;
 
   // ---- a. the bucket's positions, in position order -------------------------------------------
-  const int own = (all + kSortBlock - 1) / kSortBlock;  // positions a lane looks at, 1..8
-  for (int j = t; j < all; j += kSortBlock) skey[j] = keys[a + j];   // coalesced; re-read by ownership below
-  __syncthreads();
+  // a lane looks at `own` consecutive positions (1..8), read straight from global memory: a lane's
+  // keys share a line or two, and every request is on its way before the first is looked at
+  const int own = (all + kSortBlock - 1) / kSortBlock;
   uint32_t mine[kSortItems];
+#pragma unroll
+  for (int i = 0; i < kSortItems; ++i) {
+    const int j = t * own + i;
+    if (i < own) mine[i] = keys[a + (j < all ? j : all - 1)];
+  }
   uint32_t take = 0;
 #pragma unroll
   for (int i = 0; i < kSortItems; ++i) {
     const int j = t * own + i;
-    if (i < own && j < all) {
-      mine[i] = skey[j];
-      if (mine[i] < call.miss_key && ((mine[i] & call.row_mask) & (n_buckets - 1)) == bucket) take |= 1u << i;
-    }
+    if (i < own && j < all && mine[i] < call.miss_key && ((mine[i] & call.row_mask) & (n_buckets - 1)) == bucket)
+      take |= 1u << i;
   }
   uint32_t total;
-  uint32_t at = sort_block_scan((uint32_t)__popc(take), wave_total, total);   // its barriers follow the reads
+  uint32_t at = sort_block_scan((uint32_t)__popc(take), wave_total, total);
 #pragma unroll
   for (int i = 0; i < kSortItems; ++i) {
     if (take & (1u << i)) {
@@ -984,8 +987,8 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
   if (len == 0) return;                                // uniform
   const int per_lane = (len + kSortBlock - 1) / kSortBlock;   // 1..8
   const int padded = per_lane * kSortBlock;
-  __syncthreads();
-  for (int j = len + t; j < padded; j += kSortBlock) {
+  for (int j = len + t; j < padded; j += kSortBlock) {   // beyond what the lanes above wrote
+
     skey[j] = 0xFFFFFFFFu;                             // padding sorts behind everything
     spos[j] = 0;
   }
