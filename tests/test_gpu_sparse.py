@@ -295,3 +295,59 @@ def test_adam_amsgrad_impulse_closed_form(api, oracle):
     order = np.argsort(gid)
     assert np.array_equal(vmax[order], np.tile(a * a, (3, 1)))
     assert sorted(steps.tolist()) == [3, 5, 6]
+
+
+@pytest.mark.parametrize("dim", [32, 64, 128])
+def test_wide_rows_pull_every_path(api, oracle, dim):
+    """Rows of 32 to 128 floats are pulled by kernels of their own (sixteen ids looked up per
+    wavefront, then copied by lane groups of dim / 4 lanes). Against the oracle: request sizes on
+    both sides of sixteen and of a workgroup's 64, ids that repeat inside a request, the ids 0 and
+    all ones, new ids next to resident ones (inserted and initialised by the same launch), a
+    request above the size from which a pull runs as two launches (resident ids copied, the rest
+    queued), and the rows read back after an update."""
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "11"})
+    t = api.SparseTable(dim, gi, capacity_hint=64)
+    r = oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=11))
+    rng = np.random.default_rng(dim)
+    o_ref, o_gpu = make_optims(oracle, api, 0, {})
+    special = np.array([0, 2**64 - 1], np.uint64)
+    for n in (1, 15, 16, 17, 63, 64, 65, 1000):
+        fresh = splitmix64(rng.integers(0, 1 << 40, size=n, dtype=np.uint64))
+        ids = np.concatenate([fresh, fresh[: n // 2], special])[rng.permutation(n + n // 2 + 2)]
+        rc, got = t.Pull(ids)
+        _, want = r.pull(ids)
+        assert rc == 0
+        assert_close(got, want, "dim %d, %d ids" % (dim, ids.size), rtol=1e-6)
+        u = np.unique(ids)
+        g = (rng.standard_normal((u.size, dim)) * 0.1).astype(np.float32)
+        assert t.Push(o_gpu, u, g, 0.05) == 0 and r.push(o_ref, u, g, 0.05) == 0
+    big = splitmix64(rng.integers(0, 200_000, size=300_000, dtype=np.uint64))   # repeats, mostly new
+    for _ in range(2):                                   # the second time every id is resident
+        rc, got = t.Pull(big)
+        _, want = r.pull(big)
+        assert rc == 0
+        assert_close(got, want, "dim %d, large pull" % dim, rtol=1e-6)
+    mixed = np.concatenate([big[:280_000], splitmix64(np.arange(1 << 41, (1 << 41) + 20_000, dtype=np.uint64))])
+    rc, got = t.Pull(mixed)                              # two launches: resident rows, then the new ones
+    _, want = r.pull(mixed)
+    assert rc == 0
+    assert_close(got, want, "dim %d, resident and new ids" % dim, rtol=1e-6)
+    assert len(t) == len(r)
+
+
+def test_wide_rows_group_pull_ragged_members(api, oracle):
+    """A combined pull over tables of 64-float rows whose members bring 0, 1, 17 and 5000 ids."""
+    dim = 64
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "4"})
+    counts = [0, 1, 17, 5000, 16]
+    tables = [api.SparseTable(dim, gi) for _ in counts]
+    refs = [oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=4)) for _ in counts]
+    grp = api.TableGroup(tables)
+    rng = np.random.default_rng(5)
+    for step in range(2):
+        per = [splitmix64(rng.integers(0, 3000, size=c, dtype=np.uint64)) for c in counts]
+        rc, got = grp.CombinePull(np.concatenate(per), grp._offsets(counts))
+        assert rc == 0
+        want = np.concatenate([r.pull(p)[1] for r, p in zip(refs, per) if p.size] or [np.zeros((0, dim), np.float32)])
+        assert_close(got, want, "combined pull, step %d" % step, rtol=1e-6)
+    grp.close()
