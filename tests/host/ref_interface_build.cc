@@ -97,6 +97,23 @@ int main(int argc, char** argv) {
   CHECK(sparse->Pull(uniq, &rows) == ErrorCode::kSuccess);
   for (size_t i = 0; i < uniq.size(); ++i)
     for (int64_t j = 0; j < dim; ++j) CHECK(std::fabs(rows[i].Data<float>()[j] - (0.25f - 0.1f * 0.5f * (float)(i + 1))) < 1e-7f);
+  // a reply's rows are views of one page-locked block that belongs to the reply: a later reply
+  // does not overwrite them, and they outlive the request vector they came back in
+  {
+    std::vector<Tensor> first, second;
+    CHECK(sparse->Pull(uniq, &first) == ErrorCode::kSuccess);
+    const Tensor kept = first[1];
+    first.clear();
+    CHECK(sparse->Pull({uniq[0]}, &second) == ErrorCode::kSuccess);
+    for (int64_t j = 0; j < dim; ++j) CHECK(std::fabs(kept.Data<float>()[j] - (0.25f - 0.1f * 0.5f * 2.0f)) < 1e-7f);
+    for (int64_t j = 0; j < dim; ++j) CHECK(std::fabs(second[0].Data<float>()[j] - (0.25f - 0.1f * 0.5f)) < 1e-7f);
+    // a large reply takes a block of its own size
+    std::vector<uint64_t> many(70000);
+    for (size_t i = 0; i < many.size(); ++i) many[i] = 1000000 + i;
+    std::vector<Tensor> big;
+    CHECK(sparse->Pull(many, &big) == ErrorCode::kSuccess && big.size() == many.size());
+    CHECK(big.back().Data<float>()[dim - 1] == 0.25f && big.front().Data<float>()[0] == 0.25f);
+  }
   CHECK(sparse->Push(sgd.get(), {12345}, {grads[0]}, 0.1f) == ErrorCode::kSparseIdNotExistError);
   std::vector<Tensor> narrow = {Tensor::Dense(std::vector<int64_t>{dim - 1}, ElementType::From<float>())};
   CHECK(sparse->Push(sgd.get(), {7}, narrow, 0.1f) == ErrorCode::kGradientUnCompatibleError);
