@@ -297,7 +297,7 @@ def test_adam_amsgrad_impulse_closed_form(api, oracle):
     assert sorted(steps.tolist()) == [3, 5, 6]
 
 
-@pytest.mark.parametrize("dim", [32, 64, 128])
+@pytest.mark.parametrize("dim", [20, 32, 36, 64, 100, 124, 128])
 def test_wide_rows_pull_every_path(api, oracle, dim):
     """Rows of 32 to 128 floats are pulled by kernels of their own (sixteen ids looked up per
     wavefront, then copied by lane groups of dim / 4 lanes). Against the oracle: request sizes on
