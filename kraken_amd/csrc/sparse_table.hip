@@ -2038,6 +2038,8 @@ int32_t krk_sparse_select_routed(krk_sparse* t, uint64_t table_id, const uint64_
 // runs on the null stream.
 static std::mutex g_route_mu;
 static DeviceBuffer g_route_pool;
+static char* g_route_pinned = nullptr;      // page-locked staging for the ring and the counts
+static size_t g_route_pinned_bytes = 0;
 
 int32_t krk_route_ids(uint64_t table_id, const uint64_t* ring_hash, const uint64_t* ring_node, int64_t ring_n,
                       const uint64_t* ids, int64_t n, uint64_t* owner, int64_t* perm, uint64_t* node_ids,
@@ -2116,9 +2118,21 @@ int32_t krk_route_ids(uint64_t table_id, const uint64_t* ring_hash, const uint64
     KRK_HIP(hipMemcpy(s_ids, ids, (size_t)n * 8, hipMemcpyHostToDevice));
     d_ids = s_ids;
   }
-  KRK_HIP(hipMemcpy(d_ring_hash, ring_hash, (size_t)ring_n * 8, hipMemcpyHostToDevice));
-  KRK_HIP(hipMemcpy(d_ring_rank, ring_rank.data(), (size_t)ring_n * 4, hipMemcpyHostToDevice));
-  KRK_HIP(hipMemcpy(d_nodes, nodes.data(), (size_t)m * 8, hipMemcpyHostToDevice));
+  // the ring, its ranks and the node list travel in one copy out of page-locked memory, and the
+  // counts come back the same way: the call waits for the stream once
+  const size_t up_b = ring_hash_b + ring_rank_b + nodes_b;
+  if (g_route_pinned_bytes < up_b + count_b) {
+    if (g_route_pinned) (void)hipHostFree(g_route_pinned);
+    g_route_pinned = nullptr;
+    g_route_pinned_bytes = 0;
+    KRK_HIP(hipHostMalloc((void**)&g_route_pinned, 2 * (up_b + count_b), hipHostMallocDefault));
+    g_route_pinned_bytes = 2 * (up_b + count_b);
+  }
+  std::memcpy(g_route_pinned, ring_hash, (size_t)ring_n * 8);
+  std::memcpy(g_route_pinned + ring_hash_b, ring_rank.data(), (size_t)ring_n * 4);
+  std::memcpy(g_route_pinned + ring_hash_b + ring_rank_b, nodes.data(), (size_t)m * 8);
+  int32_t* h_count = reinterpret_cast<int32_t*>(g_route_pinned + up_b);
+  KRK_HIP(hipMemcpyAsync(d_ring_hash, g_route_pinned, up_b, hipMemcpyHostToDevice, st));
   KRK_HIP(hipMemsetAsync(d_count, 0, (size_t)m * 4, st));
   hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, st, d_ids, n,
                      (unsigned long long)route_hash64(table_id), d_ring_hash, d_ring_rank, (int)ring_n, d_nodes,
@@ -2127,14 +2141,13 @@ int32_t krk_route_ids(uint64_t table_id, const uint64_t* ring_hash, const uint64
   KRK_TRY(exclusive_scan_i32(d_bc, d_bc, m * blocks, d_total, d_scan, st));
   hipLaunchKernelGGL(route_scatter_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, st, d_rank8, n, d_bc, d_perm);
   KRK_HIP(hipGetLastError());
-  std::vector<int32_t> h_count((size_t)m);
-  KRK_HIP(hipMemcpy(h_count.data(), d_count, (size_t)m * 4, hipMemcpyDeviceToHost));
-  for (int64_t k = 0; k < m; ++k) counts[k] = h_count[(size_t)k];
+  KRK_HIP(hipMemcpyAsync(h_count, d_count, (size_t)m * 4, hipMemcpyDeviceToHost, st));
   if (host) {
     if (owner) KRK_HIP(hipMemcpy(owner, d_owner, (size_t)n * 8, hipMemcpyDeviceToHost));
     KRK_HIP(hipMemcpy(perm, d_perm, (size_t)n * 8, hipMemcpyDeviceToHost));
   }
   KRK_HIP(hipStreamSynchronize(st));
+  for (int64_t k = 0; k < m; ++k) counts[k] = h_count[k];
   return KRK_SUCCESS;
 }
 

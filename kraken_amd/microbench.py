@@ -9,6 +9,7 @@ the program the rocprofv3 summaries of the individual kernels are taken from.
 """
 import gc
 import sys
+import time
 
 import numpy as np
 
@@ -315,6 +316,56 @@ def dct():
         back.free()
 
 
+def hooks():
+    print("# routing on the device: a ring of 8 nodes x 64 virtual nodes (blocking calls, device ids)")
+    rng = np.random.default_rng(3)
+    hashes = np.sort(rng.integers(0, 1 << 63, size=8 * 64, dtype=np.uint64) * np.uint64(2))
+    ring = [(int(h), int(i % 8)) for i, h in enumerate(hashes)]
+    for n in (98_600, 1_000_000):
+        d_ids = api.DeviceArray.from_host(splitmix64(np.arange(n, dtype=np.uint64)))
+        rh = np.ascontiguousarray([h for h, _ in ring], dtype=np.uint64)
+        rn = np.ascontiguousarray([i for _, i in ring], dtype=np.uint64)
+        owner, perm = api.DeviceArray(n, np.uint64), api.DeviceArray(n, np.int64)
+        node_ids, counts, m = np.empty(8, np.uint64), np.empty(8, np.int64), api.C.c_int64()
+
+        def call():
+            rc = api.lib().krk_route_ids(7, api._ptr(rh), api._ptr(rn), len(ring), api._ptr(d_ids), n,
+                                         api._ptr(owner), api._ptr(perm), api._ptr(node_ids), api._ptr(counts), 8,
+                                         api.C.byref(m), api.DEVICE_PTRS)
+            assert rc == 0 and m.value == 8
+        call()
+        t0 = time.perf_counter()
+        reps = 10
+        for _ in range(reps):
+            call()
+        dt = (time.perf_counter() - t0) / reps
+        owner.free()
+        perm.free()
+        print("route %8d ids to their nodes (owner per id, stable partition) %8.1f us" % (n, dt * 1e6), flush=True)
+        d_ids.free()
+    init = api.Initializer.create(api.InitializerType.kConstant, {"value": "0"})
+    rows = 10_000_000
+    t = api.SparseTable(16, init, capacity_hint=rows)
+    prefill(t, rows, 16)
+    rh = np.ascontiguousarray([h for h, _ in ring], dtype=np.uint64)
+    rn = np.ascontiguousarray([i for _, i in ring], dtype=np.uint64)
+    d_sel, count = api.DeviceArray(rows, np.uint64), api.C.c_int64()
+
+    def select():
+        rc = api.lib().krk_sparse_select_routed(t.h, 7, api._ptr(rh), api._ptr(rn), len(ring), 3, 1, api._ptr(d_sel),
+                                                rows, api.C.byref(count), api.DEVICE_PTRS)
+        assert rc == 0
+    select()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        select()
+    dt = (time.perf_counter() - t0) / 5
+    print("select the rows of one node among %d rows (%d selected, ids left on the device) %8.1f us" % (
+        rows, count.value, dt * 1e6), flush=True)
+    d_sel.free()
+    t.close()
+
+
 def copy():
     nbytes = 1 << 30
     a, b = api.DeviceArray(nbytes // 4, np.float32), api.DeviceArray(nbytes // 4, np.float32)
@@ -323,7 +374,7 @@ def copy():
     print("# plain copy of 1 GiB: %.1f us, %.0f GB/s read + write" % (dt * 1e6, 2 * nbytes / dt / 1e9), flush=True)
 
 
-SECTIONS = {"copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct}
+SECTIONS = {"copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct, "hooks": hooks}
 
 
 def main(argv):
