@@ -32,7 +32,7 @@ FAMILIES = [[(3, {}), (0, {}), (1, {}), (2, {"momentum": 0.5})],
 
 @pytest.mark.parametrize("seed", range(120))
 def test_random_operation_sequences(api, oracle, tmp_path, seed):
-    _table_sequence(api, oracle, tmp_path, seed, [4, 5, 16, 32, 72])
+    _table_sequence(api, oracle, tmp_path, seed, [4, 5, 16, 32, 64, 72, 128])
 
 
 @pytest.mark.parametrize("seed", range(12))
