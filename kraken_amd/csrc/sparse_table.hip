@@ -724,6 +724,30 @@ __host__ __device__ inline unsigned long long route_hash64(unsigned long long v)
   return v;
 }
 
+// Rings of up to this many virtual nodes are searched in LDS (the same 512 or so entries are looked
+// at by every id: nine dependent reads that should not go to memory each time).
+constexpr int kRingLds = 2048;
+
+// First virtual node at or above `hv`, or the ring's first when hv lies above them all.
+__device__ __forceinline__ int ring_position(const unsigned long long* ring, int m, unsigned long long hv) {
+  int lo = 0, hi = m;
+  while (lo < hi) {
+    const int mid = lo + ((hi - lo) >> 1);
+    if (ring[mid] < hv) lo = mid + 1; else hi = mid;
+  }
+  return lo == m ? 0 : lo;
+}
+
+// the ring's hashes in LDS when they fit; every thread of the workgroup calls this
+__device__ __forceinline__ const unsigned long long* stage_ring(unsigned long long* lds,
+                                                                const unsigned long long* __restrict__ ring_hash,
+                                                                int m) {
+  if (m > kRingLds) return ring_hash;
+  for (int i = threadIdx.x; i < m; i += kBlock) lds[i] = ring_hash[i];
+  __syncthreads();
+  return lds;
+}
+
 // flag[r] = 1 where Router::Hit(utils::Hash(table_id, id of row r)) (common/router.cc:262-277,
 // common/utils.h:46-48) is node_id (want_owned) or another node (!want_owned). The ring is the
 // virtual nodes in ascending hash order: a hash belongs to the first one at or above it, or to
@@ -734,19 +758,16 @@ __global__ __launch_bounds__(kBlock) void route_flag_kernel(const unsigned long 
                                                             const unsigned long long* __restrict__ ring_node,
                                                             int m, unsigned long long node_id, bool want_owned,
                                                             int32_t* __restrict__ flag) {
-  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (r >= rows) return;
-  const unsigned long long hv = table_hash ^ route_hash64(row_key[r]);
-  unsigned long long owner = ~0ull;
-  if (m > 0) {
-    int lo = 0, hi = m;
-    while (lo < hi) {
-      const int mid = lo + ((hi - lo) >> 1);
-      if (ring_hash[mid] < hv) lo = mid + 1; else hi = mid;
-    }
-    owner = ring_node[lo == m ? 0 : lo];
+  __shared__ unsigned long long sring[kRingLds];
+  const unsigned long long* ring = stage_ring(sring, ring_hash, m);
+  // a workgroup walks several stretches of rows, so the ring is staged once for many rows
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x; r < rows; r += step) {
+    const unsigned long long hv = table_hash ^ route_hash64(__builtin_nontemporal_load(row_key + r));
+    unsigned long long owner = ~0ull;
+    if (m > 0) owner = ring_node[ring_position(ring, m, hv)];
+    flag[r] = ((owner == node_id) == want_owned) ? 1 : 0;
   }
-  flag[r] = ((owner == node_id) == want_owned) ? 1 : 0;
 }
 
 __global__ __launch_bounds__(kBlock) void route_emit_kernel(const unsigned long long* __restrict__ row_key,
@@ -772,17 +793,14 @@ __global__ __launch_bounds__(kBlock) void route_rank_kernel(const uint64_t* __re
                                                             int32_t* __restrict__ block_counts,
                                                             int32_t* __restrict__ node_count) {
   __shared__ int32_t hist[kRouteMaxNodes];
+  __shared__ unsigned long long sring[kRingLds];
   if ((int)threadIdx.x < nodes) hist[threadIdx.x] = 0;
+  const unsigned long long* ring = stage_ring(sring, ring_hash, m);
   __syncthreads();
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p < n) {
     const unsigned long long hv = table_hash ^ route_hash64(ids[p]);
-    int lo = 0, hi = m;
-    while (lo < hi) {
-      const int mid = lo + ((hi - lo) >> 1);
-      if (ring_hash[mid] < hv) lo = mid + 1; else hi = mid;
-    }
-    const uint32_t k = ring_rank[lo == m ? 0 : lo];
+    const uint32_t k = ring_rank[ring_position(ring, m, hv)];
     rank8[p] = (uint8_t)k;
     if (owner) owner[p] = node_of_rank[k];
     atomicAdd(&hist[k], 1);
@@ -2010,7 +2028,9 @@ int32_t krk_sparse_select_routed(krk_sparse* t, uint64_t table_id, const uint64_
     KRK_HIP(hipMemcpyAsync(d_ring_hash, ring_hash, (size_t)ring_n * 8, hipMemcpyHostToDevice, t->stream));
     KRK_HIP(hipMemcpyAsync(d_ring_node, ring_node, (size_t)ring_n * 8, hipMemcpyHostToDevice, t->stream));
   }
-  hipLaunchKernelGGL(route_flag_kernel, dim3(grid_for(rows, kBlock)), dim3(kBlock), 0, t->stream, t->row_key, rows,
+  // a few thousand workgroups that stride over the rows: each stages the ring once
+  const unsigned flag_grid = (unsigned)std::min<int64_t>(grid_for(rows, kBlock), 256 * 16);
+  hipLaunchKernelGGL(route_flag_kernel, dim3(flag_grid), dim3(kBlock), 0, t->stream, t->row_key, rows,
                      route_hash64(table_id), d_ring_hash, d_ring_node, (int)ring_n, (unsigned long long)node_id,
                      owned != 0, flag);
   KRK_HIP(hipGetLastError());
