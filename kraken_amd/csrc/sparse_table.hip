@@ -790,8 +790,7 @@ __global__ __launch_bounds__(kBlock) void route_rank_kernel(const uint64_t* __re
                                                             const unsigned long long* __restrict__ node_of_rank,
                                                             int nodes, unsigned long long* __restrict__ owner,
                                                             uint8_t* __restrict__ rank8,
-                                                            int32_t* __restrict__ block_counts,
-                                                            int32_t* __restrict__ node_count) {
+                                                            int32_t* __restrict__ block_counts) {
   __shared__ int32_t hist[kRouteMaxNodes];
   __shared__ unsigned long long sring[kRingLds];
   if ((int)threadIdx.x < nodes) hist[threadIdx.x] = 0;
@@ -806,11 +805,19 @@ __global__ __launch_bounds__(kBlock) void route_rank_kernel(const uint64_t* __re
     atomicAdd(&hist[k], 1);
   }
   __syncthreads();
-  if ((int)threadIdx.x < nodes) {
-    const int32_t c = hist[threadIdx.x];
-    block_counts[(int64_t)threadIdx.x * gridDim.x + blockIdx.x] = c;
-    if (c) atomicAdd(&node_count[threadIdx.x], c);
-  }
+  if ((int)threadIdx.x < nodes) block_counts[(int64_t)threadIdx.x * gridDim.x + blockIdx.x] = hist[threadIdx.x];
+}
+
+// node_count[k] = ids of node k, read off the scanned per-workgroup counts: where node k + 1's
+// ids begin minus where node k's do (thousands of workgroups adding to the same few counters
+// in memory cost more than the rest of the routing together).
+__global__ __launch_bounds__(kRouteMaxNodes) void route_counts_kernel(const int32_t* __restrict__ block_base,
+                                                                      int64_t blocks, int nodes, int32_t n,
+                                                                      int32_t* __restrict__ node_count) {
+  const int k = threadIdx.x;
+  if (k >= nodes) return;
+  const int32_t end = k + 1 < nodes ? block_base[(int64_t)(k + 1) * blocks] : n;
+  node_count[k] = end - block_base[(int64_t)k * blocks];
 }
 
 // perm[where node k's ids begin + ids of node k in earlier workgroups + earlier in this one] = p:
@@ -2060,6 +2067,8 @@ static std::mutex g_route_mu;
 static DeviceBuffer g_route_pool;
 static char* g_route_pinned = nullptr;      // page-locked staging for the ring and the counts
 static size_t g_route_pinned_bytes = 0;
+static std::vector<char> g_route_last;        // the ring block the device holds ...
+static const void* g_route_on_device = nullptr;   // ... and where (null: nothing usable there)
 
 int32_t krk_route_ids(uint64_t table_id, const uint64_t* ring_hash, const uint64_t* ring_node, int64_t ring_n,
                       const uint64_t* ids, int64_t n, uint64_t* owner, int64_t* perm, uint64_t* node_ids,
@@ -2116,13 +2125,16 @@ int32_t krk_route_ids(uint64_t table_id, const uint64_t* ring_hash, const uint64
   const size_t scan_b = r256(scan_scratch_bytes(m * blocks));
   const size_t n8 = r256((size_t)n * 8);
   std::lock_guard<std::mutex> pool_lock(g_route_mu);
-  KRK_TRY(g_route_pool.reserve(ring_hash_b + ring_rank_b + nodes_b + count_b + rank8_b + bc_b + scan_b + 256 +
-                               (host ? 3 * n8 : 0)));
+  const size_t pool_before = g_route_pool.bytes;
+  const int32_t pool_rc = g_route_pool.reserve(ring_hash_b + ring_rank_b + nodes_b + count_b + rank8_b + bc_b +
+                                               scan_b + 256 + (host ? 3 * n8 : 0));
+  if (g_route_pool.bytes != pool_before || pool_rc != KRK_SUCCESS) g_route_on_device = nullptr;   // a new allocation
+  KRK_TRY(pool_rc);
   char* cur = g_route_pool.as<char>();
   unsigned long long* d_ring_hash = reinterpret_cast<unsigned long long*>(cur); cur += ring_hash_b;
   uint32_t* d_ring_rank = reinterpret_cast<uint32_t*>(cur); cur += ring_rank_b;
   unsigned long long* d_nodes = reinterpret_cast<unsigned long long*>(cur); cur += nodes_b;
-  int32_t* d_count = reinterpret_cast<int32_t*>(cur); cur += count_b;
+  cur += count_b;
   uint8_t* d_rank8 = reinterpret_cast<uint8_t*>(cur); cur += rank8_b;
   int32_t* d_bc = reinterpret_cast<int32_t*>(cur); cur += bc_b;
   void* d_scan = cur; cur += scan_b;
@@ -2138,35 +2150,50 @@ int32_t krk_route_ids(uint64_t table_id, const uint64_t* ring_hash, const uint64
     KRK_HIP(hipMemcpy(s_ids, ids, (size_t)n * 8, hipMemcpyHostToDevice));
     d_ids = s_ids;
   }
-  // the ring, its ranks and the node list travel in one copy out of page-locked memory, and the
-  // counts come back the same way: the call waits for the stream once
+  // The ring, its ranks and the node list travel in one copy out of page-locked memory, and only
+  // when they differ from what the last call left on the device (rings change with the
+  // cluster's membership, not between requests). The counts are written by the device straight
+  // into page-locked memory: the call waits for the stream once and copies nothing back.
   const size_t up_b = ring_hash_b + ring_rank_b + nodes_b;
   if (g_route_pinned_bytes < up_b + count_b) {
     if (g_route_pinned) (void)hipHostFree(g_route_pinned);
     g_route_pinned = nullptr;
     g_route_pinned_bytes = 0;
+    g_route_on_device = nullptr;
     KRK_HIP(hipHostMalloc((void**)&g_route_pinned, 2 * (up_b + count_b), hipHostMallocDefault));
     g_route_pinned_bytes = 2 * (up_b + count_b);
   }
-  std::memcpy(g_route_pinned, ring_hash, (size_t)ring_n * 8);
-  std::memcpy(g_route_pinned + ring_hash_b, ring_rank.data(), (size_t)ring_n * 4);
-  std::memcpy(g_route_pinned + ring_hash_b + ring_rank_b, nodes.data(), (size_t)m * 8);
+  const bool same_ring = g_route_on_device == (const void*)d_ring_hash && g_route_last.size() == up_b &&
+                         std::memcmp(g_route_last.data(), ring_hash, (size_t)ring_n * 8) == 0 &&
+                         std::memcmp(g_route_last.data() + ring_hash_b, ring_rank.data(), (size_t)ring_n * 4) == 0 &&
+                         std::memcmp(g_route_last.data() + ring_hash_b + ring_rank_b, nodes.data(), (size_t)m * 8) == 0;
   int32_t* h_count = reinterpret_cast<int32_t*>(g_route_pinned + up_b);
-  KRK_HIP(hipMemcpyAsync(d_ring_hash, g_route_pinned, up_b, hipMemcpyHostToDevice, st));
-  KRK_HIP(hipMemsetAsync(d_count, 0, (size_t)m * 4, st));
+  int32_t* d_count = nullptr;
+  KRK_HIP(hipHostGetDevicePointer((void**)&d_count, h_count, 0));
+  if (!same_ring) {
+    g_route_on_device = nullptr;
+    g_route_last.assign(up_b, 0);
+    std::memcpy(g_route_last.data(), ring_hash, (size_t)ring_n * 8);
+    std::memcpy(g_route_last.data() + ring_hash_b, ring_rank.data(), (size_t)ring_n * 4);
+    std::memcpy(g_route_last.data() + ring_hash_b + ring_rank_b, nodes.data(), (size_t)m * 8);
+    std::memcpy(g_route_pinned, g_route_last.data(), up_b);
+    KRK_HIP(hipMemcpyAsync(d_ring_hash, g_route_pinned, up_b, hipMemcpyHostToDevice, st));
+  }
   hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, st, d_ids, n,
                      (unsigned long long)route_hash64(table_id), d_ring_hash, d_ring_rank, (int)ring_n, d_nodes,
-                     (int)m, d_owner, d_rank8, d_bc, d_count);
+                     (int)m, d_owner, d_rank8, d_bc);
   KRK_HIP(hipGetLastError());
   KRK_TRY(exclusive_scan_i32(d_bc, d_bc, m * blocks, d_total, d_scan, st));
+  hipLaunchKernelGGL(route_counts_kernel, dim3(1), dim3(kRouteMaxNodes), 0, st, d_bc, blocks, (int)m, (int32_t)n,
+                     d_count);
   hipLaunchKernelGGL(route_scatter_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, st, d_rank8, n, d_bc, d_perm);
   KRK_HIP(hipGetLastError());
-  KRK_HIP(hipMemcpyAsync(h_count, d_count, (size_t)m * 4, hipMemcpyDeviceToHost, st));
   if (host) {
     if (owner) KRK_HIP(hipMemcpy(owner, d_owner, (size_t)n * 8, hipMemcpyDeviceToHost));
     KRK_HIP(hipMemcpy(perm, d_perm, (size_t)n * 8, hipMemcpyDeviceToHost));
   }
   KRK_HIP(hipStreamSynchronize(st));
+  g_route_on_device = d_ring_hash;   // only now: a call that failed above leaves the ring to be sent again
   for (int64_t k = 0; k < m; ++k) counts[k] = h_count[k];
   return KRK_SUCCESS;
 }

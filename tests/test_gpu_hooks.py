@@ -224,8 +224,21 @@ def test_route_ids_partitions_a_request_like_the_worker(api, oracle):
         assert np.array_equal(perm, want_perm) and np.array_equal(d_perm.to_host()[:ids.size], want_perm)
         assert counts.tolist() == np.bincount(rank, minlength=node_ids.size).tolist() == d_counts.tolist()
         assert counts.sum() == ids.size
-    # errors: an unsorted ring, too little room for the nodes, an empty ring with ids to route
+    # the library keeps the last ring on the device: a ring of the same hashes whose virtual nodes
+    # changed hands, then the first one again, must each be answered for themselves
     ring = [(int(h), int(n)) for h, n in cases[0]["ring"]]
+    nodes = sorted(set(n for _, n in ring))
+    if len(nodes) > 1:
+        moved = [(h, nodes[(nodes.index(n) + 1) % len(nodes)]) for h, n in ring]
+        ids = splitmix64(np.arange(99, 99 + 30_000, dtype=np.uint64))
+        for r in (ring, moved, moved, ring):
+            node_ids, counts, owner, perm = api.route_ids(5, r, ids)
+            want_owner = oracle.route_owners(r, 5, ids)
+            assert np.array_equal(owner, want_owner)
+            assert counts.tolist() == np.bincount(np.searchsorted(node_ids, want_owner),
+                                                  minlength=node_ids.size).tolist()
+        assert not np.array_equal(oracle.route_owners(ring, 5, ids), oracle.route_owners(moved, 5, ids))
+    # errors: an unsorted ring, too little room for the nodes, an empty ring with ids to route
     with pytest.raises(api.KrakenHipError):
         api.route_ids(1, [(9, 0), (5, 1)], np.arange(4, dtype=np.uint64))
     with pytest.raises(api.KrakenHipError):
