@@ -37,23 +37,49 @@ __global__ void dct2_basis_kernel(float* __restrict__ fwd, float* __restrict__ i
   inv[k * kDctB + j] = (float)v;
 }
 
-// Y[M, N] = X[M, K] * Bm[K, N]; ldx / ldb / ldy are row strides in floats. K is a multiple of 32,
+// Y[M, N] = X[M, K] * Bm[K, N]; ldx / ldb / ldy are row strides in floats. K is a multiple of 64,
 // N a multiple of 32 * NT. grid.x workgroups share the row tiles, grid.y = N / (32 * NT).
 //
-// The basis tile [K][32 * NT] sits in LDS for the whole launch and is only read. X never
+// The basis tile sits in LDS for the whole launch and is only read. It is laid out
+// [K + kPadRows][32][NT]: the NT values a lane needs for one step (columns r, r + 32, ...) are one
+// vector read, at an offset from the slice's first row that is known at compile time. X never
 // passes through LDS: the matrix instruction takes, per lane (r = lane % 32, h = lane / 32),
 // one value A[r][k_h] for its two reduction indices k_0, k_1, and the order in which the
 // reduction indices are consumed is free as long as the basis rows follow it. So lane (r, h)
 // loads the 16 consecutive floats X[row r][32 s + 16 h ...] of slice s as four float4 and
 // step j multiplies them against basis rows 32 s + 16 h + j. Wavefronts never wait on each
 // other inside the loop; the next slice's loads are in flight while this one multiplies.
+//
+// A tile's results are not stored when the tile is done: the two wavefronts that share a SIMD
+// run in step, so both would store while the matrix pipe idles (10 % of the kernel's time).
+// They are kept in registers and leave between the multiplies of the next tile's first two
+// slices, two (NT = 4) or one (NT = 2) store a step; the last tile's follow the loop.
+constexpr int kPadRows = 17;   // the step after a tile's last one still reads "its" basis rows
+
+template <int NT>
+struct BasisVec;
+template <>
+struct BasisVec<4> {
+  typedef float type __attribute__((ext_vector_type(4)));
+};
+template <>
+struct BasisVec<2> {
+  typedef float type __attribute__((ext_vector_type(2)));
+};
+
+template <int V>
+struct IntTag {
+  static constexpr int value = V;
+};
+
 template <int NT>
 __global__ __launch_bounds__(kThreads) void dct2_gemm_kernel(const float* __restrict__ X, int64_t ldx,
                                                              const float* __restrict__ Bm, int ldb,
                                                              float* __restrict__ Y, int64_t ldy,
                                                              int64_t M, int K) {
+  typedef typename BasisVec<NT>::type bvec;
   constexpr int kTileN = 32 * NT;
-  extern __shared__ float Bs[];                     // [K][kTileN]
+  extern __shared__ float Bs[];                     // [K + kPadRows][32][NT]
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -64,12 +90,18 @@ __global__ __launch_bounds__(kThreads) void dct2_gemm_kernel(const float* __rest
   for (int i = tid; i < K * (kTileN / 4); i += kThreads) {
     const int br = i / (kTileN / 4);
     const int c4 = i - br * (kTileN / 4);
-    reinterpret_cast<float4*>(Bs)[i] = *reinterpret_cast<const float4*>(Bm + (size_t)br * ldb + n0 + c4 * 4);
+    const float4 v = *reinterpret_cast<const float4*>(Bm + (size_t)br * ldb + n0 + c4 * 4);
+    const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = c4 * 4 + u;                     // column c of the tile is (r, t) = (c % 32, c / 32)
+      Bs[br * kTileN + (c & 31) * NT + (c >> 5)] = e[u];
+    }
   }
   __syncthreads();
 
   const int64_t tiles = (M + kTileM - 1) / kTileM;
-  const int slices = K / kSliceK;
+  const int slices = K / kSliceK;                   // at least two
   // Rows past the end are clamped, not masked: row r of X only reaches row r of Y, and those
   // rows are never stored, so the loads carry no branch.
   auto row_ptr = [&](int64_t tile) {
@@ -77,67 +109,86 @@ __global__ __launch_bounds__(kThreads) void dct2_gemm_kernel(const float* __rest
     if (row >= M) row = M - 1;
     return X + row * ldx + 16 * h;
   };
-  const float* bs = Bs + (size_t)(16 * h) * kTileN + r;
+  const float* bs = Bs + (size_t)(16 * h) * kTileN + r * NT;
   const float* xrow = row_ptr(blockIdx.x);
-  // X runs two slices ahead of the multiplies (K >= 64, so a tile has at least two slices).
+  // X runs two slices ahead of the multiplies.
   float4 cur[4], nx1[4], nx2[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     cur[q] = reinterpret_cast<const float4*>(xrow)[q];
     nx1[q] = reinterpret_cast<const float4*>(xrow + kSliceK)[q];
   }
+  v16f acc[NT], prev[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) prev[t] = v16f{0};
+  int64_t prev_base = M;                            // first row of the tile prev holds: none yet
+  bvec bcur, bnxt;
+
+  // accumulator element i of lane l is C[(i / 4) * 8 + (l / 32) * 4 + i % 4][l % 32]
+  auto store_prev = [&](int i, int t) {
+    const int64_t orow = prev_base + (i >> 2) * 8 + h * 4 + (i & 3);
+    if (orow < M) Y[orow * ldy + n0 + r + 32 * t] = prev[t][i];
+  };
+
+  // One reduction slice: 16 steps of NT multiplies. STORE 0 / 1: the first / second half of the
+  // previous tile's results leaves between the multiplies; -1: nothing to store.
+  auto slice = [&](auto store_tag, int s, const float* xnext) {
+    constexpr int STORE = decltype(store_tag)::value;
+    // slice s + 2 of this tile, or one of the first two slices of the next tile
+    const float* ahead = s + 2 < slices ? xrow + (s + 2) * kSliceK : xnext + (s + 2 - slices) * kSliceK;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) nx2[q] = reinterpret_cast<const float4*>(ahead)[q];
+    __builtin_amdgcn_sched_barrier(0);              // keep the requests ahead of the multiplies
+    const float* brow = bs + (size_t)s * kSliceK * kTileN;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float a4[4] = {cur[q].x, cur[q].y, cur[q].z, cur[q].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int j = q * 4 + e;
+        // basis values of the following step are requested before this step multiplies: row j + 1
+        // of this slice, or row 0 of the next one (past the last slice: padding, never used)
+        bnxt = *reinterpret_cast<const bvec*>(brow + (j < 15 ? (j + 1) * kTileN : kSliceK * kTileN));
+        if constexpr (STORE >= 0) {
+          constexpr int kPerStep = NT / 2;
+#pragma unroll
+          for (int u = 0; u < kPerStep; ++u) {
+            const int idx = (STORE * 16 + j) * kPerStep + u;
+            store_prev(idx / NT, idx % NT);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[e], bcur[t], acc[t], 0, 0, 0);
+        bcur = bnxt;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      cur[q] = nx1[q];
+      nx1[q] = nx2[q];
+    }
+  };
+
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
     // the tile after this one (or this one again at the end: its values are then unused)
     const float* xnext = row_ptr(tile + gridDim.x < tiles ? tile + gridDim.x : tile);
-    v16f acc[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[t] = v16f{0};
-    float bcur[NT], bnxt[NT];
+    bcur = *reinterpret_cast<const bvec*>(bs);
+    slice(IntTag<0>{}, 0, xnext);
+    slice(IntTag<1>{}, 1, xnext);
+    for (int s = 2; s < slices; ++s) slice(IntTag<-1>{}, s, xnext);
 #pragma unroll
-    for (int t = 0; t < NT; ++t) bcur[t] = bs[32 * t];
-    for (int s = 0; s < slices; ++s) {
-      // slice s + 2 of this tile, or one of the first two slices of the next tile
-      const float* ahead = s + 2 < slices ? xrow + (s + 2) * kSliceK : xnext + (s + 2 - slices) * kSliceK;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) nx2[q] = reinterpret_cast<const float4*>(ahead)[q];
-      __builtin_amdgcn_sched_barrier(0);   // keep the requests ahead of the multiplies
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const float a4[4] = {cur[q].x, cur[q].y, cur[q].z, cur[q].w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          // basis values of the following step are requested before this step multiplies
-          const int step = s * 16 + q * 4 + e + 1;
-          const float* brow = bs + (size_t)((step >> 4) * kSliceK + (step & 15)) * kTileN;
-          const bool more = step < slices * 16;
-#pragma unroll
-          for (int t = 0; t < NT; ++t) bnxt[t] = brow[more ? 32 * t : 32 * t - kSliceK * kTileN];
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int t = 0; t < NT; ++t)
-            acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[e], bcur[t], acc[t], 0, 0, 0);
-#pragma unroll
-          for (int t = 0; t < NT; ++t) bcur[t] = bnxt[t];
-        }
-      }
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        cur[q] = nx1[q];
-        nx1[q] = nx2[q];
-      }
-    }
-    // accumulator element i of lane l is C[(i / 4) * 8 + (l / 32) * 4 + i % 4][l % 32]
-    const int64_t base = tile * kTileM + wave * 32;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int64_t orow = base + (i >> 2) * 8 + h * 4 + (i & 3);
-      if (orow < M) {
-        float* y = Y + orow * ldy + n0 + r;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) y[32 * t] = acc[t][i];
-      }
-    }
+    for (int t = 0; t < NT; ++t) prev[t] = acc[t];
+    prev_base = tile * kTileM + wave * 32;
     xrow = xnext;
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) store_prev(i, t);
   }
 }
 
@@ -194,9 +245,9 @@ static int32_t dct2_run(const float* in, float* out, int64_t n, int32_t keep, ui
   const float* basis = forward ? g_basis_fwd : g_basis_inv;
   const int nt = (N % 128 == 0) ? 4 : 2;          // 128-column tiles where the width allows
   const int tile_n = 32 * nt;
-  const size_t lds_bytes = sizeof(float) * (size_t)K * tile_n;
+  const size_t lds_bytes = sizeof(float) * (size_t)(K + kPadRows) * tile_n;
   const int64_t tiles = (M + kTileM - 1) / kTileM;
-  const int64_t per_cu = lds_bytes <= 64 * 1024 ? 2 : 1;   // workgroups that fit one CU's LDS
+  const int64_t per_cu = lds_bytes <= 80 * 1024 ? 2 : 1;   // workgroups that fit one CU's 160 KB of LDS
   int64_t gx = 256 * per_cu / (N / tile_n);
   if (gx > tiles) gx = tiles;
   if (gx < 1) gx = 1;
