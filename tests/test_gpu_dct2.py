@@ -79,6 +79,25 @@ def test_device_pointers_and_arguments(dct2):
         dct2.forward(x, 50)
 
 
+@pytest.mark.parametrize("keep", [64, 128, 192, 256])
+def test_several_tiles_per_workgroup_and_a_ragged_end(dct2, keep):
+    """70 001 blocks: workgroups walk two or three row tiles each (a tile's results are stored
+    while the next one is multiplied, the last one's after the loop) and the last tile holds 113
+    rows. Every block against scipy, forward and back; keep 192 takes three column tiles."""
+    fft = pytest.importorskip("scipy.fft")
+    rng = np.random.default_rng(1000 + keep)
+    blocks = 70_001
+    x = rng.standard_normal(blocks * 256).astype(np.float32)
+    got = dct2.forward(x, keep)
+    want = _ref(x, keep)
+    scale = np.linalg.norm(x.reshape(-1, 256).astype(np.float64), axis=1, keepdims=True)
+    assert (np.abs(got - want) <= 1e-5 * scale + 1e-7).all()
+    pad = np.zeros((blocks, 256))
+    pad[:, :keep] = want
+    back = dct2.inverse(got, blocks * 256, keep).reshape(-1, 256)
+    assert (np.abs(back - fft.idct(pad, type=2, norm="ortho", axis=1)) <= 1e-5 * scale + 1e-7).all()
+
+
 @pytest.mark.parametrize("keep", [64, 256])
 def test_config_size_tensor(dct2, keep):
     """The configuration's own shape, fp32 [4096, 16384] of N(0, 1) = 262144 blocks: scipy on a
