@@ -738,14 +738,15 @@ __device__ __forceinline__ int ring_position(const unsigned long long* ring, int
   return lo == m ? 0 : lo;
 }
 
-// the ring's hashes in LDS when they fit; every thread of the workgroup calls this
-__device__ __forceinline__ const unsigned long long* stage_ring(unsigned long long* lds,
-                                                                const unsigned long long* __restrict__ ring_hash,
-                                                                int m) {
-  if (m > kRingLds) return ring_hash;
+// the ring's hashes into LDS when they fit (-> true); every thread of the workgroup calls this.
+// The callers search `lds` or `ring_hash` by name, each in its own branch: through one pointer
+// that may be either, every read of the search would be a flat access instead of an LDS read.
+__device__ __forceinline__ bool stage_ring(unsigned long long* lds, const unsigned long long* __restrict__ ring_hash,
+                                           int m) {
+  if (m > kRingLds) return false;
   for (int i = threadIdx.x; i < m; i += kBlock) lds[i] = ring_hash[i];
   __syncthreads();
-  return lds;
+  return true;
 }
 
 // flag[r] = 1 where Router::Hit(utils::Hash(table_id, id of row r)) (common/router.cc:262-277,
@@ -759,13 +760,13 @@ __global__ __launch_bounds__(kBlock) void route_flag_kernel(const unsigned long 
                                                             int m, unsigned long long node_id, bool want_owned,
                                                             int32_t* __restrict__ flag) {
   __shared__ unsigned long long sring[kRingLds];
-  const unsigned long long* ring = stage_ring(sring, ring_hash, m);
+  const bool in_lds = stage_ring(sring, ring_hash, m);
   // a workgroup walks several stretches of rows, so the ring is staged once for many rows
   const int64_t step = (int64_t)gridDim.x * kBlock;
   for (int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x; r < rows; r += step) {
     const unsigned long long hv = table_hash ^ route_hash64(__builtin_nontemporal_load(row_key + r));
     unsigned long long owner = ~0ull;
-    if (m > 0) owner = ring_node[ring_position(ring, m, hv)];
+    if (m > 0) owner = ring_node[in_lds ? ring_position(sring, m, hv) : ring_position(ring_hash, m, hv)];
     flag[r] = ((owner == node_id) == want_owned) ? 1 : 0;
   }
 }
@@ -794,12 +795,12 @@ __global__ __launch_bounds__(kBlock) void route_rank_kernel(const uint64_t* __re
   __shared__ int32_t hist[kRouteMaxNodes];
   __shared__ unsigned long long sring[kRingLds];
   if ((int)threadIdx.x < nodes) hist[threadIdx.x] = 0;
-  const unsigned long long* ring = stage_ring(sring, ring_hash, m);
+  const bool in_lds = stage_ring(sring, ring_hash, m);
   __syncthreads();
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p < n) {
     const unsigned long long hv = table_hash ^ route_hash64(ids[p]);
-    const uint32_t k = ring_rank[ring_position(ring, m, hv)];
+    const uint32_t k = ring_rank[in_lds ? ring_position(sring, m, hv) : ring_position(ring_hash, m, hv)];
     rank8[p] = (uint8_t)k;
     if (owner) owner[p] = node_of_rank[k];
     atomicAdd(&hist[k], 1);
