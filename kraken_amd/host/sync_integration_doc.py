@@ -1,6 +1,6 @@
-"""Copies the adapters of kraken_ref_tables.h (between its integration markers) into
-INTEGRATION.md, between the document's own markers, so that the document prints the code that is
-compiled against the reference's interface and not a second typing of it.
+"""Copies the adapters of kraken_ref_tables.h (between its integration markers) into the
+repository's integration notes, between that document's own markers, so that it prints the code
+that is compiled against the reference's interface and not a second typing of it.
 
     python kraken_amd/host/sync_integration_doc.py
 """

@@ -47,7 +47,7 @@ def test_adapters_compile_against_the_reference_interface_and_fail_softly_withou
 
 
 def test_integration_document_prints_the_compiled_adapters():
-    """INTEGRATION.md shows the adapters as they are compiled, not a second typing of them."""
+    """The integration notes show the adapters as they are compiled, not a second typing of them."""
     src = open(os.path.join(ROOT, "kraken_amd", "host", "kraken_ref_tables.h")).read()
     body = src[src.index("// [integration:begin]") + len("// [integration:begin]"):src.index("// [integration:end]")]
     doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
