@@ -184,6 +184,18 @@ def test_coo_to_dense_large_tensors(api, oracle, n):
     check(rng.permutation(quarter), rng.standard_normal(quarter.size))          # not ascending
     twice = np.sort(np.concatenate([quarter[:1000], quarter[:1000], quarter[5000:6000]]))
     check(twice, (rng.integers(-8, 9, size=twice.size) / 8.0))    # repeats add up (exact sums)
+    # device indices that start 8 bytes into a 16-byte unit (a view into a larger buffer)
+    import ctypes as C
+    val = rng.standard_normal(quarter.size).astype(np.float32)
+    shifted = api.DeviceArray.from_host(np.concatenate([[0], quarter]).astype(np.int64))
+    d_val = api.DeviceArray.from_host(val)
+    out = api.DeviceArray(n, np.float32)
+    rc = api.lib().krk_coo_to_dense(C.c_void_p(shifted.ptr + 8), C.c_void_p(d_val.ptr), quarter.size,
+                                    C.c_void_p(out.ptr), n, api.DEVICE_PTRS)
+    assert rc == 0
+    want = np.zeros(n, np.float32)
+    want[quarter] = val
+    assert np.array_equal(out.to_host(), want)
 
 
 def test_dense_push_coo_large(api, oracle):
