@@ -1,6 +1,6 @@
 """Per-kernel timings of the table engine at the sizes of the benchmark configurations.
 
-    python -m kraken_amd.microbench [copy] [tables] [raw] [combined] [host] [pooled] [codec] [dense] [dct2] [copy]
+    python -m kraken_amd.microbench [lines] [copy] [tables] [raw] [combined] [host] [pooled] [codec] [dense] [dct2] [hooks]
 
 Every figure is the average of back-to-back launches between two HIP events recorded on the
 stream the kernels run on, with inputs resident in HBM; bandwidths are algorithmic bytes
@@ -374,7 +374,39 @@ def copy():
     print("# plain copy of 1 GiB: %.1f us, %.0f GB/s read + write" % (dt * 1e6, 2 * nbytes / dt / 1e9), flush=True)
 
 
-SECTIONS = {"copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct, "hooks": hooks}
+def lines():
+    """Random 128-byte lines (krk_hbm_probe_lines) out of regions of growing size, twice: as the
+    launches come (a launch's lines then fall on pages that were not touched for a while), and
+    with four million lines of the same region touched just before each timed run, which leaves
+    the region's address translations in the GPU's translation caches."""
+    print("# random independent 128-byte lines out of the first R bytes of one 16 GiB allocation")
+    print("#   cold: launch after launch of n lines; warm: 4M lines of the region touched before the timed launches")
+    region_max = 1 << 34
+    big = api.DeviceArray(region_max // 4, np.float32)
+    api.lib().krk_memset(api._ptr(big), 1, region_max)
+    api.synchronize()
+    salt = [1]
+
+    def probe(rmw, region, n):
+        salt[0] += 1
+        rc = api.lib().krk_hbm_probe_lines(rmw, api._ptr(big), region, n, salt[0] * 0x9E3779B97F4A7C15 % (1 << 64))
+        assert rc == 0
+
+    for region in (1 << 25, 1 << 28, 1 << 30, 1 << 32, 1 << 34):
+        for n in (98_600, 1 << 20):
+            cells = []
+            for rmw in (0, 1):
+                cold = timed(None, lambda: probe(rmw, region, n), 10)
+                for _ in range(3):
+                    probe(0, region, 1 << 22)
+                warm = timed(None, lambda: probe(rmw, region, n), 10)
+                cells.append("%s cold %6.1f us warm %6.1f us %5.1f G lines/s" % (
+                    "read + write" if rmw else "read", cold * 1e6, warm * 1e6, n / warm / 1e9))
+            print("R %6d MB n %8d | %s | %s" % (region >> 20, n, cells[0], cells[1]), flush=True)
+    big.free()
+
+
+SECTIONS = {"lines": lines, "copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct, "hooks": hooks}
 
 
 def main(argv):
