@@ -36,7 +36,11 @@ HBM_PEAK_GBS = 8000.0
 # summarised in profiles/wide_deep_adagrad_d16_hbm_counters.md. Counters cannot be read from
 # inside this script, so the figure is carried here for the workload it was measured on.
 COUNTER_FIGURES = {"wide_deep": {"traffic": 45.4e6, "tcc_hit_rate": 0.456,
-                                 "source": "profiles/wide_deep_adagrad_d16_hbm_counters.md"}}
+                                 "source": "profiles/wide_deep_adagrad_d16_hbm_counters.md"},
+                   "dup_heavy": {"traffic": 144.4e6, "tcc_hit_rate": 0.552,
+                                 "source": "profiles/deepfm_and_dup_heavy_bench_lines.md"},
+                   "deepfm": {"traffic": 647.8e6, "tcc_hit_rate": 0.566,
+                              "source": "profiles/deepfm_and_dup_heavy_bench_lines.md"}}
 # the same for the dim 32 and dim 64 legs of the default workload (their push kernel)
 COUNTER_FIGURES_BY_DIM = {32: {"traffic": 77.0e6, "tcc_hit_rate": 0.504,
                                "source": "profiles/wide_deep_adagrad_d32_d64_hbm_counters.md"},
