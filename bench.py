@@ -9,17 +9,29 @@ unique id (Adagrad), then one dense Adam push. The default workload is the Wide&
 batch 8192 per table, Adagrad lr 0.05 with initial accumulator 0.1, plus a dense table of
 150 000 fp32 parameters under Adam.
 
+Timing: all timed blocks of K steps are enqueued back to back; HIP events recorded on the stream
+the sparse kernels run on separate the blocks (the last one after that stream has been made to
+wait for the dense table's), and the host waits once, at the end. `ms_per_step` is the median
+block's span / K, so it does not depend on how often the host drains the queue; the figure with a
+host drain after every block is carried as `ms_per_step_host_drained`.
+
 Prints ONE JSON line. `value` is unique rows pulled and pushed per second over the whole job.
 `roofline` prices the dominant kernel (the fused Adagrad push) at its algorithmic bytes,
-U * (8 + 4D + 16D) per launch, against 8 TB/s. `cpu_baseline` times the CPU oracle (a
-restatement of the reference's table path; the checker, never the product) on the host cores of
-the same machine on a bounded sample of the same workload.
+U * (8 + 4D + 16D) per launch, against 8 TB/s; `line_floor_us` next to every `us_per_launch` is
+what the kernel's count of random 128-byte lines costs at the line rates measured in the same
+run, plus one empty launch. `secondary` holds the other configurations (ids with their repeats at
+the worker boundary, DeepFM, the duplicate-heavy shape, the codec and the blockwise DCT), each
+with its own algorithmic bytes or flops. `cpu_baseline` times the CPU oracle (a restatement of
+the reference's table path; the checker, never the product) on the host cores of the same
+machine on a bounded sample of the same workload.
 """
 import argparse
 import concurrent.futures
 import gc
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -27,55 +39,68 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+from kraken_amd.workloads import WORKLOADS, make_batches, table_ids  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+T_START = time.perf_counter()
 
-# HBM bytes per launch of the dominant kernel from hardware counters (FETCH_SIZE and WRITE_SIZE,
-# each scaled by what it reads for the plain 1 GiB copy kernel); the runs and their commands are
-# summarised in profiles/wide_deep_adagrad_d16_hbm_counters.md. Counters cannot be read from
-# inside this script, so the figure is carried here for the workload it was measured on.
-COUNTER_FIGURES = {"wide_deep": {"traffic": 45.4e6, "tcc_hit_rate": 0.456,
-                                 "source": "profiles/wide_deep_adagrad_d16_hbm_counters.md"},
-                   "dup_heavy": {"traffic": 144.4e6, "tcc_hit_rate": 0.552,
-                                 "source": "profiles/deepfm_and_dup_heavy_bench_lines.md"},
-                   "deepfm": {"traffic": 647.8e6, "tcc_hit_rate": 0.566,
-                              "source": "profiles/deepfm_and_dup_heavy_bench_lines.md"}}
-# the same for the dim 32 and dim 64 legs of the default workload (their push kernel)
-COUNTER_FIGURES_BY_DIM = {32: {"traffic": 77.0e6, "tcc_hit_rate": 0.504,
-                               "source": "profiles/wide_deep_adagrad_d32_d64_hbm_counters.md"},
-                          64: {"traffic": 140.4e6, "tcc_hit_rate": 0.535,
-                               "source": "profiles/wide_deep_adagrad_d32_d64_hbm_counters.md"}}
-
-WORKLOADS = {
-    # name: tables, id space, zipf s, dim, ids per table per step, optimizer, dense params
-    "wide_deep": dict(tables=26, space=10**6, s=1.05, dim=16, batch=8192, optim="adagrad",
-                      dense=150_000, prefill=0),
-    "wide_deep_d32": dict(tables=26, space=10**6, s=1.05, dim=32, batch=8192, optim="adagrad",
-                          dense=150_000, prefill=0),
-    "deepfm": dict(tables=1, space=10**8, s=1.1, dim=32, batch=65536 * 39, optim="adam", dense=0,
-                   prefill=0),
-    "dup_heavy": dict(tables=1, space=2 * 10**7, s=1.3, dim=128, batch=131072 * 8, optim="rmsprop",
-                      dense=0, prefill=0),
-}
+# ---------------------------------------------------------------------------------------------
+# Figures that hardware counters gave for the dominant kernel (HBM bytes per launch from
+# FETCH_SIZE and WRITE_SIZE scaled by the plain copy kernel, L2 hit rate). Counters cannot be read
+# from inside this process, so the summaries under profiles/ carry them in a machine-readable
+# block, together with a hash of the kernel sources they were measured at:
+#
+#     <!-- bench-figures
+#     {"workload": "wide_deep", "dim": 16, "kernel": "...", "traffic": 45.4e6,
+#      "tcc_hit_rate": 0.456, "kernel_sources": "<sha of the sources at measuring time>"}
+#     -->
+#
+# The bench line repeats them with their source file and says so when the sources have changed.
+# ---------------------------------------------------------------------------------------------
+KERNEL_SOURCES = ("sparse_table.hip", "sparse_internal.h", "krk_internal.h")
 
 
-def make_batches(cfg, n_batches, seed):
-    """Per batch and table: unique hashed ids (the server boundary sees unique ids,
-    worker/emitter.cc:131-149) and one gradient row per unique id."""
-    from util import zipf_ranks, splitmix64
-    rng = np.random.default_rng(seed)
-    out = []
-    for _ in range(n_batches):
-        per_table = []
-        for t in range(cfg["tables"]):
-            ranks = zipf_ranks(rng, cfg["s"], cfg["space"], cfg["batch"])
-            ids = np.unique(splitmix64(ranks + np.uint64(t) * np.uint64(cfg["space"])))
-            rng.shuffle(ids)
-            g = (rng.standard_normal((ids.size, cfg["dim"])) * 1e-2).astype(np.float32)
-            per_table.append((ids, g))
-        out.append(per_table)
+def kernel_sources_hash(names=KERNEL_SOURCES):
+    h = hashlib.sha256()
+    for n in names:
+        with open(os.path.join(ROOT, "kraken_amd", "csrc", n), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def profile_figures():
+    """Every bench-figures block under profiles/ -> {(workload, dim): figures + "source"}."""
+    out = {}
+    pdir = os.path.join(ROOT, "profiles")
+    if not os.path.isdir(pdir):
+        return out
+    for name in sorted(os.listdir(pdir)):
+        if not name.endswith(".md"):
+            continue
+        with open(os.path.join(pdir, name)) as f:
+            text = f.read()
+        for m in re.finditer(r"<!-- bench-figures\s*(.*?)-->", text, re.S):
+            for line in m.group(1).strip().splitlines():
+                line = line.strip()
+                if not line:
+                    continue
+                fig = json.loads(line)
+                fig["source"] = "profiles/" + name
+                out[(fig["workload"], int(fig["dim"]))] = fig
     return out
+
+
+def attach_counter_figures(roofline, workload, dim):
+    fig = profile_figures().get((workload, dim))
+    if not fig:
+        return
+    roofline["traffic"] = fig["traffic"]
+    roofline["tcc_hit_rate"] = fig.get("tcc_hit_rate")
+    roofline["traffic_kernel"] = fig.get("kernel")
+    roofline["traffic_source"] = fig["source"] + " (hardware counters of an earlier run of this command)"
+    roofline["traffic_kernel_sources"] = fig.get("kernel_sources")
+    roofline["traffic_stale"] = fig.get("kernel_sources") != kernel_sources_hash()
 
 
 def gpu_optim(api, name):
@@ -90,20 +115,24 @@ def state_arrays(name):
     return {"adagrad": 1, "adam": 2, "rmsprop": 1}[name]
 
 
-def table_ids(cfg, t, lo, hi):
-    """Every id table t can ever see, in rank order: the hashed Zipf ranks lo..hi-1."""
-    from util import splitmix64
-    return splitmix64(np.arange(lo, hi, dtype=np.uint64) + np.uint64(t) * np.uint64(cfg["space"]))
-
-
 def _percentiles(xs):
     xs = np.sort(np.asarray(xs, np.float64))
     return float(np.median(xs)), float(xs[int(0.1 * (xs.size - 1))]), float(xs[int(np.ceil(0.9 * (xs.size - 1)))])
 
 
-def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32):
-    """Builds the workload's tables, fills their key space, and times `blocks` blocks of `steps`
-    steps each (a synchronisation on both sides of every block). -> dict of figures."""
+def lines_per_row(dim, states, word):
+    """128-byte lines one row costs: (read only by the pull, read only by the push, read and
+    written back by the push). The index bucket is one line either way; a record's weights take
+    ceil(4 D / 128) lines, the whole record (weights, state arrays, the 64-bit word's sector)
+    ceil(bytes / 128)."""
+    w_lines = -(-4 * dim // 128)
+    rec_bytes = 4 * dim * (1 + states) + (64 if word else 0)
+    return 1 + w_lines, 1, -(-rec_bytes // 128)
+
+
+def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, drained_blocks=8):
+    """Builds the workload's tables, fills their key space and times `blocks` blocks of `steps`
+    steps each between events on the stream the sparse kernels run on. -> dict of figures."""
     import ctypes as C
     from kraken_amd import api
     L = api.lib()
@@ -196,28 +225,51 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32):
     for i in range(warmup):
         step(i)
     sync_all()
-    per_step, enq = [], []
     rows_per_step = float(np.mean([dev[i % n_batches][4] for i in range(steps)]))
-    # the interpreter's garbage is collected between blocks, not inside one: a collection stalls
+    marks = [api.Event() for _ in range(blocks + 1)]
+    dense_done = api.Event()
+    # the interpreter's garbage is collected between phases, not inside one: a collection stalls
     # the host for longer than several steps take on the device
     gc.collect()
     gc.disable()
     try:
+        # 1. every block enqueued behind the one before, events in between, one wait at the end.
+        #    An untimed block goes first so that the queue is never empty while the clock runs.
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(i)
+        marks[0].record(owner)
         for b in range(blocks):
+            for i in range(steps):
+                step(i)
+            if b == blocks - 1 and dense is not None:
+                # the span ends when the dense table's stream has finished too
+                dense_done.record(dense)
+                dense_done.wait(owner)
+            marks[b + 1].record(owner)
+        t1 = time.perf_counter()
+        sync_all()
+        per_step = [marks[b].elapsed_ms(marks[b + 1]) * 1e-3 / steps for b in range(blocks)]
+        enqueue_s = (t1 - t0) / ((blocks + 1) * steps)
+        gc.collect()
+        # 2. the same blocks with the host waiting for every queue after each of them: what a
+        #    caller that drains after K steps sees (the waits' cost is spread over K steps)
+        drained = []
+        for b in range(drained_blocks):
             t0 = time.perf_counter()
             for i in range(steps):
                 step(i)
-            t1 = time.perf_counter()
             sync_all()
-            t2 = time.perf_counter()
-            per_step.append((t2 - t0) / steps)
-            enq.append((t1 - t0) / steps)
+            drained.append((time.perf_counter() - t0) / steps)
             gc.collect()
     finally:
         gc.enable()
     med, p10, p90 = _percentiles(per_step)
-    print("dim %d: host enqueue %.1f us/step, drained %.1f us/step (median of %d blocks of %d steps)" % (
-        dim, np.median(enq) * 1e6, med * 1e6, blocks, steps), file=sys.stderr)
+    drained_med = float(np.median(drained)) if drained else None
+    print("dim %d: %.2f us/step between events (p10 %.2f, p90 %.2f; %d blocks of %d steps), %.2f us/step with a "
+          "host drain per block, host enqueue %.1f us/step" % (
+              dim, med * 1e6, p10 * 1e6, p90 * 1e6, blocks, steps, (drained_med or 0) * 1e6, enqueue_s * 1e6),
+          file=sys.stderr)
 
     # the two kernels of the step: M back-to-back launches on the owner's stream, bracketed by
     # HIP events recorded on that stream
@@ -242,25 +294,38 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32):
     extra = 16 if cfg["optim"] == "adam" else 0
     push_bytes = u * (8 + 4 * dim + 8 * dim * (1 + S) + extra)
     pull_bytes = u * (8 + 8 * dim)
+    wide = 32 <= dim <= 128 and dim % 4 == 0
+    pull_lines, push_read_lines, push_rmw_lines = lines_per_row(dim, S, cfg["optim"] == "adam")
     roofline = {
-        "bound": "hbm", "kernel": "%spush_kernel<%s,4>" % ("" if single else "group_", cfg["optim"]),
+        "bound": "hbm",
+        "kernel": "%spush%s_kernel<%s>" % ("" if single else "group_", "_wide" if wide else "", cfg["optim"]),
         "achieved": push_bytes / (push_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": push_bytes / (push_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
         "bytes_per_launch": push_bytes, "us_per_launch": push_ms * 1e3,
+        "lines_per_row": {"read": push_read_lines, "read_and_written_back": push_rmw_lines},
         "pull_kernel": {"achieved": pull_bytes / (pull_ms * 1e-3) / 1e9, "us_per_launch": pull_ms * 1e3,
                         "bytes_per_launch": pull_bytes,
-                        "frac": pull_bytes / (pull_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+                        "frac": pull_bytes / (pull_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        "lines_per_row": {"read": pull_lines}},
+        "rows_per_launch": u,
     }
     per_row = 16 + 4 * dim * (2 + 1 + 2 * (1 + S)) + extra
     res = {
         "value": rows_per_step / med, "ms_per_step": med * 1e3, "ms_per_step_p10": p10 * 1e3,
         "ms_per_step_p90": p90 * 1e3, "blocks": blocks, "rows_per_step": rows_per_step,
-        "host_enqueue_us_per_step": float(np.median(enq) * 1e6),
+        "ms_per_step_host_drained": drained_med * 1e3 if drained_med else None,
+        "host_enqueue_us_per_step": enqueue_s * 1e6,
         "algorithmic_bytes_per_row": per_row,
         "achieved_gbs_whole_step": rows_per_step / med * per_row / 1e9,
         "frac_whole_step": rows_per_step / med * per_row / 1e9 / HBM_PEAK_GBS,
         "roofline": roofline, "batches": batches,
     }
+    if with_worker_leg and group is not None:
+        from kraken_amd import microbench
+        try:
+            res["worker_boundary"] = microbench.worker_boundary_leg(cfg, tables, group, optim, lr)
+        except Exception as e:   # a secondary leg never takes the headline down with it
+            res["worker_boundary"] = {"error": repr(e)}
     # give the memory back before the next configuration is built
     if group is not None:
         group.close()
@@ -272,6 +337,20 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32):
         for a in d[:3]:
             a.free()
     return res
+
+
+def add_line_floors(roofline, ceil):
+    """line_floor_us: the kernel's random lines at the line rates this run measured (read-only
+    lines at the read rate, lines written back at the read-modify-write rate) + one empty launch."""
+    rd = ceil["random_lines"]["random_line_read_%d" % (1 << 22)]["lines_per_s"]
+    rmw = ceil["random_lines"]["random_line_rmw_%d" % (1 << 22)]["lines_per_s"]
+    empty = ceil["empty_launch_us"]
+    u = roofline["rows_per_launch"]
+    lp = roofline["lines_per_row"]
+    roofline["line_floor_us"] = (u * lp["read"] / rd + u * lp["read_and_written_back"] / rmw) * 1e6 + empty
+    pk = roofline["pull_kernel"]
+    pk["line_floor_us"] = u * pk["lines_per_row"]["read"] / rd * 1e6 + empty
+    return roofline["line_floor_us"] + pk["line_floor_us"]
 
 
 def run_cpu(cfg, batches, budget_s=20.0, threads=1, n_tables=4, prefill_cap=2 * 10**6):
@@ -357,9 +436,9 @@ def copy_calibration(nbytes=1 << 30, reps=20):
 def hbm_ceilings(nbytes=1 << 31, verbose=False):
     """What this GPU's memory delivers to the simplest kernels, measured now: streaming read, fill
     and copy (best over unroll x non-temporal x workgroup count, HIP events on the null stream
-    around 5 launches), and random independent 128-byte lines over a 16 GiB region, read only and
+    around 5 launches), random independent 128-byte lines over a 16 GiB region, read only and
     read-modify-write (the table kernels' access pattern without their index), each timed right
-    after heavy traffic. GB/s."""
+    after heavy traffic, and an empty launch. GB/s."""
     from kraken_amd import api
     L = api.lib()
     if L.krk_runtime_init(0) != 0:
@@ -398,24 +477,25 @@ def hbm_ceilings(nbytes=1 << 31, verbose=False):
     big = api.DeviceArray(region // 4, np.float32)
     L.krk_memset(api._ptr(big), 1, region)
     lines = {}
+    salt = [1]
+
+    def probe(n, kind):
+        salt[0] += 1
+        rc = L.krk_hbm_probe_lines(kind, api._ptr(big), region, n, salt[0] * 0x9E3779B97F4A7C15 % (1 << 64))
+        if rc:
+            raise RuntimeError(L.krk_last_error_string().decode())
+
     for n in (98600, 1 << 20, 1 << 22):
         for rmw, name in ((0, "random_line_read"), (1, "random_line_rmw")):
-            salt = [1]
-
-            def run(lines=n, kind=rmw):
-                salt[0] += 1
-                rc = L.krk_hbm_probe_lines(kind, api._ptr(big), region, lines,
-                                           salt[0] * 0x9E3779B97F4A7C15 % (1 << 64))
-                if rc:
-                    raise RuntimeError(L.krk_last_error_string().decode())
             # A sequence of nothing but small launches runs slower than the same launches right after
             # heavy traffic (98.6k lines over 16 GiB: 9-10 us against 4-4.5 us): the figure to hold a
             # table kernel against is the second, so every timing follows three 4M-line launches.
             for _ in range(3):
-                run(1 << 22, 0)
-            sec = timed(run, reps=10)
+                probe(1 << 22, 0)
+            sec = timed(lambda: probe(n, rmw), reps=10)
             lines["%s_%d" % (name, n)] = {"us_per_launch": sec * 1e6, "lines_per_s": n / sec,
                                           "gbs": n * 128 * (2 if rmw else 1) / sec / 1e9}
+    empty_us = timed(lambda: probe(1, 0), reps=50) * 1e6     # one workgroup that reads one line
     big.free()
     out = {
         "read_ceiling": best["read"][0], "read_variant": best["read"][1],
@@ -423,7 +503,7 @@ def hbm_ceilings(nbytes=1 << 31, verbose=False):
         "copy_ceiling": best["copy"][0], "copy_variant": best["copy"][1],
         "random_line_read_ceiling": lines["random_line_read_%d" % (1 << 22)]["gbs"],
         "random_line_rmw_ceiling": lines["random_line_rmw_%d" % (1 << 22)]["gbs"],
-        "random_lines": lines, "unit": "GB/s",
+        "random_lines": lines, "empty_launch_us": empty_us, "unit": "GB/s",
     }
     if verbose:
         out["stream_table"] = [dict(kind=k, unroll=u, nontemporal=nt, workgroups=bl, gbs=g)
@@ -449,6 +529,31 @@ def host_description():
             "pinning": "none (threads float over the usable cpus)"}
 
 
+def secondary_legs(budget_s):
+    """The other configurations, each a function of kraken_amd.microbench that returns a dict.
+    A leg is skipped, and the line says so, when the run would pass its wall-clock budget."""
+    from kraken_amd import microbench
+    legs = (("deepfm", microbench.deepfm_leg, 45.0),
+            ("dup_heavy", microbench.dup_heavy_leg, 60.0),
+            ("codec", microbench.codec_leg, 20.0),
+            ("dct2", microbench.dct2_leg, 15.0))
+    out = {}
+    for name, fn, estimate_s in legs:
+        spent = time.perf_counter() - T_START
+        if spent + estimate_s > budget_s:
+            out[name] = {"skipped": "wall-clock budget: %.0f s spent, leg estimated at %.0f s, budget %.0f s" % (
+                spent, estimate_s, budget_s)}
+            continue
+        t0 = time.perf_counter()
+        try:
+            out[name] = fn()
+        except Exception as e:
+            out[name] = {"error": repr(e)}
+        out[name]["leg_wall_s"] = time.perf_counter() - t0
+        gc.collect()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -459,6 +564,10 @@ def main():
     ap.add_argument("--workload", default="wide_deep", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dims", action="store_true", help="skip the dim 32 / dim 64 legs of the default workload")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip the secondary legs (worker boundary, DeepFM, duplicate-heavy, codec, DCT)")
+    ap.add_argument("--budget-s", type=float, default=270.0,
+                    help="wall-clock budget of the whole run: a secondary leg that would pass it is skipped")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain 1 GiB streaming-copy kernel (hardware byte counters are "
                          "scaled by what they read for it) and print its bandwidth")
@@ -476,7 +585,9 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     cfg = WORKLOADS[args.workload]
-    r = run_gpu(cfg, args.steps, args.warmup, blocks=args.blocks)
+    default = args.workload == "wide_deep"
+    secondary = default and not args.no_secondary
+    r = run_gpu(cfg, args.steps, args.warmup, blocks=args.blocks, with_worker_leg=secondary)
     batches = r.pop("batches")
     roofline = r.pop("roofline")
     ceil = hbm_ceilings()
@@ -485,17 +596,16 @@ def main():
     roofline["frac_of_random_line_rmw_ceiling"] = roofline["achieved"] / ceil["random_line_rmw_ceiling"]
     roofline["copy_ceiling"] = ceil["copy_ceiling"]
     roofline["frac_of_copy_ceiling"] = roofline["achieved"] / ceil["copy_ceiling"]
-    carried = COUNTER_FIGURES.get(args.workload)
-    if carried:
-        roofline["traffic"] = carried["traffic"]
-        roofline["traffic_source"] = carried["source"] + " (carried: hardware counters cannot be read from inside this process)"
-        roofline["tcc_hit_rate"] = carried["tcc_hit_rate"]
+    step_floor = add_line_floors(roofline, ceil)
+    attach_counter_figures(roofline, args.workload, cfg["dim"])
     dim = cfg["dim"]
     line = {
         "metric": "sparse pull+push unique-rows/sec (%s, dim %d fp32)" % (cfg["optim"], dim),
         "value": r["value"], "unit": "unique-rows/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "ms_per_step_p10": r["ms_per_step_p10"],
         "ms_per_step_p90": r["ms_per_step_p90"], "timed_blocks": r["blocks"],
+        "timing": "HIP events between blocks on the sparse kernels' stream, blocks enqueued back to back",
+        "ms_per_step_host_drained": r["ms_per_step_host_drained"],
         "host_enqueue_us_per_step": r["host_enqueue_us_per_step"],
         "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
@@ -507,30 +617,33 @@ def main():
         "algorithmic_bytes_per_row": r["algorithmic_bytes_per_row"],
         "achieved_gbs_whole_step": r["achieved_gbs_whole_step"],
         "frac_whole_step": r["frac_whole_step"],
+        "line_floor_us_whole_step": step_floor,
         "roofline": roofline,
     }
-    if args.workload == "wide_deep" and not args.no_dims:
+    worker = r.pop("worker_boundary", None)
+    if default and not args.no_dims:
         by_dim = {}
         for d in (32, 64):
             c2 = dict(cfg, dim=d)
             r2 = run_gpu(c2, args.steps, args.warmup, blocks=args.blocks)
             r2.pop("batches")
-            carried = COUNTER_FIGURES_BY_DIM.get(d)
-            if carried:
-                r2["roofline"]["traffic"] = carried["traffic"]
-                r2["roofline"]["traffic_source"] = carried["source"] + " (carried)"
-                r2["roofline"]["tcc_hit_rate"] = carried["tcc_hit_rate"]
+            r2["line_floor_us_whole_step"] = add_line_floors(r2["roofline"], ceil)
+            attach_counter_figures(r2["roofline"], args.workload, d)
             by_dim[str(d)] = r2
         line["by_dim"] = by_dim
+    if secondary:
+        sec = {"worker_boundary": worker} if worker is not None else {}
+        sec.update(secondary_legs(args.budget_s - (0 if args.no_cpu else 30.0)))
+        line["secondary"] = sec
     if not args.no_cpu:
         host = host_description()
         ncpu = min(16, host["usable_cpus"] or 1)
         # three points: one caller thread, the reference server's default of two
         # (ps_server_main.cc:6), and eight (its eight slot locks bound the concurrency)
-        v1, s1 = run_cpu(cfg, batches, budget_s=8.0, threads=1)
-        v2, s2 = run_cpu(cfg, batches, budget_s=8.0, threads=min(2, ncpu))
+        v1, s1 = run_cpu(cfg, batches, budget_s=7.0, threads=1)
+        v2, s2 = run_cpu(cfg, batches, budget_s=7.0, threads=min(2, ncpu))
         threads = min(8, ncpu)
-        v8, s8 = run_cpu(cfg, batches, budget_s=8.0, threads=threads)
+        v8, s8 = run_cpu(cfg, batches, budget_s=7.0, threads=threads)
         line["cpu_baseline"] = {
             "value": v2, "unit": "unique-rows/s", "cores": min(2, ncpu), "kind": "port",
             "threads_1": v1, "threads_2": v2, "threads_%d" % threads: v8, "host": host,
@@ -538,6 +651,7 @@ def main():
                       "(same ids, gradients, optimizer) through the CPU oracle in process; value = the "
                       "reference server's default of 2 caller threads" % (cfg["tables"], s1 + s2 + s8),
         }
+    line["wall_s"] = time.perf_counter() - T_START
     print(json.dumps(line))
 
 

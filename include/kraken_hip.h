@@ -487,6 +487,10 @@ int32_t krk_event_destroy(krk_event* e);
  * object's stream, behind the work already enqueued there. NULL = the null stream, where the
  * calls that own no object (krk_dedup, krk_dct2_*, krk_coo_to_dense, krk_stream_copy) run. */
 int32_t krk_event_record(krk_event* e, void* object);
+/* Work enqueued on object's stream after this call starts only once e (recorded before, on any
+ * stream) has happened: how a span measured on one object's stream is made to include work that
+ * ran on another's, without the host waiting for either. */
+int32_t krk_event_wait(krk_event* e, void* object);
 int32_t krk_event_elapsed_ms(krk_event* start, krk_event* stop, float* ms);
 
 #ifdef __cplusplus

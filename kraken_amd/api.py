@@ -149,6 +149,7 @@ EXPORTS = {
     "krk_event_create": (C.c_int32, [C.POINTER(C.c_void_p)]),
     "krk_event_destroy": (C.c_int32, [C.c_void_p]),
     "krk_event_record": (C.c_int32, [C.c_void_p, C.c_void_p]),
+    "krk_event_wait": (C.c_int32, [C.c_void_p, C.c_void_p]),
     "krk_group_create": (C.c_int32, [C.POINTER(C.c_void_p), C.c_int32, C.POINTER(C.c_void_p)]),
     "krk_group_destroy": (C.c_int32, [C.c_void_p]),
     "krk_group_sync": (C.c_int32, [C.c_void_p]),
@@ -841,6 +842,10 @@ class Event:
     def record(self, obj):
         # obj None: the null stream, where the calls that own no object (dedup, dct2) run
         _check(lib().krk_event_record(self.h, obj.h if obj is not None else None), "krk_event_record")
+
+    def wait(self, obj):
+        # what is enqueued on obj's stream from now on starts after this (already recorded) event
+        _check(lib().krk_event_wait(self.h, obj.h if obj is not None else None), "krk_event_wait")
 
     def elapsed_ms(self, stop):
         ms = C.c_float()

@@ -477,6 +477,12 @@ int32_t krk_event_record(krk_event* e, void* object) {
   KRK_HIP(hipEventRecord(e->ev, b ? b->stream : nullptr));
   return KRK_SUCCESS;
 }
+int32_t krk_event_wait(krk_event* e, void* object) {
+  if (!e) return KRK_E_ARGUMENT;
+  ObjBase* b = reinterpret_cast<ObjBase*>(object);
+  KRK_HIP(hipStreamWaitEvent(b ? b->stream : nullptr, e->ev, 0));
+  return KRK_SUCCESS;
+}
 int32_t krk_event_elapsed_ms(krk_event* start, krk_event* stop, float* ms) {
   if (!start || !stop || !ms) return KRK_E_ARGUMENT;
   KRK_HIP(hipEventSynchronize(stop->ev));

@@ -14,21 +14,7 @@ import time
 import numpy as np
 
 from . import api
-
-
-def splitmix64(x):
-    with np.errstate(over="ignore"):
-        z = np.asarray(x, dtype=np.uint64) + np.uint64(0x9E3779B97F4A7C15)
-        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
-        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
-        return z ^ (z >> np.uint64(31))
-
-
-def zipf_ranks(rng, s, space, size):
-    w = 1.0 / np.arange(1, space + 1, dtype=np.float64) ** s
-    cdf = np.cumsum(w)
-    cdf /= cdf[-1]
-    return np.searchsorted(cdf, rng.random(size)).astype(np.uint64)
+from .workloads import splitmix64, zipf_ranks
 
 
 def timed(owner, fn, reps=10, sync=None):
@@ -406,7 +392,299 @@ def lines():
     big.free()
 
 
-SECTIONS = {"lines": lines, "copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct, "hooks": hooks}
+# ---------------------------------------------------------------------------------------------
+# The legs bench.py reports under "secondary": each returns a dict of figures. Times are HIP
+# events around back-to-back launches on the stream the kernels run on, inputs resident in HBM.
+# ---------------------------------------------------------------------------------------------
+HBM_PEAK = 8.0e12
+MFMA_F32_PEAK = 157.3e12
+
+
+def _leg(ms, nbytes=None, flops=None, **more):
+    out = {"ms": ms}
+    if nbytes is not None:
+        out.update(algorithmic_bytes=float(nbytes), achieved_gbs=nbytes / (ms * 1e-3) / 1e9,
+                   frac=nbytes / (ms * 1e-3) / HBM_PEAK, bound="hbm")
+    if flops is not None:
+        out.update(flops=float(flops), achieved_tflops=flops / (ms * 1e-3) / 1e12,
+                   frac=flops / (ms * 1e-3) / MFMA_F32_PEAK, bound="mfma")
+    out.update(more)
+    return out
+
+
+def _states(optim_name):
+    return {"adagrad": 1, "adam": 2, "rmsprop": 1}[optim_name]
+
+
+def pull_bytes_expanded(n, u, dim):
+    """Pull with the re-expansion on the device: ids in, each distinct row read once, n rows out."""
+    return 8 * n + 4 * dim * u + 4 * dim * n
+
+
+def push_raw_bytes(n, u, dim, states, adam=False):
+    """Push with the dedup on the device: ids and one gradient row per position in, one fused
+    read-modify-write per distinct row."""
+    return u * (8 + 4 * dim + 8 * dim * (1 + states) + (16 if adam else 0)) + 8 * n + 4 * dim * n
+
+
+def worker_boundary_leg(cfg, tables, group, optim, lr, n_batches=8, reps=20):
+    """The Wide&Deep step as the worker holds it: every table's ids with their repeats. One
+    combined pull of all N ids and one combined push that dedups, sums the gradients of equal
+    ids and updates (worker/emitter.cc:185-283, 552-632 + ps/sparse_table.cc:33-108)."""
+    from .workloads import make_batches
+    dim = cfg["dim"]
+    batches = make_batches(cfg, n_batches, seed=11, unique=False)
+    dev, n_ids, n_unique = [], [], []
+    for per_table in batches:
+        off = api.TableGroup._offsets([ids.size for ids, _ in per_table])
+        ids = np.concatenate([ids for ids, _ in per_table])
+        g = np.concatenate([g for _, g in per_table])
+        dev.append((api.DeviceArray.from_host(ids), api.DeviceArray.from_host(g), off))
+        n_ids.append(ids.size)
+        n_unique.append(sum(np.unique(i).size for i, _ in per_table))
+    d_out = api.DeviceArray((max(n_ids), dim), np.float32)
+    k = [0]
+
+    def pull():
+        k[0] += 1
+        d_ids, _, off = dev[k[0] % n_batches]
+        assert group.CombinePull(d_ids, off, out=d_out, async_=True)[0] == 0
+
+    def push():
+        k[0] += 1
+        d_ids, d_g, off = dev[k[0] % n_batches]
+        assert group.CombinePushRaw(optim, d_ids, off, d_g, lr, async_=True) == 0
+
+    def step():
+        pull()
+        k[0] -= 1
+        push()
+
+    t_pull, t_push, t_step = (timed(group, f, reps) for f in (pull, push, step))
+    n, u, S = float(np.mean(n_ids)), float(np.mean(n_unique)), _states(cfg["optim"])
+    b_pull, b_push = pull_bytes_expanded(n, u, dim), push_raw_bytes(n, u, dim, S)
+    for d in dev:
+        d[0].free()
+        d[1].free()
+    d_out.free()
+    return {"workload": "wide_deep, ids with repeats: %d tables x %d ids, dim %d, %s" % (
+                cfg["tables"], cfg["batch"], dim, cfg["optim"]),
+            "ids_per_step": n, "distinct_rows_per_step": u,
+            "step": _leg(t_step * 1e3, b_pull + b_push), "group_pull": _leg(t_pull * 1e3, b_pull),
+            "group_push_raw": _leg(t_push * 1e3, b_push), "ids_per_s": n / t_step}
+
+
+def _single_table(cfg, seed, extra_rows=0):
+    from .workloads import table_ids
+    dim = cfg["dim"]
+    init = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": str(seed)})
+    t = api.SparseTable(dim, init, capacity_hint=min(cfg["space"], 4 * 10**6))
+    chunk = 1 << 22
+    scratch = api.DeviceArray((min(chunk, cfg["space"]), dim), np.float32)
+    t.reserve(cfg["space"] + cfg["space"] // 8 + extra_rows)
+    for lo in range(0, cfg["space"], chunk):
+        d = api.DeviceArray.from_host(table_ids(cfg, 0, lo, min(lo + chunk, cfg["space"])))
+        t.Pull(d, out=scratch, async_=True)
+        assert t.sync() == 0
+        d.free()
+    scratch.free()
+    return t
+
+
+def deepfm_leg(n_batches=3, reps=6):
+    """cfg3: one table of 1e8 resident rows, dim 32, Adam; a step's 2.56M ids (Zipf 1.1) with
+    their repeats: pull of all ids, push_raw (dedup + sum + update), and the same step at the
+    server boundary (unique ids: pull + fused push)."""
+    from .workloads import WORKLOADS, raw_batch
+    cfg = WORKLOADS["deepfm"]
+    dim, n = cfg["dim"], cfg["batch"]
+    t = _single_table(cfg, seed=0)
+    rng = np.random.default_rng(21)
+    o = api.Optim.create(api.OptimType.kAdam)
+    d_g = api.DeviceArray.from_host(rng.standard_normal((n, dim), dtype=np.float32) * np.float32(1e-3))
+    d_out = api.DeviceArray((n, dim), np.float32)
+    raw, uniq, us = [], [], []
+    for _ in range(n_batches):
+        ids = raw_batch(rng, cfg)
+        u = np.unique(ids)
+        rng.shuffle(u)
+        raw.append(api.DeviceArray.from_host(ids))
+        uniq.append(api.DeviceArray.from_host(u))
+        us.append(u.size)
+    k = [0]
+
+    def nxt(arrs):
+        k[0] += 1
+        return arrs[k[0] % n_batches]
+
+    def chk(rc):
+        assert (rc[0] if isinstance(rc, tuple) else rc) == 0
+
+    t_pull_all = timed(t, lambda: chk(t.Pull(nxt(raw), out=d_out, async_=True)), reps)
+    t_push_raw = timed(t, lambda: chk(t.PushRaw(o, nxt(raw), d_g, 1e-3, async_=True)), reps)
+
+    def unique_step():
+        d = nxt(uniq)
+        chk(t.Pull(d, out=d_out, async_=True))
+        chk(t.Push(o, d, d_g, 1e-3, async_=True))
+    t_unique = timed(t, unique_step, reps)
+    u = float(np.mean(us))
+    out = {"workload": "deepfm: 1 table, 1e8 resident rows, dim 32, Zipf 1.1, %d ids a step, Adam" % n,
+           "ids_per_step": n, "distinct_rows_per_step": u,
+           "pull_all_ids": _leg(t_pull_all * 1e3, pull_bytes_expanded(n, u, dim)),
+           "push_raw": _leg(t_push_raw * 1e3, push_raw_bytes(n, u, dim, 2, adam=True)),
+           "unique_boundary_step": _leg(t_unique * 1e3, u * (16 + 4 * dim * (2 + 1 + 2 * 3) + 16)),
+           "unique_rows_per_s": u / t_unique}
+    for a in raw + uniq + [d_g, d_out]:
+        a.free()
+    t.close()
+    return out
+
+
+def dup_heavy_leg(steps=8, warm=2):
+    """cfg4: one table of 2e7 resident rows, dim 128, 1 048 576 Zipf(1.3) ids a step of which 5 %
+    are ids the table has never seen (every timed step has its own), RMSprop (alpha 0.9) and
+    Adagrad as separate passes. A step = pull of all ids (inserting and initialising the unseen
+    ones) + push_raw."""
+    from .workloads import WORKLOADS, raw_batch, splitmix64
+    cfg = WORKLOADS["dup_heavy"]
+    dim, n = cfg["dim"], cfg["batch"]
+    total_steps = 2 * (steps + warm)
+    fresh_per_step = n // 20
+    t = _single_table(cfg, seed=0, extra_rows=total_steps * fresh_per_step)
+    rng = np.random.default_rng(31)
+    d_g = api.DeviceArray.from_host(rng.standard_normal((n, dim), dtype=np.float32) * np.float32(1e-2))
+    d_out = api.DeviceArray((n, dim), np.float32)
+    batches, us = [], []
+    for i in range(total_steps):
+        ids = raw_batch(rng, cfg)
+        where = rng.choice(n, size=fresh_per_step, replace=False)
+        # ids beyond the key space: never drawn by the Zipf ranks, new to the table at their step
+        ids[where] = splitmix64(np.uint64(cfg["space"]) + np.arange(i * fresh_per_step, (i + 1) * fresh_per_step,
+                                                                    dtype=np.uint64))
+        batches.append(api.DeviceArray.from_host(ids))
+        us.append(np.unique(ids).size)
+    out = {"workload": "dup_heavy: 1 table, 2e7 resident rows, dim 128, Zipf 1.3, %d ids a step, 5 %% unseen" % n,
+           "ids_per_step": n, "distinct_rows_per_step": float(np.mean(us))}
+    e = [api.Event() for _ in range(3)]
+    nxt = 0
+    for name, o in (("rmsprop", api.Optim.create(api.OptimType.kRMSprop, {"alpha": "0.9"})),
+                    ("adagrad", api.Optim.create(api.OptimType.kAdagrad))):
+        pulls, pushes, u_timed = [], [], []
+        for s in range(warm + steps):
+            d = batches[nxt]
+            e[0].record(t)
+            assert t.Pull(d, out=d_out, async_=True)[0] == 0
+            e[1].record(t)
+            assert t.PushRaw(o, d, d_g, 1e-3, async_=True) == 0
+            e[2].record(t)
+            assert t.sync() == 0
+            if s >= warm:
+                pulls.append(e[0].elapsed_ms(e[1]))
+                pushes.append(e[1].elapsed_ms(e[2]))
+                u_timed.append(us[nxt])
+            nxt += 1
+        u = float(np.mean(u_timed))
+        tp, tq = float(np.median(pulls)), float(np.median(pushes))
+        b_pull, b_push = pull_bytes_expanded(n, u, dim), push_raw_bytes(n, u, dim, 1)
+        out[name] = {"step": _leg(tp + tq, b_pull + b_push), "pull_with_inserts": _leg(tp, b_pull),
+                     "push_raw": _leg(tq, b_push), "ids_per_s": n / ((tp + tq) * 1e-3)}
+    for a in batches + [d_g, d_out]:
+        a.free()
+    t.close()
+    return out
+
+
+def codec_leg(reps=5):
+    """cfg5 through the reference's emitter (worker/dct_emitter.cc:16-43): the error-feedback
+    threshold codec on a fp32 [4096, 16384] N(0, 1) gradient, eta 0.75, life_span 1000. The first
+    call selects the threshold, the timed ones run with it; decode = CooToDense."""
+    n = 4096 * 16384
+    rng = np.random.default_rng(5)
+    g = rng.standard_normal(n, dtype=np.float32)
+    d_g = api.DeviceArray.from_host(g)
+    bag = api.DenseBag(n)
+    idx, val = api.DeviceArray(n, np.int64), api.DeviceArray(n, np.float32)
+    e0, e1 = api.Event(), api.Event()
+    e0.record(bag)
+    nnz = bag.MaybeToCoo(1000, 0.75, d_g, idx, val)[2]
+    e1.record(bag)
+    api.synchronize()
+    t_select = e0.elapsed_ms(e1)
+    dense = api.DeviceArray(n, np.float32)
+    assert api.lib().krk_coo_to_dense(api._ptr(idx), api._ptr(val), nnz, api._ptr(dense), n, api.DEVICE_PTRS) == 0
+    # decode(coo) + residual restores the gradient exactly (the first call starts from a zero residual)
+    back = dense.to_host() + bag.residual
+    err = float(np.max(np.abs(back - g)))
+    kept = dense.to_host()
+    kept_err = float(np.max(np.abs(kept[kept != 0] - g[kept != 0]))) if nnz else 0.0
+    nnz2 = [nnz]
+
+    def compress():
+        nnz2[0] = bag.MaybeToCoo(1000, 0.75, d_g, idx, val)[2]
+    t_c = timed(bag, compress, reps, sync=api.synchronize)
+
+    def decode():
+        assert api.lib().krk_coo_to_dense(api._ptr(idx), api._ptr(val), nnz2[0], api._ptr(dense), n,
+                                          api.DEVICE_PTRS) == 0
+    t_d = timed(None, decode, reps)
+    out = {"workload": "threshold codec, fp32 [4096, 16384] N(0,1), eta 0.75, life_span 1000",
+           "n": n, "nnz_first_call": nnz, "nnz_timed_calls": nnz2[0],
+           "compress_selecting_threshold": _leg(t_select, 16 * n + 12 * nnz),
+           "compress": _leg(t_c * 1e3, 12 * n + 12 * nnz2[0]),
+           "decode": _leg(t_d * 1e3, 4 * n + 16 * nnz2[0]),
+           "max_abs_error_of_kept_values": kept_err,
+           "max_abs_error_decode_plus_residual_vs_gradient": err,
+           "max_rel_error": 0.0 if err == 0.0 and kept_err == 0.0 else err / float(np.max(np.abs(g)))}
+    for a in (d_g, idx, val, dense):
+        a.free()
+    bag.close()
+    return out
+
+
+def dct2_leg(reps=10):
+    """cfg5 through the blockwise DCT-II (block 256; no reference counterpart): forward and inverse
+    at keep 64 (the emitter's retention 1 - eta = 0.25) and keep 256 (round trip). Errors: the
+    coefficients of the first 4096 blocks against scipy.fft.dct(norm="ortho") in float64, relative
+    to the largest coefficient, and the keep-256 round trip against the input."""
+    import scipy.fft
+    n = 4096 * 16384
+    x = np.random.default_rng(0).standard_normal(n, dtype=np.float32)
+    d_x = api.DeviceArray.from_host(x)
+    out = {"workload": "blockwise DCT-II, block 256, fp32 [4096, 16384] N(0,1)", "n": n}
+    fl = api.DEVICE_PTRS | api.ASYNC
+    for keep in (64, 256):
+        y = api.DeviceArray((n // 256, keep), np.float32)
+        back = api.DeviceArray(n, np.float32)
+        tf = timed(None, lambda: api.lib().krk_dct2_forward(api._ptr(d_x), api._ptr(y), n, keep, fl), reps)
+        ti = timed(None, lambda: api.lib().krk_dct2_inverse(api._ptr(y), api._ptr(back), n, keep, fl), reps)
+        flops, nbytes = 2.0 * n * keep, 4.0 * (n + n // 256 * keep)
+        # what bounds a launch: the matrix pipe at keep 256, memory at keep 64
+        leg = (lambda t: _leg(t * 1e3, flops=flops)) if keep == 256 else (lambda t: _leg(t * 1e3, nbytes=nbytes))
+        rec = {"forward": leg(tf), "inverse": leg(ti)}
+        for r in rec.values():
+            r.update(flops=flops, algorithmic_bytes=nbytes)
+        coeff = y.to_host()[:4096].astype(np.float64)
+        want = scipy.fft.dct(x[:4096 * 256].reshape(4096, 256).astype(np.float64), type=2, norm="ortho")[:, :keep]
+        rec["max_rel_error_vs_scipy"] = float(np.max(np.abs(coeff - want)) / np.max(np.abs(want)))
+        if keep == 256:
+            rt = back.to_host()
+            rec["max_rel_error_round_trip"] = float(np.max(np.abs(rt - x)) / np.max(np.abs(x)))
+        out["keep_%d" % keep] = rec
+        y.free()
+        back.free()
+    d_x.free()
+    return out
+
+
+def legs():
+    import json
+    from .workloads import WORKLOADS
+    for fn in (deepfm_leg, dup_heavy_leg, codec_leg, dct2_leg):
+        print(fn.__name__, json.dumps(fn()), flush=True)
+
+
+SECTIONS = {"legs": legs, "lines": lines, "copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct, "hooks": hooks}
 
 
 def main(argv):

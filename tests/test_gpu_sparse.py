@@ -351,3 +351,80 @@ def test_wide_rows_group_pull_ragged_members(api, oracle):
         want = np.concatenate([r.pull(p)[1] for r, p in zip(refs, per) if p.size] or [np.zeros((0, dim), np.float32)])
         assert_close(got, want, "combined pull, step %d" % step, rtol=1e-6)
     grp.close()
+
+
+_WIDE_PUSH_CASES = [c for c in OPTIM_CASES if c[0] in ("sgd", "sgd_damp", "adagrad", "adam_wd", "adam_amsgrad",
+                                                        "rmsprop_all")]
+_WIDE_GROUP_CASES = [c for c in OPTIM_CASES if c[0] in ("adagrad", "adam", "sgd_mom")]
+
+
+@pytest.mark.parametrize("name,type_,conf", _WIDE_PUSH_CASES, ids=[c[0] for c in _WIDE_PUSH_CASES])
+@pytest.mark.parametrize("dim", [20, 32, 36, 64, 100, 128])
+def test_wide_rows_push_every_path(api, oracle, name, type_, conf, dim):
+    """Rows of 32 to 128 floats are pushed by kernels of their own (sixteen ids looked up per
+    wavefront, then lane groups of 8, 16 or 32 lanes update the records, several rows' loads in
+    flight). Against the oracle: request sizes on both sides of sixteen and of a workgroup's 64,
+    the ids 0 and all ones, a request with ids the table does not hold (code 12, the others
+    updated), repeated pushes of the same rows (state columns, Adam's per-row counter, SGD's first
+    momentum step), and every state column afterwards."""
+    gi, oi = _const_init(api, oracle, 0.5)
+    t = api.SparseTable(dim, gi)
+    r = oracle.SparseTable(dim, oi)
+    rng = np.random.default_rng(dim * 7 + type_)
+    o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    pool = np.concatenate([splitmix64(np.arange(3000, dtype=np.uint64)), np.array([0, 2**64 - 1], np.uint64)])
+    w0 = rng.standard_normal((pool.size, dim)).astype(np.float32)
+    t.load(pool, w0)
+    r.load(pool, w0)
+    for n in (1, 15, 16, 17, 63, 64, 65, 1000, 3002):
+        sub = pool[rng.permutation(pool.size)[:n]]
+        g = (rng.standard_normal((n, dim)) * 0.5).astype(np.float32)
+        assert t.Push(o_gpu, sub, g, 0.05) == 0
+        assert r.push(o_ref, sub, g, 0.05) == 0
+    # ids the table does not hold: the call reports them and still updates the rest
+    absent = splitmix64(np.arange(10**6, 10**6 + 5, dtype=np.uint64))
+    sub = np.concatenate([pool[:40], absent])[rng.permutation(45)]
+    g = (rng.standard_normal((45, dim)) * 0.5).astype(np.float32)
+    assert t.Push(o_gpu, sub, g, 0.05) == 12
+    held = np.isin(sub, pool)
+    assert r.push(o_ref, sub[held], g[held], 0.05) == 0
+    rc, got = t.Pull(pool)
+    _, want = r.pull(pool)
+    assert rc == 0 and len(t) == len(r)
+    assert_close(got, want, "%s dim %d weights" % (name, dim))
+    gid, _, _, gsteps = t.export()
+    rid, _, _, rsteps = r.export()
+    order_g, order_r = np.argsort(gid), np.argsort(rid)
+    if type_ == 1:
+        assert np.array_equal(gsteps[order_g], rsteps[order_r])
+    for st in STATE_OF[type_]:
+        _, _, gs, _ = t.export(state_type=st)
+        _, _, rs, _ = r.export(state_type=st)
+        assert_close(gs[order_g], rs[order_r], "%s dim %d state %d" % (name, dim, st))
+
+
+@pytest.mark.parametrize("name,type_,conf", _WIDE_GROUP_CASES, ids=[c[0] for c in _WIDE_GROUP_CASES])
+@pytest.mark.parametrize("dim", [32, 64, 128])
+def test_wide_rows_group_push_ragged_members(api, oracle, name, type_, conf, dim):
+    """A combined push over tables of wide rows whose members bring 0, 1, 17, 5000 and 16 ids."""
+    gi, oi = _const_init(api, oracle, -0.25)
+    counts = [0, 1, 17, 5000, 16]
+    tables = [api.SparseTable(dim, gi) for _ in counts]
+    refs = [oracle.SparseTable(dim, oi) for _ in counts]
+    grp = api.TableGroup(tables)
+    rng = np.random.default_rng(dim + type_)
+    o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    pool = splitmix64(np.arange(6000, dtype=np.uint64))
+    for t, r in zip(tables, refs):
+        t.Pull(pool)
+        r.pull(pool)
+    for step in range(3):
+        per = [pool[rng.permutation(pool.size)[:c]] for c in counts]
+        grads = [(rng.standard_normal((c, dim)) * 0.3).astype(np.float32) for c in counts]
+        assert grp.CombinePush(o_gpu, np.concatenate(per), grp._offsets(counts), np.concatenate(grads), 0.02) == 0
+        for r, p, g in zip(refs, per, grads):
+            if p.size:
+                assert r.push(o_ref, p, g, 0.02) == 0
+    for i, (t, r) in enumerate(zip(tables, refs)):
+        assert_close(t.Pull(pool)[1], r.pull(pool)[1], "%s dim %d member %d" % (name, dim, i))
+    grp.close()

@@ -1,30 +1,17 @@
 """Shared helpers for the parity tests: seeded inputs and optimizer pairs."""
+import os
+import sys
+
 import numpy as np
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
 RTOL = 1e-5     # north-star tolerance for fp32 values
 ATOL = 1e-7
 
 
-def splitmix64(x):
-    """Vectorised splitmix64 output function on uint64 arrays."""
-    with np.errstate(over="ignore"):
-        z = (np.asarray(x, dtype=np.uint64) + np.uint64(0x9E3779B97F4A7C15))
-        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
-        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
-        return z ^ (z >> np.uint64(31))
-
-
-def zipf_ranks(rng, s, space, size):
-    """Zipf(s) ranks in [0, space) by inverse-CDF on the truncated distribution."""
-    w = 1.0 / np.arange(1, space + 1, dtype=np.float64) ** s
-    cdf = np.cumsum(w)
-    cdf /= cdf[-1]
-    return np.searchsorted(cdf, rng.random(size)).astype(np.uint64)
-
-
-def zipf_ids(rng, s, space, size):
-    """Ids of the benchmark configurations: splitmix64 of a Zipf rank."""
-    return splitmix64(zipf_ranks(rng, s, space, size))
+# the workload generators live with the package: the bench and the tests draw the same inputs
+from kraken_amd.workloads import splitmix64, zipf_ids, zipf_ranks  # noqa: E402,F401
 
 
 OPTIM_CASES = [
