@@ -22,19 +22,45 @@ namespace krk {
 constexpr int kBlock = 256;
 constexpr int64_t kTwoLaunchPull = 1 << 18;   // ids from which a pull runs as two launches
 constexpr int kMissingGrid = 2048;            // workgroups of the launch that inserts missing ids
+// The positions whose id is missing are queued in kQueues lists, each with a counter on a line
+// of its own: workgroup b of the first launch appends to list b mod kQueues. One counter for the
+// whole request serialises on its address: 36k additions of a 5 %-new request of a million ids
+// made the first launch take 428 us instead of 131.
+constexpr int kQueues = 64;
+constexpr int kQueueCounterStride = 32;       // 32-bit words between two lists' counters: 128 bytes
+constexpr int kQueueCounterWords = 2 * kQueues * kQueueCounterStride;   // two sets, used in turn
+constexpr int kCounterWords = 4 + kQueueCounterWords;                    // what t->counters holds
+
+// Entries list q of a request of n positions can hold: every workgroup appends at most
+// ids_per_block entries to its list.
+__host__ __device__ inline int64_t queue_capacity(int64_t n, int ids_per_block) {
+  const int64_t blocks = (n + ids_per_block - 1) / ids_per_block;
+  return ((blocks + kQueues - 1) / kQueues) * ids_per_block;
+}
+__device__ __forceinline__ uint32_t* queue_counter(const TableView& tv, int parity, int q) {
+  return tv.counters + 4 + (parity * kQueues + q) * kQueueCounterStride;
+}
 
 // VEC initial values of a new row, evaluated one after the other: the loop stays rolled so that
 // the double-precision Box-Muller of the rare branch is live once, not VEC times, and the
 // kernels that carry it keep their occupancy (the pulls are bound by the reads in flight).
-template <int VEC>
+// (UNROLLED: the kernels that only handle new ids evaluate the VEC values side by side instead;
+// an evaluation is a long chain of dependent double-precision operations, and those kernels have
+// few wavefronts to hide it behind.)
+template <int VEC, bool UNROLLED = false>
 __device__ __forceinline__ void init_vec(const InitK& init, uint64_t id, int64_t first, float (&v)[VEC]) {
+  if constexpr (UNROLLED) {
 #pragma unroll
-  for (int c = 0; c < VEC; ++c) v[c] = 0.0f;
+    for (int c = 0; c < VEC; ++c) v[c] = init_element(init, id, first + c);
+  } else {
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) v[c] = 0.0f;
 #pragma unroll 1
-  for (int c = 0; c < VEC; ++c) {
-    const float x = init_element(init, id, first + c);
+    for (int c = 0; c < VEC; ++c) {
+      const float x = init_element(init, id, first + c);
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) v[k] = k == c ? x : v[k];
+      for (int k = 0; k < VEC; ++k) v[k] = k == c ? x : v[k];
+    }
   }
 }
 
@@ -81,7 +107,7 @@ __device__ __forceinline__ void vstore(float* p, const float (&v)[VEC]) {
 // pull: gather rows, inserting and initialising the ones that are missing.
 // `i` is this lane group's position in ids/out, gl the lane's index in the group.
 // ---------------------------------------------------------------------------
-template <int VEC>
+template <int VEC, bool MOSTLY_NEW = false>
 __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init,
                                           const uint64_t* __restrict__ ids, int64_t i, bool active,
                                           int gl, float* __restrict__ out, int dim, int elems,
@@ -110,7 +136,7 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
     if (fresh) {
       // the value of a new row is a pure function of (seed, id, element): every group that
       // meets it computes the same numbers, only the creator stores them
-      init_vec<VEC>(init, id, (int64_t)e * VEC, v);
+      init_vec<VEC, MOSTLY_NEW>(init, id, (int64_t)e * VEC, v);
       if (owner) vstore<VEC>(rec + e * VEC, v);
     } else {
       vload<VEC>(rec + e * VEC, v);
@@ -220,8 +246,8 @@ __global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, InitK init,
 // large request first runs a kernel that only searches and copies (eight wavefronts per SIMD)
 // and queues the positions whose id is missing; a second, small launch walks that queue with
 // pull_body. In steady state the queue is empty and the second launch ends at once.
-// counters[2 + parity] counts the queue; the second launch clears the other parity's counter
-// for the request after it (same stream, so that request's first kernel has not started).
+// Two sets of list counters are used in turn; the second launch clears the other set for the
+// request after it (same stream, so that request's first kernel has not started).
 template <int VEC>
 __global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, const uint64_t* __restrict__ ids,
                                                                int64_t n, float* __restrict__ out,
@@ -232,16 +258,19 @@ __global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, con
   const int gl = threadIdx.x & (group - 1);
   const bool active = i < n;
   const uint32_t row = probe_find(tv, active ? ids[i] : 0, active, gl, group);
-  // one atomic per wavefront reserves queue entries for all of its missing ids
+  // one atomic per wavefront reserves entries of the workgroup's list for all of its missing ids
   const bool queue = active && row == kEmptyRow && gl == 0;
   const unsigned long long votes = __ballot(queue);
   if (votes) {
     const int lane = wave_lane();
     const int first = __ffsll(votes) - 1;
+    const int q = blockIdx.x & (kQueues - 1);
     uint32_t base = 0;
-    if (lane == first) base = atomicAdd(&tv.counters[2 + parity], (uint32_t)__popcll(votes));
+    if (lane == first) base = atomicAdd(queue_counter(tv, parity, q), (uint32_t)__popcll(votes));
     base = __shfl(base, first);
-    if (queue) todo[base + (uint32_t)__popcll(votes & ((1ull << lane) - 1ull))] = (uint32_t)i;
+    if (queue)
+      todo[q * queue_capacity(n, per_block) + base + (uint32_t)__popcll(votes & ((1ull << lane) - 1ull))] =
+          (uint32_t)i;
   }
   if (!active || row == kEmptyRow) return;
   const float* rec = tv.recs + (int64_t)row * tv.stride;
@@ -258,17 +287,20 @@ __global__ __launch_bounds__(kBlock) void pull_missing_kernel(TableView tv, Init
                                                               const uint64_t* __restrict__ ids,
                                                               float* __restrict__ out,
                                                               const uint32_t* __restrict__ todo, int parity,
-                                                              int dim, int elems, int group) {
-  const uint32_t count = __atomic_load_n(&tv.counters[2 + parity], __ATOMIC_RELAXED);
-  if (blockIdx.x == 0 && threadIdx.x == 0) tv.counters[2 + (parity ^ 1)] = 0u;
+                                                              int64_t n, int dim, int elems, int group) {
+  // workgroup b walks list b mod kQueues, together with the other gridDim.x / kQueues of that list
+  const int q = blockIdx.x & (kQueues - 1);
+  const uint32_t count = __atomic_load_n(queue_counter(tv, parity, q), __ATOMIC_RELAXED);
+  if (blockIdx.x < kQueues && threadIdx.x == 0) *queue_counter(tv, parity ^ 1, q) = 0u;
   const int per_block = kBlock / group;
-  const uint32_t stride = gridDim.x * per_block;
+  const uint32_t* list = todo + q * queue_capacity(n, per_block);
+  const uint32_t stride = (gridDim.x / kQueues) * per_block;
   const int gl = threadIdx.x & (group - 1);
   // block-uniform trip count: pull_body votes across the wavefront
-  for (uint32_t k0 = blockIdx.x * per_block; k0 < count; k0 += stride) {
+  for (uint32_t k0 = (blockIdx.x / kQueues) * per_block; k0 < count; k0 += stride) {
     const uint32_t k = k0 + threadIdx.x / group;
     const bool active = k < count;
-    pull_body<VEC>(tv, init, ids, active ? (int64_t)todo[k] : 0, active, gl, out, dim, elems, group);
+    pull_body<VEC, true>(tv, init, ids, active ? (int64_t)list[k] : 0, active, gl, out, dim, elems, group);
   }
 }
 
@@ -383,7 +415,8 @@ __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64
 // otherwise they are queued for pull_missing_kernel as in pull_resident_kernel.
 constexpr int kWideIds = kWave / kBucket;        // ids a wavefront takes: 16
 
-template <int VEC, bool INSERT>
+// VIA (with INSERT): first..end count entries of the queue `todo`, which names the positions.
+template <int VEC, bool INSERT, bool VIA = false>
 __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init,
                                           const uint64_t* __restrict__ ids, int64_t first, int64_t end,
                                           float* __restrict__ out, int dim, int elems, int group,
@@ -392,7 +425,8 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
   const int gl4 = lane & (kBucket - 1);
   const int64_t i = first + (lane >> 2);
   const bool active = i < end;
-  const uint64_t id = active ? ids[i] : 0;
+  const uint32_t my_pos = (VIA && active) ? todo[i] : 0u;
+  const uint64_t id = active ? ids[VIA ? (int64_t)my_pos : i] : 0;
   const FindResult f = probe_find_slot(tv, id, active, gl4, kBucket);
   ProbeResult pr;
   pr.row = (uint32_t)f.row_epoch;
@@ -406,15 +440,19 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
       if (miss) pr = q;
     }
   } else {
-    // one atomic per wavefront reserves queue entries for all of its missing ids
+    // one atomic per wavefront reserves entries of the workgroup's list for all of its missing ids
+    // (here `end` is the request's length: the lists' capacity follows from it)
     const bool queue = miss && gl4 == 0;
     const unsigned long long votes = __ballot(queue);
     if (votes) {
       const int leader = __ffsll(votes) - 1;
+      const int q = blockIdx.x & (kQueues - 1);
       uint32_t base = 0;
-      if (lane == leader) base = atomicAdd(&tv.counters[2 + parity], (uint32_t)__popcll(votes));
+      if (lane == leader) base = atomicAdd(queue_counter(tv, parity, q), (uint32_t)__popcll(votes));
       base = __shfl(base, leader);
-      if (queue) todo[base + (uint32_t)__popcll(votes & ((1ull << lane) - 1ull))] = (uint32_t)i;
+      if (queue)
+        todo[q * queue_capacity(end, (kBlock / kWave) * kWideIds) + base +
+             (uint32_t)__popcll(votes & ((1ull << lane) - 1ull))] = (uint32_t)i;
     }
     copy = active && f.found;
     pr.fresh = false;                              // nothing is created here: what was found is read
@@ -426,6 +464,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
   const int gl = lane & (group - 1);
   const uint32_t id_lo = (uint32_t)id, id_hi = (uint32_t)(id >> 32);
   float v[8][VEC];
+  uint32_t where[VIA ? 8 : 1];                   // VIA: the position each step's row goes to
   uint32_t live = 0;                             // bit s: this lane has a slice of step s to store
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
@@ -436,12 +475,13 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
       const int owner = __shfl((int)pr.owner, src);
       const int on = __shfl((int)copy, src);
       const uint64_t its_id = (uint64_t)__shfl(id_lo, src) | ((uint64_t)__shfl(id_hi, src) << 32);
+      if constexpr (VIA) where[s] = __shfl(my_pos, src);
       if (on && gl < elems) {
         float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
         if (fresh) {
           // the value of a new row is a pure function of (seed, id, element): every group that
           // meets it computes the same numbers, only the creator stores them
-          init_vec<VEC>(init, its_id, (int64_t)gl * VEC, v[s]);
+          init_vec<VEC, VIA>(init, its_id, (int64_t)gl * VEC, v[s]);
           if (owner) vstore<VEC>(rec + gl * VEC, v[s]);
         } else {
           vload<VEC>(rec + gl * VEC, v[s]);
@@ -452,8 +492,10 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
   }
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
-    if (live & (1u << s))
-      vstore_once<VEC>(out + (first + s * rows_per_step + sub) * (int64_t)dim + gl * VEC, v[s]);
+    if (live & (1u << s)) {
+      const int64_t p = VIA ? (int64_t)where[VIA ? s : 0] : first + s * rows_per_step + sub;
+      vstore_once<VEC>(out + p * (int64_t)dim + gl * VEC, v[s]);
+    }
   }
 }
 
@@ -582,6 +624,23 @@ __global__ __launch_bounds__(kBlock) void pull_resident_wide_kernel(TableView tv
   if (first >= n) return;
   InitK none{};
   pull_wide<VEC, false>(tv, none, ids, first, n, out, dim, elems, group, todo, parity);
+}
+
+// the second launch of a large pull for wide rows: sixteen queued positions per wavefront
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pull_missing_wide_kernel(TableView tv, InitK init,
+                                                                   const uint64_t* __restrict__ ids,
+                                                                   float* __restrict__ out,
+                                                                   uint32_t* __restrict__ todo, int parity,
+                                                                   int64_t n, int dim, int elems, int group) {
+  const int q = blockIdx.x & (kQueues - 1);
+  const uint32_t count = __atomic_load_n(queue_counter(tv, parity, q), __ATOMIC_RELAXED);
+  if (blockIdx.x < kQueues && threadIdx.x == 0) *queue_counter(tv, parity ^ 1, q) = 0u;
+  uint32_t* list = todo + q * queue_capacity(n, (kBlock / kWave) * kWideIds);
+  const uint32_t stride = (gridDim.x / kQueues) * (kBlock / kWave) * kWideIds;
+  for (uint32_t k0 = ((blockIdx.x / kQueues) * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds; k0 < count;
+       k0 += stride)
+    pull_wide<VEC, true, true>(tv, init, ids, k0, count, out, dim, elems, group, list, parity);
 }
 
 // ---- one launch over several tables of equal row width ------------------------
@@ -1511,8 +1570,8 @@ int32_t krk_sparse_create(int64_t dim, const krk_init* init, int64_t capacity_hi
   int32_t rc = t->open_stream();
   t->own_stream = t->stream;
   if (rc == KRK_SUCCESS) {
-    hipError_t e = hipMalloc((void**)&t->counters, 16);
-    if (e == hipSuccess) e = hipMemsetAsync(t->counters, 0, 16, t->stream);
+    hipError_t e = hipMalloc((void**)&t->counters, kCounterWords * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMemsetAsync(t->counters, 0, kCounterWords * sizeof(uint32_t), t->stream);
     if (e == hipSuccess) e = hipHostMalloc((void**)&t->host_counters, 16, hipHostMallocDefault);
     if (e == hipSuccess) e = hipHostMalloc((void**)&t->host_pub, 8, hipHostMallocCoherent);
     if (e == hipSuccess) *t->host_pub = 0ull;
@@ -1607,7 +1666,7 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
   // of about the table's size is the other case: many repeats of resident ids (8.9 million ids
   // over a table of ten million rows: 590 us in two launches, 730 us fused).
   if (n >= kTwoLaunchPull && rows_before >= n) {
-    KRK_TRY(t->scratch[5].reserve((size_t)n * sizeof(uint32_t)));
+    KRK_TRY(t->scratch[5].reserve((size_t)kQueues * queue_capacity(n, per_block) * sizeof(uint32_t)));
     uint32_t* todo = t->scratch[5].as<uint32_t>();
     const int parity = t->pull_parity;
     t->pull_parity ^= 1;
@@ -1620,13 +1679,18 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
         hipLaunchKernelGGL((pull_resident_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
                            parity, (int)t->dim, t->elems, t->group);
       }
-      hipLaunchKernelGGL((pull_missing_kernel<4>), small, block, 0, t->stream, t->view(), t->initk, d_ids, d_out,
-                         todo, parity, (int)t->dim, t->elems, t->group);
+      if (wide) {
+        hipLaunchKernelGGL((pull_missing_wide_kernel<4>), small, block, 0, t->stream, t->view(), t->initk, d_ids,
+                           d_out, todo, parity, n, (int)t->dim, t->elems, t->group);
+      } else {
+        hipLaunchKernelGGL((pull_missing_kernel<4>), small, block, 0, t->stream, t->view(), t->initk, d_ids,
+                           d_out, todo, parity, n, (int)t->dim, t->elems, t->group);
+      }
     } else {
       hipLaunchKernelGGL((pull_resident_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
                          parity, (int)t->dim, t->elems, t->group);
       hipLaunchKernelGGL((pull_missing_kernel<1>), small, block, 0, t->stream, t->view(), t->initk, d_ids, d_out,
-                         todo, parity, (int)t->dim, t->elems, t->group);
+                         todo, parity, n, (int)t->dim, t->elems, t->group);
     }
   } else if (t->vec == 4 && wide) {
     hipLaunchKernelGGL((pull_wide_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
