@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libkraken_hip.so")
 
-SOURCES = ["runtime.hip", "sparse_table.hip", "push_raw.hip", "dense_table.hip", "codec.hip",
+SOURCES = ["runtime.hip", "sparse_table.hip", "push_raw.hip", "radix_sort.hip", "dense_table.hip", "codec.hip",
            "dct2.hip", "checkpoint.hip"]
 
 # -ffp-contract=off: the reference rounds after every elementwise op (one Eigen pass per op),

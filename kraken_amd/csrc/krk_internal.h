@@ -277,6 +277,15 @@ size_t coo_densify_work_bytes(int64_t n);
 int32_t coo_densify(const long long* d_idx, const float* d_val, int64_t nnz, float* d_dense, int64_t n,
                     void* work, uint32_t* err, hipStream_t stream);
 
+// Stable radix sort of n (key, payload) pairs by the low `bits` bits of the key (radix_sort.hip).
+// keys / vals are overwritten; keys_alt / vals_alt hold n entries each; work holds
+// radix_sort_work_bytes(n). *keys_sorted / *vals_sorted say which of the two pairs of arrays the
+// result is in.
+size_t radix_sort_work_bytes(int64_t n);
+int32_t radix_sort_pairs(uint32_t* keys, uint32_t* vals, uint32_t* keys_alt, uint32_t* vals_alt, int64_t n,
+                         int bits, void* work, hipStream_t stream, uint32_t** keys_sorted,
+                         uint32_t** vals_sorted);
+
 // scratch must hold scan_scratch_bytes(n).
 size_t scan_scratch_bytes(int64_t n);
 int32_t exclusive_scan_i32(const int32_t* in, int32_t* out, int64_t n, int32_t* total_out,

@@ -15,8 +15,6 @@
 #include <cstring>
 #include <new>
 
-#include <rocprim/block/block_radix_sort.hpp>
-#include <rocprim/device/device_radix_sort.hpp>
 
 #include "sparse_internal.h"
 
@@ -475,7 +473,7 @@ __device__ __forceinline__ void apply_row(const TableView& tv, uint32_t row, con
 // other, 36 us against four launches of about 8 us for the tail of an 8192-id request.
 constexpr int kPrefetch = 4;
 constexpr int kPrefetchCarry = 4;
-constexpr int kCarryTile = 4;
+constexpr int kCarryTile = 4;   // 16, 32 and 64 were measured: 254, 272 and 304 us for a million dim-128 ids against 244
 
 // Weighted bags (level 0 only): the sorted payload is a position p, its gradient row is
 // vals[bag_of[p]] times weight[p]. Both null otherwise: the payload itself names the row.
@@ -798,42 +796,6 @@ static int pick_tile(int64_t cnt) {
   // (measured 4 to 64). The carry lists themselves are short: tiles of 4 there.
   if (cnt >= (1 << 19)) return 16;
   return 8;
-}
-
-// The library's radix sort switches from a merge sort (one block sort plus log2(n / block)
-// merge passes, each two launches) to its one-pass-per-digit radix sort above a size limit that
-// defaults to 2^20 items, and its default radix blocks hold 16k items, i.e. 64 workgroups for a
-// million pairs on 256 CUs. For (u32, u32) pairs on this GPU the radix path with 8-bit digits
-// and the wavefront-matching rank is the faster one from about 2^16 items on; blocks of 4096
-// items serve up to two million pairs best, blocks of 8192 beyond (measured per sort of 2^20
-// pairs of 26-bit keys: 160 us merge sort, 110 us with 4096-item blocks). Up to 8192 pairs one
-// workgroup sorts them all in a single launch (the default switches to block sort plus merge
-// passes above 2048: six launches and 26 us for 8192 pairs). All paths are stable.
-template <unsigned ItemsPerThread, unsigned DigitBits>
-using SortConfig = rocprim::radix_sort_config<
-    rocprim::kernel_config<1024, 8>, rocprim::default_config,
-    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<256, 12>, rocprim::kernel_config<1024, ItemsPerThread>,
-                                        DigitBits, rocprim::block_radix_rank_algorithm::match>,
-    (size_t)1 << 16>;
-
-template <unsigned DigitBits>
-static hipError_t sort_pairs_with(void* tmp, size_t& tmp_bytes, uint32_t* keys, uint32_t* keys_out, uint32_t* vals,
-                                  uint32_t* vals_out, int64_t n, int bits, hipStream_t stream) {
-  if (n <= ((int64_t)1 << 21))
-    return rocprim::radix_sort_pairs<SortConfig<4, DigitBits>>(tmp, tmp_bytes, keys, keys_out, vals, vals_out,
-                                                               (size_t)n, 0, bits, stream);
-  return rocprim::radix_sort_pairs<SortConfig<8, DigitBits>>(tmp, tmp_bytes, keys, keys_out, vals, vals_out,
-                                                             (size_t)n, 0, bits, stream);
-}
-
-// One pass over the pairs per digit: 9-bit digits where they save a pass over 8-bit ones (17-18
-// and 25-27 key bits; a 9-bit pass is about 5 % slower than an 8-bit one, 10-bit passes lose more
-// than they save).
-static hipError_t sort_pairs(void* tmp, size_t& tmp_bytes, uint32_t* keys, uint32_t* keys_out, uint32_t* vals,
-                             uint32_t* vals_out, int64_t n, int bits, hipStream_t stream) {
-  if ((bits + 8) / 9 < (bits + 7) / 8)
-    return sort_pairs_with<9>(tmp, tmp_bytes, keys, keys_out, vals, vals_out, n, bits, stream);
-  return sort_pairs_with<8>(tmp, tmp_bytes, keys, keys_out, vals, vals_out, n, bits, stream);
 }
 
 // ---------------------------------------------------------------------------
@@ -1231,8 +1193,7 @@ static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, Device
   const int per_block = kBlock / sh.group;
   const int64_t groups0 = ((n + tile0 - 1) / tile0 + per_block - 1) / per_block;   // workgroups of level 0
   const size_t n4 = (size_t)n * sizeof(uint32_t);
-  size_t sort_bytes = 0;
-  KRK_HIP(sort_pairs(nullptr, sort_bytes, nullptr, nullptr, nullptr, nullptr, n, bits, stream));
+  const size_t sort_bytes = radix_sort_work_bytes(n);
   const size_t carry_entries = (size_t)(2 * groups0);
   KRK_TRY(scratch[0].reserve(4 * n4));                       // keys, payload, sorted keys, sorted payload
   KRK_TRY(scratch[1].reserve(sort_bytes));
@@ -1241,12 +1202,12 @@ static int32_t sort_and_reduce(const ReduceShape& sh, hipStream_t stream, Device
   KRK_TRY(scratch[4].reserve((carry_entries / 2 + 16) * (size_t)sh.dim * sizeof(float)));  // B
   uint32_t* keys = scratch[0].as<uint32_t>();
   uint32_t* pos = keys + n;
-  uint32_t* skeys = pos + n;
-  uint32_t* spos = skeys + n;
+  uint32_t* skeys = nullptr;
+  uint32_t* spos = nullptr;
 
   fill(keys, pos);
   KRK_HIP(hipGetLastError());
-  KRK_HIP(sort_pairs(scratch[1].ptr, sort_bytes, keys, skeys, pos, spos, n, bits, stream));
+  KRK_TRY(radix_sort_pairs(keys, pos, pos + n, pos + 2 * n, n, bits, scratch[1].ptr, stream, &skeys, &spos));
 
   // level 0 reads value rows through the sorted payloads; later levels read the carry list
   uint32_t* ckeys[2] = {scratch[2].as<uint32_t>(), scratch[2].as<uint32_t>() + carry_entries};
