@@ -433,6 +433,22 @@ int32_t krk_dense_states(krk_dense* t, uint32_t* mask);
  * leaves it) of a table built from a saved Value (checkpoint/checkpoint.cc:535-557). */
 int32_t krk_dense_import_state(krk_dense* t, int32_t state_type, const float* state, int64_t steps,
                                uint32_t flags);
+/* Several dense tables served by one launch. Ps::CombinePullDenseTable (ps/ps_op.cc:177-252) pulls
+ * every dense parameter of a model in one request, which the worker issues after every step
+ * (pytorch/optimizer.py:151-173): pull writes the members' values one after the other, in member
+ * order, into out[sum of sizes]. push applies Optim::Update to every member with its part of
+ * grads[n] laid out the same way (the loop of Ps::PushDenseTable calls, ps/ps_op.cc:254-300, that a
+ * step's gradient hooks make): n != the sum of the members' sizes returns 11; every member's Adam
+ * counter advances by one. While a table is a member its own calls run on the group's stream,
+ * ordered with the group's; destroy the group before its tables. */
+typedef struct krk_dense_group krk_dense_group;
+int32_t krk_dense_group_create(krk_dense** tables, int32_t n, krk_dense_group** out);
+int32_t krk_dense_group_destroy(krk_dense_group* g);
+int32_t krk_dense_group_sync(krk_dense_group* g);
+int32_t krk_dense_group_size(krk_dense_group* g, int64_t* total);
+int32_t krk_dense_group_pull(krk_dense_group* g, float* out, uint32_t flags);
+int32_t krk_dense_group_push(krk_dense_group* g, const krk_optim* o, const float* grads, int64_t n, float lr,
+                             uint32_t flags);
 /* Checkpoint::SaveDenseTable / LoadDenseTable (checkpoint/checkpoint.cc:444-463, 535-557): a
  * *.dense file holds the table's type, id, name and Value. shape/rank give the tensor shape to
  * record (rank 0 = one dimension of n elements). Loading creates the table; *rank holds the

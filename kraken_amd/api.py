@@ -137,6 +137,12 @@ EXPORTS = {
                                        C.c_int64, C.c_float, C.c_uint32]),
     "krk_dense_state": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_uint32]),
     "krk_dense_steps": (C.c_int32, [C.c_void_p, C.POINTER(C.c_int64)]),
+    "krk_dense_group_create": (C.c_int32, [C.POINTER(C.c_void_p), C.c_int32, C.POINTER(C.c_void_p)]),
+    "krk_dense_group_destroy": (C.c_int32, [C.c_void_p]),
+    "krk_dense_group_sync": (C.c_int32, [C.c_void_p]),
+    "krk_dense_group_size": (C.c_int32, [C.c_void_p, C.POINTER(C.c_int64)]),
+    "krk_dense_group_pull": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_uint32]),
+    "krk_dense_group_push": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float, C.c_uint32]),
     "krk_dct_create": (C.c_int32, [C.c_int64, C.POINTER(C.c_void_p)]),
     "krk_dct_destroy": (C.c_int32, [C.c_void_p]),
     "krk_dct_compress": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_float, C.c_void_p,
@@ -679,6 +685,45 @@ class DenseTable:
         s = C.c_int64()
         _check(lib().krk_dense_steps(self.h, C.byref(s)), "krk_dense_steps")
         return s.value
+
+
+class DenseGroup:
+    """The dense tables of one combined request (Ps::CombinePullDenseTable, ps/ps_op.cc:177-252):
+    one launch serves all of them; values and gradients are the members' arrays one after the
+    other."""
+
+    def __init__(self, tables):
+        self.tables = list(tables)
+        arr = (C.c_void_p * len(self.tables))(*[t.h for t in self.tables])
+        h = C.c_void_p()
+        _check(lib().krk_dense_group_create(arr, len(self.tables), C.byref(h)), "krk_dense_group_create")
+        self.h = h
+        n = C.c_int64()
+        _check(lib().krk_dense_group_size(h, C.byref(n)), "krk_dense_group_size")
+        self.n = n.value
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().krk_dense_group_destroy(self.h)
+            self.h = None
+
+    __del__ = close
+
+    def sync(self):
+        return lib().krk_dense_group_sync(self.h)
+
+    def CombinePull(self, out=None, async_=False):
+        """-> (code, the members' values concatenated)"""
+        if out is None:
+            out = np.empty(self.n, np.float32)
+        rc = lib().krk_dense_group_pull(self.h, _ptr(out), _flags(out, extra=ASYNC if async_ else 0))
+        return rc, out
+
+    def CombinePush(self, optim, grads, lr, async_=False):
+        if not isinstance(grads, DeviceArray):
+            grads = np.ascontiguousarray(grads, dtype=np.float32).ravel()
+        return lib().krk_dense_group_push(self.h, C.byref(optim.raw), _ptr(grads), grads.size, lr,
+                                          _flags(grads, extra=ASYNC if async_ else 0))
 
 
 def dedup(ids):

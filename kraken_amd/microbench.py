@@ -284,6 +284,49 @@ def dense():
         t.close()
 
 
+def dense_group():
+    print("# dense parameters of one model, Adam: 40 tables (2 x 150k, 6 x 16k, 32 x 64..2048) table by table and")
+    print("# as one combined request (krk_dense_group_pull / _push)")
+    rng = np.random.default_rng(0)
+    sizes = [150_000, 150_000] + [16_384] * 6 + [int(x) for x in rng.integers(64, 2048, size=32)]
+    tables = [api.DenseTable(np.zeros(n, np.float32)) for n in sizes]
+    o = api.Optim.create(api.OptimType.kAdam)
+    grads = [api.DeviceArray.from_host(np.ones(n, np.float32)) for n in sizes]
+    outs = [api.DeviceArray(n, np.float32) for n in sizes]
+    total = sum(sizes)
+
+    def each_push():
+        for t, g in zip(tables, grads):
+            t.Push(o, g, 1e-3, async_=True)
+
+    def each_pull():
+        for t, d in zip(tables, outs):
+            api.lib().krk_dense_pull(t.h, api._ptr(d), api.DEVICE_PTRS | api.ASYNC)
+
+    def sync_each():
+        for t in tables:
+            t.sync()
+    def wall(fn, reps=20):
+        fn()
+        sync_each()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        sync_each()
+        return (time.perf_counter() - t0) / reps
+    t_each_push, t_each_pull = wall(each_push), wall(each_pull)
+    grp = api.DenseGroup(tables)
+    d_g, d_out = api.DeviceArray.from_host(np.ones(total, np.float32)), api.DeviceArray(total, np.float32)
+    t_push = timed(grp, lambda: grp.CombinePush(o, d_g, 1e-3, async_=True), 20)
+    t_pull = timed(grp, lambda: grp.CombinePull(out=d_out, async_=True), 20)
+    print("%d tables, %d parameters | push: one call a table %7.1f us (wall clock; the tables' streams run side by side), "
+          "combined %6.1f us | pull: one call a table %7.1f us, combined %6.1f us" % (
+              len(sizes), total, t_each_push * 1e6, t_push * 1e6, t_each_pull * 1e6, t_pull * 1e6), flush=True)
+    grp.close()
+    for t in tables:
+        t.close()
+
+
 def dct():
     print("# blockwise DCT-II, block 256, n = 4096 x 16384: 2 n keep flop, 4 (n + n keep / 256) bytes")
     n = 4096 * 16384
@@ -684,7 +727,7 @@ def legs():
         print(fn.__name__, json.dumps(fn()), flush=True)
 
 
-SECTIONS = {"legs": legs, "lines": lines, "copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dct2": dct, "hooks": hooks}
+SECTIONS = {"legs": legs, "lines": lines, "copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dense_group": dense_group, "dct2": dct, "hooks": hooks}
 
 
 def main(argv):

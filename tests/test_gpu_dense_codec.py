@@ -217,3 +217,56 @@ def test_dense_push_coo_large(api, oracle):
     one = np.ones(2, np.float32)
     assert t.PushCoo(o_gpu, bad, one, 0.01) == 0 and r.push_coo(o_ref, bad[:1], one[:1], 0.01) == 0
     assert_close(t.Pull()[1], r.pull(), "after an out-of-range entry")
+
+
+_GROUP_CASES = [c for c in OPTIM_CASES if c[0] in ("sgd_mom", "adagrad_wd", "adam", "adam_amsgrad", "rmsprop_all")]
+
+
+@pytest.mark.parametrize("name,type_,conf", _GROUP_CASES, ids=[c[0] for c in _GROUP_CASES])
+def test_dense_group_matches_the_per_table_loop(api, oracle, name, type_, conf):
+    """Ps::CombinePullDenseTable (ps/ps_op.cc:177-252) and a step's PushDenseTable calls for every
+    dense parameter of a model, as one launch each: against the oracle's loop over the tables.
+    Member sizes put some members off the 16-byte grid of the concatenated arrays (the scalar
+    path), one member is empty, 40 members take two launches, and a member that was updated on its
+    own before joining keeps its own Adam step count."""
+    rng = np.random.default_rng(type_ + 40)
+    sizes = [64, 1, 150_000, 4099, 0, 7, 1024, 333] + [int(x) for x in rng.integers(1, 3000, size=32)]
+    w0 = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+    tables = [api.DenseTable(w) for w in w0]
+    refs = [oracle.DenseTable(w) for w in w0]
+    o_ref, o_gpu = make_optims(oracle, api, type_, conf)
+    g = (rng.standard_normal(sizes[2]) * 1e-3).astype(np.float32)
+    assert tables[2].Push(o_gpu, g, 0.01) == 0 and refs[2].push(o_ref, g, 0.01) == 0
+    grp = api.DenseGroup(tables)
+    assert grp.n == sum(sizes)
+    for step in range(3):
+        grads = (rng.standard_normal(grp.n) * 1e-3).astype(np.float32)
+        assert grp.CombinePush(o_gpu, grads, 0.01) == 0
+        at = 0
+        for r, n in zip(refs, sizes):
+            if n:
+                assert r.push(o_ref, grads[at:at + n], 0.01) == 0
+            at += n
+        if step == 1:    # a member's own call in between is ordered with the group's
+            g = (rng.standard_normal(sizes[3]) * 1e-3).astype(np.float32)
+            assert tables[3].Push(o_gpu, g, 0.01) == 0 and refs[3].push(o_ref, g, 0.01) == 0
+    rc, got = grp.CombinePull()
+    assert rc == 0
+    want = np.concatenate([r.pull() for r in refs])
+    assert_close(got, want, name + " combined pull")
+    for t, r, n in zip(tables, refs, sizes):
+        if n:
+            assert np.array_equal(t.Pull()[1], got[sum(sizes[:tables.index(t)]):][:n])
+            for st in STATE_OF[type_]:
+                ws = r.state(st)
+                assert_close(t.state(st), ws if ws is not None else np.zeros(n, np.float32), "%s state %d" % (name, st))
+    if type_ == 1:
+        assert [t.steps for t in tables if t.n] == [r.steps for r, n in zip(refs, sizes) if n]
+        assert tables[2].steps == 4 and tables[3].steps == 4
+    # the wrong total is the reference's code 11; device pointers work the same way
+    assert grp.CombinePush(o_gpu, np.zeros(grp.n - 1, np.float32), 0.01) == 11
+    d_out = api.DeviceArray(grp.n, np.float32)
+    assert grp.CombinePull(out=d_out, async_=True)[0] == 0 and grp.sync() == 0
+    assert np.array_equal(d_out.to_host(), got)
+    grp.close()
+    assert tables[0].Pull()[0] == 0       # members work on their own again
