@@ -31,6 +31,8 @@ int32_t hip_fail(hipError_t e, const char* what, const char* file, int line);
 
 int32_t ensure_runtime();
 int current_device();
+// Resolves, for the current device, the address of the fixed work space krk_dedup_noalloc uses.
+int32_t noalloc_prepare();
 
 // A device buffer that only ever grows; used for staging and scratch.
 struct DeviceBuffer {

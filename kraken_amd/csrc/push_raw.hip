@@ -1504,6 +1504,17 @@ static int32_t noalloc_scratch(unsigned char** out) {
   return KRK_SUCCESS;
 }
 
+// Called when the library binds a device (krk_runtime_init, or the first call of anything): the
+// array's address is resolved there, with whatever that costs the runtime the first time (loading
+// the code object, backing the array), so that krk_dedup_noalloc itself finds it ready, also
+// under stream capture.
+}  // extern "C"
+int32_t krk::noalloc_prepare() {
+  unsigned char* base = nullptr;
+  return noalloc_scratch(&base);
+}
+extern "C" {
+
 int32_t krk_dedup_noalloc(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv,
                           int64_t* n_unique, void* stream) {
   if (n < 0 || !n_unique || (n > 0 && (!ids || !uids))) return KRK_E_ARGUMENT;

@@ -47,6 +47,7 @@ static int32_t init_device(int device) {
   }
   KRK_HIP(hipSetDevice(device));
   g_device = device;
+  KRK_TRY(noalloc_prepare());
   g_ready = true;
   return KRK_SUCCESS;
 }

@@ -61,10 +61,18 @@ inline const krk_optim* ToKrkOptim(Optim* optim) {
 // Page-locked host blocks for replies and gradients. A reply's rows are views of one such block,
 // which the GPU writes across PCIe in place (no device-side staging, no pageable copy: a pull of
 // 8192 rows of 16 floats takes 27 us instead of 58); the block goes back to the pool when the last
-// Tensor of the reply is gone. Blocks are powers of two from 64 KB; a few of each size are kept.
+// Tensor of the reply is gone. Blocks are powers of two from 64 KB. Page-locking and releasing
+// memory takes milliseconds and waits for the device, so the request path should almost never do
+// either: a request takes the smallest idle block that holds it (up to eight times its size, so
+// that requests of varying size share blocks), and the pool keeps idle blocks up to kMaxIdleBytes
+// in all and kMaxIdlePerSize of one size; beyond that a returned block is released.
 class PinnedPool {
+  static constexpr size_t kMinBlock = 64 * 1024;
+  static constexpr size_t kMaxIdleBytes = (size_t)1 << 30;
+  static constexpr int kMaxIdlePerSize = 8;
   std::mutex mu_;
   std::vector<std::pair<void*, size_t>> free_;
+  size_t idle_bytes_ = 0;
 
  public:
   ~PinnedPool() {
@@ -72,18 +80,22 @@ class PinnedPool {
   }
   // nullptr when page-locked memory cannot be had: the caller falls back to ordinary memory
   void* Take(size_t bytes, size_t* size) {
-    size_t want = 64 * 1024;
+    size_t want = kMinBlock;
     while (want < bytes) want <<= 1;
     {
       std::lock_guard<std::mutex> lk(mu_);
+      size_t best = free_.size();
       for (size_t i = 0; i < free_.size(); ++i) {
-        if (free_[i].second == want) {
-          void* p = free_[i].first;
-          free_[i] = free_.back();
-          free_.pop_back();
-          *size = want;
-          return p;
-        }
+        const size_t have = free_[i].second;
+        if (have >= want && have <= 8 * want && (best == free_.size() || have < free_[best].second)) best = i;
+      }
+      if (best != free_.size()) {
+        void* p = free_[best].first;
+        *size = free_[best].second;
+        idle_bytes_ -= *size;
+        free_[best] = free_.back();
+        free_.pop_back();
+        return p;
       }
     }
     void* p = nullptr;
@@ -94,8 +106,11 @@ class PinnedPool {
   void Give(void* p, size_t size) {
     {
       std::lock_guard<std::mutex> lk(mu_);
-      if (free_.size() < 16) {
+      int same = 0;
+      for (auto& b : free_) same += b.second == size;
+      if (same < kMaxIdlePerSize && idle_bytes_ + size <= kMaxIdleBytes) {
         free_.emplace_back(p, size);
+        idle_bytes_ += size;
         return;
       }
     }

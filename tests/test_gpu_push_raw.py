@@ -226,3 +226,65 @@ def test_dedup_sum_random_gradients_and_device_arrays(api, oracle):
     bad[5] = count + 3
     rc, _ = api.expand_rows(got, bad)
     assert rc == api.E_ARGUMENT
+
+
+@pytest.mark.parametrize("dim", [5, 16, 64])
+@pytest.mark.parametrize("shape", ["one_id", "one_bucket", "long_and_short", "boundary"])
+def test_push_raw_short_path_extremes(api, oracle, dim, shape):
+    """Requests of at most 8192 ids take the two-launch path (one workgroup per bucket of rows, LDS
+    sort, runs above 64 positions shared out over the workgroup). Its corners, against the oracle's
+    dedup + sum + push: 8192 copies of one id (one run that fills the bucket), 8192 distinct rows that
+    all fall into one bucket (the workgroup's arrays at their fullest), long runs next to short ones
+    at an odd row width, and the same ids as a request of 8192 and of 8193 (the second takes the
+    path of large requests). Dyadic gradients: exact whatever the order of additions. Random
+    gradients: the long runs are added as per-lane-group stretches combined in a fixed tree, not
+    strictly in position order, so they are held to the float64 sum."""
+    rng = np.random.default_rng(dim * 10 + len(shape))
+    gi = api.Initializer.create(api.InitializerType.kConstant, {"value": "1"})
+    t = api.SparseTable(dim, gi)
+    r = oracle.SparseTable(dim, oracle.init(oracle.INIT_CONSTANT, 1.0))
+    o_ref, o_gpu = make_optims(oracle, api, 0, {})          # Adagrad: a non-linear update
+    if shape == "one_id":
+        requests = [np.full(8192, 4242, np.uint64)]
+    elif shape == "one_bucket":
+        pool = splitmix64(np.arange(300_000, dtype=np.uint64))
+        t.Pull(pool)
+        r.pull(pool)
+        rows = t.lookup(pool)
+        same = pool[rows % 32 == 0][:8192]                    # the short path's buckets are row mod 8..32
+        assert same.size == 8192
+        requests = [same]
+    elif shape == "long_and_short":
+        hot = splitmix64(np.arange(5, dtype=np.uint64))
+        ids = np.concatenate([np.repeat(hot, [3000, 900, 65, 64, 63]), splitmix64(np.arange(100, 4200, dtype=np.uint64))])
+        requests = [ids[rng.permutation(ids.size)]]
+    else:
+        base = zipf_ids(rng, 1.05, 10**5, 8193)
+        requests = [base[:8192], base]
+    for ids in requests:
+        t.Pull(ids)
+        r.pull(ids)
+        for grads in (_dyadic_grads(rng, (ids.size, dim)),
+                      (rng.standard_normal((ids.size, dim)) * 1e-2).astype(np.float32)):
+            assert t.PushRaw(o_gpu, ids, grads, 0.05) == 0
+            u, gs = oracle.dedup_sum(ids, grads)
+            assert r.push(o_ref, u, gs, 0.05) == 0
+            got, want = t.Pull(u)[1], r.pull(u)[1]
+            if grads is not None and np.array_equal(grads * 4096, np.round(grads * 4096)):
+                assert_close(got, want, "%s dim %d, dyadic" % (shape, dim), rtol=1e-6, atol=1e-7)
+            else:
+                # the two orders of fp32 additions differ by a few ulps of the mass that was added
+                assert_close(got, want, "%s dim %d, random" % (shape, dim), rtol=1e-5, atol=1e-6)
+    # SGD makes the sum itself visible: against the float64 sum of the long runs
+    if shape in ("one_id", "long_and_short"):
+        ids = requests[0]
+        grads = (rng.standard_normal((ids.size, dim)) * 1e-2).astype(np.float32)
+        before = t.Pull(np.unique(ids))[1].astype(np.float64)
+        assert t.PushRaw(api.Optim.create(api.OptimType.kSGD), ids, grads, 1.0) == 0
+        u, inv = np.unique(ids, return_inverse=True)
+        exact = np.zeros((u.size, dim), np.float64)
+        mass = np.zeros((u.size, dim), np.float64)
+        np.add.at(exact, inv, grads.astype(np.float64))
+        np.add.at(mass, inv, np.abs(grads).astype(np.float64))
+        after = t.Pull(u)[1].astype(np.float64)
+        assert (np.abs((before - after) - exact) <= 4e-7 * mass + 2e-7 * np.abs(before) + 1e-30).all()
