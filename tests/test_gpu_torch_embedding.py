@@ -234,10 +234,13 @@ def test_modules_take_the_reference_descriptions(mods, oracle):
     """Initializers and optimizers given as the reference's Python classes
     (pytorch/initializer.py, pytorch/optim.py) reach the engine with the same meaning."""
     api, te = mods
-    from kraken_amd import configs
+
+    class Described:       # what kraken.pytorch.initializer / optim objects answer
+        def __init__(self, type_, conf):
+            self.type, self.conf = (lambda: type_), (lambda: conf)
     dim = 4
-    emb = te.Embedding(dim, initializer=configs.ConstantInitializer(0.5),
-                       optim=configs.Adagrad(eps=1e-6), lr=0.25)
+    emb = te.Embedding(dim, initializer=Described(0, {"value": "0.5"}),        # ConstantInitializer(0.5)
+                       optim=Described(0, {"eps": "1e-06"}), lr=0.25)          # Adagrad(eps=1e-6)
     ref = oracle.SparseTable(dim, oracle.init(oracle.INIT_CONSTANT, 0.5, 0.0))
     o_ref, _ = make_optims(oracle, api, 0, {"eps": 1e-6})
     ids = np.array([5, 9, 5, 2], np.uint64)
