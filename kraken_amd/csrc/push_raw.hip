@@ -838,7 +838,11 @@ constexpr int kMaxBucketBits = 5;                      // up to 32 buckets a tab
 constexpr int kDigitBits = 9;
 constexpr int kDigits = 1 << kDigitBits;
 constexpr int kRunAhead = 8;                           // gradient rows requested ahead of the sums
-constexpr int kLongRun = 64;                           // runs longer than this are shared out over the workgroup
+constexpr int kShortRun = 16;                          // runs up to this length: one lane group each
+constexpr int kWaveRunPerGroup = 16;                   // a wavefront takes runs of up to this many entries per lane group;
+                                                       // longer runs are shared out over the whole workgroup
+constexpr int kRunListMax = kSortMax / (kShortRun + 1) + 1;   // runs above kShortRun a bucket can hold
+constexpr int kPartOffset = (kSortMax + 1 + 2 * kRunListMax + 3) & ~3;   // the partial sums start on 16 bytes
 constexpr int kShortMaxDim = 64;
 static_assert(kSortWaves * kDigits <= kSortMax + 1, "the histogram fits the work space");
 
@@ -898,7 +902,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
   // histogram [wave][digit] while sorting; partial sums and their keys while reducing
   // histogram [wave][digit] while sorting; then run starts, the list of long runs, and the
   // wavefronts' partial sums of a long run
-  __shared__ uint32_t work[kSortMax + 1 + kSortMax / kLongRun + 1 + kSortWaves * kWave * 4];
+  __shared__ __align__(16) uint32_t work[kPartOffset + kSortWaves * kWave * 4];
   __shared__ uint32_t wave_total[kSortWaves];
   const int mb = blockIdx.x;
   const int bucket_bits = call.bucket_bits;
@@ -1027,8 +1031,9 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
 
   // ---- c. runs of equal rows: sums in position order, one update per row -----------------------
   uint32_t* run_start = work;                          // [runs + 1]; the histogram is done with
-  uint32_t* long_run = work + kSortMax + 1;            // [<= kSortMax / kLongRun] runs longer than kLongRun
-  __shared__ uint32_t n_long;
+  uint32_t* long_run = work + kSortMax + 1;            // [kRunListMax] runs for the whole workgroup
+  uint32_t* wave_run = long_run + kRunListMax;         // [kRunListMax] runs for one wavefront each
+  __shared__ uint32_t n_long, n_wave;
   uint32_t runs;
   {
     // lane t looks at entries [t * per_lane, (t + 1) * per_lane): where does a new row begin?
@@ -1039,7 +1044,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
       const int j = j0 + i;
       if (i < per_lane && j < len && (j == 0 || skey[j - 1] != skey[j])) heads |= 1u << i;
     }
-    if (t == 0) n_long = 0u;
+    if (t == 0) n_long = n_wave = 0u;
     uint32_t r = sort_block_scan((uint32_t)__popc(heads), wave_total, runs);
 #pragma unroll
     for (int i = 0; i < kSortItems; ++i)
@@ -1052,6 +1057,21 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
   const int gl = t & (group - 1);
   const bool lane_on = gl < elems;
   const float* g_base = grads + a * (int64_t)dim;
+  // Who adds a run up: a lane group (up to kShortRun entries, the reference's order exactly), a
+  // wavefront (its lane groups take a stretch each and the stretches' sums are added in order),
+  // or the whole workgroup. A lane group walking 64 entries on its own took eight trips to memory
+  // while the others waited at the barrier: 10 of the kernel's 30 us for 26 tables of 8192 ids.
+  const int groups_per_wave = kWave / group;
+  const int wave_run_max = kWaveRunPerGroup * groups_per_wave;
+  for (uint32_t q = (uint32_t)t; q < runs; q += kSortBlock) {
+    const int count = (int)(run_start[q + 1] - run_start[q]);
+    if (count > wave_run_max) {
+      long_run[atomicAdd(&n_long, 1u)] = q;
+    } else if (count > kShortRun) {
+      wave_run[atomicAdd(&n_wave, 1u)] = q;
+    }
+  }
+  __syncthreads();
 
   // adds entries [lo, hi) of the sorted list in list order; the first addend is copied, not added
   // to zero (worker/emitter.cc:527 clones it)
@@ -1083,24 +1103,110 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
     }
   };
 
-  // runs of at most kLongRun entries: one lane group each, exactly the reference's order
-  for (uint32_t q = (uint32_t)lt; q < runs; q += (uint32_t)per_block) {
-    const int start = (int)run_start[q], end = (int)run_start[q + 1];
-    if (end - start > kLongRun) {
-      if (gl == 0) long_run[atomicAdd(&n_long, 1u)] = q;
-      continue;
+  // Runs of at most kShortRun entries: one lane group each, exactly the reference's order. A lane
+  // group takes two runs at a time: both records and the first kPairAhead gradient rows of both
+  // are requested before anything is added, so a round costs one trip to memory for two rows (a
+  // bucket's workgroup has 256 lane groups for some 500 runs, and the trips were most of the
+  // phase: 13 of 39 us for 26 tables of 8192 ids).
+  constexpr int kPairAhead = 2;
+  auto request_head = [&](int lo, int hi, float (&v)[kPairAhead][VEC]) {
+#pragma unroll
+    for (int u = 0; u < kPairAhead; ++u) {
+      if (lo + u < hi && lane_on) {
+        vload<VEC>(g_base + (int64_t)spos[lo + u] * dim + gl * VEC, v[u]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) v[u][c] = 0.0f;
+      }
     }
-    const uint32_t row = (skey[start] << bucket_bits) | bucket;
-    RowRegs<VEC> rec;
-    load_row<OPT, VEC>(tv, row, gl, lane_on, args, rec);   // on its way while the gradients are added
-    float acc[VEC];
-    sum_entries(start, end, acc);
-    finish_row<OPT, VEC>(tv, row, acc, gl, lane_on, gl, true, dim, args, rec);
+  };
+  // the head's rows first (already requested), then the rest of the run in chunks
+  auto sum_from_head = [&](int lo, int hi, const float (&v)[kPairAhead][VEC], float (&acc)[VEC]) {
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) acc[c] = v[0][c];      // the first addend is copied (emitter.cc:527)
+#pragma unroll
+    for (int u = 1; u < kPairAhead; ++u) {
+      if (lo + u < hi) {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) acc[c] = acc[c] + v[u][c];
+      }
+    }
+    for (int j0 = lo + kPairAhead; j0 < hi; j0 += kRunAhead) {
+      float w[kRunAhead][VEC];
+#pragma unroll
+      for (int u = 0; u < kRunAhead; ++u) {
+        if (j0 + u < hi && lane_on) {
+          vload<VEC>(g_base + (int64_t)spos[j0 + u] * dim + gl * VEC, w[u]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) w[u][c] = 0.0f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kRunAhead; ++u) {
+        if (j0 + u >= hi) break;
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) acc[c] = acc[c] + w[u][c];
+      }
+    }
+  };
+  // runs for one wavefront each: lane group i of the wavefront adds the i-th stretch, then the
+  // stretches' sums are added in order inside the wavefront (neighbours first, by doubling)
+  {
+    const int sub = lane / group;
+    const uint32_t waves_runs = n_wave;
+    for (uint32_t k = (uint32_t)wave; k < waves_runs; k += kSortWaves) {
+      const uint32_t q = wave_run[k];                  // in any order: the runs are different rows
+      const int first = (int)run_start[q], count = (int)run_start[q + 1] - first;
+      const int stretch = (count + groups_per_wave - 1) / groups_per_wave;
+      const int lo = first + sub * stretch < first + count ? first + sub * stretch : first + count;
+      const int hi = lo + stretch < first + count ? lo + stretch : first + count;
+      const uint32_t row = (skey[first] << bucket_bits) | bucket;
+      RowRegs<VEC> rec;
+      if (sub == 0) load_row<OPT, VEC>(tv, row, gl, lane_on, args, rec);
+      float acc[VEC];
+      sum_entries(lo, hi, acc);
+      for (int d = group; d < kWave; d <<= 1) {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+          const float other = __shfl_down(acc[c], d);
+          if ((sub & ((2 * d / group) - 1)) == 0) acc[c] = acc[c] + other;
+        }
+      }
+      if (sub == 0) finish_row<OPT, VEC>(tv, row, acc, gl, lane_on, gl, true, dim, args, rec);
+    }
+  }
+  for (uint32_t q0 = (uint32_t)lt; q0 < runs; q0 += 2u * (uint32_t)per_block) {
+    int start[2], end[2];
+    bool on[2];
+    uint32_t row[2];
+    RowRegs<VEC> rec[2];
+    float head[2][kPairAhead][VEC];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const uint32_t q = q0 + (uint32_t)h * (uint32_t)per_block;
+      on[h] = q < runs;
+      start[h] = on[h] ? (int)run_start[q] : 0;
+      end[h] = on[h] ? (int)run_start[q + 1] : 0;
+      if (on[h] && end[h] - start[h] > kShortRun) on[h] = false;   // a wavefront's or the workgroup's
+      row[h] = on[h] ? ((skey[start[h]] << bucket_bits) | bucket) : 0u;
+      if (on[h]) {
+        load_row<OPT, VEC>(tv, row[h], gl, lane_on, args, rec[h]);
+        request_head(start[h], end[h], head[h]);
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (!on[h]) continue;
+      float acc[VEC];
+      sum_from_head(start[h], end[h], head[h], acc);
+      finish_row<OPT, VEC>(tv, row[h], acc, gl, lane_on, gl, true, dim, args, rec[h]);
+    }
   }
   __syncthreads();
   // hot ids: every lane group adds a stretch of the run; the stretches' sums are added in order,
   // first inside each wavefront (neighbouring lane groups, by doubling), then across wavefronts
-  float* part = reinterpret_cast<float*>(work + kSortMax + 1 + kSortMax / kLongRun + 1);   // [kSortWaves][group * VEC]
+  float* part = reinterpret_cast<float*>(work + kPartOffset);   // [2][kSortWaves][group * VEC]
   const uint32_t longs = n_long;
   const int lane_floats = group * VEC;
   for (uint32_t k = 0; k < longs; ++k) {
