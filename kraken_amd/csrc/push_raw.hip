@@ -53,6 +53,29 @@ __device__ __forceinline__ void vstore_once(float* p, const float (&v)[VEC]) {
     __builtin_nontemporal_store(v[0], p);
   }
 }
+// The same accesses through pointers the compiler is told lie in global memory. A table's record
+// pointer that a kernel reads out of a descriptor is a generic pointer to the compiler, which
+// then uses flat instructions; those count as LDS operations too, so every wait for an LDS read
+// (the sorted positions, the run starts) would also wait for the records requested before it.
+#define KRK_GLOBAL __attribute__((address_space(1)))
+template <int VEC>
+__device__ __forceinline__ void gload(const float* p, float (&v)[VEC]) {
+  if constexpr (VEC == 4) {
+    const vfloat4_t x = *(const KRK_GLOBAL vfloat4_t*)p;
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  } else {
+    v[0] = *(const KRK_GLOBAL float*)p;
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void gstore_once(float* p, const float (&v)[VEC]) {
+  if constexpr (VEC == 4) {
+    const vfloat4_t x = {v[0], v[1], v[2], v[3]};
+    __builtin_nontemporal_store(x, (KRK_GLOBAL vfloat4_t*)p);
+  } else {
+    __builtin_nontemporal_store(v[0], (KRK_GLOBAL float*)p);
+  }
+}
 template <int VEC>
 __device__ __forceinline__ void vstore(float* p, const float (&v)[VEC]) {
   if constexpr (VEC == 4) {
@@ -388,10 +411,10 @@ __device__ __forceinline__ void load_row(const TableView& tv, uint32_t row, int 
   if constexpr (OPT == kOptStore) return;
   const float* rec = tv.recs + (int64_t)row * tv.stride;
   if (lane_on) {
-    vload<VEC>(rec + e * VEC, r.w);
-    if (a.c0 >= 0) vload<VEC>(rec + a.c0 + e * VEC, r.s0);
-    if (a.c1 >= 0) vload<VEC>(rec + a.c1 + e * VEC, r.s1);
-    if (a.c2 >= 0) vload<VEC>(rec + a.c2 + e * VEC, r.s2);
+    gload<VEC>(rec + e * VEC, r.w);
+    if (a.c0 >= 0) gload<VEC>(rec + a.c0 + e * VEC, r.s0);
+    if (a.c1 >= 0) gload<VEC>(rec + a.c1 + e * VEC, r.s1);
+    if (a.c2 >= 0) gload<VEC>(rec + a.c2 + e * VEC, r.s2);
   }
 }
 
@@ -409,7 +432,7 @@ __device__ __forceinline__ void finish_row(const TableView& tv, uint32_t row, co
   float bc1 = 1.0f, bc2 = 1.0f;
   uint64_t steps = 0;
   if (a.meta_off >= 0) {
-    const uint32_t* meta = reinterpret_cast<const uint32_t*>(rec + a.meta_off);
+    const KRK_GLOBAL uint32_t* meta = (const KRK_GLOBAL uint32_t*)(rec + a.meta_off);
     steps = (uint64_t)meta[0] | ((uint64_t)meta[1] << 32);
     if (OPT == KRK_ADAM) {
       steps += 1;                           // the flag bit rides along untouched
@@ -433,10 +456,10 @@ __device__ __forceinline__ void finish_row(const TableView& tv, uint32_t row, co
     }
     // a record is written once per request: past the caches, so the kernel ends with no dirty
     // lines to write back
-    vstore_once<VEC>(rec + e * VEC, r.w);
-    if (a.c0 >= 0) vstore_once<VEC>(rec + a.c0 + e * VEC, r.s0);
-    if (a.c1 >= 0) vstore_once<VEC>(rec + a.c1 + e * VEC, r.s1);
-    if (a.c2 >= 0) vstore_once<VEC>(rec + a.c2 + e * VEC, r.s2);
+    gstore_once<VEC>(rec + e * VEC, r.w);
+    if (a.c0 >= 0) gstore_once<VEC>(rec + a.c0 + e * VEC, r.s0);
+    if (a.c1 >= 0) gstore_once<VEC>(rec + a.c1 + e * VEC, r.s1);
+    if (a.c2 >= 0) gstore_once<VEC>(rec + a.c2 + e * VEC, r.s2);
   }
   // The counter is read by every chunk of the row before the last chunk advances it.
   if (a.meta_off >= 0 && last_chunk) store_row_word<VEC>(rec + a.meta_off, steps, gl, dim, (int)tv.stride - a.meta_off);
@@ -867,6 +890,13 @@ __device__ __forceinline__ unsigned long long match_digit(uint32_t digit) {
   return same;
 }
 
+// A barrier for phases that exchange data through LDS only: waits for the wavefront's LDS
+// operations, not for its global loads and stores as __syncthreads() does. (Requesting the
+// records' lines ahead of the sort, behind such barriers, was measured too: no gain.)
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // exclusive prefix sum of one value per lane over the workgroup (1024 lanes); total to all
 __device__ __forceinline__ uint32_t sort_block_scan(uint32_t v, uint32_t* wave_total, uint32_t& total) {
   const int lane = threadIdx.x & (kWave - 1);
@@ -877,9 +907,9 @@ __device__ __forceinline__ uint32_t sort_block_scan(uint32_t v, uint32_t* wave_t
     const uint32_t y = __shfl_up(incl, d);
     if (lane >= d) incl += y;
   }
-  __syncthreads();                                     // wave_total may still be read from a previous scan
+  lds_barrier();                                     // wave_total may still be read from a previous scan
   if (lane == kWave - 1) wave_total[wave] = incl;
-  __syncthreads();
+  lds_barrier();
   uint32_t offset = incl - v;
   uint32_t sum = 0;
   for (int w = 0; w < kSortWaves; ++w) {
@@ -960,7 +990,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
     skey[j] = 0xFFFFFFFFu;                             // padding sorts behind everything
     spos[j] = 0;
   }
-  __syncthreads();
+  lds_barrier();
 
   // ---- b. stable radix sort by row -----------------------------------------------------------
   // element i of lane l in wavefront w is pair w * 64 * per_lane + i * 64 + l: a wavefront's
@@ -984,7 +1014,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
         }
       }
       for (int i = t; i < kSortWaves * kDigits; i += kSortBlock) hist[i] = 0u;
-      __syncthreads();                                 // everyone holds its pairs; the histogram is clear
+      lds_barrier();                                 // everyone holds its pairs; the histogram is clear
 #pragma unroll
       for (int i = 0; i < kSortItems; ++i) {
         if (i < per_lane) {                            // uniform
@@ -998,7 +1028,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
           rank[i] = old + before;
         }
       }
-      __syncthreads();
+      lds_barrier();
       // exclusive scan over (digit, wavefront): lane t owns digit t / 2, wavefronts 8 (t % 2) .. + 7
       {
         const int digit = t >> 1;
@@ -1016,7 +1046,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
           offset += c[k];
         }
       }
-      __syncthreads();
+      lds_barrier();
 #pragma unroll
       for (int i = 0; i < kSortItems; ++i) {
         if (i < per_lane) {
@@ -1025,7 +1055,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
           spos[dest] = pos[i];
         }
       }
-      __syncthreads();
+      lds_barrier();
     }
   }
 
@@ -1050,7 +1080,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
     for (int i = 0; i < kSortItems; ++i)
       if (heads & (1u << i)) run_start[r++] = (uint32_t)(j0 + i);
     if (t == 0) run_start[runs] = (uint32_t)len;
-    __syncthreads();
+    lds_barrier();
   }
   const int per_block = kSortBlock / group;
   const int lt = t / group;
@@ -1071,7 +1101,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
       wave_run[atomicAdd(&n_wave, 1u)] = q;
     }
   }
-  __syncthreads();
+  lds_barrier();
 
   // adds entries [lo, hi) of the sorted list in list order; the first addend is copied, not added
   // to zero (worker/emitter.cc:527 clones it)
@@ -1083,7 +1113,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
 #pragma unroll
       for (int u = 0; u < kRunAhead; ++u) {
         if (j0 + u < hi && lane_on) {
-          vload<VEC>(g_base + (int64_t)spos[j0 + u] * dim + gl * VEC, v[u]);
+          gload<VEC>(g_base + (int64_t)spos[j0 + u] * dim + gl * VEC, v[u]);
         } else {
 #pragma unroll
           for (int c = 0; c < VEC; ++c) v[u][c] = 0.0f;
@@ -1113,7 +1143,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
 #pragma unroll
     for (int u = 0; u < kPairAhead; ++u) {
       if (lo + u < hi && lane_on) {
-        vload<VEC>(g_base + (int64_t)spos[lo + u] * dim + gl * VEC, v[u]);
+        gload<VEC>(g_base + (int64_t)spos[lo + u] * dim + gl * VEC, v[u]);
       } else {
 #pragma unroll
         for (int c = 0; c < VEC; ++c) v[u][c] = 0.0f;
@@ -1136,7 +1166,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
 #pragma unroll
       for (int u = 0; u < kRunAhead; ++u) {
         if (j0 + u < hi && lane_on) {
-          vload<VEC>(g_base + (int64_t)spos[j0 + u] * dim + gl * VEC, w[u]);
+          gload<VEC>(g_base + (int64_t)spos[j0 + u] * dim + gl * VEC, w[u]);
         } else {
 #pragma unroll
           for (int c = 0; c < VEC; ++c) w[u][c] = 0.0f;
