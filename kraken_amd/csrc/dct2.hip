@@ -50,6 +50,7 @@ __global__ void dct2_basis_kernel(float* __restrict__ fwd, float* __restrict__ i
 // step j multiplies them against basis rows 32 s + 16 h + j. Wavefronts never wait on each
 // other inside the loop; the next slice's loads are in flight while this one multiplies.
 //
+// (This kernel serves the 64-column tiles, keep = 64 and 192.)
 // A tile's results are not stored when the tile is done: the two wavefronts that share a SIMD
 // run in step, so both would store while the matrix pipe idles (10 % of the kernel's time).
 // They are kept in registers and leave between the multiplies of the next tile's first two
@@ -192,6 +193,103 @@ __global__ __launch_bounds__(kThreads) void dct2_gemm_kernel(const float* __rest
   }
 }
 
+// The 128-column tiles run with sixteen wavefronts a workgroup (four per SIMD instead of two): a
+// wavefront keeps 128 registers, so a tile's results are stored as soon as the tile is done
+// (no copy of them survives into the next tile) and X runs one slice ahead, not two. What the
+// wavefronts of a SIMD lose while one of them stores, the other three fill in. Against the
+// eight-wavefront kernel above at the same tile width: keep 128 forward 160 -> 152 us, inverse
+// 175 -> 160 us; keep 256 is the same 302 us either way (113 TFLOP/s: with four wavefronts a SIMD
+// the matrix pipe is not waiting for anybody any more, and the rate still moves with the operand
+// values, which is what a clock held down by power looks like).
+constexpr int kThreads16 = 1024;
+constexpr int kTileM16 = 512;
+
+template <int NT>
+__global__ __launch_bounds__(kThreads16) void dct2_gemm16_kernel(const float* __restrict__ X, int64_t ldx,
+                                                                 const float* __restrict__ Bm, int ldb,
+                                                                 float* __restrict__ Y, int64_t ldy,
+                                                                 int64_t M, int K) {
+  typedef typename BasisVec<NT>::type bvec;
+  constexpr int kTileN = 32 * NT;
+  extern __shared__ float Bs[];                     // [K + kPadRows][32][NT]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int r = lane & 31;
+  const int h = lane >> 5;
+  const int n0 = blockIdx.y * kTileN;
+
+  for (int i = tid; i < K * (kTileN / 4); i += kThreads16) {
+    const int br = i / (kTileN / 4);
+    const int c4 = i - br * (kTileN / 4);
+    const float4 v = *reinterpret_cast<const float4*>(Bm + (size_t)br * ldb + n0 + c4 * 4);
+    const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = c4 * 4 + u;
+      Bs[br * kTileN + (c & 31) * NT + (c >> 5)] = e[u];
+    }
+  }
+  __syncthreads();
+
+  const int64_t tiles = (M + kTileM16 - 1) / kTileM16;
+  const int slices = K / kSliceK;
+  auto row_ptr = [&](int64_t tile) {
+    int64_t row = tile * kTileM16 + wave * 32 + r;
+    if (row >= M) row = M - 1;
+    return X + row * ldx + 16 * h;
+  };
+  const float* bs = Bs + (size_t)(16 * h) * kTileN + r * NT;
+  const float* xrow = row_ptr(blockIdx.x);
+  float4 cur[4], nxt[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) cur[q] = reinterpret_cast<const float4*>(xrow)[q];
+  v16f acc[NT];
+  bvec bcur, bnxt;
+
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const float* xnext = row_ptr(tile + gridDim.x < tiles ? tile + gridDim.x : tile);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = v16f{0};
+    bcur = *reinterpret_cast<const bvec*>(bs);
+    for (int s = 0; s < slices; ++s) {
+      // the next slice of this tile, or the first slice of the next tile
+      const float* ahead = s + 1 < slices ? xrow + (s + 1) * kSliceK : xnext;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) nxt[q] = reinterpret_cast<const float4*>(ahead)[q];
+      __builtin_amdgcn_sched_barrier(0);            // keep the requests ahead of the multiplies
+      const float* brow = bs + (size_t)s * kSliceK * kTileN;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float a4[4] = {cur[q].x, cur[q].y, cur[q].z, cur[q].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int j = q * 4 + e;
+          bnxt = *reinterpret_cast<const bvec*>(brow + (j < 15 ? (j + 1) * kTileN : kSliceK * kTileN));
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[e], bcur[t], acc[t], 0, 0, 0);
+          bcur = bnxt;
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) cur[q] = nxt[q];
+    }
+    // accumulator element i of lane l is C[(i / 4) * 8 + (l / 32) * 4 + i % 4][l % 32]
+    const int64_t base = tile * kTileM16 + wave * 32;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int64_t orow = base + (i >> 2) * 8 + h * 4 + (i & 3);
+      if (orow < M) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) Y[orow * ldy + n0 + r + 32 * t] = acc[t][i];
+      }
+    }
+    xrow = xnext;
+  }
+}
+
 static std::mutex g_basis_mu;
 static float* g_basis_fwd = nullptr;
 static float* g_basis_inv = nullptr;
@@ -251,13 +349,28 @@ static int32_t dct2_run(const float* in, float* out, int64_t n, int32_t keep, ui
   int64_t gx = 256 * per_cu / (N / tile_n);
   if (gx > tiles) gx = tiles;
   if (gx < 1) gx = 1;
-  auto kernel = nt == 4 ? dct2_gemm_kernel<4> : dct2_gemm_kernel<2>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-  if (e == hipSuccess) {
-    hipLaunchKernelGGL(kernel, dim3((unsigned)gx, (unsigned)(N / tile_n)), dim3(kThreads), lds_bytes, s,
-                       d_in, (int64_t)K, basis, kDctB, d_out, (int64_t)N, M, K);
-    e = hipGetLastError();
+  hipError_t e;
+  if (nt == 4) {
+    const int64_t tiles16 = (M + kTileM16 - 1) / kTileM16;
+    int64_t gx16 = 256 / (N / tile_n);
+    if (gx16 > tiles16) gx16 = tiles16;
+    if (gx16 < 1) gx16 = 1;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(dct2_gemm16_kernel<4>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(dct2_gemm16_kernel<4>, dim3((unsigned)gx16, (unsigned)(N / tile_n)), dim3(kThreads16),
+                         lds_bytes, s, d_in, (int64_t)K, basis, kDctB, d_out, (int64_t)N, M, K);
+      e = hipGetLastError();
+    }
+  } else {
+    auto kernel = dct2_gemm_kernel<2>;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds_bytes);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(kernel, dim3((unsigned)gx, (unsigned)(N / tile_n)), dim3(kThreads), lds_bytes, s,
+                         d_in, (int64_t)K, basis, kDctB, d_out, (int64_t)N, M, K);
+      e = hipGetLastError();
+    }
   }
   if (e == hipSuccess && host)
     e = hipMemcpy(out, d_out, sizeof(float) * (size_t)out_count, hipMemcpyDeviceToHost);
