@@ -822,7 +822,7 @@ static int pick_tile(int64_t cnt) {
 }
 
 // ---------------------------------------------------------------------------
-// Requests of at most 8192 ids per table: two launches, no carry levels, no library sort.
+// Requests of at most 8192 ids per table: two launches, no carry levels, no global sort.
 //   1. ids -> rows for every position, over the whole chip (rows_of_ids / group_rows_of_ids).
 //   2. bucket_push_kernel, one workgroup of 1024 lanes for each of a table's 8 to 32 buckets
 //      (bucket = row mod the number of buckets; as many as keep the request at about one
@@ -834,11 +834,12 @@ static int pick_tile(int64_t cnt) {
 //         elements with wave-wide votes (lanes holding the same digit find each other through
 //         nine ballots), a per-wavefront histogram in LDS turns into offsets by one scan over
 //         (digit, wavefront), and the pairs are scattered through LDS;
-//      c. the sorted list is cut into one tile per lane group; a group adds the gradient rows of
-//         each run of equal rows in position order (worker/emitter.cc:527-529; eight rows are
-//         requested ahead of the sums) and applies every run that lies inside its tile. Runs
-//         that cross tile borders (hot ids) leave partial sums in LDS, and after a barrier the
-//         group that owns a run's first partial adds the others in order and applies the sum.
+//      c. every run of equal rows is summed in position order (worker/emitter.cc:527-529) and
+//         applied once. Who adds a run up depends on its length: a lane group (up to 16
+//         positions, two runs in flight per group), a wavefront (up to 16 positions per lane
+//         group of it: the groups add a stretch each and the stretches' sums are added in order
+//         inside the wavefront), or the whole workgroup the same way (the very head of a skewed
+//         distribution). The three lists are made in one pass over the run lengths.
 //      Nothing but the row numbers passes through global memory between the stages.
 // Measured on the way here, 8192 Zipf ids, dim 16: the whole push in one workgroup per table
 // 88 us (one compute unit keeps too few random reads in flight for index, gradients and
