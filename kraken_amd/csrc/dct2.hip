@@ -1,4 +1,5 @@
-// Blockwise orthonormal DCT-II / DCT-III over blocks of 256 floats on the fp32 matrix cores.
+// Blockwise orthonormal DCT-II / DCT-III over blocks of 256 floats on the matrix cores, at fp32
+// accuracy.
 //
 // There is NO reference counterpart: the reference's "DCT" emitter is a threshold codec
 // (worker/dct_emitter.cc:16-43) and contains no cosine transform. This file exists because the
@@ -8,10 +9,10 @@
 // each block (keep = B * (1 - eta) = 64 for the emitter's default eta = 0.75) is the compression.
 //
 // Shape of the work: Y[M, N] = X[M, K] * Basis[K, N] with M = n / 256 blocks (forward: K = 256,
-// N = keep; inverse: K = keep, N = 256), folded in half by the basis' mirror symmetry (below) and
-// fed to v_mfma_f32_32x32x2_f32: a workgroup keeps its basis tile resident in LDS and walks over
-// row tiles of 512 blocks; each of its sixteen wavefronts owns 32 rows and holds their X values
-// in registers.
+// N = keep; inverse: K = keep, N = 256), (1) folded in half by the basis' mirror symmetry and
+// (2) multiplied as six bf16 products per fp32 product on v_mfma_f32_32x32x16_bf16, both below.
+// A workgroup keeps its basis tile resident in LDS and walks over row tiles of 512 blocks; each
+// of its sixteen wavefronts owns 32 rows and holds their X values in registers.
 #include <cmath>
 #include <mutex>
 
@@ -27,124 +28,197 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 
-// fwd[j * B + k] = inv[k * B + j] = s_k cos(pi (2j+1) k / (2B)), evaluated in double.
-__global__ void dct2_basis_kernel(float* __restrict__ fwd, float* __restrict__ inv) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= kDctB * kDctB) return;
-  const int k = t / kDctB;
-  const int j = t - k * kDctB;
-  const double s = k == 0 ? sqrt(1.0 / kDctB) : sqrt(2.0 / kDctB);
-  const double v = s * cos(3.14159265358979323846 * (2.0 * j + 1.0) * k / (2.0 * kDctB));
-  fwd[j * kDctB + k] = (float)v;
-  inv[k * kDctB + j] = (float)v;
-}
-
-// The cosine basis is mirror symmetric: c[255 - j][k] = (-1)^k c[j][k]. So the even coefficients
-// of a block are a 128-term sum over x[j] + x[255 - j] and the odd ones over x[j] - x[255 - j]
-// (forward), and a block's values come back as x[j] = E[j] + O[j], x[255 - j] = E[j] - O[j] with
-// E over the even and O over the odd coefficients (inverse): half the multiplies of the plain
-// product, at one more fp32 rounding per input pair (forward) or output pair (inverse).
+// (1) The cosine basis is mirror symmetric: c[255 - j][k] = (-1)^k c[j][k]. So the even
+// coefficients of a block are a 128-term sum over x[j] + x[255 - j] and the odd ones over
+// x[j] - x[255 - j] (forward), and a block's values come back as x[j] = E[j] + O[j],
+// x[255 - j] = E[j] - O[j] with E over the even and O over the odd coefficients (inverse): half
+// the multiplies of the plain product, at one more fp32 rounding per input pair (forward) or
+// output pair (inverse).
 //
 // Shape of the work per workgroup: 512 blocks (rows) by 32 * NT folded columns, each folded
 // column carrying two results (forward: coefficients 2c and 2c + 1; inverse: positions j and
 // 255 - j), so a wavefront owns 32 rows and 2 * NT accumulator tiles, the first NT fed with the
 // first operand of a pair (sum, or even coefficient), the others with the second (difference,
-// or odd coefficient).
-//
-// The basis tile sits in LDS for the whole launch and is only read. It is laid out
-// [KF + kPadRows][32][2 NT]: the 2 NT values a lane needs for one step are one vector read, at an
-// offset from the slice's first row that is known at compile time. X never passes through LDS:
-// the matrix instruction takes, per lane (r = lane % 32, h = lane / 32), one value A[r][k_h] for
-// its two reduction indices k_0, k_1, and the order in which the reduction indices are consumed
-// is free as long as the basis rows follow it. So lane (r, h) holds the operands of 8 or 16
-// consecutive folded indices per slice (two or four float4 from the row and as many from its
-// mirror image) and step e multiplies operand e against the basis row of its index.
+// or odd coefficient). X never passes through LDS: the matrix instruction takes, per lane
+// (r = lane % 32, h = lane / 32), the values A[r][k] of eight reduction indices k, a set that
+// depends on h only, and the order in which the reduction indices are consumed is free as long
+// as the basis follows it. So lane (r, h) holds the operands of 8 or 16 consecutive folded
+// indices per slice (two or four float4 from the row and as many from its mirror image).
 // Sixteen wavefronts a workgroup (four per SIMD, 128 registers each): wavefronts never wait on
 // each other inside the loop, the next slice's loads are in flight while this one multiplies,
 // and what the wavefronts of a SIMD lose while one of them stores its tile, the other three fill in.
 //
-// Measured on fp32 [4096, 16384] against the plain 256-term product this replaces (same tiling,
-// every multiply done): keep 256 forward 302 -> 160-175 us, keep 128 152 -> 93 us, keep 64 93 ->
-// 58 us; inverse 302 -> 166-175, 160 -> 100, 100 -> 61 us. Two wavefronts side by side on the
-// same rows (all of keep 256's columns in one workgroup, X read from memory once) was slower,
-// 200 us: the second read is already served by the L2 the two workgroups of a row tile share.
-constexpr int kPadRows = 17;   // the step after a tile's last one still reads "its" basis rows
+// Measured on fp32 [4096, 16384], forward / inverse, microseconds:
+//                                                        keep 64      keep 128     keep 256
+//   plain 256-term product, v_mfma_f32_32x32x2_f32       93 / 100     152 / 160    302 / 302
+//   folded, same instruction, stores past the caches     58 / 61       93 / 100    165 / 170
+//   folded, six bf16 products (this file)                56 / 55       88 / 72     117 / 128
+// The last row moves 4.2 to 6.0 TB/s of the bytes the transform has to read and write: memory,
+// not the matrix pipe, is what it waits for. Two wavefronts side by side on the same rows (all
+// of keep 256's columns in one workgroup, X read from memory once) was slower (200 against
+// 172 us with the fp32 instruction): the second read is already served by the L2 that the two
+// workgroups of a row tile share. 64-column tiles for keep 128 and 256 (whole-line loads, more
+// workgroups a row tile): 89 and 163 us.
 constexpr int kFoldB = kDctB / 2;
 
-template <int NT2>
-struct BasisVec;
-template <>
-struct BasisVec<4> {
-  typedef float type __attribute__((ext_vector_type(4)));
-};
-template <>
-struct BasisVec<2> {
-  typedef float type __attribute__((ext_vector_type(2)));
+// A wavefront's finished tile. Accumulator element i of lane l is
+// C[(i / 4) * 8 + (l / 32) * 4 + i % 4][l % 32]. ybase points at the wavefront's first row
+// (uniform), `rows` is how many rows exist from there on, and the lane's part of the address is
+// a 32-bit offset: no 64-bit address is kept in registers across the multiplies. Lane r holds
+// the folded columns cl = c0 + NT r + t, t < NT: neighbours, so that a row's results leave as
+// one vector per lane (forward: coefficients 2 cl .. 2 cl + 2 NT; inverse: positions
+// cl .. cl + NT and their mirror images 255 - cl - NT + 1 .. 255 - cl). The results are written
+// once and not read again here: the stores go past the caches, which took keep 64 from 68 to
+// 58 us forward and from 81 to 61 us back. (The same hint on the X loads costs a factor of two:
+// a row's 128-byte lines are asked for in two or four pieces.)
+template <int NT, bool FWD>
+__device__ __forceinline__ void store_tile(const v16f (&acc)[2 * NT], float* __restrict__ ybase, int ldy,
+                                           int64_t rows, int h, int cl) {
+  // (the two offsets are a handful of operations: made here, once per tile, not kept in
+  // registers for the whole launch)
+  asm volatile("" : "+v"(h), "+v"(cl));
+  const int left = (int)(rows < 32 ? rows : 32) - 4 * h;
+  const uint32_t lane_off = (uint32_t)(4 * h * ldy + (FWD ? 2 * cl : cl));
+  const uint32_t mirror_off = (uint32_t)(4 * h * ldy + kDctB - NT - cl);   // position 255 - (cl + NT - 1)
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int off = (i >> 2) * 8 + (i & 3);
+    if (off < left) {
+      float* row = ybase + off * ldy;               // uniform
+      if (FWD) {
+        if constexpr (NT == 2) {
+          __builtin_nontemporal_store(v4f{acc[0][i], acc[2][i], acc[1][i], acc[3][i]},
+                                      reinterpret_cast<v4f*>(row + lane_off));
+        } else {
+          __builtin_nontemporal_store(v2f{acc[0][i], acc[1][i]}, reinterpret_cast<v2f*>(row + lane_off));
+        }
+      } else {
+        if constexpr (NT == 2) {
+          __builtin_nontemporal_store(v2f{acc[0][i] + acc[2][i], acc[1][i] + acc[3][i]},
+                                      reinterpret_cast<v2f*>(row + lane_off));
+          __builtin_nontemporal_store(v2f{acc[1][i] - acc[3][i], acc[0][i] - acc[2][i]},
+                                      reinterpret_cast<v2f*>(row + mirror_off));
+        } else {
+          row[lane_off] = acc[0][i] + acc[1][i];
+          row[mirror_off] = acc[0][i] - acc[1][i];
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// (2) The folded product on the bf16 matrix instruction, at fp32 accuracy: every fp32 operand is
+// split into three bf16 pieces, x = x0 + x1 + x2 with x0 = bf16(x), x1 = bf16(x - x0),
+// x2 = bf16(x - x0 - x1) (round to nearest: |x1| <= 2^-9 |x|, |x2| <= 2^-18 |x|, and the three
+// carry all 24 bits of x but for a last piece below 2^-27 |x|), and a product a b becomes the six
+// pieces a0 b0 + a0 b1 + a1 b0 + a1 b1 + a0 b2 + a2 b0; the three left out are below 2^-26 |a b|,
+// under the rounding of the fp32 sum they would be added to. A bf16 x bf16 product is exact in
+// fp32 and v_mfma_f32_32x32x16_bf16 adds in fp32, sixteen reduction indices an instruction at
+// sixteen times the fp32 instruction's rate: six of them cost 3/8 of the fp32 multiplies they
+// replace. The basis is split once, from its double-precision values; X is split in registers,
+// a slice at a time (about five VALU operations a value). Against scipy's float64 transform on
+// N(0, 1) blocks the coefficients are off by 1.0e-8 of the block norm (rms; 1.5e-7 at worst),
+// the fp32 instruction's by 1.3e-8 (1.7e-7), a plain fp32 matrix product's by 1.8e-8 (2.3e-7).
+//
+// LDS holds the basis pieces as [reduction group of 8][piece][tile][32 lanes][8 bf16]: the eight
+// values a lane feeds to one instruction are one 16-byte read, and the global arrays are laid
+// out so that the tile is filled with 16-byte copies.
+// ---------------------------------------------------------------------------
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+struct Split3 {
+  bf16x8 p0, p1, p2;
 };
 
+__device__ __forceinline__ Split3 split3(const float (&x)[8]) {
+  Split3 o;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const v2f a = {x[2 * q], x[2 * q + 1]};
+    const bf16x2 h0 = __builtin_convertvector(a, bf16x2);
+    const v2f r1 = a - __builtin_convertvector(h0, v2f);
+    const bf16x2 h1 = __builtin_convertvector(r1, bf16x2);
+    const v2f r2 = r1 - __builtin_convertvector(h1, v2f);
+    const bf16x2 h2 = __builtin_convertvector(r2, bf16x2);
+    o.p0[2 * q] = h0[0];
+    o.p0[2 * q + 1] = h0[1];
+    o.p1[2 * q] = h1[0];
+    o.p1[2 * q + 1] = h1[1];
+    o.p2[2 * q] = h2[0];
+    o.p2[2 * q + 1] = h2[1];
+  }
+  return o;
+}
+
+// The basis in pieces. fwd3[g][piece][k][i] = piece of c[8 g + i][k] (g < 16: the folded rows
+// j < 128); inv3[second][g][piece][j][i] = piece of c[j][2 (8 g + i) + second] (j < 128).
+__global__ void dct2_basis3_kernel(__bf16* __restrict__ fwd3, __bf16* __restrict__ inv3) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= kFoldB * kDctB) return;
+  const int j = t / kDctB;                           // position, < 128
+  const int k = t - j * kDctB;                       // coefficient
+  const double s = k == 0 ? sqrt(1.0 / kDctB) : sqrt(2.0 / kDctB);
+  const double v = s * cos(3.14159265358979323846 * (2.0 * j + 1.0) * k / (2.0 * kDctB));
+  const __bf16 b0 = (__bf16)(float)v;
+  const double r1 = v - (double)(float)b0;
+  const __bf16 b1 = (__bf16)(float)r1;
+  const double r2 = r1 - (double)(float)b1;
+  const __bf16 b2 = (__bf16)(float)r2;
+  const __bf16 piece[3] = {b0, b1, b2};
+#pragma unroll
+  for (int p = 0; p < 3; ++p) {
+    fwd3[(((size_t)(j >> 3) * 3 + p) * kDctB + k) * 8 + (j & 7)] = piece[p];
+    const int c = k >> 1, second = k & 1;
+    inv3[((((size_t)second * 16 + (c >> 3)) * 3 + p) * kFoldB + j) * 8 + (c & 7)] = piece[p];
+  }
+}
+
 template <int NT, bool FWD>
-__global__ __launch_bounds__(kThreads) void dct2_fold_kernel(const float* __restrict__ X, int64_t ldx,
-                                                             const float* __restrict__ Bm,
-                                                             float* __restrict__ Y, int64_t ldy,
-                                                             int64_t M, int KF) {
+__global__ __launch_bounds__(kThreads) void dct2_split_kernel(const float* __restrict__ X, int64_t ldx,
+                                                              const __bf16* __restrict__ B3,
+                                                              float* __restrict__ Y, int64_t ldy,
+                                                              int64_t M, int KF) {
   constexpr int NT2 = 2 * NT;
-  typedef typename BasisVec<NT2>::type bvec;
-  constexpr int kRow = 32 * NT2;                    // floats per basis row in LDS
-  extern __shared__ float Bs[];                     // [KF + kPadRows][32][NT2]
+  // Folded indices a lane holds per slice: one group of 8, or two where the accumulators leave
+  // the registers for it (a row's loads are then whole 64-byte pieces, which memory serves
+  // better; the narrow tiles are the ones that wait for memory). Either way the groups are taken
+  // in the same order, so the kernels of all widths add a coefficient's products up alike.
+  constexpr int E = (FWD && NT == 1) ? 16 : 8;
+  constexpr int V = E / 2;                          // float4 per lane and slice
+  constexpr int kSliceK = 2 * E;
+  extern __shared__ uint4 Bl[];                     // [KF / 8][3][NT2][32] x 8 bf16
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int r = lane & 31;
   const int h = lane >> 5;
   const int c0 = blockIdx.y * 32 * NT;              // first folded column of this workgroup
+  const int groups = KF / 8;
 
-  if (FWD) {
-    // row j of the tile: fwd[j][2 c0 .. 2 c0 + 64 NT), consecutive in memory
-    for (int i = tid; i < KF * kRow; i += kThreads) {
-      const int j = i / kRow;
-      const int kk = i - j * kRow;
-      const int cl = kk >> 1, second = kk & 1;
-      Bs[(j * 32 + cl / NT) * NT2 + second * NT + cl % NT] = Bm[(size_t)j * kDctB + 2 * c0 + kk];
-    }
-  } else {
-    // reduction index c: inv[2 c][c0 ..] feeds E, inv[2 c + 1][c0 ..] feeds O
-    for (int i = tid; i < KF * kRow; i += kThreads) {
-      const int kk = i / (32 * NT);                 // coefficient 2 c + second
-      const int cl = i - kk * (32 * NT);
-      const int c = kk >> 1, second = kk & 1;
-      Bs[(c * 32 + cl / NT) * NT2 + second * NT + cl % NT] = Bm[(size_t)kk * kDctB + c0 + cl];
-    }
+  for (int i = tid; i < groups * 3 * NT2 * 32; i += kThreads) {
+    const int rr = i & 31;
+    const int t = (i >> 5) % NT2;
+    const int gp = (i >> 5) / NT2;                  // group * 3 + piece
+    const int cl = c0 + NT * rr + t % NT, second = t / NT;
+    const uint4* src = reinterpret_cast<const uint4*>(B3);
+    Bl[i] = FWD ? src[(size_t)gp * kDctB + 2 * cl + second]
+                : src[((size_t)second * 16 * 3 + gp) * kFoldB + cl];
   }
   __syncthreads();
 
-  // Folded reduction indices a lane holds per slice: 8, or 16 where the accumulators leave the
-  // registers for it (a row's loads are then whole 64-byte pieces, which memory serves better;
-  // the narrow tiles are the ones that wait for memory).
-  constexpr int E = NT == 1 ? 16 : 8;
-  constexpr int kSliceK = 2 * E;                    // both halves of the wavefront
-  constexpr int V = E / 2;                          // float4 per lane and slice
   const int64_t tiles = (M + kTileM - 1) / kTileM;
   const int slices = KF / kSliceK;
-  // A lane's loads are addressed as (uniform tile and slice base) + (32-bit lane offset): two
-  // registers per lane instead of a 64-bit pointer per stream. Rows past the end are clamped,
-  // not masked: row r of X only reaches row r of Y, and those rows are never stored, so the
-  // loads carry no branch.
   auto lane_row = [&](int64_t tile) -> uint32_t {
-    int64_t row = wave * 32 + r;
-    const int64_t last = M - 1 - tile * kTileM;
+    const int64_t left = M - 1 - tile * kTileM;      // uniform
+    const int last = left < kTileM - 1 ? (int)left : kTileM - 1;
+    int row = wave * 32 + r;
     if (row > last) row = last;
-    return (uint32_t)(row * ldx);                   // at most 512 rows of 256 floats
+    return (uint32_t)row * (uint32_t)ldx;
   };
-  // Which folded indices lane half h holds in step e of slice s: first(s) + kHalf h + e. Forward,
-  // the two halves are 16 apart whatever E is, so that the kernels of all widths add a
-  // coefficient's products up in the same order and keep-64 output equals the first 64 columns
-  // of keep-256 output bit for bit. Inverse: the halves follow each other (a lane pair then
-  // reads 128 consecutive bytes).
   constexpr int kHalf = FWD ? 16 : E;
   auto first = [&](int s) { return FWD && E == 8 ? 32 * (s >> 1) + 8 * (s & 1) : kSliceK * s; };
-  // Slice s of a row. Forward: x[j ..+E) from j = first(s) + 16 h and its mirror image
-  // x[256 - E - j ..+E) (element e pairs with element E - 1 - e of the mirror). Inverse: the 2E
-  // coefficients 2 j ..+2E, even and odd ones interleaved.
   auto load_slice = [&](int64_t tile, uint32_t lrow, int s, float4 (&v)[V]) {
     const float* tb = X + tile * kTileM * ldx;       // uniform
     if (FWD) {
@@ -163,33 +237,18 @@ __global__ __launch_bounds__(kThreads) void dct2_fold_kernel(const float* __rest
       for (int q = 0; q < V; ++q) v[q] = *reinterpret_cast<const float4*>(a + ia + 4 * q);
     }
   };
-  const float* bs = Bs + (size_t)(kHalf * h) * kRow + r * NT2;
   uint32_t lrow = lane_row(blockIdx.x);
-  float4 cur[V], nxt[V];
+  float4 cur[V];
   load_slice(blockIdx.x, lrow, 0, cur);
   v16f acc[NT2];
-  bvec bcur, bnxt;
+  const uint4* bl = Bl + r;
 
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    // the tile after this one (or this one again at the end: its values are then unused)
     const int64_t tile_next = tile + gridDim.x < tiles ? tile + gridDim.x : tile;
 #pragma unroll
     for (int t = 0; t < NT2; ++t) acc[t] = v16f{0};
-    bcur = *reinterpret_cast<const bvec*>(bs);
 #pragma unroll 1
     for (int s = 0; s < slices; ++s) {
-      // the next slice of this tile, or the first slice of the next tile
-      if (s + 1 < slices) {
-        load_slice(tile, lrow, s + 1, nxt);
-      } else {
-        lrow = lane_row(tile_next);
-        load_slice(tile_next, lrow, 0, nxt);
-      }
-      __builtin_amdgcn_sched_barrier(0);            // keep the requests ahead of the multiplies
-      const float* brow = bs + first(s) * kRow;
-      const float* brow_next = bs + first(s + 1) * kRow;
-      // the slice as scalars: the values, then their mirror images (forward), or the
-      // interleaved even and odd coefficients (inverse)
       float v[2 * E];
 #pragma unroll
       for (int q = 0; q < V; ++q) {
@@ -198,79 +257,78 @@ __global__ __launch_bounds__(kThreads) void dct2_fold_kernel(const float* __rest
         v[4 * q + 2] = cur[q].z;
         v[4 * q + 3] = cur[q].w;
       }
+      // forward: the values, then their mirror images; inverse: even and odd coefficients interleaved
+      float one[E], two[E];
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        // basis values of the following step are requested before this step multiplies: row e + 1
-        // of this slice, or the first row of the next one (past the last slice: padding, never used)
-        bnxt = *reinterpret_cast<const bvec*>(e < E - 1 ? brow + (e + 1) * kRow : brow_next);
-        const float first = FWD ? v[e] + v[2 * E - 1 - e] : v[2 * e];
-        const float second = FWD ? v[e] - v[2 * E - 1 - e] : v[2 * e + 1];
-        __builtin_amdgcn_sched_barrier(0);
+        one[e] = FWD ? v[e] + v[2 * E - 1 - e] : v[2 * e];
+        two[e] = FWD ? v[e] - v[2 * E - 1 - e] : v[2 * e + 1];
+      }
+      Split3 piece[E / 8][2];
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(first, bcur[t], acc[t], 0, 0, 0);
+      for (int g = 0; g < E / 8; ++g) {
+        float x8[8];
 #pragma unroll
-        for (int t = NT; t < NT2; ++t)
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(second, bcur[t], acc[t], 0, 0, 0);
-        bcur = bnxt;
+        for (int e = 0; e < 8; ++e) x8[e] = one[8 * g + e];
+        piece[g][0] = split3(x8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x8[e] = two[8 * g + e];
+        piece[g][1] = split3(x8);
+      }
+      // the slice's values are used up: the next slice's take their registers
+      if (s + 1 < slices) {
+        load_slice(tile, lrow, s + 1, cur);
+      } else {
+        lrow = lane_row(tile_next);
+        load_slice(tile_next, lrow, 0, cur);
       }
 #pragma unroll
-      for (int q = 0; q < V; ++q) cur[q] = nxt[q];
-    }
-    // accumulator element i of lane l is C[(i / 4) * 8 + (l / 32) * 4 + i % 4][l % 32]. The
-    // row offsets are compile-time numbers times the (uniform) row stride, so that no address
-    // is kept in registers across the multiplies.
-    const int64_t row0 = tile * kTileM + wave * 32 + h * 4;
-    const int64_t left = M - row0;
-    // lane r holds the folded columns c0 + NT r + t, t < NT: neighbours, so that a row's results
-    // leave as one vector per lane (forward: coefficients 2 c .. 2 c + 2 NT; inverse: positions
-    // c .. c + NT and their mirror images 255 - c - NT + 1 .. 255 - c). The results are written
-    // once and not read again here: the stores go past the caches, which took keep 64 from 68 to
-    // 58 us forward and from 81 to 61 us back. (The same hint on the X loads costs a factor of
-    // two: a row's 128-byte lines are asked for in two or four pieces.)
-    const int cl = c0 + NT * r;
-    float* yp = Y + row0 * ldy + (FWD ? 2 * cl : cl);
+      for (int g = 0; g < E / 8; ++g) {
+        // group g of the slice: folded indices first(s) + 8 g + kHalf h ..+8
+        const uint4* bg = bl + (size_t)((first(s) + 8 * g + kHalf * h) >> 3) * (3 * NT2 * 32);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int off = (i >> 2) * 8 + (i & 3);
-      if (off < left) {
-        float* p = yp + off * ldy;
-        if (FWD) {
-          if constexpr (NT == 2) {
-            __builtin_nontemporal_store(v4f{acc[0][i], acc[2][i], acc[1][i], acc[3][i]}, reinterpret_cast<v4f*>(p));
-          } else {
-            __builtin_nontemporal_store(v2f{acc[0][i], acc[1][i]}, reinterpret_cast<v2f*>(p));
-          }
-        } else {
-          float* q = p + (kDctB - NT - 2 * cl);     // position 255 - (cl + NT - 1)
-          if constexpr (NT == 2) {
-            __builtin_nontemporal_store(v2f{acc[0][i] + acc[2][i], acc[1][i] + acc[3][i]}, reinterpret_cast<v2f*>(p));
-            __builtin_nontemporal_store(v2f{acc[1][i] - acc[3][i], acc[0][i] - acc[2][i]}, reinterpret_cast<v2f*>(q));
-          } else {
-            p[0] = acc[0][i] + acc[1][i];
-            q[0] = acc[0][i] - acc[1][i];
+        for (int half = 0; half < 2; ++half) {
+          const Split3& a = piece[g][half];
+#pragma unroll
+          for (int tt = 0; tt < NT; ++tt) {
+            const int t = half * NT + tt;
+            const uint4 u0 = bg[(0 * NT2 + t) * 32], u1 = bg[(1 * NT2 + t) * 32], u2 = bg[(2 * NT2 + t) * 32];
+            const bf16x8 b0 = __builtin_bit_cast(bf16x8, u0), b1 = __builtin_bit_cast(bf16x8, u1),
+                         b2 = __builtin_bit_cast(bf16x8, u2);
+            // the small pieces first
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.p2, b0, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.p0, b2, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.p1, b1, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.p1, b0, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.p0, b1, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.p0, b0, acc[t], 0, 0, 0);
           }
         }
       }
+    }
+    {
+      const int64_t row0 = tile * kTileM + __builtin_amdgcn_readfirstlane(wave) * 32;
+      store_tile<NT, FWD>(acc, Y + row0 * ldy, (int)ldy, M - row0, h, c0 + NT * r);
     }
   }
 }
 
 static std::mutex g_basis_mu;
-static float* g_basis_fwd = nullptr;
-static float* g_basis_inv = nullptr;
+static __bf16* g_basis3_fwd = nullptr;
+static __bf16* g_basis3_inv = nullptr;
+constexpr size_t kBasis3Count = (size_t)16 * 3 * kDctB * 8;   // per direction
 
 static int32_t ensure_basis(hipStream_t s) {
   std::lock_guard<std::mutex> lk(g_basis_mu);
-  if (g_basis_fwd) return KRK_SUCCESS;
+  if (g_basis3_fwd) return KRK_SUCCESS;
   DeviceGuard guard;
-  KRK_HIP(hipMalloc(&guard.p, 2 * sizeof(float) * kDctB * kDctB));
-  float* p = reinterpret_cast<float*>(guard.p);
-  hipLaunchKernelGGL(dct2_basis_kernel, dim3(kDctB * kDctB / 256), dim3(256), 0, s, p, p + kDctB * kDctB);
+  KRK_HIP(hipMalloc(&guard.p, 2 * sizeof(__bf16) * kBasis3Count));
+  __bf16* p3 = reinterpret_cast<__bf16*>(guard.p);
+  hipLaunchKernelGGL(dct2_basis3_kernel, dim3(kFoldB * kDctB / 256), dim3(256), 0, s, p3, p3 + kBasis3Count);
   KRK_HIP(hipGetLastError());
   KRK_HIP(hipStreamSynchronize(s));
-  g_basis_fwd = guard.release<float>();
-  g_basis_inv = p + kDctB * kDctB;
+  g_basis3_fwd = guard.release<__bf16>();
+  g_basis3_inv = p3 + kBasis3Count;
   return KRK_SUCCESS;
 }
 
@@ -310,12 +368,12 @@ static int32_t dct2_run(const float* in, float* out, int64_t n, int32_t keep, ui
   const int NF = forward ? keep / 2 : kFoldB;
   const int nt = (NF % 64 == 0) ? 2 : 1;          // 64 folded columns a wavefront where the width allows
   const int gy = NF / (32 * nt);
-  const size_t lds_bytes = sizeof(float) * (size_t)(KF + kPadRows) * 64 * nt;
+  const size_t lds_bytes = (size_t)(KF / 8) * 3 * 2 * nt * 32 * 16;   // [KF / 8][3][2 nt][32] x 16 bytes
   const int64_t tiles = (M + kTileM - 1) / kTileM;
   int64_t gx = 256 / gy;                           // one workgroup a compute unit
   if (gx > tiles) gx = tiles;
   if (gx < 1) gx = 1;
-  const float* basis = forward ? g_basis_fwd : g_basis_inv;
+  const __bf16* basis = forward ? g_basis3_fwd : g_basis3_inv;
   const dim3 grid((unsigned)gx, (unsigned)gy), block(kThreads);
   const int64_t ldx = forward ? kDctB : keep, ldy = forward ? keep : kDctB;
   hipError_t e = hipSuccess;
@@ -327,11 +385,11 @@ static int32_t dct2_run(const float* in, float* out, int64_t n, int32_t keep, ui
     e = hipGetLastError();
   };
   if (!forward) {
-    launch(dct2_fold_kernel<2, false>);
+    launch(dct2_split_kernel<2, false>);
   } else if (nt == 2) {
-    launch(dct2_fold_kernel<2, true>);             // keep 128 and 256
+    launch(dct2_split_kernel<2, true>);            // keep 128 and 256
   } else {
-    launch(dct2_fold_kernel<1, true>);             // keep 64 and 192
+    launch(dct2_split_kernel<1, true>);            // keep 64 and 192
   }
   if (e == hipSuccess && host)
     e = hipMemcpy(out, d_out, sizeof(float) * (size_t)out_count, hipMemcpyDeviceToHost);

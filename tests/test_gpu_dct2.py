@@ -3,7 +3,8 @@ emitter is the threshold codec), so there is no reference output to match: the t
 pinned by the library definition scipy.fft.dct(type=2, norm="ortho") on blocks of 256, by the
 orthonormality of the basis (Parseval) and by the round trip. Tolerance: 1e-5 relative to the
 block's norm (a coefficient is a sum of 256 fp32 products; relative to a single coefficient no
-bound exists, since coefficients pass through zero)."""
+bound exists, since coefficients pass through zero); test_fp32_accuracy_of_the_split_products
+holds the kernels (fp32 products made of bf16 pieces) to what a plain fp32 product achieves."""
 import numpy as np
 import pytest
 
@@ -64,6 +65,35 @@ def test_round_trip_and_parseval(dct2):
     want = fft.idct(pad, type=2, norm="ortho", axis=1).ravel()
     got = dct2.inverse(y64, n, 64)
     assert np.abs(got - want).max() < 1e-5 * 16
+
+
+def test_fp32_accuracy_of_the_split_products(dct2):
+    """The kernels multiply every fp32 operand as three bf16 pieces (six piece products out of
+    nine, fp32 sums). What that must not cost: against float64 the coefficients stay within
+    1e-6 of the block norm (a plain fp32 matrix product of the same data is at 2.3e-7 at worst,
+    1.8e-8 rms; bf16 operands alone would be at 4e-3), also when the values of a block span
+    e^-20 .. e^20, when they are exact small integers (every piece product exact: the result is
+    the fp32 product's), and for powers of two near the ends of the fp32 range."""
+    fft = pytest.importorskip("scipy.fft")
+    rng = np.random.default_rng(77)
+    blocks = 4096
+    normal = rng.standard_normal(blocks * 256).astype(np.float32)
+    wide = (normal * np.exp(rng.uniform(-20, 20, normal.size))).astype(np.float32)
+    for x in (normal, wide, normal * np.float32(2.0 ** 100), normal * np.float32(2.0 ** -100)):
+        want = fft.dct(x.reshape(-1, 256).astype(np.float64), type=2, norm="ortho", axis=1)
+        nrm = np.linalg.norm(x.reshape(-1, 256).astype(np.float64), axis=1, keepdims=True)
+        got = dct2.forward(x, 256)
+        err = np.abs(got - want) / nrm
+        assert err.max() <= 1e-6, err.max()
+        assert np.sqrt(np.mean(err ** 2)) <= 3e-8
+        back = dct2.inverse(got, x.size, 256).reshape(-1, 256)
+        wb = fft.idct(got.astype(np.float64), type=2, norm="ortho", axis=1)
+        errb = np.abs(back - wb) / np.linalg.norm(got.astype(np.float64), axis=1, keepdims=True)
+        assert errb.max() <= 1e-6, errb.max()
+    # a constant block of an integer: sums and differences exact, one nonzero coefficient
+    x = np.full(256, 3.0, np.float32)
+    y = dct2.forward(x, 256)[0]
+    assert y[0] == np.float32(48.0) and np.abs(y[1:]).max() < 1e-5
 
 
 def test_device_pointers_and_arguments(dct2):
