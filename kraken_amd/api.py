@@ -15,6 +15,8 @@ LIB_PATH = os.path.join(_HERE, "libkraken_hip.so")
 
 DEVICE_PTRS = 0x1
 ASYNC = 0x2
+NOTE_ROWS = 0x4          # on a pull: keep the row of every position for a push_raw of the same ids
+IDS_AS_PULLED = 0x8      # on a push_raw: ids is the unchanged buffer of that pull
 
 SUCCESS = 0
 UNSUPPORTED_OPTIM = 6
@@ -366,8 +368,8 @@ class SparseTable:
     def sync(self):
         return lib().krk_sparse_sync(self.h)
 
-    def Pull(self, sparse_ids, out=None, async_=False):
-        """-> (code, vals[n, dimension])"""
+    def Pull(self, sparse_ids, out=None, async_=False, note_rows=False):
+        """-> (code, vals[n, dimension]). note_rows (device ids): see KRK_NOTE_ROWS."""
         if isinstance(sparse_ids, DeviceArray):
             n = sparse_ids.size
             if out is None:
@@ -378,10 +380,11 @@ class SparseTable:
             if out is None:
                 out = np.empty((n, self.dimension), np.float32)
         rc = lib().krk_sparse_pull(self.h, _ptr(sparse_ids), n, _ptr(out),
-                                   _flags(sparse_ids, out, extra=ASYNC if async_ else 0))
+                                   _flags(sparse_ids, out, extra=(ASYNC if async_ else 0) |
+                                          (NOTE_ROWS if note_rows else 0)))
         return rc, out
 
-    def Push(self, optim, sparse_ids, grads, lr, async_=False, raw=False):
+    def Push(self, optim, sparse_ids, grads, lr, async_=False, raw=False, as_pulled=False):
         if isinstance(sparse_ids, DeviceArray):
             n = sparse_ids.size
             gd = grads.shape[-1]
@@ -392,11 +395,13 @@ class SparseTable:
             gd = grads.shape[-1] if grads.ndim > 1 else (grads.size // max(n, 1))
         fn = lib().krk_sparse_push_raw if raw else lib().krk_sparse_push
         return fn(self.h, C.byref(optim.raw), _ptr(sparse_ids), n, _ptr(grads), gd, lr,
-                  _flags(sparse_ids, grads, extra=ASYNC if async_ else 0))
+                  _flags(sparse_ids, grads, extra=(ASYNC if async_ else 0) |
+                         (IDS_AS_PULLED if as_pulled else 0)))
 
-    def PushRaw(self, optim, ids, grads, lr, async_=False):
-        """Emitter::PushSparseTable's dedup + sum fused with Push: ids may repeat."""
-        return self.Push(optim, ids, grads, lr, async_=async_, raw=True)
+    def PushRaw(self, optim, ids, grads, lr, async_=False, as_pulled=False):
+        """Emitter::PushSparseTable's dedup + sum fused with Push: ids may repeat. as_pulled:
+        ids is the unchanged device buffer of the last Pull(note_rows=True) (KRK_IDS_AS_PULLED)."""
+        return self.Push(optim, ids, grads, lr, async_=async_, raw=True, as_pulled=as_pulled)
 
     _POOL = {"sum": 0, "mean": 1}
 
@@ -577,8 +582,9 @@ class TableGroup:
         np.cumsum(counts, out=off[1:])
         return off
 
-    def CombinePull(self, ids, offsets, out=None, async_=False):
-        """ids: concatenated per-table ids; offsets: int64[n_tables + 1] -> (code, vals)"""
+    def CombinePull(self, ids, offsets, out=None, async_=False, note_rows=False):
+        """ids: concatenated per-table ids; offsets: int64[n_tables + 1] -> (code, vals).
+        note_rows (device ids): see KRK_NOTE_ROWS."""
         offsets = np.ascontiguousarray(offsets, dtype=np.int64)
         total = int(offsets[-1])
         if isinstance(ids, DeviceArray):
@@ -589,10 +595,11 @@ class TableGroup:
             if out is None:
                 out = np.empty((total, self.dimension), np.float32)
         rc = lib().krk_group_pull(self.h, _ptr(ids), _ptr(offsets), _ptr(out),
-                                  _flags(ids, out, extra=ASYNC if async_ else 0))
+                                  _flags(ids, out, extra=(ASYNC if async_ else 0) |
+                                         (NOTE_ROWS if note_rows else 0)))
         return rc, out
 
-    def CombinePush(self, optim, ids, offsets, grads, lr, async_=False, raw=False):
+    def CombinePush(self, optim, ids, offsets, grads, lr, async_=False, raw=False, as_pulled=False):
         offsets = np.ascontiguousarray(offsets, dtype=np.int64)
         if not isinstance(ids, DeviceArray):
             ids = np.ascontiguousarray(ids, dtype=np.uint64)
@@ -600,11 +607,13 @@ class TableGroup:
         gd = grads.shape[-1]
         fn = lib().krk_group_push_raw if raw else lib().krk_group_push
         return fn(self.h, C.byref(optim.raw), _ptr(ids), _ptr(offsets), _ptr(grads),
-                  gd, lr, _flags(ids, grads, extra=ASYNC if async_ else 0))
+                  gd, lr, _flags(ids, grads, extra=(ASYNC if async_ else 0) |
+                                 (IDS_AS_PULLED if as_pulled else 0)))
 
-    def CombinePushRaw(self, optim, ids, offsets, grads, lr, async_=False):
-        """Emitter::CombinePushSparseTable's dedup + sum fused with CombinePush: ids may repeat."""
-        return self.CombinePush(optim, ids, offsets, grads, lr, async_=async_, raw=True)
+    def CombinePushRaw(self, optim, ids, offsets, grads, lr, async_=False, as_pulled=False):
+        """Emitter::CombinePushSparseTable's dedup + sum fused with CombinePush: ids may repeat.
+        as_pulled: ids is the unchanged device buffer of the last CombinePull(note_rows=True)."""
+        return self.CombinePush(optim, ids, offsets, grads, lr, async_=async_, raw=True, as_pulled=as_pulled)
 
 
 class DenseTable:

@@ -121,7 +121,7 @@ struct ObjBase {
 };
 
 inline int32_t check_flags(uint32_t flags) {
-  if (flags & ~(KRK_DEVICE_PTRS | KRK_ASYNC)) {
+  if (flags & ~(KRK_DEVICE_PTRS | KRK_ASYNC | KRK_NOTE_ROWS | KRK_IDS_AS_PULLED)) {
     set_error("unknown flag bits 0x%x", flags);
     return KRK_E_ARGUMENT;
   }

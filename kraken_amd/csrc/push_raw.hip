@@ -857,6 +857,7 @@ static int pick_tile(int64_t cnt) {
 constexpr int kSortBlock = 1024;
 constexpr int kSortItems = 8;
 constexpr int kSortMax = kSortBlock * kSortItems;      // ids per table
+static_assert(kSortMax == kNotedMax, "row notes are kept for exactly the requests that take this path");
 constexpr int kSortWaves = kSortBlock / kWave;
 constexpr int kMaxBucketBits = 5;                      // up to 32 buckets a table
 constexpr int kDigitBits = 9;
@@ -876,6 +877,11 @@ struct SortCall {
   int32_t row_bits;                                    // bits of a row number
   uint32_t row_mask;                                   // a key's row (member bits above it)
   uint32_t miss_key;                                   // keys at or above it stand for missing ids
+  // Not null: `keys` are the row notes of the pull of these ids (a member's own row numbers).
+  // A note of kEmptyRow was taken while the row's creator, another wavefront of that pull, had
+  // not published the row number yet (further occurrences of an id that the pull inserted):
+  // such a position is looked up here.
+  const uint64_t* note_ids;
   int64_t row_start[kMaxGroupTables + 1];
 };
 
@@ -964,6 +970,13 @@ __global__ __launch_bounds__(kSortBlock) void bucket_push_kernel(const TableDesc
   for (int i = 0; i < kSortItems; ++i) {
     const int j = t * own + i;
     if (i < own) mine[i] = keys[a + (j < all ? j : all - 1)];
+  }
+  if (call.note_ids) {
+#pragma unroll
+    for (int i = 0; i < kSortItems; ++i) {
+      const int j = t * own + i;
+      if (i < own && j < all && mine[i] == kEmptyRow) mine[i] = probe_find_alone(tv, call.note_ids[a + j]);
+    }
   }
   uint32_t take = 0;
 #pragma unroll
@@ -1858,6 +1871,7 @@ int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* i
     while (((int64_t)1 << sc.row_bits) < t->row_cap) ++sc.row_bits;
     sc.row_mask = 0xFFFFFFFFu;
     sc.miss_key = kNoRow;
+    sc.note_ids = nullptr;
     sc.row_start[0] = 0;
     sc.row_start[1] = n;
     ApplyArgs args;
@@ -1869,11 +1883,21 @@ int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* i
     args.c1 = cols[1];
     args.c2 = cols[2];
     args.meta_off = ((optim_state_mask(*o) >> KRK_ST_STEPS) & 1u) ? t->meta_off : -1;
-    KRK_TRY(t->scratch[0].reserve((size_t)n * sizeof(uint32_t)));
-    uint32_t* keys = t->scratch[0].as<uint32_t>();
     const TableView tv = t->view();
-    hipLaunchKernelGGL(rows_of_ids_kernel, dim3(grid_for(n, kBlock / kBucket)), dim3(kBlock), 0, t->stream, tv,
-                       d_ids, n, kNoRow, (const uint32_t*)nullptr, false, keys, (uint32_t*)nullptr);
+    // KRK_IDS_AS_PULLED: the rows of these very ids were noted by the pull before (and nothing
+    // has moved since): the look-up launch is not needed
+    const bool noted = (flags & KRK_IDS_AS_PULLED) && t->noted_ids == ids && t->noted_n == n &&
+                       t->noted_version == t->layout_version;
+    const uint32_t* keys = t->notes.as<uint32_t>();
+    if (!noted) {
+      KRK_TRY(t->scratch[0].reserve((size_t)n * sizeof(uint32_t)));
+      uint32_t* found = t->scratch[0].as<uint32_t>();
+      hipLaunchKernelGGL(rows_of_ids_kernel, dim3(grid_for(n, kBlock / kBucket)), dim3(kBlock), 0, t->stream, tv,
+                         d_ids, n, kNoRow, (const uint32_t*)nullptr, false, found, (uint32_t*)nullptr);
+      keys = found;
+    } else {
+      sc.note_ids = d_ids;
+    }
     const GroupSrc none{nullptr, 0, -1, -1, -1, 0};
     if (t->vec == 4) {
       launch_bucket_push<4, false>(o->type, 1u << sc.bucket_bits, t->stream, nullptr, tv, sc, keys, d_g, (int)t->dim, t->elems,
@@ -1967,11 +1991,27 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
     sc.row_bits = row_bits;
     sc.row_mask = row_bits >= 32 ? 0xFFFFFFFFu : ((1u << row_bits) - 1u);
     sc.miss_key = miss_key;
+    sc.note_ids = nullptr;
     for (int m = 0; m <= n_tables; ++m) sc.row_start[m] = offsets[m];
-    KRK_TRY(g->scratch[0].reserve((size_t)total * sizeof(uint32_t)));
-    uint32_t* keys = g->scratch[0].as<uint32_t>();
-    hipLaunchKernelGGL(group_rows_of_ids_kernel, dim3(rows_call.block_start[n_tables]), dim3(kBlock), 0, g->stream,
-                       g->d_descs, rows_call, d_ids, total, row_bits, miss_key, keys, (uint32_t*)nullptr);
+    // KRK_IDS_AS_PULLED: the rows of these very ids were noted by the combined pull before (and
+    // nothing has moved since): the look-up launch is not needed. A note is a member's own row
+    // number, which is all the bucket kernel reads of a key.
+    bool noted = (flags & KRK_IDS_AS_PULLED) && g->noted_ids == ids &&
+                 g->noted_offsets.size() == (size_t)n_tables + 1 && g->noted_versions.size() == (size_t)n_tables;
+    for (int m = 0; noted && m < n_tables; ++m)
+      noted = g->noted_offsets[m] == offsets[m] && g->noted_offsets[m + 1] == offsets[m + 1] &&
+              g->noted_versions[m] == g->tables[m]->layout_version;
+    const uint32_t* keys = g->notes.as<uint32_t>();
+    if (!noted) {
+      KRK_TRY(g->scratch[0].reserve((size_t)total * sizeof(uint32_t)));
+      uint32_t* found = g->scratch[0].as<uint32_t>();
+      hipLaunchKernelGGL(group_rows_of_ids_kernel, dim3(rows_call.block_start[n_tables]), dim3(kBlock), 0,
+                         g->stream, g->d_descs, rows_call, d_ids, total, row_bits, miss_key, found,
+                         (uint32_t*)nullptr);
+      keys = found;
+    } else {
+      sc.note_ids = d_ids;
+    }
     if (g->vec == 4) {
       launch_bucket_push<4, true>(o->type, (unsigned)n_tables << sc.bucket_bits, g->stream, g->d_descs, TableView{}, sc,
                                   keys, d_g, (int)g->dim, g->elems, g->group, args, gs);

@@ -334,6 +334,12 @@ __device__ inline uint32_t probe_find_alone(const TableView& tv, uint64_t id) {
 
 struct krk_group;
 
+namespace krk {
+// Requests of at most this many ids a table keep row notes (KRK_NOTE_ROWS): the size up to
+// which push_raw runs as look-up + one launch per bucket, where the look-up is a fifth of it.
+constexpr int64_t kNotedMax = 8192;
+}  // namespace krk
+
 // The handle behind krk_sparse*.
 struct krk_sparse : krk::ObjBase {
   int64_t dim = 0;
@@ -368,6 +374,13 @@ struct krk_sparse : krk::ObjBase {
   krk_group* member_of = nullptr;
 
   krk::DeviceBuffer scratch[6];       // push_raw work space
+
+  // Row notes (KRK_NOTE_ROWS): the row of every position of one pull, kept for a push_raw of the
+  // same ids. Valid while noted_ids is not null and noted_version == layout_version.
+  krk::DeviceBuffer notes;
+  const uint64_t* noted_ids = nullptr;
+  int64_t noted_n = 0;
+  uint64_t noted_version = 0;
 
   krk::TableView view() const {
     krk::TableView tv;
@@ -419,6 +432,12 @@ struct krk_group : krk::ObjBase {
   int vec = 1, elems = 0, group = 1;
   hipStream_t own_stream = nullptr;    // the stream created with the group
   krk::DeviceBuffer scratch[5];        // push_raw work space
+  // Row notes of one combined pull (see krk_sparse::notes): valid while noted_ids is not null
+  // and every member's layout_version is what it was.
+  krk::DeviceBuffer notes;
+  const uint64_t* noted_ids = nullptr;
+  std::vector<int64_t> noted_offsets;
+  std::vector<uint64_t> noted_versions;
 };
 
 namespace krk {

@@ -111,7 +111,7 @@ template <int VEC, bool MOSTLY_NEW = false>
 __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init,
                                           const uint64_t* __restrict__ ids, int64_t i, bool active,
                                           int gl, float* __restrict__ out, int dim, int elems,
-                                          int group) {
+                                          int group, uint32_t* __restrict__ notes = nullptr) {
   const uint64_t id = active ? ids[i] : 0;
   // Most ids are resident: a search that never writes settles them, and only a wavefront that
   // holds a missing id goes through the claiming search as well.
@@ -129,6 +129,8 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
   const uint32_t row = pr.row;
   const bool owner = pr.owner;
   const bool fresh = pr.fresh;
+  // where the id lives, for a push of the same ids that follows (kEmptyRow: the table is full)
+  if (notes && gl == 0) notes[i] = row;
   float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
   float* dst = out + i * (int64_t)dim;
   for (int e = gl; e < elems; e += group) {
@@ -234,10 +236,10 @@ template <int VEC>
 __global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, InitK init,
                                                       const uint64_t* __restrict__ ids, int64_t n,
                                                       float* __restrict__ out, int dim, int elems,
-                                                      int group) {
+                                                      int group, uint32_t* __restrict__ notes) {
   const int per_block = kBlock / group;
   const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
-  pull_body<VEC>(tv, init, ids, i, i < n, threadIdx.x & (group - 1), out, dim, elems, group);
+  pull_body<VEC>(tv, init, ids, i, i < n, threadIdx.x & (group - 1), out, dim, elems, group, notes);
 }
 
 // ---- large pulls in two launches ------------------------------------------------
@@ -420,7 +422,8 @@ template <int VEC, bool INSERT, bool VIA = false>
 __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init,
                                           const uint64_t* __restrict__ ids, int64_t first, int64_t end,
                                           float* __restrict__ out, int dim, int elems, int group,
-                                          uint32_t* __restrict__ todo, int parity) {
+                                          uint32_t* __restrict__ todo, int parity,
+                                          uint32_t* __restrict__ notes = nullptr) {
   const int lane = wave_lane();
   const int gl4 = lane & (kBucket - 1);
   const int64_t i = first + (lane >> 2);
@@ -439,6 +442,8 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
       const ProbeResult q = probe_insert(tv, id, miss, gl4, kBucket);
       if (miss) pr = q;
     }
+    // where the id lives, for a push of the same ids that follows (kEmptyRow: the table is full)
+    if (!VIA && notes && active && gl4 == 0) notes[i] = pr.row;
   } else {
     // one atomic per wavefront reserves entries of the workgroup's list for all of its missing ids
     // (here `end` is the request's length: the lists' capacity follows from it)
@@ -608,10 +613,10 @@ template <int VEC>
 __global__ __launch_bounds__(kBlock) void pull_wide_kernel(TableView tv, InitK init,
                                                            const uint64_t* __restrict__ ids, int64_t n,
                                                            float* __restrict__ out, int dim, int elems,
-                                                           int group) {
+                                                           int group, uint32_t* __restrict__ notes) {
   const int64_t first = ((int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds;
   if (first >= n) return;                        // the whole wavefront
-  pull_wide<VEC, true>(tv, init, ids, first, n, out, dim, elems, group, nullptr, 0);
+  pull_wide<VEC, true>(tv, init, ids, first, n, out, dim, elems, group, nullptr, 0, notes);
 }
 
 template <int VEC>
@@ -659,7 +664,7 @@ __global__ __launch_bounds__(kBlock) void group_pull_kernel(const TableDesc* __r
                                                             GroupCall call,
                                                             const uint64_t* __restrict__ ids,
                                                             float* __restrict__ out, int dim, int elems,
-                                                            int group) {
+                                                            int group, uint32_t* __restrict__ notes) {
   const int t = find_table(call);
   TableView tv = descs[t].tv;
   tv.epoch = call.epoch[t];
@@ -668,7 +673,7 @@ __global__ __launch_bounds__(kBlock) void group_pull_kernel(const TableDesc* __r
   const int64_t local = (int64_t)(blockIdx.x - call.block_start[t]) * per_block + threadIdx.x / group;
   const int64_t i = call.row_start[t] + local;
   pull_body<VEC>(tv, init, ids, i, i < call.row_start[t + 1], threadIdx.x & (group - 1), out, dim,
-                 elems, group);
+                 elems, group, notes);
 }
 
 // the same for rows 32 to 128 floats wide: a workgroup takes 64 positions of its table
@@ -677,7 +682,8 @@ __global__ __launch_bounds__(kBlock) void group_pull_wide_kernel(const TableDesc
                                                                  GroupCall call,
                                                                  const uint64_t* __restrict__ ids,
                                                                  float* __restrict__ out, int dim,
-                                                                 int elems, int group) {
+                                                                 int elems, int group,
+                                                                 uint32_t* __restrict__ notes) {
   const int t = find_table(call);
   TableView tv = descs[t].tv;
   tv.epoch = call.epoch[t];
@@ -686,7 +692,7 @@ __global__ __launch_bounds__(kBlock) void group_pull_wide_kernel(const TableDesc
                         kWideIds;
   const int64_t first = call.row_start[t] + local;
   if (first >= call.row_start[t + 1]) return;    // the whole wavefront
-  pull_wide<VEC, true>(tv, init, ids, first, call.row_start[t + 1], out, dim, elems, group, nullptr, 0);
+  pull_wide<VEC, true>(tv, init, ids, first, call.row_start[t + 1], out, dim, elems, group, nullptr, 0, notes);
 }
 
 template <int OPT, int VEC>
@@ -1603,6 +1609,7 @@ int32_t krk_sparse_destroy(krk_sparse* t) {
   if (t->host_counters) (void)hipHostFree(t->host_counters);
   if (t->host_pub) (void)hipHostFree(t->host_pub);
   for (auto& b : t->scratch) b.release();
+  t->notes.release();
   t->stream = t->own_stream;
   t->close_stream();
   delete t;
@@ -1655,7 +1662,8 @@ int32_t krk_sparse_sync(krk_sparse* t) {
 
 // The launches of one pull of n > 0 ids into d_out [n, dim]; the caller holds the table's lock
 // and has made room for n more rows.
-static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, float* d_out) {
+static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, float* d_out,
+                            uint32_t* notes = nullptr) {
   const int64_t rows_before = t->size_ub;           // upper bound of the rows the table holds
   KRK_TRY(sparse_next_epoch(t, n));
   const bool wide = t->vec == 4 && pull_is_wide(t->group, t->elems);
@@ -1694,13 +1702,13 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
     }
   } else if (t->vec == 4 && wide) {
     hipLaunchKernelGGL((pull_wide_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
-                       (int)t->dim, t->elems, t->group);
+                       (int)t->dim, t->elems, t->group, notes);
   } else if (t->vec == 4) {
     hipLaunchKernelGGL((pull_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
-                       (int)t->dim, t->elems, t->group);
+                       (int)t->dim, t->elems, t->group, notes);
   } else {
     hipLaunchKernelGGL((pull_kernel<1>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
-                       (int)t->dim, t->elems, t->group);
+                       (int)t->dim, t->elems, t->group, notes);
   }
   KRK_HIP(hipGetLastError());
   return KRK_SUCCESS;
@@ -1726,7 +1734,21 @@ int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* ou
   float* d_out;
   KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
   KRK_TRY(t->output(out, (size_t)n * t->dim, flags, 1, &d_out));
-  KRK_TRY(pull_enqueue(t, d_ids, n, d_out));
+  // KRK_NOTE_ROWS: short requests (one launch) leave the row of every position behind
+  uint32_t* notes = nullptr;
+  if (flags & KRK_NOTE_ROWS) {
+    t->noted_ids = nullptr;
+    if ((flags & KRK_DEVICE_PTRS) && n <= kNotedMax) {
+      KRK_TRY(t->notes.reserve((size_t)n * sizeof(uint32_t)));
+      notes = t->notes.as<uint32_t>();
+    }
+  }
+  KRK_TRY(pull_enqueue(t, d_ids, n, d_out, notes));
+  if (notes) {
+    t->noted_ids = ids;
+    t->noted_n = n;
+    t->noted_version = t->layout_version;
+  }
   if ((flags & KRK_ASYNC) && sparse_near_full(t)) KRK_TRY(sparse_publish(&t, 1, t->stream));
   KRK_TRY(t->output_back(out, (size_t)n * t->dim, flags, 1));
   return sparse_finish(t, flags);
@@ -2458,6 +2480,7 @@ int32_t krk_group_destroy(krk_group* g) {
   if (g->d_descs) (void)hipFree(g->d_descs);
   if (g->h_descs) (void)hipHostFree(g->h_descs);
   for (auto& b : g->scratch) b.release();
+  g->notes.release();
   g->stream = g->own_stream;
   g->close_stream();
   delete g;
@@ -2597,17 +2620,34 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
   KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
   KRK_TRY(g->output(out, (size_t)total * g->dim, flags, 1, &d_out));
   const dim3 grid(call.block_start[call.n_tables]), block(kBlock);
+  // KRK_NOTE_ROWS: requests of at most 8192 ids a member leave the row of every position behind
+  uint32_t* notes = nullptr;
+  if (flags & KRK_NOTE_ROWS) {
+    g->noted_ids = nullptr;
+    bool fits = (flags & KRK_DEVICE_PTRS) != 0;
+    for (int i = 0; i < call.n_tables; ++i) fits = fits && offsets[i + 1] - offsets[i] <= kNotedMax;
+    if (fits) {
+      KRK_TRY(g->notes.reserve((size_t)total * sizeof(uint32_t)));
+      notes = g->notes.as<uint32_t>();
+    }
+  }
   if (wide) {
     hipLaunchKernelGGL((group_pull_wide_kernel<4>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
-                       (int)g->dim, g->elems, g->group);
+                       (int)g->dim, g->elems, g->group, notes);
   } else if (g->vec == 4) {
     hipLaunchKernelGGL((group_pull_kernel<4>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
-                       (int)g->dim, g->elems, g->group);
+                       (int)g->dim, g->elems, g->group, notes);
   } else {
     hipLaunchKernelGGL((group_pull_kernel<1>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
-                       (int)g->dim, g->elems, g->group);
+                       (int)g->dim, g->elems, g->group, notes);
   }
   KRK_HIP(hipGetLastError());
+  if (notes) {
+    g->noted_ids = ids;
+    g->noted_offsets.assign(offsets, offsets + call.n_tables + 1);
+    g->noted_versions.clear();
+    for (krk_sparse* t : g->tables) g->noted_versions.push_back(t->layout_version);
+  }
   if (flags & KRK_ASYNC) {
     bool any = false;
     for (krk_sparse* t : g->tables) any = any || sparse_near_full(t);

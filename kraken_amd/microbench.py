@@ -129,6 +129,13 @@ def raw():
         print("dim %3d N %8d U %7d zipf %.2f | push_raw %7.1f us %5.0f GB/s | pull of the N ids %7.1f us | "
               "dedup (blocking call) %7.1f us" % (dim, n, u, s, dt * 1e6, alg / dt / 1e9, dp * 1e6, dd * 1e6),
               flush=True)
+        if n <= 8192:
+            def both(noted):
+                t.Pull(d_ids, out=d_out, async_=True, note_rows=noted)
+                t.PushRaw(o, d_ids, d_g, 0.01, async_=True, as_pulled=noted)
+            plain, noted = timed(t, lambda: both(False)), timed(t, lambda: both(True))
+            print("                                       | pull + push_raw of the same ids %7.1f us, with the pull's "
+                  "row notes %7.1f us" % (plain * 1e6, noted * 1e6), flush=True)
         for a in (d_ids, d_g, d_out, uids, inv):
             a.free()
         t.close()
@@ -160,9 +167,15 @@ def combined():
         for t, d in zip(tables, d_one):
             t.PushRaw(o, d, d_g1, 0.01, async_=True)
 
+    def both(noted):
+        grp.CombinePull(d_ids, off, out=d_out, async_=True, note_rows=noted)
+        grp.CombinePushRaw(o, d_ids, off, d_g, 0.01, async_=True, as_pulled=noted)
+
     for name, fn in (
             ("combined pull of all ids", lambda: grp.CombinePull(d_ids, off, out=d_out, async_=True)),
             ("combined push with repeats", lambda: grp.CombinePushRaw(o, d_ids, off, d_g, 0.01, async_=True)),
+            ("pull + push of the same ids", lambda: both(False)),
+            ("the same with the pull's row notes", lambda: both(True)),
             ("push_raw table by table (26 calls)", per_table)):
         print("%-36s %8.1f us" % (name, timed(grp, fn, 10) * 1e6), flush=True)
     grp.close()
@@ -499,12 +512,15 @@ def worker_boundary_leg(cfg, tables, group, optim, lr, n_batches=8, reps=20):
         d_ids, d_g, off = dev[k[0] % n_batches]
         assert group.CombinePushRaw(optim, d_ids, off, d_g, lr, async_=True) == 0
 
-    def step():
-        pull()
-        k[0] -= 1
-        push()
+    def step(noted):
+        # the worker's sequence: the rows of a batch's ids, then the gradients of the same ids
+        k[0] += 1
+        d_ids, d_g, off = dev[k[0] % n_batches]
+        assert group.CombinePull(d_ids, off, out=d_out, async_=True, note_rows=noted)[0] == 0
+        assert group.CombinePushRaw(optim, d_ids, off, d_g, lr, async_=True, as_pulled=noted) == 0
 
-    t_pull, t_push, t_step = (timed(group, f, reps) for f in (pull, push, step))
+    t_pull, t_push, t_plain, t_step = (timed(group, f, reps) for f in (
+        pull, push, lambda: step(False), lambda: step(True)))
     n, u, S = float(np.mean(n_ids)), float(np.mean(n_unique)), _states(cfg["optim"])
     b_pull, b_push = pull_bytes_expanded(n, u, dim), push_raw_bytes(n, u, dim, S)
     for d in dev:
@@ -514,7 +530,10 @@ def worker_boundary_leg(cfg, tables, group, optim, lr, n_batches=8, reps=20):
     return {"workload": "wide_deep, ids with repeats: %d tables x %d ids, dim %d, %s" % (
                 cfg["tables"], cfg["batch"], dim, cfg["optim"]),
             "ids_per_step": n, "distinct_rows_per_step": u,
-            "step": _leg(t_step * 1e3, b_pull + b_push), "group_pull": _leg(t_pull * 1e3, b_pull),
+            # step: the push reuses the rows the pull noted (KRK_NOTE_ROWS / KRK_IDS_AS_PULLED)
+            "step": _leg(t_step * 1e3, b_pull + b_push),
+            "step_ids_looked_up_twice": _leg(t_plain * 1e3, b_pull + b_push),
+            "group_pull": _leg(t_pull * 1e3, b_pull),
             "group_push_raw": _leg(t_push * 1e3, b_push), "ids_per_s": n / t_step}
 
 
