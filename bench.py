@@ -130,7 +130,8 @@ def lines_per_row(dim, states, word):
     return 1 + w_lines, 1, -(-rec_bytes // 128)
 
 
-def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, drained_blocks=8):
+def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, drained_blocks=8,
+            noted_blocks=10):
     """Builds the workload's tables, fills their key space and times `blocks` blocks of `steps`
     steps each between events on the stream the sparse kernels run on. -> dict of figures."""
     import ctypes as C
@@ -201,10 +202,15 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, 
         if dense is not None:
             dpush = (L.krk_dense_push, (dense.h, C.byref(dense_opt.raw), C.c_void_p(d_dense_g[i].ptr),
                                         cfg["dense"], 1e-3, flags))
-        calls.append((pull, push, dpush))
+        # the same two calls with the push told that its ids are the pull's (a second figure,
+        # not the headline: the pull then notes every position's row and the push skips its look-up)
+        noted_pull = (pull[0], pull[1][:-1] + (flags | api.NOTE_ROWS,))
+        noted_push = (push[0], push[1][:-1] + (flags | api.IDS_AS_PULLED,))
+        calls.append((pull, push, dpush, noted_pull, noted_push))
 
-    def step(i):
-        pull, push, dpush = calls[i % n_batches]
+    def step(i, noted=False):
+        pull, push, dpush = calls[i % n_batches][3 if noted else 0], calls[i % n_batches][4 if noted else 1], \
+            calls[i % n_batches][2]
         rc = pull[0](*pull[1]) | push[0](*push[1])
         if dpush is not None:
             rc |= dpush[0](*dpush[1])
@@ -262,13 +268,29 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, 
             sync_all()
             drained.append((time.perf_counter() - t0) / steps)
             gc.collect()
+        # 3. as 1., with KRK_NOTE_ROWS on the pull and KRK_IDS_AS_PULLED on the push
+        noted_marks = [api.Event() for _ in range(noted_blocks + 1)]
+        for i in range(steps):
+            step(i, True)
+        noted_marks[0].record(owner)
+        for b in range(noted_blocks):
+            for i in range(steps):
+                step(i, True)
+            if b == noted_blocks - 1 and dense is not None:
+                dense_done.record(dense)
+                dense_done.wait(owner)
+            noted_marks[b + 1].record(owner)
+        sync_all()
+        noted = [noted_marks[b].elapsed_ms(noted_marks[b + 1]) * 1e-3 / steps for b in range(noted_blocks)]
     finally:
         gc.enable()
+    noted_med = float(np.median(noted))
     med, p10, p90 = _percentiles(per_step)
     drained_med = float(np.median(drained)) if drained else None
     print("dim %d: %.2f us/step between events (p10 %.2f, p90 %.2f; %d blocks of %d steps), %.2f us/step with a "
-          "host drain per block, host enqueue %.1f us/step" % (
-              dim, med * 1e6, p10 * 1e6, p90 * 1e6, blocks, steps, (drained_med or 0) * 1e6, enqueue_s * 1e6),
+          "host drain per block, host enqueue %.1f us/step; %.2f us/step when the push reuses the pull's rows" % (
+              dim, med * 1e6, p10 * 1e6, p90 * 1e6, blocks, steps, (drained_med or 0) * 1e6, enqueue_s * 1e6,
+              noted_med * 1e6),
           file=sys.stderr)
 
     # the two kernels of the step: M back-to-back launches on the owner's stream, bracketed by
@@ -314,6 +336,11 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, 
         "value": rows_per_step / med, "ms_per_step": med * 1e3, "ms_per_step_p10": p10 * 1e3,
         "ms_per_step_p90": p90 * 1e3, "blocks": blocks, "rows_per_step": rows_per_step,
         "ms_per_step_host_drained": drained_med * 1e3 if drained_med else None,
+        # KRK_NOTE_ROWS on the pull, KRK_IDS_AS_PULLED on the push: the worker's pull-then-push of
+        # one batch with the second look-up of the ids left out. Not what `value` is computed from.
+        "ms_per_step_ids_as_pulled": noted_med * 1e3,
+        "frac_whole_step_ids_as_pulled": rows_per_step / noted_med * (16 + 4 * dim * (2 + 1 + 2 * (1 + S)) + (
+            16 if cfg["optim"] == "adam" else 0)) / 1e9 / HBM_PEAK_GBS,
         "host_enqueue_us_per_step": enqueue_s * 1e6,
         "algorithmic_bytes_per_row": per_row,
         "achieved_gbs_whole_step": rows_per_step / med * per_row / 1e9,

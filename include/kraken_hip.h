@@ -45,13 +45,15 @@ extern "C" {
  * KRK_DEVICE_PTRS and are ignored by every other call.
  * KRK_NOTE_ROWS on krk_sparse_pull / krk_group_pull: the table (group) also keeps the row
  * number of every position of this request (4 bytes a position, in memory of its own) until
- * its next pull with the flag; requests above 8192 ids a table are not noted.
- * KRK_IDS_AS_PULLED on krk_sparse_push_raw / krk_group_push_raw: the caller states that `ids`
- * is the buffer of that pull (same pointer, same counts) with its contents unchanged. The call
- * then skips its own look-up of the ids. It looks the ids up as usual when the pointer or the
- * counts differ from what was noted, when nothing was noted, or when rows have moved since
- * (krk_sparse_erase, a table that grew or gained optimizer columns). Results are the same
- * either way; ids whose contents did change give the updates of the old ids' rows. */
+ * its next pull with the flag; single-table requests of 2^18 ids and more are not noted.
+ * KRK_IDS_AS_PULLED on krk_sparse_push / krk_sparse_push_raw / krk_group_push /
+ * krk_group_push_raw: the caller states that `ids` is the buffer of that pull (same pointer,
+ * same counts) with its contents unchanged. The call then skips its own look-up of the ids
+ * (push_raw: for requests of at most 8192 ids a table, where the look-up is a launch of its
+ * own). It looks the ids up as usual when the pointer or the counts differ from what was
+ * noted, when nothing was noted, or when rows have moved since (krk_sparse_erase, a table that
+ * grew or gained optimizer columns). Results are the same either way; ids whose contents did
+ * change give the updates of the old ids' rows. */
 #define KRK_NOTE_ROWS 0x4u
 #define KRK_IDS_AS_PULLED 0x8u
 

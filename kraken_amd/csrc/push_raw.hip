@@ -857,7 +857,7 @@ static int pick_tile(int64_t cnt) {
 constexpr int kSortBlock = 1024;
 constexpr int kSortItems = 8;
 constexpr int kSortMax = kSortBlock * kSortItems;      // ids per table
-static_assert(kSortMax == kNotedMax, "row notes are kept for exactly the requests that take this path");
+static_assert(kSortMax <= kNotedMax, "row notes are kept for the requests that take this path");
 constexpr int kSortWaves = kSortBlock / kWave;
 constexpr int kMaxBucketBits = 5;                      // up to 32 buckets a table
 constexpr int kDigitBits = 9;
@@ -1886,9 +1886,8 @@ int32_t krk_sparse_push_raw(krk_sparse* t, const krk_optim* o, const uint64_t* i
     const TableView tv = t->view();
     // KRK_IDS_AS_PULLED: the rows of these very ids were noted by the pull before (and nothing
     // has moved since): the look-up launch is not needed
-    const bool noted = (flags & KRK_IDS_AS_PULLED) && t->noted_ids == ids && t->noted_n == n &&
-                       t->noted_version == t->layout_version;
-    const uint32_t* keys = t->notes.as<uint32_t>();
+    const uint32_t* keys = noted_rows(t, ids, n, flags);
+    const bool noted = keys != nullptr;
     if (!noted) {
       KRK_TRY(t->scratch[0].reserve((size_t)n * sizeof(uint32_t)));
       uint32_t* found = t->scratch[0].as<uint32_t>();
@@ -1996,12 +1995,8 @@ int32_t krk_group_push_raw(krk_group* g, const krk_optim* o, const uint64_t* ids
     // KRK_IDS_AS_PULLED: the rows of these very ids were noted by the combined pull before (and
     // nothing has moved since): the look-up launch is not needed. A note is a member's own row
     // number, which is all the bucket kernel reads of a key.
-    bool noted = (flags & KRK_IDS_AS_PULLED) && g->noted_ids == ids &&
-                 g->noted_offsets.size() == (size_t)n_tables + 1 && g->noted_versions.size() == (size_t)n_tables;
-    for (int m = 0; noted && m < n_tables; ++m)
-      noted = g->noted_offsets[m] == offsets[m] && g->noted_offsets[m + 1] == offsets[m + 1] &&
-              g->noted_versions[m] == g->tables[m]->layout_version;
-    const uint32_t* keys = g->notes.as<uint32_t>();
+    const uint32_t* keys = noted_rows(g, ids, offsets, flags);
+    const bool noted = keys != nullptr;
     if (!noted) {
       KRK_TRY(g->scratch[0].reserve((size_t)total * sizeof(uint32_t)));
       uint32_t* found = g->scratch[0].as<uint32_t>();

@@ -335,9 +335,9 @@ __device__ inline uint32_t probe_find_alone(const TableView& tv, uint64_t id) {
 struct krk_group;
 
 namespace krk {
-// Requests of at most this many ids a table keep row notes (KRK_NOTE_ROWS): the size up to
-// which push_raw runs as look-up + one launch per bucket, where the look-up is a fifth of it.
-constexpr int64_t kNotedMax = 8192;
+// Requests of at most this many ids a table keep row notes (KRK_NOTE_ROWS): the pulls that run
+// as one launch.
+constexpr int64_t kNotedMax = (1 << 18) - 1;
 }  // namespace krk
 
 // The handle behind krk_sparse*.
@@ -441,6 +441,23 @@ struct krk_group : krk::ObjBase {
 };
 
 namespace krk {
+// KRK_IDS_AS_PULLED: the row notes of the pull of these very ids, or null when they do not apply
+// (another buffer or count, nothing noted, rows moved since). The caller holds the lock(s).
+inline const uint32_t* noted_rows(const krk_sparse* t, const uint64_t* ids, int64_t n, uint32_t flags) {
+  const bool ok = (flags & KRK_IDS_AS_PULLED) && t->noted_ids && t->noted_ids == ids && t->noted_n == n &&
+                  t->noted_version == t->layout_version;
+  return ok ? t->notes.as<uint32_t>() : nullptr;
+}
+inline const uint32_t* noted_rows(const krk_group* g, const uint64_t* ids, const int64_t* offsets, uint32_t flags) {
+  const size_t n = g->tables.size();
+  bool ok = (flags & KRK_IDS_AS_PULLED) && g->noted_ids && g->noted_ids == ids && g->noted_offsets.size() == n + 1 &&
+            g->noted_versions.size() == n;
+  for (size_t m = 0; ok && m < n; ++m)
+    ok = g->noted_offsets[m] == offsets[m] && g->noted_offsets[m + 1] == offsets[m + 1] &&
+         g->noted_versions[m] == g->tables[m]->layout_version;
+  return ok ? g->notes.as<uint32_t>() : nullptr;
+}
+
 // Takes the group's lock and then every member's, in member order.
 struct GroupLock {
   krk_group* g;

@@ -154,11 +154,28 @@ struct PushCols {
   int c0, c1, c2, meta;
 };
 
+// The row of ids[i] for a push: looked up, or taken from the notes of the pull of the same ids
+// (KRK_IDS_AS_PULLED). A note of kEmptyRow was taken before the row's creator had published the
+// number (or the table was full): those are looked up after all. Wave-wide like probe_find.
+__device__ __forceinline__ uint32_t row_for_push(const TableView& tv, const uint64_t* __restrict__ ids,
+                                                 int64_t i, bool active, int gl, int group,
+                                                 const uint32_t* __restrict__ notes) {
+  if (!notes) return probe_find(tv, active ? ids[i] : 0, active, gl, group);
+  uint32_t row = active ? notes[i] : kEmptyRow;
+  const bool again = active && row == kEmptyRow;
+  if (__any(again)) {
+    const uint32_t r = probe_find(tv, again ? ids[i] : 0, again, gl, group);
+    if (again) row = r;
+  }
+  return row;
+}
+
 template <int OPT, int VEC>
 __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* __restrict__ ids,
                                           int64_t i, bool active, int gl,
                                           const float* __restrict__ grads, int dim, int elems,
-                                          int group, float lr, const OptimK& k, const PushCols& pc) {
+                                          int group, float lr, const OptimK& k, const PushCols& pc,
+                                          const uint32_t* __restrict__ notes = nullptr) {
   // The gradient row does not depend on the index: its first slice is requested before the
   // probe so that it travels while the probe waits for its bucket.
   const float* g = grads + i * (int64_t)dim;
@@ -166,7 +183,7 @@ __device__ __forceinline__ void push_body(const TableView& tv, const uint64_t* _
 #pragma unroll
   for (int c = 0; c < VEC; ++c) g_first[c] = 0.0f;
   if (active && gl < elems) vload_once<VEC>(g + gl * VEC, g_first);
-  const uint32_t row = probe_find(tv, active ? ids[i] : 0, active, gl, group);
+  const uint32_t row = row_for_push(tv, ids, i, active, gl, group, notes);
   if (!active) return;
   if (row == kEmptyRow) {
     if (gl == 0) atomicOr(&tv.counters[1], kErrMissingId);
@@ -401,10 +418,11 @@ template <int OPT, int VEC>
 __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64_t* __restrict__ ids,
                                                       int64_t n, const float* __restrict__ grads,
                                                       int dim, int elems, int group, float lr,
-                                                      OptimK k, PushCols pc) {
+                                                      OptimK k, PushCols pc,
+                                                      const uint32_t* __restrict__ notes) {
   const int per_block = kBlock / group;
   const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
-  push_body<OPT, VEC>(tv, ids, i, i < n, threadIdx.x & (group - 1), grads, dim, elems, group, lr, k, pc);
+  push_body<OPT, VEC>(tv, ids, i, i < n, threadIdx.x & (group - 1), grads, dim, elems, group, lr, k, pc, notes);
 }
 
 // ---- pulls of rows 32 to 128 floats wide -------------------------------------------------------
@@ -522,7 +540,7 @@ template <int OPT, int STEPS>
 __device__ __forceinline__ void push_wide(const TableView& tv, const uint64_t* __restrict__ ids,
                                           int64_t first, int64_t end, const float* __restrict__ grads,
                                           int dim, int elems, float lr, const OptimK& k,
-                                          const PushCols& pc) {
+                                          const PushCols& pc, const uint32_t* __restrict__ notes = nullptr) {
   constexpr int VEC = 4;
   constexpr int rows_per_step = kWideIds / STEPS;   // 8, 4 or 2
   constexpr int group = kWave / rows_per_step;      // 8, 16 or 32
@@ -541,7 +559,7 @@ __device__ __forceinline__ void push_wide(const TableView& tv, const uint64_t* _
   }
   const int64_t i = first + (lane >> 2);
   const bool active = i < end;
-  const uint32_t my_row = probe_find(tv, active ? ids[i] : 0, active, lane & (kBucket - 1), kBucket);
+  const uint32_t my_row = row_for_push(tv, ids, i, active, lane & (kBucket - 1), kBucket, notes);
   if (active && my_row == kEmptyRow && (lane & (kBucket - 1)) == 0) atomicOr(&tv.counters[1], kErrMissingId);
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
@@ -603,10 +621,10 @@ template <int OPT, int STEPS>
 __global__ __launch_bounds__(kBlock) void push_wide_kernel(TableView tv, const uint64_t* __restrict__ ids,
                                                            int64_t n, const float* __restrict__ grads,
                                                            int dim, int elems, float lr, OptimK k,
-                                                           PushCols pc) {
+                                                           PushCols pc, const uint32_t* __restrict__ notes) {
   const int64_t first = ((int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds;
   if (first >= n) return;                        // the whole wavefront
-  push_wide<OPT, STEPS>(tv, ids, first, n, grads, dim, elems, lr, k, pc);
+  push_wide<OPT, STEPS>(tv, ids, first, n, grads, dim, elems, lr, k, pc, notes);
 }
 
 template <int VEC>
@@ -701,7 +719,8 @@ __global__ __launch_bounds__(kBlock) void group_push_kernel(const TableDesc* __r
                                                             const uint64_t* __restrict__ ids,
                                                             const float* __restrict__ grads, int dim,
                                                             int elems, int group, float lr, OptimK k,
-                                                            int st0, int st1, int st2, int use_meta) {
+                                                            int st0, int st1, int st2, int use_meta,
+                                                            const uint32_t* __restrict__ notes) {
   const uint32_t bx = blockIdx.x;
   const int t = find_table(call, bx);
   const TableView tv = descs[t].tv;
@@ -714,7 +733,7 @@ __global__ __launch_bounds__(kBlock) void group_push_kernel(const TableDesc* __r
   const int64_t local = (int64_t)(bx - call.block_start[t]) * per_block + threadIdx.x / group;
   const int64_t i = call.row_start[t] + local;
   push_body<OPT, VEC>(tv, ids, i, i < call.row_start[t + 1], threadIdx.x & (group - 1), grads, dim,
-                      elems, group, lr, k, pc);
+                      elems, group, lr, k, pc, notes);
 }
 
 // the same for rows 32 to 128 floats wide: a workgroup takes 64 positions of its table
@@ -724,7 +743,8 @@ __global__ __launch_bounds__(kBlock) void group_push_wide_kernel(const TableDesc
                                                                  const uint64_t* __restrict__ ids,
                                                                  const float* __restrict__ grads, int dim,
                                                                  int elems, float lr, OptimK k, int st0,
-                                                                 int st1, int st2, int use_meta) {
+                                                                 int st1, int st2, int use_meta,
+                                                                 const uint32_t* __restrict__ notes) {
   const uint32_t bx = blockIdx.x;
   const int t = find_table(call, bx);
   const TableView tv = descs[t].tv;
@@ -737,7 +757,7 @@ __global__ __launch_bounds__(kBlock) void group_push_wide_kernel(const TableDesc
                         kWideIds;
   const int64_t first = call.row_start[t] + local;
   if (first >= call.row_start[t + 1]) return;    // the whole wavefront
-  push_wide<OPT, STEPS>(tv, ids, first, call.row_start[t + 1], grads, dim, elems, lr, k, pc);
+  push_wide<OPT, STEPS>(tv, ids, first, call.row_start[t + 1], grads, dim, elems, lr, k, pc, notes);
 }
 
 __global__ __launch_bounds__(kBlock) void lookup_kernel(TableView tv, const uint64_t* __restrict__ ids,
@@ -1491,7 +1511,7 @@ static InitK make_init_k(const krk_init& in, int64_t dim) {
 // Enqueues push_kernel or, for whole rows of 32 to 128 floats, push_wide_kernel.
 template <int OPT, int VEC>
 static void launch_push_opt(krk_sparse* t, const uint64_t* ids, int64_t n, const float* grads, float lr,
-                            const OptimK& k, const PushCols& pc) {
+                            const OptimK& k, const PushCols& pc, const uint32_t* notes) {
   const TableView tv = t->view();
   const int dim = (int)t->dim;
   const dim3 block(kBlock);
@@ -1500,32 +1520,32 @@ static void launch_push_opt(krk_sparse* t, const uint64_t* ids, int64_t n, const
       const dim3 grid(grid_for(n, (kBlock / kWave) * kWideIds));
       if (t->group == 8) {
         hipLaunchKernelGGL((push_wide_kernel<OPT, 2>), grid, block, 0, t->stream, tv, ids, n, grads, dim,
-                           t->elems, lr, k, pc);
+                           t->elems, lr, k, pc, notes);
       } else {
         hipLaunchKernelGGL((push_wide_kernel<OPT, 4>), grid, block, 0, t->stream, tv, ids, n, grads, dim,
-                           t->elems, lr, k, pc);
+                           t->elems, lr, k, pc, notes);
       }
       return;
     }
   }
   const dim3 grid(grid_for(n, kBlock / t->group));
   hipLaunchKernelGGL((push_kernel<OPT, VEC>), grid, block, 0, t->stream, tv, ids, n, grads, dim, t->elems,
-                     t->group, lr, k, pc);
+                     t->group, lr, k, pc, notes);
 }
 
 template <int VEC>
 static void launch_push(krk_sparse* t, const krk_optim& o, const uint64_t* ids, int64_t n,
-                        const float* grads, float lr) {
+                        const float* grads, float lr, const uint32_t* notes = nullptr) {
   const OptimK k = make_optim_k(o);
   int32_t cols[3];
   sparse_optim_columns(t, o, cols);
   const bool needs_meta = (optim_state_mask(o) >> KRK_ST_STEPS) & 1u;
   const PushCols pc{cols[0], cols[1], cols[2], needs_meta ? t->meta_off : -1};
   switch (o.type) {
-    case KRK_SGD: launch_push_opt<KRK_SGD, VEC>(t, ids, n, grads, lr, k, pc); break;
-    case KRK_ADAGRAD: launch_push_opt<KRK_ADAGRAD, VEC>(t, ids, n, grads, lr, k, pc); break;
-    case KRK_ADAM: launch_push_opt<KRK_ADAM, VEC>(t, ids, n, grads, lr, k, pc); break;
-    default: launch_push_opt<KRK_RMSPROP, VEC>(t, ids, n, grads, lr, k, pc); break;
+    case KRK_SGD: launch_push_opt<KRK_SGD, VEC>(t, ids, n, grads, lr, k, pc, notes); break;
+    case KRK_ADAGRAD: launch_push_opt<KRK_ADAGRAD, VEC>(t, ids, n, grads, lr, k, pc, notes); break;
+    case KRK_ADAM: launch_push_opt<KRK_ADAM, VEC>(t, ids, n, grads, lr, k, pc, notes); break;
+    default: launch_push_opt<KRK_RMSPROP, VEC>(t, ids, n, grads, lr, k, pc, notes); break;
   }
 }
 
@@ -1734,7 +1754,7 @@ int32_t krk_sparse_pull(krk_sparse* t, const uint64_t* ids, int64_t n, float* ou
   float* d_out;
   KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
   KRK_TRY(t->output(out, (size_t)n * t->dim, flags, 1, &d_out));
-  // KRK_NOTE_ROWS: short requests (one launch) leave the row of every position behind
+  // KRK_NOTE_ROWS: requests served by one launch leave the row of every position behind
   uint32_t* notes = nullptr;
   if (flags & KRK_NOTE_ROWS) {
     t->noted_ids = nullptr;
@@ -1845,10 +1865,11 @@ int32_t krk_sparse_push(krk_sparse* t, const krk_optim* o, const uint64_t* ids, 
   const float* d_g;
   KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
   KRK_TRY(t->input(grads, (size_t)n * t->dim, flags, 1, &d_g));
+  const uint32_t* notes = noted_rows(t, ids, n, flags);   // KRK_IDS_AS_PULLED: no second look-up
   if (t->vec == 4) {
-    launch_push<4>(t, *o, d_ids, n, d_g, lr);
+    launch_push<4>(t, *o, d_ids, n, d_g, lr, notes);
   } else {
-    launch_push<1>(t, *o, d_ids, n, d_g, lr);
+    launch_push<1>(t, *o, d_ids, n, d_g, lr, notes);
   }
   KRK_HIP(hipGetLastError());
   return sparse_finish(t, flags);
@@ -2620,13 +2641,11 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
   KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
   KRK_TRY(g->output(out, (size_t)total * g->dim, flags, 1, &d_out));
   const dim3 grid(call.block_start[call.n_tables]), block(kBlock);
-  // KRK_NOTE_ROWS: requests of at most 8192 ids a member leave the row of every position behind
+  // KRK_NOTE_ROWS: the row of every position stays behind
   uint32_t* notes = nullptr;
   if (flags & KRK_NOTE_ROWS) {
     g->noted_ids = nullptr;
-    bool fits = (flags & KRK_DEVICE_PTRS) != 0;
-    for (int i = 0; i < call.n_tables; ++i) fits = fits && offsets[i + 1] - offsets[i] <= kNotedMax;
-    if (fits) {
+    if (flags & KRK_DEVICE_PTRS) {
       KRK_TRY(g->notes.reserve((size_t)total * sizeof(uint32_t)));
       notes = g->notes.as<uint32_t>();
     }
@@ -2662,40 +2681,41 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
 template <int OPT, int VEC>
 static void launch_group_push_opt(krk_group* g, const GroupCall& call, const uint64_t* ids,
                                   const float* grads, float lr, const OptimK& k, const int32_t st[3],
-                                  int use_meta, bool wide) {
+                                  int use_meta, bool wide, const uint32_t* notes) {
   const dim3 grid(call.block_start[call.n_tables]), block(kBlock);
   const int dim = (int)g->dim;
   if constexpr (VEC == 4) {
     if (wide) {
       if (g->group == 8) {
         hipLaunchKernelGGL((group_push_wide_kernel<OPT, 2>), grid, block, 0, g->stream, g->d_descs, call,
-                           ids, grads, dim, g->elems, lr, k, st[0], st[1], st[2], use_meta);
+                           ids, grads, dim, g->elems, lr, k, st[0], st[1], st[2], use_meta, notes);
       } else {
         hipLaunchKernelGGL((group_push_wide_kernel<OPT, 4>), grid, block, 0, g->stream, g->d_descs, call,
-                           ids, grads, dim, g->elems, lr, k, st[0], st[1], st[2], use_meta);
+                           ids, grads, dim, g->elems, lr, k, st[0], st[1], st[2], use_meta, notes);
       }
       return;
     }
   }
   hipLaunchKernelGGL((group_push_kernel<OPT, VEC>), grid, block, 0, g->stream, g->d_descs, call, ids, grads,
-                     dim, g->elems, g->group, lr, k, st[0], st[1], st[2], use_meta);
+                     dim, g->elems, g->group, lr, k, st[0], st[1], st[2], use_meta, notes);
 }
 
 // wide: the request was laid out for group_push_wide_kernel (64 positions a workgroup)
 template <int VEC>
 static void launch_group_push(krk_group* g, const krk_optim& o, const GroupCall& call,
-                              const uint64_t* ids, const float* grads, float lr, bool wide) {
+                              const uint64_t* ids, const float* grads, float lr, bool wide,
+                              const uint32_t* notes) {
   const OptimK k = make_optim_k(o);
   int32_t st[3];
   optim_state_slots(o, st);
   const int use_meta = (optim_state_mask(o) >> KRK_ST_STEPS) & 1u;
   switch (o.type) {
-    case KRK_SGD: launch_group_push_opt<KRK_SGD, VEC>(g, call, ids, grads, lr, k, st, use_meta, wide); break;
+    case KRK_SGD: launch_group_push_opt<KRK_SGD, VEC>(g, call, ids, grads, lr, k, st, use_meta, wide, notes); break;
     case KRK_ADAGRAD:
-      launch_group_push_opt<KRK_ADAGRAD, VEC>(g, call, ids, grads, lr, k, st, use_meta, wide);
+      launch_group_push_opt<KRK_ADAGRAD, VEC>(g, call, ids, grads, lr, k, st, use_meta, wide, notes);
       break;
-    case KRK_ADAM: launch_group_push_opt<KRK_ADAM, VEC>(g, call, ids, grads, lr, k, st, use_meta, wide); break;
-    default: launch_group_push_opt<KRK_RMSPROP, VEC>(g, call, ids, grads, lr, k, st, use_meta, wide); break;
+    case KRK_ADAM: launch_group_push_opt<KRK_ADAM, VEC>(g, call, ids, grads, lr, k, st, use_meta, wide, notes); break;
+    default: launch_group_push_opt<KRK_RMSPROP, VEC>(g, call, ids, grads, lr, k, st, use_meta, wide, notes); break;
   }
 }
 
@@ -2731,10 +2751,11 @@ int32_t krk_group_push(krk_group* g, const krk_optim* o, const uint64_t* ids, co
   KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
   KRK_TRY(g->input(grads, (size_t)total * g->dim, flags, 1, &d_g));
   for (int i = 0; i < call.n_tables; ++i) call.epoch[i] = 0;
+  const uint32_t* notes = noted_rows(g, ids, offsets, flags);   // KRK_IDS_AS_PULLED: no second look-up
   if (g->vec == 4) {
-    launch_group_push<4>(g, *o, call, d_ids, d_g, lr, wide);
+    launch_group_push<4>(g, *o, call, d_ids, d_g, lr, wide, notes);
   } else {
-    launch_group_push<1>(g, *o, call, d_ids, d_g, lr, false);
+    launch_group_push<1>(g, *o, call, d_ids, d_g, lr, false, notes);
   }
   KRK_HIP(hipGetLastError());
   return group_finish(g, flags);

@@ -157,7 +157,7 @@ def test_notes_are_dropped_when_they_do_not_apply(api):
     big = np.arange(300000, 300000 + 9000, dtype=np.uint64)
     d_big = api.DeviceArray.from_host(big)
     d_gbig = api.DeviceArray.from_host(np.ones((big.size, dim), np.float32))
-    assert t.Pull(d_big, note_rows=True)[0] == 0         # too long to be noted: drops the older notes too
+    assert t.Pull(d_big, note_rows=True)[0] == 0         # noted, but a push_raw this long sorts by itself
     before = t.Pull(big)[1]
     assert t.Push(o, d_big, d_gbig, float(lr), raw=True, as_pulled=True) == 0
     assert np.array_equal(t.Pull(big)[1], before - lr)
@@ -204,5 +204,78 @@ def test_group_with_notes_equals_without(api, dim):
     counts2 = [3000, 0, 1, 8192 - 5, 777 + 5]
     off2 = ga._offsets(counts2)
     assert ga.CombinePushRaw(o, d_ids, off2, d_g, 0.05, as_pulled=True) in (0, 12)
+    ga.close()
+    gb.close()
+
+
+@pytest.mark.parametrize("dim", [16, 64, 5])
+@pytest.mark.parametrize("optim", ["adagrad", "adam"])
+def test_push_of_unique_ids_with_notes_equals_without(api, dim, optim):
+    """krk_sparse_push after a noting pull of the same unique ids (narrow rows, the wide kernels,
+    rows that are no multiple of four floats), three steps with fresh ids, against the plain calls."""
+    rng = np.random.default_rng(100 + dim)
+    o = api.Optim.create(api.OptimType.kAdagrad if optim == "adagrad" else api.OptimType.kAdam)
+    a, b = api.SparseTable(dim, _init(api)), api.SparseTable(dim, _init(api))
+    for step in range(3):
+        ids = np.unique(zipf_ids(rng, 1.05, 40000, 12000) + np.uint64(step * 9000))
+        rng.shuffle(ids)
+        d_ids = api.DeviceArray.from_host(ids)
+        d_g = api.DeviceArray.from_host((rng.standard_normal((ids.size, dim)) * 0.1).astype(np.float32))
+        assert a.Pull(d_ids, note_rows=True)[0] == 0
+        assert b.Pull(d_ids)[0] == 0
+        assert a.Push(o, d_ids, d_g, 0.05, as_pulled=True) == 0
+        assert b.Push(o, d_ids, d_g, 0.05) == 0
+    S = api.StateType
+    _same_tables(api, a, b, [S.kStateSum] if optim == "adagrad" else [S.kFirstMoment, S.kSecondMoment])
+    a.close()
+    b.close()
+
+
+def test_flagged_push_reads_the_notes_and_drops_stale_ones(api):
+    """As for push_raw: with the buffer overwritten after the pull the flagged push updates the
+    rows that were pulled; after an erase it looks the ids up (and reports the missing ones)."""
+    dim, n = 32, 5000
+    o = api.Optim.create(api.OptimType.kSGD)
+    t = api.SparseTable(dim, _init(api))
+    x = np.arange(1, n + 1, dtype=np.uint64)
+    y = x + np.uint64(100000)
+    t.Pull(y)
+    before_y = t.Pull(y)[1]
+    d_ids = api.DeviceArray.from_host(x)
+    d_g = api.DeviceArray.from_host(np.ones((n, dim), np.float32))
+    before_x = t.Pull(d_ids, note_rows=True)[1].to_host()
+    _h2d(api, d_ids, y)
+    assert t.Push(o, d_ids, d_g, 0.5, as_pulled=True) == 0
+    assert np.array_equal(t.Pull(y)[1], before_y)
+    assert np.array_equal(t.Pull(x)[1], before_x - np.float32(0.5))
+    _h2d(api, d_ids, x)
+    assert t.Pull(d_ids, note_rows=True)[0] == 0
+    t.erase(x[:100])
+    assert t.Push(o, d_ids, d_g, 0.5, as_pulled=True) == 12            # the erased ids are gone
+    assert np.array_equal(t.Pull(x[100:])[1], before_x[100:] - np.float32(0.5) - np.float32(0.5))
+    t.close()
+
+
+@pytest.mark.parametrize("dim", [16, 32])
+def test_group_push_of_unique_ids_with_notes_equals_without(api, dim):
+    rng = np.random.default_rng(7 + dim)
+    o = api.Optim.create(api.OptimType.kAdagrad)
+    counts = [3790, 0, 1, 9000, 64]
+    ta = [api.SparseTable(dim, _init(api)) for _ in counts]
+    tb = [api.SparseTable(dim, _init(api)) for _ in counts]
+    ga, gb = api.TableGroup(ta), api.TableGroup(tb)
+    off = ga._offsets(counts)
+    total = int(off[-1])
+    for step in range(3):
+        per = [rng.permutation(np.arange(1, 20001, dtype=np.uint64))[:c] + np.uint64(step * 3000) for c in counts]
+        d_ids = api.DeviceArray.from_host(np.concatenate(per))
+        d_g = api.DeviceArray.from_host((rng.standard_normal((total, dim)) * 0.1).astype(np.float32))
+        assert ga.CombinePull(d_ids, off, note_rows=True)[0] == 0
+        assert gb.CombinePull(d_ids, off)[0] == 0
+        assert ga.CombinePush(o, d_ids, off, d_g, 0.05, as_pulled=True) == 0
+        assert gb.CombinePush(o, d_ids, off, d_g, 0.05) == 0
+    for a, b, c in zip(ta, tb, counts):
+        if c:
+            _same_tables(api, a, b, [api.StateType.kStateSum])
     ga.close()
     gb.close()
