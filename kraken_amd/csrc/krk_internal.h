@@ -162,17 +162,40 @@ struct InitK {
   uint64_t seed_mix;  // splitmix64(seed)
 };
 
+// Normal draws come in pairs: elements 2q and 2q + 1 of a row are the two values of one
+// Box-Muller step on the bits drawn for q (radius from the upper 24 bits, angle from the next
+// 24: radius * cos(angle) and radius * cos(angle - pi/2), independent standard normals; the
+// second is written as a cosine so that both take the same code). A kernel that makes whole
+// rows pays the logarithm and the square root once per two elements (init_normal_pair); one
+// that makes a single element evaluates only the half it needs.
+constexpr double kHalfPi = 1.5707963267948966192313216916398;
+__device__ inline void normal_polar(uint64_t key, int64_t q, double& radius, double& angle) {
+  const uint64_t r = splitmix64(key + (uint64_t)q * 0x9E3779B97F4A7C15ull);
+  const double u1 = (double)((r >> 40) + 1) * (1.0 / 16777216.0);
+  const double u2 = (double)((r >> 16) & 0xFFFFFFull) * (1.0 / 16777216.0);
+  radius = sqrt(-2.0 * log(u1));
+  angle = 6.283185307179586476925286766559 * u2;
+}
+
+__device__ inline void init_normal_pair(const InitK& k, uint64_t key, int64_t q, float& even, float& odd) {
+  double radius, angle;
+  normal_polar(key, q, radius, angle);
+  even = (float)((double)k.p0 + (double)k.p1 * (radius * cos(angle)));
+  odd = (float)((double)k.p0 + (double)k.p1 * (radius * cos(angle - kHalfPi)));
+}
+
 __device__ inline float init_element(const InitK& k, uint64_t id, int64_t j) {
   if (k.kind == 0) return k.p0;
   uint64_t key = splitmix64(id ^ k.seed_mix);
-  uint64_t r = splitmix64(key + (uint64_t)j * 0x9E3779B97F4A7C15ull);
+  // uniform: bits drawn for element j; normal: for the pair j / 2
+  uint64_t r = splitmix64(key + (uint64_t)(k.kind == 1 ? j : j >> 1) * 0x9E3779B97F4A7C15ull);
   if (k.kind == 1) {
     double u = (double)(r >> 40) * (1.0 / 16777216.0);
     return (float)((double)k.p0 + ((double)k.p1 - (double)k.p0) * u);
   }
   double u1 = (double)((r >> 40) + 1) * (1.0 / 16777216.0);
   double u2 = (double)((r >> 16) & 0xFFFFFFull) * (1.0 / 16777216.0);
-  double z = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2);
+  double z = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2 - ((j & 1) ? kHalfPi : 0.0));
   return (float)((double)k.p0 + (double)k.p1 * z);
 }
 

@@ -41,15 +41,24 @@ __device__ __forceinline__ uint32_t* queue_counter(const TableView& tv, int pari
   return tv.counters + 4 + (parity * kQueues + q) * kQueueCounterStride;
 }
 
-// VEC initial values of a new row, evaluated one after the other: the loop stays rolled so that
-// the double-precision Box-Muller of the rare branch is live once, not VEC times, and the
-// kernels that carry it keep their occupancy (the pulls are bound by the reads in flight).
-// (UNROLLED: the kernels that only handle new ids evaluate the VEC values side by side instead;
-// an evaluation is a long chain of dependent double-precision operations, and those kernels have
-// few wavefronts to hide it behind.)
+// VEC initial values of a new row (first is a multiple of VEC), evaluated one after the other:
+// the loop stays rolled so that the double-precision Box-Muller of the rare branch is live once,
+// not VEC times, and the kernels that carry it keep their occupancy (the pulls are bound by the
+// reads in flight).
+// (UNROLLED: the kernels that only handle new ids evaluate the values side by side instead, and
+// normal draws a pair at a time: an evaluation is a long chain of dependent double-precision
+// operations, and those kernels have few wavefronts to hide it behind.)
 template <int VEC, bool UNROLLED = false>
 __device__ __forceinline__ void init_vec(const InitK& init, uint64_t id, int64_t first, float (&v)[VEC]) {
   if constexpr (UNROLLED) {
+    if constexpr (VEC == 4) {
+      if (init.kind == 2) {
+        const uint64_t key = splitmix64(id ^ init.seed_mix);
+        init_normal_pair(init, key, first >> 1, v[0], v[1]);
+        init_normal_pair(init, key, (first >> 1) + 1, v[2], v[3]);
+        return;
+      }
+    }
 #pragma unroll
     for (int c = 0; c < VEC; ++c) v[c] = init_element(init, id, first + c);
   } else {

@@ -421,10 +421,16 @@ static float draw_uniform(uint64_t r, float lower, float upper) {
   double u = (double)(r >> 40) * (1.0 / 16777216.0);
   return (float)((double)lower + ((double)upper - (double)lower) * u);
 }
-static float draw_normal(uint64_t r, float mean, float stddev) {
+/* Elements 2q and 2q + 1 of a row are the two values of one Box-Muller step on the bits drawn
+ * for q: radius * cos(angle) and radius * cos(angle - pi/2), independent standard normals (the
+ * second is written as a cosine, with the subtraction in double, so that every implementation
+ * of this definition evaluates the same expression). */
+static float draw_normal(uint64_t key, int64_t j, float mean, float stddev) {
+  uint64_t r = elem_bits(key, j >> 1);
   double u1 = (double)((r >> 40) + 1) * (1.0 / 16777216.0);
   double u2 = (double)((r >> 16) & 0xFFFFFFULL) * (1.0 / 16777216.0);
-  double z = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2);
+  double angle = 6.283185307179586476925286766559 * u2;
+  double z = sqrt(-2.0 * log(u1)) * cos((j & 1) ? angle - 1.5707963267948966192313216916398 : angle);
   return (float)((double)mean + (double)stddev * z);
 }
 
@@ -438,7 +444,7 @@ void kro_init_row(const kro_init* init, uint64_t id, int64_t dim, float* out) {
       for (int64_t j = 0; j < dim; ++j) out[j] = draw_uniform(elem_bits(key, j), init->a, init->b);
       break;
     case KRO_INIT_NORMAL:                       /* t/math.cc:455-474 (distribution only) */
-      for (int64_t j = 0; j < dim; ++j) out[j] = draw_normal(elem_bits(key, j), init->a, init->b);
+      for (int64_t j = 0; j < dim; ++j) out[j] = draw_normal(key, j, init->a, init->b);
       break;
     case KRO_INIT_XAVIER_UNIFORM: {             /* t/math.cc:507-517 */
       float std = kro_xavier_std(init->a, dim);
@@ -448,7 +454,7 @@ void kro_init_row(const kro_init* init, uint64_t id, int64_t dim, float* out) {
     }
     case KRO_INIT_XAVIER_NORMAL: {              /* t/math.cc:476-484 */
       float std = kro_xavier_std(init->a, dim);
-      for (int64_t j = 0; j < dim; ++j) out[j] = draw_normal(elem_bits(key, j), 0.0f, std);
+      for (int64_t j = 0; j < dim; ++j) out[j] = draw_normal(key, j, 0.0f, std);
       break;
     }
     default:
