@@ -270,7 +270,7 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, 
             gc.collect()
         # 3. as 1., with KRK_NOTE_ROWS on the pull and KRK_IDS_AS_PULLED on the push
         noted_marks = [api.Event() for _ in range(noted_blocks + 1)]
-        for i in range(steps):
+        for i in range(steps if noted_blocks else 0):
             step(i, True)
         noted_marks[0].record(owner)
         for b in range(noted_blocks):
@@ -284,7 +284,7 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, 
         noted = [noted_marks[b].elapsed_ms(noted_marks[b + 1]) * 1e-3 / steps for b in range(noted_blocks)]
     finally:
         gc.enable()
-    noted_med = float(np.median(noted))
+    noted_med = float(np.median(noted)) if noted else float("nan")
     med, p10, p90 = _percentiles(per_step)
     drained_med = float(np.median(drained)) if drained else None
     print("dim %d: %.2f us/step between events (p10 %.2f, p90 %.2f; %d blocks of %d steps), %.2f us/step with a "
@@ -338,9 +338,9 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, 
         "ms_per_step_host_drained": drained_med * 1e3 if drained_med else None,
         # KRK_NOTE_ROWS on the pull, KRK_IDS_AS_PULLED on the push: the worker's pull-then-push of
         # one batch with the second look-up of the ids left out. Not what `value` is computed from.
-        "ms_per_step_ids_as_pulled": noted_med * 1e3,
+        "ms_per_step_ids_as_pulled": noted_med * 1e3 if noted else None,
         "frac_whole_step_ids_as_pulled": rows_per_step / noted_med * (16 + 4 * dim * (2 + 1 + 2 * (1 + S)) + (
-            16 if cfg["optim"] == "adam" else 0)) / 1e9 / HBM_PEAK_GBS,
+            16 if cfg["optim"] == "adam" else 0)) / 1e9 / HBM_PEAK_GBS if noted else None,
         "host_enqueue_us_per_step": enqueue_s * 1e6,
         "algorithmic_bytes_per_row": per_row,
         "achieved_gbs_whole_step": rows_per_step / med * per_row / 1e9,
@@ -588,6 +588,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--blocks", type=int, default=30,
                     help="timed blocks of --steps steps each; the line carries their median, p10 and p90")
+    ap.add_argument("--noted-blocks", type=int, default=10,
+                    help="blocks of the second figure (push told that its ids are the pull's); 0 leaves it "
+                         "out, as the committed profiles of the plain step do")
     ap.add_argument("--workload", default="wide_deep", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-dims", action="store_true", help="skip the dim 32 / dim 64 legs of the default workload")
@@ -614,7 +617,8 @@ def main():
     cfg = WORKLOADS[args.workload]
     default = args.workload == "wide_deep"
     secondary = default and not args.no_secondary
-    r = run_gpu(cfg, args.steps, args.warmup, blocks=args.blocks, with_worker_leg=secondary)
+    r = run_gpu(cfg, args.steps, args.warmup, blocks=args.blocks, with_worker_leg=secondary,
+                noted_blocks=args.noted_blocks)
     batches = r.pop("batches")
     roofline = r.pop("roofline")
     ceil = hbm_ceilings()
@@ -652,7 +656,7 @@ def main():
         by_dim = {}
         for d in (32, 64):
             c2 = dict(cfg, dim=d)
-            r2 = run_gpu(c2, args.steps, args.warmup, blocks=args.blocks)
+            r2 = run_gpu(c2, args.steps, args.warmup, blocks=args.blocks, noted_blocks=args.noted_blocks)
             r2.pop("batches")
             r2["line_floor_us_whole_step"] = add_line_floors(r2["roofline"], ceil)
             attach_counter_figures(r2["roofline"], args.workload, d)
