@@ -1,6 +1,7 @@
 """Per-kernel timings of the table engine at the sizes of the benchmark configurations.
 
-    python -m kraken_amd.microbench [lines] [copy] [tables] [raw] [combined] [host] [pooled] [codec] [dense] [dct2] [hooks]
+    python -m kraken_amd.microbench [lines] [copy] [tables] [raw] [combined] [host] [pooled] [codec] [dense] [dense_group]
+                                    [dct2] [hooks] [legs]
 
 Every figure is the average of back-to-back launches between two HIP events recorded on the
 stream the kernels run on, with inputs resident in HBM; bandwidths are algorithmic bytes
@@ -757,7 +758,8 @@ def main(argv):
     rc = api.lib().krk_runtime_init(0)
     if rc != 0:
         raise RuntimeError("no usable GPU: " + api.lib().krk_last_error_string().decode())
-    for name in argv or list(SECTIONS):
+    # `legs` (the bench's secondary legs as json lines) only runs when it is named
+    for name in argv or [n for n in SECTIONS if n != "legs"]:
         SECTIONS[name]()
 
 
