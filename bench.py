@@ -320,7 +320,8 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, 
     pull_lines, push_read_lines, push_rmw_lines = lines_per_row(dim, S, cfg["optim"] == "adam")
     roofline = {
         "bound": "hbm",
-        "kernel": "%spush%s_kernel<%s>" % ("" if single else "group_", "_wide" if wide else "", cfg["optim"]),
+        "kernel": "%spush%s_kernel<%s>" % ("" if single else "group_", "_wide" if wide and dim <= 64 else "",
+                                            cfg["optim"]),
         "achieved": push_bytes / (push_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": push_bytes / (push_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
         "bytes_per_launch": push_bytes, "us_per_launch": push_ms * 1e3,
