@@ -520,8 +520,13 @@ def worker_boundary_leg(cfg, tables, group, optim, lr, n_batches=8, reps=20):
         assert group.CombinePull(d_ids, off, out=d_out, async_=True, note_rows=noted)[0] == 0
         assert group.CombinePushRaw(optim, d_ids, off, d_g, lr, async_=True, as_pulled=noted) == 0
 
-    t_pull, t_push, t_plain, t_step = (timed(group, f, reps) for f in (
-        pull, push, lambda: step(False), lambda: step(True)))
+    def noting_pull():
+        k[0] += 1
+        d_ids, _, off = dev[k[0] % n_batches]
+        assert group.CombinePull(d_ids, off, out=d_out, async_=True, note_rows=True)[0] == 0
+
+    t_pull, t_push, t_plain, t_step, t_noting = (timed(group, f, reps) for f in (
+        pull, push, lambda: step(False), lambda: step(True), noting_pull))
     n, u, S = float(np.mean(n_ids)), float(np.mean(n_unique)), _states(cfg["optim"])
     b_pull, b_push = pull_bytes_expanded(n, u, dim), push_raw_bytes(n, u, dim, S)
     for d in dev:
@@ -535,7 +540,10 @@ def worker_boundary_leg(cfg, tables, group, optim, lr, n_batches=8, reps=20):
             "step": _leg(t_step * 1e3, b_pull + b_push),
             "step_ids_looked_up_twice": _leg(t_plain * 1e3, b_pull + b_push),
             "group_pull": _leg(t_pull * 1e3, b_pull),
-            "group_push_raw": _leg(t_push * 1e3, b_push), "ids_per_s": n / t_step}
+            "group_push_raw": _leg(t_push * 1e3, b_push),
+            # what the push adds to a step whose pull noted the rows: the flagged step less the noting pull
+            "group_push_raw_ids_as_pulled": _leg((t_step - t_noting) * 1e3, b_push),
+            "group_pull_noting_rows": _leg(t_noting * 1e3, b_pull), "ids_per_s": n / t_step}
 
 
 def _single_table(cfg, seed, extra_rows=0):
