@@ -66,8 +66,10 @@ class EmbeddingFunction(torch.autograd.Function):
         dim = sparse_table.dimension()
         out = torch.empty(tuple(indices.shape) + (dim,), dtype=torch.float32, device=indices.device)
         h = sparse_table._on_current_stream()
+        # the table notes where it found every id: backward pushes gradients for this very
+        # tensor (autograd keeps it alive and unchanged), so its look-up need not be repeated
         api._check(api.lib().krk_sparse_pull(h, p_ids, ids.numel(), C.c_void_p(out.data_ptr()),
-                                             api.DEVICE_PTRS | api.ASYNC), "krk_sparse_pull")
+                                             api.DEVICE_PTRS | api.ASYNC | api.NOTE_ROWS), "krk_sparse_pull")
         ctx.table = sparse_table
         ctx.save_for_backward(ids)
         return out
@@ -80,7 +82,8 @@ class EmbeddingFunction(torch.autograd.Function):
         h = t._on_current_stream()
         api._check(api.lib().krk_sparse_push_raw(h, C.byref(t._optim.raw), C.c_void_p(ids.data_ptr()), ids.numel(),
                                                  C.c_void_p(grad.data_ptr()), t.dimension(), t.lr,
-                                                 api.DEVICE_PTRS | api.ASYNC), "krk_sparse_push_raw")
+                                                 api.DEVICE_PTRS | api.ASYNC | api.IDS_AS_PULLED),
+                   "krk_sparse_push_raw")
         return None, None
 
 
@@ -257,7 +260,7 @@ class CombineEmbeddingFunction(torch.autograd.Function):
             out = torch.empty((ids.numel(), dim), dtype=torch.float32, device=ids.device)
             h = table._on_current_stream(dim)
             api._check(api.lib().krk_group_pull(h, C.c_void_p(ids.data_ptr()), off, C.c_void_p(out.data_ptr()),
-                                                api.DEVICE_PTRS | api.ASYNC), "krk_group_pull")
+                                                api.DEVICE_PTRS | api.ASYNC | api.NOTE_ROWS), "krk_group_pull")
             for k, i in enumerate(members):
                 outs[i] = out[off[k]:off[k + 1]].view(tuple(indices[i].shape) + (dim,))
             saved.append(ids)
@@ -280,7 +283,8 @@ class CombineEmbeddingFunction(torch.autograd.Function):
             h = t._on_current_stream(dim)
             api._check(api.lib().krk_group_push_raw(h, C.byref(t._optim.raw), C.c_void_p(ids.data_ptr()), off,
                                                     C.c_void_p(g.data_ptr()), dim, t.lr,
-                                                    api.DEVICE_PTRS | api.ASYNC), "krk_group_push_raw")
+                                                    api.DEVICE_PTRS | api.ASYNC | api.IDS_AS_PULLED),
+                       "krk_group_push_raw")
         return (None,) * (1 + len(grads))
 
 

@@ -57,6 +57,39 @@ def test_embedding_forward_backward(mods, oracle):
     assert_close(t.Pull(rid)[1], rval, "rows after three steps", rtol=1e-4, atol=1e-6)
 
 
+def test_embedding_used_twice_before_backward(mods, oracle):
+    """The module's pull leaves the row of every index behind for its backward's push. Two
+    forwards on one table before either backward: the second pull's notes replace the first's,
+    and the first backward (another index tensor) must look its ids up again; both updates land
+    on the right rows."""
+    api, te = mods
+    dim = 16
+    gi, oi = _init(api, oracle, 5)
+    o_ref, o_gpu = make_optims(oracle, api, 0, {})                      # plain SGD: updates commute
+    emb = te.Embedding(dim, initializer=gi, optim=o_gpu, lr=0.1)
+    ref = oracle.SparseTable(dim, oi)
+    g = torch.Generator(device="cpu").manual_seed(4)
+    a = torch.randint(0, 300, (512,), generator=g).cuda()
+    b = torch.randint(200, 600, (640,), generator=g).cuda()
+    out_a, out_b = emb(a), emb(b)
+    wa = torch.linspace(-1.0, 1.0, dim).cuda()
+    (out_a * wa).sum().backward()
+    (out_b * (2.0 * wa)).sum().backward()
+    torch.cuda.synchronize()
+    for idx, scale in ((a, 1.0), (b, 2.0)):
+        ids = idx.cpu().numpy().astype(np.uint64)
+        ref.pull(np.unique(ids))
+    for idx, scale in ((a, 1.0), (b, 2.0)):
+        ids = idx.cpu().numpy().astype(np.uint64)
+        grad = np.tile((scale * wa.cpu().numpy()).astype(np.float32), (ids.size, 1))
+        u, gs = oracle.dedup_sum(ids, grad)
+        assert ref.push(o_ref, u, gs, 0.1) == 0
+    rid, rval, _, _ = ref.export()
+    t = emb.sparse_table.table()
+    assert len(t) == len(ref)
+    assert_close(t.Pull(rid)[1], rval, "rows after two interleaved uses", rtol=1e-5, atol=1e-6)
+
+
 @pytest.mark.parametrize("mode", ["sum", "mean"])
 @pytest.mark.parametrize("weighted", [False, True])
 def test_jagged_embedding_forward_backward(mods, oracle, mode, weighted):
