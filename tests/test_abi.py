@@ -31,6 +31,16 @@ def test_every_declared_symbol_is_exported(api):
     assert not [n for n in names if n not in api.EXPORTS]
 
 
+def test_flag_bits_of_the_binding_are_the_headers(api):
+    """The call flags are single, distinct bits, and the ctypes binding carries the header's values."""
+    header = open(os.path.join(ROOT, "include", "kraken_hip.h")).read()
+    flags = {n: int(v, 16) for n, v in re.findall(r"#define (KRK_(?:DEVICE_PTRS|ASYNC|NOTE_ROWS|IDS_AS_PULLED)) (0x[0-9a-f]+)u", header)}
+    assert flags == {"KRK_DEVICE_PTRS": api.DEVICE_PTRS, "KRK_ASYNC": api.ASYNC, "KRK_NOTE_ROWS": api.NOTE_ROWS,
+                     "KRK_IDS_AS_PULLED": api.IDS_AS_PULLED}
+    bits = sorted(flags.values())
+    assert all(b and b & (b - 1) == 0 for b in bits) and len(set(bits)) == len(bits)
+
+
 def test_optim_conf_parsing_matches_oracle_defaults(api, oracle):
     """Optim::Create (ps/optim/optim.cc:18-105): defaults and has_* flags."""
     for type_ in (0, 1, 2, 3):
