@@ -13,7 +13,9 @@ Timing: all timed blocks of K steps are enqueued back to back; HIP events record
 the sparse kernels run on separate the blocks (the last one after that stream has been made to
 wait for the dense table's), and the host waits once, at the end. `ms_per_step` is the median
 block's span / K, so it does not depend on how often the host drains the queue; the figure with a
-host drain after every block is carried as `ms_per_step_host_drained`.
+host drain after every block is carried as `ms_per_step_host_drained`, and the step whose push is
+told that its ids are the pull's (KRK_NOTE_ROWS / KRK_IDS_AS_PULLED: no second look-up) as
+`ms_per_step_ids_as_pulled`. `value` comes from the plain step.
 
 Prints ONE JSON line. `value` is unique rows pulled and pushed per second over the whole job.
 `roofline` prices the dominant kernel (the fused Adagrad push) at its algorithmic bytes,
