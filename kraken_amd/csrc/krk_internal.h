@@ -163,40 +163,92 @@ struct InitK {
 };
 
 // Normal draws come in pairs: elements 2q and 2q + 1 of a row are the two values of one
-// Box-Muller step on the bits drawn for q (radius from the upper 24 bits, angle from the next
-// 24: radius * cos(angle) and radius * cos(angle - pi/2), independent standard normals; the
-// second is written as a cosine so that both take the same code). A kernel that makes whole
-// rows pays the logarithm and the square root once per two elements (init_normal_pair); one
-// that makes a single element evaluates only the half it needs.
-constexpr double kHalfPi = 1.5707963267948966192313216916398;
-__device__ inline void normal_polar(uint64_t key, int64_t q, double& radius, double& angle) {
-  const uint64_t r = splitmix64(key + (uint64_t)q * 0x9E3779B97F4A7C15ull);
-  const double u1 = (double)((r >> 40) + 1) * (1.0 / 16777216.0);
-  const double u2 = (double)((r >> 16) & 0xFFFFFFull) * (1.0 / 16777216.0);
-  radius = sqrt(-2.0 * log(u1));
-  angle = 6.283185307179586476925286766559 * u2;
+// Box-Muller step on the bits drawn for q: k = upper 24 bits + 1 gives the radius
+// sqrt(-2 log(k / 2^24)), j = the next 24 bits the angle 2 pi j / 2^24; the values are
+// radius * cos(angle) and radius * sin(angle), independent standard normals.
+//
+// The logarithm and the sine / cosine are written out here, in double-precision +, -, *, /
+// only (no library call, no fused multiply-add: the build contracts nothing), so that this file
+// and the CPU oracle evaluate the same sequence of IEEE operations and agree to the bit, and so
+// that the rare branch of a pull that creates rows stays small: the general-purpose library
+// routines handle every argument there is and take several times the instructions and registers.
+// Their arguments here are 24-bit fractions, which makes the argument reductions exact.
+
+// log(k / 2^24) for k in [1, 2^24]: k = m 2^e with m in (1/sqrt 2, sqrt 2], log m by the atanh
+// series in f = (m - 1) / (m + 1), |f| <= 0.1716 (eight terms: below 1e-14).
+__device__ inline double log_u24(uint32_t k) {
+  int e = 31 - __clz((int)k);
+  double m = (double)k * (1.0 / (double)(1u << e));   // exact, in [1, 2)
+  if (m > 1.4142135623730951) {
+    m = m * 0.5;
+    e = e + 1;
+  }
+  const double f = (m - 1.0) / (m + 1.0);
+  const double z = f * f;
+  double p = 0.066666666666666666;                    // 1/15
+  p = p * z + 0.076923076923076927;                   // 1/13
+  p = p * z + 0.090909090909090912;                   // 1/11
+  p = p * z + 0.11111111111111111;                    // 1/9
+  p = p * z + 0.14285714285714285;                    // 1/7
+  p = p * z + 0.2;                                    // 1/5
+  p = p * z + 0.33333333333333331;                    // 1/3
+  p = p * z + 1.0;
+  return 2.0 * f * p + (double)(e - 24) * 0.69314718055994529;
 }
 
+// sin and cos of 2 pi j / 2^24 for j in [0, 2^24): the nearest quarter turn is taken off in
+// integers (exact), the rest, at most pi/4 either way, goes through the Taylor polynomials
+// (degree 13 and 14: below 3e-14), and the quarter turns are put back by swapping and negating.
+__device__ inline void sincos_u24(uint32_t j, double& sn, double& cs) {
+  const int32_t quarter = (int32_t)((j + (1u << 21)) >> 22);
+  const int32_t rest = (int32_t)j - (quarter << 22);          // in [-2^21, 2^21)
+  const double t = (double)rest * 3.7450702829239286e-07;      // 2 pi / 2^24
+  const double z = t * t;
+  double s = 1.6059043836821613e-10;                  // 1/13!
+  s = s * z - 2.505210838544172e-08;                  // 1/11!
+  s = s * z + 2.7557319223985893e-06;                 // 1/9!
+  s = s * z - 0.00019841269841269841;                 // 1/7!
+  s = s * z + 0.0083333333333333332;                  // 1/5!
+  s = s * z - 0.16666666666666666;                    // 1/3!
+  s = s * z + 1.0;
+  s = s * t;
+  double c = -1.1470745597729725e-11;                 // 1/14!
+  c = c * z + 2.08767569878681e-09;                   // 1/12!
+  c = c * z - 2.7557319223985888e-07;                 // 1/10!
+  c = c * z + 2.4801587301587302e-05;                 // 1/8!
+  c = c * z - 0.0013888888888888889;                  // 1/6!
+  c = c * z + 0.041666666666666664;                   // 1/4!
+  c = c * z - 0.5;
+  c = c * z + 1.0;
+  switch (quarter & 3) {
+    case 0: sn = s; cs = c; break;
+    case 1: sn = c; cs = -s; break;
+    case 2: sn = -s; cs = -c; break;
+    default: sn = -c; cs = s; break;
+  }
+}
+
+// both values of pair q of the row whose bits start at `key`
 __device__ inline void init_normal_pair(const InitK& k, uint64_t key, int64_t q, float& even, float& odd) {
-  double radius, angle;
-  normal_polar(key, q, radius, angle);
-  even = (float)((double)k.p0 + (double)k.p1 * (radius * cos(angle)));
-  odd = (float)((double)k.p0 + (double)k.p1 * (radius * cos(angle - kHalfPi)));
+  const uint64_t r = splitmix64(key + (uint64_t)q * 0x9E3779B97F4A7C15ull);
+  const double radius = sqrt(-2.0 * log_u24((uint32_t)(r >> 40) + 1u));
+  double sn, cs;
+  sincos_u24((uint32_t)(r >> 16) & 0xFFFFFFu, sn, cs);
+  even = (float)((double)k.p0 + (double)k.p1 * (radius * cs));
+  odd = (float)((double)k.p0 + (double)k.p1 * (radius * sn));
 }
 
 __device__ inline float init_element(const InitK& k, uint64_t id, int64_t j) {
   if (k.kind == 0) return k.p0;
   uint64_t key = splitmix64(id ^ k.seed_mix);
-  // uniform: bits drawn for element j; normal: for the pair j / 2
-  uint64_t r = splitmix64(key + (uint64_t)(k.kind == 1 ? j : j >> 1) * 0x9E3779B97F4A7C15ull);
   if (k.kind == 1) {
+    uint64_t r = splitmix64(key + (uint64_t)j * 0x9E3779B97F4A7C15ull);
     double u = (double)(r >> 40) * (1.0 / 16777216.0);
     return (float)((double)k.p0 + ((double)k.p1 - (double)k.p0) * u);
   }
-  double u1 = (double)((r >> 40) + 1) * (1.0 / 16777216.0);
-  double u2 = (double)((r >> 16) & 0xFFFFFFull) * (1.0 / 16777216.0);
-  double z = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2 - ((j & 1) ? kHalfPi : 0.0));
-  return (float)((double)k.p0 + (double)k.p1 * z);
+  float even, odd;
+  init_normal_pair(k, key, j >> 1, even, odd);
+  return (j & 1) ? odd : even;
 }
 
 // ---- optimizer arithmetic, one element at a time ---------------------------

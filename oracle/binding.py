@@ -84,6 +84,8 @@ def lib():
         "kro_optim_update": (i32, [C.POINTER(Optim), pf, i64, f32, vp]),
         "kro_init_row": (None, [C.POINTER(Init), u64, i64, pf]),
         "kro_xavier_std": (f32, [f32, i64]),
+        "kro_log_u24": (C.c_double, [C.c_uint32]),
+        "kro_sincos_u24": (None, [C.c_uint32, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
         "kro_sparse_create": (vp, [i64, C.POINTER(Init)]),
         "kro_sparse_destroy": (None, [vp]),
         "kro_sparse_size": (i64, [vp]),

@@ -422,15 +422,72 @@ static float draw_uniform(uint64_t r, float lower, float upper) {
   return (float)((double)lower + ((double)upper - (double)lower) * u);
 }
 /* Elements 2q and 2q + 1 of a row are the two values of one Box-Muller step on the bits drawn
- * for q: radius * cos(angle) and radius * cos(angle - pi/2), independent standard normals (the
- * second is written as a cosine, with the subtraction in double, so that every implementation
- * of this definition evaluates the same expression). */
+ * for q: k = upper 24 bits + 1 gives the radius sqrt(-2 log(k / 2^24)), j = the next 24 bits the
+ * angle 2 pi j / 2^24; the values are radius * cos(angle) and radius * sin(angle).
+ *
+ * The logarithm and the sine / cosine are part of the definition: they are written out below in
+ * double-precision +, -, *, / (this file is compiled without contraction), so that every
+ * implementation of the definition evaluates the same IEEE operations in the same order and
+ * agrees to the bit. Both are exact in their argument reduction because their arguments are
+ * 24-bit fractions, and accurate to a few 1e-14 (tests/test_oracle_pins.py holds them against
+ * libm). */
+double kro_log_u24(uint32_t k) {                      /* log(k / 2^24), k in [1, 2^24] */
+  int e = 31 - __builtin_clz(k);
+  double m = (double)k * (1.0 / (double)(1u << e));   /* exact, in [1, 2) */
+  if (m > 1.4142135623730951) {
+    m = m * 0.5;
+    e = e + 1;
+  }
+  /* log m = 2 atanh f, f = (m - 1) / (m + 1), |f| <= 0.1716: eight terms of the series */
+  const double f = (m - 1.0) / (m + 1.0);
+  const double z = f * f;
+  double p = 0.066666666666666666;                    /* 1/15 */
+  p = p * z + 0.076923076923076927;                   /* 1/13 */
+  p = p * z + 0.090909090909090912;                   /* 1/11 */
+  p = p * z + 0.11111111111111111;                    /* 1/9 */
+  p = p * z + 0.14285714285714285;                    /* 1/7 */
+  p = p * z + 0.2;                                    /* 1/5 */
+  p = p * z + 0.33333333333333331;                    /* 1/3 */
+  p = p * z + 1.0;
+  return 2.0 * f * p + (double)(e - 24) * 0.69314718055994529;
+}
+
+void kro_sincos_u24(uint32_t j, double* sn, double* cs) {   /* of 2 pi j / 2^24, j in [0, 2^24) */
+  /* the nearest quarter turn comes off in integers; the rest is at most pi/4 either way */
+  const int32_t quarter = (int32_t)((j + (1u << 21)) >> 22);
+  const int32_t rest = (int32_t)j - (int32_t)((uint32_t)quarter << 22);
+  const double t = (double)rest * 3.7450702829239286e-07;      /* 2 pi / 2^24 */
+  const double z = t * t;
+  double s = 1.6059043836821613e-10;                  /* Taylor: 1/13! */
+  s = s * z - 2.505210838544172e-08;                  /* 1/11! */
+  s = s * z + 2.7557319223985893e-06;                 /* 1/9! */
+  s = s * z - 0.00019841269841269841;                 /* 1/7! */
+  s = s * z + 0.0083333333333333332;                  /* 1/5! */
+  s = s * z - 0.16666666666666666;                    /* 1/3! */
+  s = s * z + 1.0;
+  s = s * t;
+  double c = -1.1470745597729725e-11;                 /* 1/14! */
+  c = c * z + 2.08767569878681e-09;                   /* 1/12! */
+  c = c * z - 2.7557319223985888e-07;                 /* 1/10! */
+  c = c * z + 2.4801587301587302e-05;                 /* 1/8! */
+  c = c * z - 0.0013888888888888889;                  /* 1/6! */
+  c = c * z + 0.041666666666666664;                   /* 1/4! */
+  c = c * z - 0.5;
+  c = c * z + 1.0;
+  switch (quarter & 3) {
+    case 0: *sn = s; *cs = c; break;
+    case 1: *sn = c; *cs = -s; break;
+    case 2: *sn = -s; *cs = -c; break;
+    default: *sn = -c; *cs = s; break;
+  }
+}
+
 static float draw_normal(uint64_t key, int64_t j, float mean, float stddev) {
   uint64_t r = elem_bits(key, j >> 1);
-  double u1 = (double)((r >> 40) + 1) * (1.0 / 16777216.0);
-  double u2 = (double)((r >> 16) & 0xFFFFFFULL) * (1.0 / 16777216.0);
-  double angle = 6.283185307179586476925286766559 * u2;
-  double z = sqrt(-2.0 * log(u1)) * cos((j & 1) ? angle - 1.5707963267948966192313216916398 : angle);
+  double radius = sqrt(-2.0 * kro_log_u24((uint32_t)(r >> 40) + 1u));
+  double sn, cs;
+  kro_sincos_u24((uint32_t)(r >> 16) & 0xFFFFFFu, &sn, &cs);
+  double z = radius * ((j & 1) ? sn : cs);
   return (float)((double)mean + (double)stddev * z);
 }
 

@@ -124,6 +124,9 @@ int32_t kro_optim_update(const kro_optim* o, const float* grad, int64_t n,
  * repository's counter-based definition keyed by (seed, id, element). */
 void kro_init_row(const kro_init* init, uint64_t id, int64_t dim, float* out);
 float kro_xavier_std(float gain, int64_t dim);     /* t/math.cc:24-50,476-484 */
+/* The two elementary functions inside the normal draw, written out as part of the definition. */
+double kro_log_u24(uint32_t k);                                /* log(k / 2^24), k in [1, 2^24] */
+void kro_sincos_u24(uint32_t j, double* sn, double* cs);       /* of 2 pi j / 2^24, j in [0, 2^24) */
 
 /* ---- sparse table -------------------------------------------------------- */
 typedef struct kro_sparse kro_sparse;

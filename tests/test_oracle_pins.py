@@ -515,6 +515,35 @@ def test_initialisers(oracle):
     assert not np.array_equal(a, b) and np.array_equal(a, c)
 
 
+def test_elementary_functions_of_the_normal_draw(oracle):
+    """The normal initialiser's logarithm and sine / cosine are written out (so that the oracle
+    and the kernels agree to the bit); here they are held against libm: every power of two, the
+    ends of the ranges, and a random sample, to 1e-13 absolute (the draw is rounded to fp32)."""
+    import ctypes as C
+    import math
+    L = oracle.lib()
+    rng = np.random.default_rng(12)
+    ks = [1, 2, 3, 2**24, 2**24 - 1, 11863283, 11863284] + [2**e for e in range(25)] + [2**e + 1 for e in range(24)]
+    ks += [int(x) for x in rng.integers(1, 2**24 + 1, 20000)]
+    worst = max(abs(L.kro_log_u24(k) - math.log(k / 2.0**24)) for k in ks)
+    assert worst < 1e-13, worst
+    assert L.kro_log_u24(2**24) == 0.0
+    sn, cs = C.c_double(), C.c_double()
+    js = [0, 1, 2**21 - 1, 2**21, 2**21 + 1, 2**22, 3 * 2**21, 2**23, 2**24 - 2**21 - 1, 2**24 - 2**21, 2**24 - 1]
+    js += [int(x) for x in rng.integers(0, 2**24, 20000)]
+    worst = 0.0
+    for j in js:
+        L.kro_sincos_u24(j, C.byref(sn), C.byref(cs))
+        a = 2.0 * math.pi * j / 2.0**24
+        worst = max(worst, abs(sn.value - math.sin(a)), abs(cs.value - math.cos(a)))
+        assert abs(sn.value ** 2 + cs.value ** 2 - 1.0) < 1e-13
+    assert worst < 1e-13, worst
+    L.kro_sincos_u24(0, C.byref(sn), C.byref(cs))
+    assert (sn.value, cs.value) == (0.0, 1.0)
+    L.kro_sincos_u24(2**22, C.byref(sn), C.byref(cs))
+    assert (sn.value, cs.value) == (1.0, 0.0)
+
+
 def _brute_dedup(ids, grads=None):
     seen = {}
     uids = []
