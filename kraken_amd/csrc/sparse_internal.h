@@ -180,8 +180,14 @@ __device__ inline uint32_t probe_find(const TableView& tv, uint64_t id, bool act
 }
 
 // id -> row, claiming a slot and the next free row when absent.
-__device__ inline ProbeResult probe_insert(const TableView& tv, uint64_t id, bool active, int gl,
-                                           int group) {
+// DEFER: the slot is claimed here and the row is numbered by the caller (number_claimed_rows),
+// for a whole workgroup with one addition to the row counter. The lane that claimed a slot
+// reports it in won / slot; every lane of its group gets owner = true, row = kEmptyRow and in src
+// the wavefront lane that holds the claim. Until the caller stores the row number the slot reads
+// as a row whose creator has not published it yet.
+template <bool DEFER>
+__device__ inline ProbeResult probe_insert_impl(const TableView& tv, uint64_t id, bool active, int gl,
+                                                int group, bool& won_out, Slot*& slot_out, int& src_out) {
   const int lane = wave_lane();
   const int base = lane & ~(group - 1);
   const uint64_t nb_mask = tv.mask >> 2;
@@ -200,6 +206,11 @@ __device__ inline ProbeResult probe_insert(const TableView& tv, uint64_t id, boo
         const unsigned long long re = __atomic_load_n(&slot->row_epoch, __ATOMIC_RELAXED);
         res.row = (uint32_t)re;
         res.fresh = res.row == kEmptyRow || (uint32_t)(re >> 32) == tv.epoch;
+      } else if constexpr (DEFER) {
+        won_out = true;
+        slot_out = slot;
+        res.owner = true;
+        res.fresh = true;
       } else {
         const uint32_t row = atomicAdd(&tv.counters[0], 1u);
         if (row < tv.row_cap) {
@@ -254,7 +265,13 @@ __device__ inline ProbeResult probe_insert(const TableView& tv, uint64_t id, boo
     // The slots claimed in this step get consecutive rows from one addition to the row counter per
     // wavefront: one addition per new id serialises on the counter's address (40 ns each, which
     // made 52k new ids in a request of a million cost 0.76 ms).
-    const unsigned long long winners = __ballot(won);
+    if constexpr (DEFER) {
+      if (won) {
+        won_out = true;
+        slot_out = mine;
+      }
+    }
+    const unsigned long long winners = DEFER ? 0ull : __ballot(won);
     if (winners) {
       const int first_winner = __ffsll(winners) - 1;
       uint32_t first_row = 0;
@@ -281,8 +298,9 @@ __device__ inline ProbeResult probe_insert(const TableView& tv, uint64_t id, boo
       done = true;
     } else if (action == 2 && old_b == kEmptyKey) {
       res.row = new_b;
-      res.owner = new_b != kEmptyRow;
+      res.owner = DEFER || new_b != kEmptyRow;
       res.fresh = true;
+      if (DEFER) src_out = src;
       done = true;
     } else if (action == 3) {
       b = (b + 1) & nb_mask;
@@ -304,9 +322,18 @@ __device__ inline ProbeResult probe_insert(const TableView& tv, uint64_t id, boo
       res.row = row0;
       res.owner = own0 != 0;
       res.fresh = fresh0 != 0;
+      if (DEFER) src_out = base;
     }
   }
   return res;
+}
+
+__device__ inline ProbeResult probe_insert(const TableView& tv, uint64_t id, bool active, int gl,
+                                           int group) {
+  bool won = false;
+  Slot* slot = nullptr;
+  int src = 0;
+  return probe_insert_impl<false>(tv, id, active, gl, group, won, slot, src);
 }
 
 // One lane looking an id up by itself (no votes): the rare second look of pooled_sum_kernel.

@@ -21,7 +21,7 @@ namespace krk {
 
 constexpr int kBlock = 256;
 constexpr int64_t kTwoLaunchPull = 1 << 18;   // ids from which a pull runs as two launches
-constexpr int kMissingGrid = 2048;            // workgroups of the launch that inserts missing ids
+constexpr int kMissingGrid = 512;             // workgroups (of 1024 lanes) of the launch that inserts missing ids
 // The positions whose id is missing are queued in kQueues lists, each with a counter on a line
 // of its own: workgroup b of the first launch appends to list b mod kQueues. One counter for the
 // whole request serialises on its address: 36k additions of a 5 %-new request of a million ids
@@ -269,11 +269,11 @@ __global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, InitK init,
 }
 
 // ---- large pulls in two launches ------------------------------------------------
-// A large pull is bound by the random reads in flight, i.e. by wavefronts per SIMD, and the
-// claiming search plus the initialiser of new rows cost pull_kernel a quarter of them. So a
-// large request first runs a kernel that only searches and copies (eight wavefronts per SIMD)
-// and queues the positions whose id is missing; a second, small launch walks that queue with
-// pull_body. In steady state the queue is empty and the second launch ends at once.
+// A large pull is bound by the random reads in flight, and in the fused kernels a wavefront that
+// inserts holds up the other ids it carries and adds to the row counter on its own. So a large
+// request first runs a kernel that only searches and copies and queues the positions whose id is
+// missing; a second, small launch walks those lists (pull_missing_kernel). In steady state the
+// lists are empty and the second launch ends at once.
 // Two sets of list counters are used in turn; the second launch clears the other set for the
 // request after it (same stream, so that request's first kernel has not started).
 template <int VEC>
@@ -310,25 +310,113 @@ __global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, con
   }
 }
 
+// The second launch: workgroups of 1024 lanes walk the lists, 256 entries at a time.
+//   1. Four lanes per entry claim a slot for its id (or find that another entry did).
+//   2. The rows of everything the workgroup claimed are numbered with one addition to the row
+//      counter. Additions to one address are served one after the other, some 15 ns each, and one
+//      per wavefront made a million new ids take 0.87 ms and 98 600 take 131 us, twelve times a
+//      pull of resident ids, at every row width.
+//   3. The lanes regroup, one lane group per entry as in pull_body, and initialise, store and
+//      copy the rows; an entry's id, position, row and state pass through LDS.
+// The trip count is the same for every lane of a workgroup (barriers inside).
+constexpr int kMissBlock = 1024;
+constexpr int kMissEntries = kMissBlock / kBucket;
+constexpr int kMissWaves = kMissBlock / kWave;
+
 template <int VEC>
-__global__ __launch_bounds__(kBlock) void pull_missing_kernel(TableView tv, InitK init,
-                                                              const uint64_t* __restrict__ ids,
-                                                              float* __restrict__ out,
-                                                              const uint32_t* __restrict__ todo, int parity,
-                                                              int64_t n, int dim, int elems, int group) {
+__global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, InitK init,
+                                                                  const uint64_t* __restrict__ ids,
+                                                                  float* __restrict__ out,
+                                                                  const uint32_t* __restrict__ todo, int parity,
+                                                                  int64_t list_capacity, int dim, int elems,
+                                                                  int group) {
+  __shared__ unsigned long long s_id[kMissEntries];
+  __shared__ uint32_t s_pos[kMissEntries], s_row[kMissEntries], s_state[kMissEntries];
+  __shared__ uint32_t s_wave[kMissWaves];
   // workgroup b walks list b mod kQueues, together with the other gridDim.x / kQueues of that list
   const int q = blockIdx.x & (kQueues - 1);
   const uint32_t count = __atomic_load_n(queue_counter(tv, parity, q), __ATOMIC_RELAXED);
   if (blockIdx.x < kQueues && threadIdx.x == 0) *queue_counter(tv, parity ^ 1, q) = 0u;
-  const int per_block = kBlock / group;
-  const uint32_t* list = todo + q * queue_capacity(n, per_block);
-  const uint32_t stride = (gridDim.x / kQueues) * per_block;
+  const uint32_t* list = todo + q * list_capacity;
+  const uint32_t stride = (gridDim.x / kQueues) * kMissEntries;
+  const int lane = wave_lane();
+  const int wave = threadIdx.x / kWave;
+  const int gl4 = threadIdx.x & (kBucket - 1);
+  const int entry = threadIdx.x / kBucket;
   const int gl = threadIdx.x & (group - 1);
-  // block-uniform trip count: pull_body votes across the wavefront
-  for (uint32_t k0 = (blockIdx.x / kQueues) * per_block; k0 < count; k0 += stride) {
-    const uint32_t k = k0 + threadIdx.x / group;
+  for (uint32_t k0 = (blockIdx.x / kQueues) * kMissEntries; k0 < count; k0 += stride) {
+    const uint32_t k = k0 + (uint32_t)entry;
     const bool active = k < count;
-    pull_body<VEC, true>(tv, init, ids, active ? (int64_t)list[k] : 0, active, gl, out, dim, elems, group);
+    const uint32_t pos = active ? list[k] : 0u;
+    const uint64_t id = active ? ids[pos] : 0;
+    bool won = false;
+    Slot* slot = nullptr;
+    int src = lane;
+    ProbeResult pr = probe_insert_impl<true>(tv, id, active, gl4, kBucket, won, slot, src);
+    // one addition for the workgroup: the wavefronts' counts meet in LDS
+    const unsigned long long winners = __ballot(won);
+    if (lane == 0) s_wave[wave] = (uint32_t)__popcll(winners);
+    __syncthreads();
+    if (wave == 0) {
+      const uint32_t mine = lane < kMissWaves ? s_wave[lane] : 0u;
+      uint32_t incl = mine;
+#pragma unroll
+      for (int d = 1; d < kMissWaves; d <<= 1) {
+        const uint32_t y = __shfl_up(incl, d);
+        if (lane >= d) incl += y;
+      }
+      const uint32_t total = __shfl(incl, kMissWaves - 1);
+      uint32_t first_row = 0;
+      if (lane == 0 && total) first_row = atomicAdd(&tv.counters[0], total);
+      first_row = __shfl(first_row, 0);
+      if (lane < kMissWaves) s_wave[lane] = first_row + incl - mine;
+    }
+    __syncthreads();
+    uint32_t new_row = kEmptyRow;
+    if (won) {
+      const uint32_t row = s_wave[wave] + (uint32_t)__popcll(winners & ((1ull << lane) - 1ull));
+      if (row < tv.row_cap) {
+        __atomic_store_n(&slot->row_epoch, (unsigned long long)row | ((unsigned long long)tv.epoch << 32),
+                         __ATOMIC_RELAXED);
+        tv.row_key[row] = id;
+        new_row = row;
+      } else {
+        atomicOr(&tv.counters[1], kErrOverflow);
+      }
+    }
+    const uint32_t numbered = __shfl(new_row, src);
+    if (pr.owner) {
+      pr.row = numbered;
+      pr.owner = numbered != kEmptyRow;
+    }
+    if (gl4 == 0) {
+      s_id[entry] = id;
+      s_pos[entry] = pos;
+      s_row[entry] = pr.row;
+      s_state[entry] = (active ? 1u : 0u) | (pr.owner ? 2u : 0u) | (pr.fresh ? 4u : 0u);
+    }
+    __syncthreads();
+    for (int j = threadIdx.x / group; j < kMissEntries; j += kMissBlock / group) {
+      const uint32_t state = s_state[j];
+      if (!(state & 1u)) break;                      // the entries past the list's end come last
+      const uint32_t row = s_row[j];
+      const uint64_t its_id = s_id[j];
+      float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
+      float* dst = out + (int64_t)s_pos[j] * dim;
+      for (int e = gl; e < elems; e += group) {
+        float v[VEC];
+        if (state & 4u) {
+          // the value of a new row is a pure function of (seed, id, element): every entry that
+          // meets it computes the same numbers, only the creator stores them
+          init_vec<VEC, true>(init, its_id, (int64_t)e * VEC, v);
+          if (state & 2u) vstore<VEC>(rec + e * VEC, v);
+        } else {
+          vload<VEC>(rec + e * VEC, v);
+        }
+        vstore_once<VEC>(dst + e * VEC, v);
+      }
+    }
+    __syncthreads();                                   // the next trip writes the same LDS
   }
 }
 
@@ -444,8 +532,7 @@ __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64
 // otherwise they are queued for pull_missing_kernel as in pull_resident_kernel.
 constexpr int kWideIds = kWave / kBucket;        // ids a wavefront takes: 16
 
-// VIA (with INSERT): first..end count entries of the queue `todo`, which names the positions.
-template <int VEC, bool INSERT, bool VIA = false>
+template <int VEC, bool INSERT>
 __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init,
                                           const uint64_t* __restrict__ ids, int64_t first, int64_t end,
                                           float* __restrict__ out, int dim, int elems, int group,
@@ -455,8 +542,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
   const int gl4 = lane & (kBucket - 1);
   const int64_t i = first + (lane >> 2);
   const bool active = i < end;
-  const uint32_t my_pos = (VIA && active) ? todo[i] : 0u;
-  const uint64_t id = active ? ids[VIA ? (int64_t)my_pos : i] : 0;
+  const uint64_t id = active ? ids[i] : 0;
   const FindResult f = probe_find_slot(tv, id, active, gl4, kBucket);
   ProbeResult pr;
   pr.row = (uint32_t)f.row_epoch;
@@ -470,7 +556,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
       if (miss) pr = q;
     }
     // where the id lives, for a push of the same ids that follows (kEmptyRow: the table is full)
-    if (!VIA && notes && active && gl4 == 0) notes[i] = pr.row;
+    if (notes && active && gl4 == 0) notes[i] = pr.row;
   } else {
     // one atomic per wavefront reserves entries of the workgroup's list for all of its missing ids
     // (here `end` is the request's length: the lists' capacity follows from it)
@@ -496,7 +582,6 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
   const int gl = lane & (group - 1);
   const uint32_t id_lo = (uint32_t)id, id_hi = (uint32_t)(id >> 32);
   float v[8][VEC];
-  uint32_t where[VIA ? 8 : 1];                   // VIA: the position each step's row goes to
   uint32_t live = 0;                             // bit s: this lane has a slice of step s to store
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
@@ -507,13 +592,12 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
       const int owner = __shfl((int)pr.owner, src);
       const int on = __shfl((int)copy, src);
       const uint64_t its_id = (uint64_t)__shfl(id_lo, src) | ((uint64_t)__shfl(id_hi, src) << 32);
-      if constexpr (VIA) where[s] = __shfl(my_pos, src);
       if (on && gl < elems) {
         float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
         if (fresh) {
           // the value of a new row is a pure function of (seed, id, element): every group that
           // meets it computes the same numbers, only the creator stores them
-          init_vec<VEC, VIA>(init, its_id, (int64_t)gl * VEC, v[s]);
+          init_vec<VEC>(init, its_id, (int64_t)gl * VEC, v[s]);
           if (owner) vstore<VEC>(rec + gl * VEC, v[s]);
         } else {
           vload<VEC>(rec + gl * VEC, v[s]);
@@ -525,7 +609,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
     if (live & (1u << s)) {
-      const int64_t p = VIA ? (int64_t)where[VIA ? s : 0] : first + s * rows_per_step + sub;
+      const int64_t p = first + s * rows_per_step + sub;
       vstore_once<VEC>(out + p * (int64_t)dim + gl * VEC, v[s]);
     }
   }
@@ -656,23 +740,6 @@ __global__ __launch_bounds__(kBlock) void pull_resident_wide_kernel(TableView tv
   if (first >= n) return;
   InitK none{};
   pull_wide<VEC, false>(tv, none, ids, first, n, out, dim, elems, group, todo, parity);
-}
-
-// the second launch of a large pull for wide rows: sixteen queued positions per wavefront
-template <int VEC>
-__global__ __launch_bounds__(kBlock) void pull_missing_wide_kernel(TableView tv, InitK init,
-                                                                   const uint64_t* __restrict__ ids,
-                                                                   float* __restrict__ out,
-                                                                   uint32_t* __restrict__ todo, int parity,
-                                                                   int64_t n, int dim, int elems, int group) {
-  const int q = blockIdx.x & (kQueues - 1);
-  const uint32_t count = __atomic_load_n(queue_counter(tv, parity, q), __ATOMIC_RELAXED);
-  if (blockIdx.x < kQueues && threadIdx.x == 0) *queue_counter(tv, parity ^ 1, q) = 0u;
-  uint32_t* list = todo + q * queue_capacity(n, (kBlock / kWave) * kWideIds);
-  const uint32_t stride = (gridDim.x / kQueues) * (kBlock / kWave) * kWideIds;
-  for (uint32_t k0 = ((blockIdx.x / kQueues) * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds; k0 < count;
-       k0 += stride)
-    pull_wide<VEC, true, true>(tv, init, ids, k0, count, out, dim, elems, group, list, parity);
 }
 
 // ---- one launch over several tables of equal row width ------------------------
@@ -1693,21 +1760,20 @@ int32_t krk_sparse_sync(krk_sparse* t) {
 // and has made room for n more rows.
 static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, float* d_out,
                             uint32_t* notes = nullptr) {
-  const int64_t rows_before = t->size_ub;           // upper bound of the rows the table holds
   KRK_TRY(sparse_next_epoch(t, n));
   const bool wide = t->vec == 4 && pull_is_wide(t->group, t->elems);
   const int per_block = wide ? (kBlock / kWave) * kWideIds : kBlock / t->group;
   const dim3 grid(grid_for(n, per_block)), block(kBlock);
-  // Two launches pay when most ids are resident; a request larger than the table is mostly new
-  // ids (a cold start), which the fused launch inserts in one go at twice the rate. A request
-  // of about the table's size is the other case: many repeats of resident ids (8.9 million ids
-  // over a table of ten million rows: 590 us in two launches, 730 us fused).
-  if (n >= kTwoLaunchPull && rows_before >= n) {
+  // Two launches pay for many repeats of resident ids (8.9 million ids over a table of ten
+  // million rows: 590 us in two launches, 730 us fused) and for requests of new ids alike (a
+  // million ids that are all new, 16 floats a row: 195 us, 870 us fused).
+  if (n >= kTwoLaunchPull) {
     KRK_TRY(t->scratch[5].reserve((size_t)kQueues * queue_capacity(n, per_block) * sizeof(uint32_t)));
     uint32_t* todo = t->scratch[5].as<uint32_t>();
     const int parity = t->pull_parity;
     t->pull_parity ^= 1;
-    const dim3 small(kMissingGrid);
+    const dim3 small(kMissingGrid), missing_block(kMissBlock);
+    const int64_t list_capacity = queue_capacity(n, per_block);
     if (t->vec == 4) {
       if (wide) {
         hipLaunchKernelGGL((pull_resident_wide_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
@@ -1716,18 +1782,13 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
         hipLaunchKernelGGL((pull_resident_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
                            parity, (int)t->dim, t->elems, t->group);
       }
-      if (wide) {
-        hipLaunchKernelGGL((pull_missing_wide_kernel<4>), small, block, 0, t->stream, t->view(), t->initk, d_ids,
-                           d_out, todo, parity, n, (int)t->dim, t->elems, t->group);
-      } else {
-        hipLaunchKernelGGL((pull_missing_kernel<4>), small, block, 0, t->stream, t->view(), t->initk, d_ids,
-                           d_out, todo, parity, n, (int)t->dim, t->elems, t->group);
-      }
+      hipLaunchKernelGGL((pull_missing_kernel<4>), small, missing_block, 0, t->stream, t->view(), t->initk, d_ids,
+                         d_out, todo, parity, list_capacity, (int)t->dim, t->elems, t->group);
     } else {
       hipLaunchKernelGGL((pull_resident_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
                          parity, (int)t->dim, t->elems, t->group);
-      hipLaunchKernelGGL((pull_missing_kernel<1>), small, block, 0, t->stream, t->view(), t->initk, d_ids, d_out,
-                         todo, parity, n, (int)t->dim, t->elems, t->group);
+      hipLaunchKernelGGL((pull_missing_kernel<1>), small, missing_block, 0, t->stream, t->view(), t->initk, d_ids,
+                         d_out, todo, parity, list_capacity, (int)t->dim, t->elems, t->group);
     }
   } else if (t->vec == 4 && wide) {
     hipLaunchKernelGGL((pull_wide_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,

@@ -335,6 +335,39 @@ def test_wide_rows_pull_every_path(api, oracle, dim):
     assert len(t) == len(r)
 
 
+@pytest.mark.parametrize("dim", [4, 6, 16, 48, 256])
+def test_large_pull_numbers_its_new_rows_once(api, oracle, dim):
+    """A pull of 300 000 ids over a table that already holds as many rows runs as two launches;
+    the second one numbers the rows of all new ids that a workgroup claims with one addition to
+    the row counter. New ids that repeat inside the request (next to each other and far apart),
+    the ids 0 and all ones among the new ones, resident ids between them: every value as the
+    oracle's, every new id in the table exactly once, the rows dense, and the same values again
+    when every id is resident."""
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "23"})
+    t = api.SparseTable(dim, gi, capacity_hint=64)
+    r = oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=23))
+    rng = np.random.default_rng(1000 + dim)
+    resident = splitmix64(np.arange(300_000, dtype=np.uint64))
+    assert t.Pull(resident)[0] == 0 and r.pull(resident)[0] == 0
+    fresh = splitmix64(np.arange(1 << 42, (1 << 42) + 40_000, dtype=np.uint64))
+    fresh = np.concatenate([fresh, np.array([0, 2**64 - 1], np.uint64)])
+    ids = np.concatenate([resident[:200_000], fresh, fresh[:30_000], np.repeat(fresh[30_000:30_100], 7)])
+    ids = ids[rng.permutation(ids.size)]
+    ids = np.concatenate([ids, np.repeat(fresh[100:164], 4)])     # one new id in neighbouring positions
+    assert ids.size >= 262_144
+    rc, got = t.Pull(ids)
+    _, want = r.pull(ids)
+    assert rc == 0
+    assert_close(got, want, "dim %d, new and resident ids" % dim, rtol=1e-6)
+    assert len(t) == len(r) == resident.size + fresh.size
+    gid, gval, _, _ = t.export()
+    assert np.array_equal(np.sort(gid), np.sort(np.concatenate([resident, fresh])))
+    rid, rval, _, _ = r.export()
+    order_g, order_r = np.argsort(gid), np.argsort(rid)
+    assert_close(gval[order_g], rval[order_r], "dim %d, the records of the new rows" % dim, rtol=1e-6)
+    rc, again = t.Pull(ids)
+    assert rc == 0 and np.array_equal(again, got)
+
 def test_wide_rows_group_pull_ragged_members(api, oracle):
     """A combined pull over tables of 64-float rows whose members bring 0, 1, 17 and 5000 ids."""
     dim = 64
