@@ -640,6 +640,8 @@ def main():
         "ms_per_step_p90": r["ms_per_step_p90"], "timed_blocks": r["blocks"],
         "timing": "HIP events between blocks on the sparse kernels' stream, blocks enqueued back to back",
         "ms_per_step_host_drained": r["ms_per_step_host_drained"],
+        "ms_per_step_ids_as_pulled": r["ms_per_step_ids_as_pulled"],
+        "frac_whole_step_ids_as_pulled": r["frac_whole_step_ids_as_pulled"],
         "host_enqueue_us_per_step": r["host_enqueue_us_per_step"],
         "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
