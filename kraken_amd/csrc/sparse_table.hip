@@ -532,10 +532,13 @@ __global__ __launch_bounds__(kBlock) void push_kernel(TableView tv, const uint64
 // otherwise they are queued for pull_missing_kernel as in pull_resident_kernel.
 constexpr int kWideIds = kWave / kBucket;        // ids a wavefront takes: 16
 
-template <int VEC, bool INSERT>
+// STEPS: the copy's trips, 2, 4 or 8 for lane groups of 8, 16 or 32 lanes (a template argument so
+// that a lane holds STEPS slices and not eight: the fused kernel for rows of 32 and 64 floats then
+// keeps all wavefronts of a 98k-id request on the chip at once instead of five sixths of them).
+template <int VEC, bool INSERT, int STEPS>
 __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init,
                                           const uint64_t* __restrict__ ids, int64_t first, int64_t end,
-                                          float* __restrict__ out, int dim, int elems, int group,
+                                          float* __restrict__ out, int dim, int elems,
                                           uint32_t* __restrict__ todo, int parity,
                                           uint32_t* __restrict__ notes = nullptr) {
   const int lane = wave_lane();
@@ -576,16 +579,16 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
     pr.fresh = false;                              // nothing is created here: what was found is read
   }
   // the copy: lane group `sub` of the wavefront takes ids sub, sub + rows_per_step, ...
-  const int rows_per_step = kWave / group;       // 8, 4 or 2
-  const int steps = kWideIds / rows_per_step;    // 2, 4 or 8
+  constexpr int rows_per_step = kWideIds / STEPS;   // 8, 4 or 2
+  constexpr int group = kWave / rows_per_step;      // 8, 16 or 32
   const int sub = lane / group;
   const int gl = lane & (group - 1);
   const uint32_t id_lo = (uint32_t)id, id_hi = (uint32_t)(id >> 32);
-  float v[8][VEC];
+  float v[STEPS][VEC];
   uint32_t live = 0;                             // bit s: this lane has a slice of step s to store
 #pragma unroll
-  for (int s = 0; s < 8; ++s) {
-    if (s < steps) {                             // uniform
+  for (int s = 0; s < STEPS; ++s) {
+    {
       const int src = kBucket * (s * rows_per_step + sub);
       const uint32_t row = __shfl(pr.row, src);
       const int fresh = __shfl((int)pr.fresh, src);
@@ -607,7 +610,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
     }
   }
 #pragma unroll
-  for (int s = 0; s < 8; ++s) {
+  for (int s = 0; s < STEPS; ++s) {
     if (live & (1u << s)) {
       const int64_t p = first + s * rows_per_step + sub;
       vstore_once<VEC>(out + p * (int64_t)dim + gl * VEC, v[s]);
@@ -720,26 +723,26 @@ __global__ __launch_bounds__(kBlock) void push_wide_kernel(TableView tv, const u
   push_wide<OPT, STEPS>(tv, ids, first, n, grads, dim, elems, lr, k, pc, notes);
 }
 
-template <int VEC>
+template <int VEC, int STEPS>
 __global__ __launch_bounds__(kBlock) void pull_wide_kernel(TableView tv, InitK init,
                                                            const uint64_t* __restrict__ ids, int64_t n,
                                                            float* __restrict__ out, int dim, int elems,
-                                                           int group, uint32_t* __restrict__ notes) {
+                                                           uint32_t* __restrict__ notes) {
   const int64_t first = ((int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds;
   if (first >= n) return;                        // the whole wavefront
-  pull_wide<VEC, true>(tv, init, ids, first, n, out, dim, elems, group, nullptr, 0, notes);
+  pull_wide<VEC, true, STEPS>(tv, init, ids, first, n, out, dim, elems, nullptr, 0, notes);
 }
 
-template <int VEC>
+template <int VEC, int STEPS>
 __global__ __launch_bounds__(kBlock) void pull_resident_wide_kernel(TableView tv,
                                                                     const uint64_t* __restrict__ ids,
                                                                     int64_t n, float* __restrict__ out,
                                                                     uint32_t* __restrict__ todo, int parity,
-                                                                    int dim, int elems, int group) {
+                                                                    int dim, int elems) {
   const int64_t first = ((int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds;
   if (first >= n) return;
   InitK none{};
-  pull_wide<VEC, false>(tv, none, ids, first, n, out, dim, elems, group, todo, parity);
+  pull_wide<VEC, false, STEPS>(tv, none, ids, first, n, out, dim, elems, todo, parity);
 }
 
 // ---- one launch over several tables of equal row width ------------------------
@@ -771,13 +774,12 @@ __global__ __launch_bounds__(kBlock) void group_pull_kernel(const TableDesc* __r
 }
 
 // the same for rows 32 to 128 floats wide: a workgroup takes 64 positions of its table
-template <int VEC>
+template <int VEC, int STEPS>
 __global__ __launch_bounds__(kBlock) void group_pull_wide_kernel(const TableDesc* __restrict__ descs,
                                                                  GroupCall call,
                                                                  const uint64_t* __restrict__ ids,
                                                                  float* __restrict__ out, int dim,
-                                                                 int elems, int group,
-                                                                 uint32_t* __restrict__ notes) {
+                                                                 int elems, uint32_t* __restrict__ notes) {
   const int t = find_table(call);
   TableView tv = descs[t].tv;
   tv.epoch = call.epoch[t];
@@ -786,7 +788,7 @@ __global__ __launch_bounds__(kBlock) void group_pull_wide_kernel(const TableDesc
                         kWideIds;
   const int64_t first = call.row_start[t] + local;
   if (first >= call.row_start[t + 1]) return;    // the whole wavefront
-  pull_wide<VEC, true>(tv, init, ids, first, call.row_start[t + 1], out, dim, elems, group, nullptr, 0, notes);
+  pull_wide<VEC, true, STEPS>(tv, init, ids, first, call.row_start[t + 1], out, dim, elems, nullptr, 0, notes);
 }
 
 template <int OPT, int VEC>
@@ -1775,9 +1777,15 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
     const dim3 small(kMissingGrid), missing_block(kMissBlock);
     const int64_t list_capacity = queue_capacity(n, per_block);
     if (t->vec == 4) {
-      if (wide) {
-        hipLaunchKernelGGL((pull_resident_wide_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
-                           todo, parity, (int)t->dim, t->elems, t->group);
+      if (wide && t->group == 8) {
+        hipLaunchKernelGGL((pull_resident_wide_kernel<4, 2>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
+                           todo, parity, (int)t->dim, t->elems);
+      } else if (wide && t->group == 16) {
+        hipLaunchKernelGGL((pull_resident_wide_kernel<4, 4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
+                           todo, parity, (int)t->dim, t->elems);
+      } else if (wide) {
+        hipLaunchKernelGGL((pull_resident_wide_kernel<4, 8>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
+                           todo, parity, (int)t->dim, t->elems);
       } else {
         hipLaunchKernelGGL((pull_resident_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
                            parity, (int)t->dim, t->elems, t->group);
@@ -1790,9 +1798,15 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
       hipLaunchKernelGGL((pull_missing_kernel<1>), small, missing_block, 0, t->stream, t->view(), t->initk, d_ids,
                          d_out, todo, parity, list_capacity, (int)t->dim, t->elems, t->group);
     }
+  } else if (t->vec == 4 && wide && t->group == 8) {
+    hipLaunchKernelGGL((pull_wide_kernel<4, 2>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
+                       (int)t->dim, t->elems, notes);
+  } else if (t->vec == 4 && wide && t->group == 16) {
+    hipLaunchKernelGGL((pull_wide_kernel<4, 4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
+                       (int)t->dim, t->elems, notes);
   } else if (t->vec == 4 && wide) {
-    hipLaunchKernelGGL((pull_wide_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
-                       (int)t->dim, t->elems, t->group, notes);
+    hipLaunchKernelGGL((pull_wide_kernel<4, 8>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
+                       (int)t->dim, t->elems, notes);
   } else if (t->vec == 4) {
     hipLaunchKernelGGL((pull_kernel<4>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
                        (int)t->dim, t->elems, t->group, notes);
@@ -2720,9 +2734,15 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
       notes = g->notes.as<uint32_t>();
     }
   }
-  if (wide) {
-    hipLaunchKernelGGL((group_pull_wide_kernel<4>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
-                       (int)g->dim, g->elems, g->group, notes);
+  if (wide && g->group == 8) {
+    hipLaunchKernelGGL((group_pull_wide_kernel<4, 2>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
+                       (int)g->dim, g->elems, notes);
+  } else if (wide && g->group == 16) {
+    hipLaunchKernelGGL((group_pull_wide_kernel<4, 4>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
+                       (int)g->dim, g->elems, notes);
+  } else if (wide) {
+    hipLaunchKernelGGL((group_pull_wide_kernel<4, 8>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
+                       (int)g->dim, g->elems, notes);
   } else if (g->vec == 4) {
     hipLaunchKernelGGL((group_pull_kernel<4>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
                        (int)g->dim, g->elems, g->group, notes);
