@@ -21,7 +21,9 @@ Prints ONE JSON line. `value` is unique rows pulled and pushed per second over t
 `roofline` prices the dominant kernel (the fused Adagrad push) at its algorithmic bytes,
 U * (8 + 4D + 16D) per launch, against 8 TB/s; `line_floor_us` next to every `us_per_launch` is
 what the kernel's count of random 128-byte lines costs at the line rates measured in the same
-run, plus one empty launch. `secondary` holds the other configurations (ids with their repeats at
+run, plus one empty launch, and `lines_and_streams_us` adds the ids and gradient rows the
+kernel streams in or the pulled rows it streams out at the streaming rates of the same run.
+`secondary` holds the other configurations (ids with their repeats at
 the worker boundary, DeepFM, the duplicate-heavy shape, the codec and the blockwise DCT), each
 with its own algorithmic bytes or flops. `cpu_baseline` times the CPU oracle (a restatement of
 the reference's table path; the checker, never the product) on the host cores of the same
@@ -369,17 +371,23 @@ def run_gpu(cfg, steps, warmup, blocks=30, n_batches=32, with_worker_leg=False, 
     return res
 
 
-def add_line_floors(roofline, ceil):
+def add_line_floors(roofline, ceil, dim):
     """line_floor_us: the kernel's random lines at the line rates this run measured (read-only
-    lines at the read rate, lines written back at the read-modify-write rate) + one empty launch."""
+    lines at the read rate, lines written back at the read-modify-write rate) + one empty launch:
+    a bound. lines_and_streams_us adds what the kernel streams besides (ids and gradient rows
+    read, pulled rows written) at the streaming rates of the same run: an estimate of a launch in
+    which the scattered lines and the streams take turns at the memory."""
     rd = ceil["random_lines"]["random_line_read_%d" % (1 << 22)]["lines_per_s"]
     rmw = ceil["random_lines"]["random_line_rmw_%d" % (1 << 22)]["lines_per_s"]
     empty = ceil["empty_launch_us"]
     u = roofline["rows_per_launch"]
     lp = roofline["lines_per_row"]
     roofline["line_floor_us"] = (u * lp["read"] / rd + u * lp["read_and_written_back"] / rmw) * 1e6 + empty
+    roofline["lines_and_streams_us"] = roofline["line_floor_us"] + u * (8 + 4 * dim) / (ceil["read_ceiling"] * 1e9) * 1e6
     pk = roofline["pull_kernel"]
     pk["line_floor_us"] = u * pk["lines_per_row"]["read"] / rd * 1e6 + empty
+    pk["lines_and_streams_us"] = pk["line_floor_us"] + (u * 8 / (ceil["read_ceiling"] * 1e9) +
+                                                          u * 4 * dim / (ceil["write_ceiling"] * 1e9)) * 1e6
     return roofline["line_floor_us"] + pk["line_floor_us"]
 
 
@@ -630,7 +638,7 @@ def main():
     roofline["frac_of_random_line_rmw_ceiling"] = roofline["achieved"] / ceil["random_line_rmw_ceiling"]
     roofline["copy_ceiling"] = ceil["copy_ceiling"]
     roofline["frac_of_copy_ceiling"] = roofline["achieved"] / ceil["copy_ceiling"]
-    step_floor = add_line_floors(roofline, ceil)
+    step_floor = add_line_floors(roofline, ceil, cfg["dim"])
     attach_counter_figures(roofline, args.workload, cfg["dim"])
     dim = cfg["dim"]
     line = {
@@ -663,7 +671,7 @@ def main():
             c2 = dict(cfg, dim=d)
             r2 = run_gpu(c2, args.steps, args.warmup, blocks=args.blocks, noted_blocks=args.noted_blocks)
             r2.pop("batches")
-            r2["line_floor_us_whole_step"] = add_line_floors(r2["roofline"], ceil)
+            r2["line_floor_us_whole_step"] = add_line_floors(r2["roofline"], ceil, d)
             attach_counter_figures(r2["roofline"], args.workload, d)
             by_dim[str(d)] = r2
         line["by_dim"] = by_dim
