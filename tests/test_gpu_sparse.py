@@ -335,7 +335,7 @@ def test_wide_rows_pull_every_path(api, oracle, dim):
     assert len(t) == len(r)
 
 
-@pytest.mark.parametrize("dim", [4, 6, 16, 48, 256])
+@pytest.mark.parametrize("dim", [4, 6, 16, 48, 130, 256])
 def test_large_pull_numbers_its_new_rows_once(api, oracle, dim):
     """A pull of 300 000 ids over a table that already holds as many rows runs as two launches;
     the second one numbers the rows of all new ids that a workgroup claims with one addition to
