@@ -100,6 +100,60 @@ def tables():
         t.close()
 
 
+def inserts():
+    """Pulls that insert: every id new (a cold start), and 5 % of a million ids new. A request of
+    262 144 ids or more runs as two launches (rows numbered once per workgroup of the second); a
+    smaller one inserts inside the fused kernel, one addition to the row counter per wavefront."""
+    print("# pulls that insert rows (each call brings ids the table has not seen); the same ids again: resident")
+    for dim in (16, 64, 128):
+        for n in (98_600, 1 << 20):
+            init = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "3"})
+            t = api.SparseTable(dim, init, capacity_hint=1 << 20)
+            t.reserve(6 * n + 1024)
+            out = api.DeviceArray((n, dim), np.float32)
+            e0, e1 = api.Event(), api.Event()
+            cold = []
+            for i in range(5):
+                d = api.DeviceArray.from_host(splitmix64(np.arange(i * n, (i + 1) * n, dtype=np.uint64) + np.uint64(12345)))
+                e0.record(t)
+                assert t.Pull(d, out=out, async_=True)[0] == 0
+                e1.record(t)
+                assert t.sync() == 0
+                cold.append(e0.elapsed_ms(e1) * 1e3)
+                if i < 4:
+                    d.free()
+            warm = timed(t, lambda: t.Pull(d, out=out, async_=True), 5)
+            print("dim %3d n %8d | every id new %7.1f us (median of calls 2 to 5) | resident %7.1f us"
+                  % (dim, n, float(np.median(cold[1:])), warm * 1e6), flush=True)
+            d.free()
+            out.free()
+            t.close()
+    dim, n, rows = 128, 1 << 20, 4 * 10**6
+    init = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "3"})
+    t = api.SparseTable(dim, init, capacity_hint=rows)
+    prefill(t, rows, dim)
+    t.reserve(rows + n)
+    rng = np.random.default_rng(8)
+    out = api.DeviceArray((n, dim), np.float32)
+    e0, e1 = api.Event(), api.Event()
+    some = []
+    for i in range(6):
+        ids = splitmix64(rng.integers(0, rows, size=n, dtype=np.uint64))
+        where = rng.choice(n, size=n // 20, replace=False)
+        ids[where] = splitmix64(np.uint64(1 << 40) + np.arange(i * (n // 20), (i + 1) * (n // 20), dtype=np.uint64))
+        d = api.DeviceArray.from_host(ids)
+        e0.record(t)
+        assert t.Pull(d, out=out, async_=True)[0] == 0
+        e1.record(t)
+        assert t.sync() == 0
+        some.append(e0.elapsed_ms(e1) * 1e3)
+        d.free()
+    print("dim %3d n %8d | 5 %% of the ids new %7.1f us (median of calls 2 to 6)" % (dim, n, float(np.median(some[1:]))),
+          flush=True)
+    out.free()
+    t.close()
+
+
 def raw():
     print("# push_raw (dedup + duplicate-gradient sum + update fused) and stand-alone dedup of N ids")
     print("#   bytes: U(8+4D+8D(1+S)) + 8N + 4DN")
@@ -768,7 +822,7 @@ def legs():
         print(fn.__name__, json.dumps(fn()), flush=True)
 
 
-SECTIONS = {"legs": legs, "lines": lines, "copy": copy, "tables": tables, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dense_group": dense_group, "dct2": dct, "hooks": hooks}
+SECTIONS = {"legs": legs, "lines": lines, "copy": copy, "tables": tables, "inserts": inserts, "raw": raw, "combined": combined, "host": host, "pooled": pooled, "codec": codec, "dense": dense, "dense_group": dense_group, "dct2": dct, "hooks": hooks}
 
 
 def main(argv):
