@@ -19,6 +19,9 @@
 //                                   the host enqueues behind an inserting launch when the table
 //                                   is close to full, so that it can bound the row count later
 //                                   without waiting for the stream
+//   + 4 B behind it                 set by a pull that found ids to insert; the host looks at it
+//                                   when it enqueues the next pull and picks the launches for a
+//                                   request that inserts if so
 #pragma once
 
 #include <vector>
@@ -45,6 +48,7 @@ struct TableView {
   uint32_t* counters;   // [0] rows used, [1] error bits
   uint32_t row_cap;
   uint32_t epoch;       // number of this launch, for launches that may insert
+  uint32_t* inserted;   // pinned host word: a pull that makes rows sets it (see pull_enqueue)
 };
 
 constexpr int kBucket = 4;   // slots per bucket: one aligned 64-byte sector
@@ -113,6 +117,12 @@ struct ProbeResult {
 };
 
 __device__ __forceinline__ int wave_lane() { return (int)(threadIdx.x & (kWave - 1)); }
+
+// Called by one lane of a wavefront that found ids to insert. A relaxed store to host memory:
+// nothing waits for it, and the host only reads it as a hint.
+__device__ __forceinline__ void note_inserting(const TableView& tv) {
+  if (tv.inserted) __hip_atomic_store(tv.inserted, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 // What a search that never writes reports: whether the id has a slot, and the slot's second
 // word (row number in the low half, number of the launch that created the row in the high half).
@@ -386,6 +396,7 @@ struct krk_sparse : krk::ObjBase {
   uint32_t* host_counters = nullptr;  // pinned
   int64_t size_ub = 0;                // upper bound of rows used, exact after a blocking call
   unsigned long long* host_pub = nullptr;   // pinned, written by the device (publish_kernel)
+  uint32_t* host_inserted = nullptr;        // pinned, behind host_pub: set by pulls that insert
   int64_t last_request = 0;           // size of the last inserting request
   uint64_t enq_total = 0;             // ids handed to inserting launches so far
   uint64_t enq_at[256] = {};          // enq_total right after the launch with number e (mod 256)
@@ -419,6 +430,7 @@ struct krk_sparse : krk::ObjBase {
     tv.counters = counters;
     tv.row_cap = (uint32_t)row_cap;
     tv.epoch = epoch;
+    tv.inserted = host_inserted;
     return tv;
   }
 };

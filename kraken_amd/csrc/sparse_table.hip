@@ -21,6 +21,7 @@ namespace krk {
 
 constexpr int kBlock = 256;
 constexpr int64_t kTwoLaunchPull = 1 << 18;   // ids from which a pull runs as two launches
+constexpr int64_t kTwoLaunchWhileFilling = 1 << 15;   // the same while the pulls before it inserted rows
 constexpr int kMissingGrid = 512;             // workgroups (of 1024 lanes) of the launch that inserts missing ids
 // The positions whose id is missing are queued in kQueues lists, each with a counter on a line
 // of its own: workgroup b of the first launch appends to list b mod kQueues. One counter for the
@@ -133,6 +134,7 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
   if (__any(miss)) {
     const ProbeResult q = probe_insert(tv, id, miss, gl, group);
     if (miss) pr = q;
+    if (wave_lane() == 0) note_inserting(tv);
   }
   if (!active) return;
   const uint32_t row = pr.row;
@@ -336,7 +338,10 @@ __global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, 
   // workgroup b walks list b mod kQueues, together with the other gridDim.x / kQueues of that list
   const int q = blockIdx.x & (kQueues - 1);
   const uint32_t count = __atomic_load_n(queue_counter(tv, parity, q), __ATOMIC_RELAXED);
-  if (blockIdx.x < kQueues && threadIdx.x == 0) *queue_counter(tv, parity ^ 1, q) = 0u;
+  if (blockIdx.x < kQueues && threadIdx.x == 0) {
+    *queue_counter(tv, parity ^ 1, q) = 0u;
+    if (count) note_inserting(tv);
+  }
   const uint32_t* list = todo + q * list_capacity;
   const uint32_t stride = (gridDim.x / kQueues) * kMissEntries;
   const int lane = wave_lane();
@@ -557,6 +562,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
     if (__any(miss)) {
       const ProbeResult q = probe_insert(tv, id, miss, gl4, kBucket);
       if (miss) pr = q;
+      if (lane == 0) note_inserting(tv);
     }
     // where the id lives, for a push of the same ids that follows (kEmptyRow: the table is full)
     if (notes && active && gl4 == 0) notes[i] = pr.row;
@@ -1677,8 +1683,12 @@ int32_t krk_sparse_create(int64_t dim, const krk_init* init, int64_t capacity_hi
     hipError_t e = hipMalloc((void**)&t->counters, kCounterWords * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMemsetAsync(t->counters, 0, kCounterWords * sizeof(uint32_t), t->stream);
     if (e == hipSuccess) e = hipHostMalloc((void**)&t->host_counters, 16, hipHostMallocDefault);
-    if (e == hipSuccess) e = hipHostMalloc((void**)&t->host_pub, 8, hipHostMallocCoherent);
-    if (e == hipSuccess) *t->host_pub = 0ull;
+    if (e == hipSuccess) e = hipHostMalloc((void**)&t->host_pub, 16, hipHostMallocCoherent);
+    if (e == hipSuccess) {
+      *t->host_pub = 0ull;
+      t->host_inserted = reinterpret_cast<uint32_t*>(t->host_pub + 1);
+      *t->host_inserted = 0u;
+    }
     if (e != hipSuccess) rc = hip_fail(e, "krk_sparse_create allocations", __FILE__, __LINE__);
   }
   if (rc == KRK_SUCCESS) {
@@ -1768,8 +1778,14 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
   const dim3 grid(grid_for(n, per_block)), block(kBlock);
   // Two launches pay for many repeats of resident ids (8.9 million ids over a table of ten
   // million rows: 590 us in two launches, 730 us fused) and for requests of new ids alike (a
-  // million ids that are all new, 16 floats a row: 195 us, 870 us fused).
-  if (n >= kTwoLaunchPull) {
+  // million ids that are all new, 16 floats a row: 195 us, 870 us fused). A smaller request takes
+  // them while the table is being filled: the fused kernel adds to the row counter once per
+  // wavefront that inserts, and those additions are served one after the other (98 600 new ids:
+  // 137 us fused). Whether the table is being filled is what the pull before this one left
+  // behind in host memory; it may lag by the requests that are still queued, and either choice
+  // gives the same rows. Row notes are kept by the fused kernels only.
+  const bool filling = t->host_inserted && __atomic_exchange_n(t->host_inserted, 0u, __ATOMIC_RELAXED) != 0u;
+  if (n >= kTwoLaunchPull || (filling && !notes && n >= kTwoLaunchWhileFilling)) {
     KRK_TRY(t->scratch[5].reserve((size_t)kQueues * queue_capacity(n, per_block) * sizeof(uint32_t)));
     uint32_t* todo = t->scratch[5].as<uint32_t>();
     const int parity = t->pull_parity;

@@ -368,6 +368,55 @@ def test_large_pull_numbers_its_new_rows_once(api, oracle, dim):
     rc, again = t.Pull(ids)
     assert rc == 0 and np.array_equal(again, got)
 
+@pytest.mark.parametrize("dim", [8, 64])
+def test_pulls_while_a_table_is_being_filled(api, oracle, dim):
+    """A pull that inserted rows leaves a word behind in host memory, and the next pull of 32 768
+    ids or more then runs as two launches (the second numbers new rows once per workgroup) instead
+    of the fused kernel. Which of the two ran must not show: steps that bring half new ids, then
+    the same ids twice (the first of them still takes the two launches, the second the fused
+    kernel), then new ids again, every step against the oracle; a request that asks for row notes
+    keeps the fused kernel and the push that reuses them updates the same rows."""
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "29"})
+    t = api.SparseTable(dim, gi, capacity_hint=64)
+    r = oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=29))
+    rng = np.random.default_rng(dim)
+    o_ref, o_gpu = make_optims(oracle, api, 0, {})
+    seen = splitmix64(np.arange(50_000, dtype=np.uint64))
+    n = 100_000
+    for step in range(7):
+        if step in (4, 5):
+            ids = last
+        else:
+            fresh = splitmix64(np.arange((step + 1) << 32, ((step + 1) << 32) + n // 2, dtype=np.uint64))
+            ids = np.concatenate([fresh, rng.choice(seen, size=n // 2 - 2), np.array([0, 2**64 - 1], np.uint64)])
+            ids = ids[rng.permutation(ids.size)]
+            seen = np.concatenate([seen, fresh])
+        last = ids
+        rc, got = t.Pull(ids)
+        _, want = r.pull(ids)
+        assert rc == 0
+        assert_close(got, want, "dim %d, step %d" % (dim, step), rtol=1e-6)
+        assert len(t) == len(r)
+        u = np.unique(ids)
+        g = (rng.standard_normal((u.size, dim)) * 0.1).astype(np.float32)
+        assert t.Push(o_gpu, u, g, 0.05) == 0 and r.push(o_ref, u, g, 0.05) == 0
+    # notes asked for while the table is being filled
+    fresh = splitmix64(np.arange(99 << 32, (99 << 32) + 40_000, dtype=np.uint64))
+    d_ids = api.DeviceArray.from_host(fresh)
+    d_out = api.DeviceArray((fresh.size, dim), np.float32)
+    assert t.Pull(d_ids, out=d_out, note_rows=True)[0] == 0
+    _, want = r.pull(fresh)
+    assert_close(d_out.to_host(), want, "dim %d, noted pull of new ids" % dim, rtol=1e-6)
+    g = (rng.standard_normal((fresh.size, dim)) * 0.1).astype(np.float32)
+    d_g = api.DeviceArray.from_host(g)
+    assert t.Push(o_gpu, d_ids, d_g, 0.05, as_pulled=True) == 0 and r.push(o_ref, fresh, g, 0.05) == 0
+    rc, got = t.Pull(fresh)
+    _, want = r.pull(fresh)
+    assert rc == 0
+    assert_close(got, want, "dim %d, rows after the push that reused the notes" % dim, rtol=1e-6)
+    for a in (d_ids, d_out, d_g):
+        a.free()
+
 def test_wide_rows_group_pull_ragged_members(api, oracle):
     """A combined pull over tables of 64-float rows whose members bring 0, 1, 17 and 5000 ids."""
     dim = 64
