@@ -321,17 +321,20 @@ __global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, con
 //   3. The lanes regroup, one lane group per entry as in pull_body, and initialise, store and
 //      copy the rows; an entry's id, position, row and state pass through LDS.
 // The trip count is the same for every lane of a workgroup (barriers inside).
+// ROWS_ONLY (the pooled pull while a table is being filled): nothing is copied; the creator
+// initialises the record and every entry's row number goes to rows_out[position] (kEmptyRow where
+// the creator, another entry, has not published it yet: pooled_sum_kernel looks those up).
 constexpr int kMissBlock = 1024;
 constexpr int kMissEntries = kMissBlock / kBucket;
 constexpr int kMissWaves = kMissBlock / kWave;
 
-template <int VEC>
+template <int VEC, bool ROWS_ONLY = false>
 __global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, InitK init,
                                                                   const uint64_t* __restrict__ ids,
                                                                   float* __restrict__ out,
                                                                   const uint32_t* __restrict__ todo, int parity,
                                                                   int64_t list_capacity, int dim, int elems,
-                                                                  int group) {
+                                                                  int group, uint32_t* __restrict__ rows_out = nullptr) {
   __shared__ unsigned long long s_id[kMissEntries];
   __shared__ uint32_t s_pos[kMissEntries], s_row[kMissEntries], s_state[kMissEntries];
   __shared__ uint32_t s_wave[kMissWaves];
@@ -399,6 +402,7 @@ __global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, 
       s_pos[entry] = pos;
       s_row[entry] = pr.row;
       s_state[entry] = (active ? 1u : 0u) | (pr.owner ? 2u : 0u) | (pr.fresh ? 4u : 0u);
+      if (ROWS_ONLY && active) rows_out[pos] = pr.row;
     }
     __syncthreads();
     for (int j = threadIdx.x / group; j < kMissEntries; j += kMissBlock / group) {
@@ -407,6 +411,16 @@ __global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, 
       const uint32_t row = s_row[j];
       const uint64_t its_id = s_id[j];
       float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
+      if constexpr (ROWS_ONLY) {
+        if ((state & 6u) == 6u) {                    // created here: the record's initial values
+          for (int e = gl; e < elems; e += group) {
+            float v[VEC];
+            init_vec<VEC, true>(init, its_id, (int64_t)e * VEC, v);
+            vstore<VEC>(rec + e * VEC, v);
+          }
+        }
+        continue;
+      }
       float* dst = out + (int64_t)s_pos[j] * dim;
       for (int e = gl; e < elems; e += group) {
         float v[VEC];
@@ -438,6 +452,32 @@ __global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, 
 //      on each other and are issued four at a time.
 // The n pulled rows themselves are never written anywhere.
 // ---------------------------------------------------------------------------
+// The first launch while the table is being filled: positions are only looked up, the ones whose
+// id is missing are queued as in pull_resident_kernel and inserted by pull_missing_kernel.
+__global__ __launch_bounds__(kBlock) void pooled_find_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                             int64_t n, uint32_t* __restrict__ rows,
+                                                             uint32_t* __restrict__ todo, int parity) {
+  constexpr int per_block = kBlock / kBucket;
+  const int64_t p = (int64_t)blockIdx.x * per_block + threadIdx.x / kBucket;
+  const int gl = threadIdx.x & (kBucket - 1);
+  const bool active = p < n;
+  const uint32_t row = probe_find(tv, active ? ids[p] : 0, active, gl, kBucket);
+  const bool queue = active && row == kEmptyRow && gl == 0;
+  const unsigned long long votes = __ballot(queue);
+  if (votes) {
+    const int lane = wave_lane();
+    const int first = __ffsll(votes) - 1;
+    const int q = blockIdx.x & (kQueues - 1);
+    uint32_t base = 0;
+    if (lane == first) base = atomicAdd(queue_counter(tv, parity, q), (uint32_t)__popcll(votes));
+    base = __shfl(base, first);
+    if (queue)
+      todo[q * queue_capacity(n, per_block) + base + (uint32_t)__popcll(votes & ((1ull << lane) - 1ull))] =
+          (uint32_t)p;
+  }
+  if (active && gl == 0) rows[p] = row;
+}
+
 template <int VEC>
 __global__ __launch_bounds__(kBlock) void pooled_probe_kernel(TableView tv, InitK init,
                                                               const uint64_t* __restrict__ ids, int64_t n,
@@ -447,6 +487,7 @@ __global__ __launch_bounds__(kBlock) void pooled_probe_kernel(TableView tv, Init
   const bool active = p < n;
   const uint64_t id = active ? ids[p] : 0;
   const ProbeResult pr = probe_insert(tv, id, active, gl, kBucket);
+  if (__any(active && pr.owner) && wave_lane() == 0) note_inserting(tv);
   if (!active) return;
   if (pr.fresh && pr.owner && pr.row != kEmptyRow) {
     float* rec = tv.recs + (int64_t)pr.row * tv.stride;
@@ -1911,19 +1952,41 @@ int32_t krk_sparse_pull_pooled(krk_sparse* t, const uint64_t* ids, int64_t n, co
   if (weights && n > 0) KRK_TRY(t->input(weights, (size_t)n, flags, 2, &d_w));
   KRK_TRY(t->output(out, (size_t)bags * t->dim, flags, 3, &d_out));
   KRK_TRY(sparse_next_epoch(t, n));
-  KRK_TRY(t->scratch[5].reserve((size_t)(n > 0 ? n : 1) * sizeof(uint32_t)));
+  // While the table is being filled (see pull_enqueue) the positions are looked up by a launch
+  // that inserts nothing and the missing ones go through pull_missing_kernel: the probing
+  // kernel that inserts adds to the row counter once per wavefront, 8.9 million positions of
+  // which one in ten is new cost it half a million additions, served one after the other.
+  const bool filling = t->host_inserted && __atomic_exchange_n(t->host_inserted, 0u, __ATOMIC_RELAXED) != 0u;
+  const bool queued = filling && n >= kTwoLaunchWhileFilling;
+  const int64_t list_capacity = queued ? queue_capacity(n, kBlock / kBucket) : 0;
+  const size_t rows_words = ((size_t)(n > 0 ? n : 1) + 63) & ~(size_t)63;
+  KRK_TRY(t->scratch[5].reserve((rows_words + (size_t)kQueues * (size_t)list_capacity) * sizeof(uint32_t)));
   uint32_t* rows = t->scratch[5].as<uint32_t>();
+  uint32_t* todo = rows + rows_words;
   const int per_block = kBlock / t->group;
   const dim3 probe_grid(grid_for(n, kBlock / kBucket)), grid(grid_for(bags, per_block)), block(kBlock);
+  const dim3 small(kMissingGrid), missing_block(kMissBlock);
   const int mean = mode == KRK_POOL_MEAN;
+  int parity = 0;
+  if (queued) {
+    parity = t->pull_parity;
+    t->pull_parity ^= 1;
+    hipLaunchKernelGGL(pooled_find_kernel, probe_grid, block, 0, t->stream, t->view(), d_ids, n, rows, todo, parity);
+  }
   if (t->vec == 4) {
-    if (n > 0)
+    if (queued)
+      hipLaunchKernelGGL((pull_missing_kernel<4, true>), small, missing_block, 0, t->stream, t->view(), t->initk,
+                         d_ids, nullptr, todo, parity, list_capacity, (int)t->dim, t->elems, t->group, rows);
+    else if (n > 0)
       hipLaunchKernelGGL((pooled_probe_kernel<4>), probe_grid, block, 0, t->stream, t->view(), t->initk, d_ids,
                          n, rows, t->elems);
     hipLaunchKernelGGL((pooled_sum_kernel<4>), grid, block, 0, t->stream, t->view(), rows, d_ids, n, d_off, bags, d_w,
                        mean, patch_value, d_out, (int)t->dim, t->elems, t->group);
   } else {
-    if (n > 0)
+    if (queued)
+      hipLaunchKernelGGL((pull_missing_kernel<1, true>), small, missing_block, 0, t->stream, t->view(), t->initk,
+                         d_ids, nullptr, todo, parity, list_capacity, (int)t->dim, t->elems, t->group, rows);
+    else if (n > 0)
       hipLaunchKernelGGL((pooled_probe_kernel<1>), probe_grid, block, 0, t->stream, t->view(), t->initk, d_ids,
                          n, rows, t->elems);
     hipLaunchKernelGGL((pooled_sum_kernel<1>), grid, block, 0, t->stream, t->view(), rows, d_ids, n, d_off, bags, d_w,

@@ -317,6 +317,24 @@ def pooled():
             ("pooled push (sum)", lambda: t.PushPooled(opt, d_ids, d_off, d_g, 1e-3, mode="sum", async_=True))):
         print("%-36s %8.1f us" % (name, timed(t, fn, 5) * 1e6), flush=True)
     t.close()
+    # the same field over a table that starts empty: each step draws its own ids
+    t = api.SparseTable(dim, init, capacity_hint=space)
+    t.reserve(space + space // 8)
+    e0, e1 = api.Event(), api.Event()
+    steps = []
+    for i in range(6):
+        d = api.DeviceArray.from_host(splitmix64(zipf_ranks(rng, 1.1, space, n)))
+        rows_before = len(t)
+        e0.record(t)
+        assert t.PullPooled(d, d_off, "mean", out=d_out, async_=True)[0] == 0
+        e1.record(t)
+        assert t.sync() == 0
+        steps.append("%.0f us (%d new rows)" % (e0.elapsed_ms(e1) * 1e3, len(t) - rows_before))
+        d.free()
+    print("pooled pull (mean), table empty at first, step by step: " + ", ".join(steps), flush=True)
+    for a in (d_ids, d_off, d_g, d_out, d_rows):
+        a.free()
+    t.close()
 
 
 def codec():

@@ -89,6 +89,30 @@ def test_pooled_pull_device_arrays_and_edge_shapes(api, oracle):
     assert rc == 0 and np.array_equal(got, _oracle_pooled_pull(oracle, ref, rep, off2, "sum", 0.0, None))
 
 
+@pytest.mark.parametrize("dim", [16, 6])
+def test_pooled_pulls_while_a_table_is_being_filled(api, oracle, dim):
+    """A pooled pull of 32 768 positions or more that follows a pull which inserted rows looks its
+    positions up without inserting, queues the missing ones and inserts them in a launch of their
+    own (rows numbered once per workgroup). Steps whose id space keeps growing (every step brings
+    new ids, repeated inside and across bags), then the same request twice: the pooled rows are
+    the oracle's bit for bit, and the rows in the table are the rows a plain pull returns."""
+    rng = np.random.default_rng(dim)
+    t, ref = _tables(api, oracle, dim, seed=40 + dim)
+    ids = off = None
+    for step in range(6):
+        if step < 4:
+            ids, off = _bags(rng, 9000, 12, 30_000 * (step + 1))
+        assert ids.size >= 32_768
+        rc, got = t.PullPooled(ids, off, "mean" if step % 2 else "sum", patch_value=0.5)
+        assert rc == 0
+        want = _oracle_pooled_pull(oracle, ref, ids, off, "mean" if step % 2 else "sum", 0.5, None)
+        assert np.array_equal(got, want), step
+        assert len(t) == len(ref)
+    u = np.unique(ids)
+    assert np.array_equal(t.Pull(u)[1], ref.pull(u)[1])
+    gid = t.export()[0]
+    assert np.unique(gid).size == gid.size == len(ref)
+
 def test_pooled_argument_errors(api, oracle):
     t, _ = _tables(api, oracle, 16, seed=1)
     ids = np.arange(10, dtype=np.uint64)
