@@ -1728,7 +1728,7 @@ int32_t krk_sparse_create(int64_t dim, const krk_init* init, int64_t capacity_hi
     if (e == hipSuccess) {
       *t->host_pub = 0ull;
       t->host_inserted = reinterpret_cast<uint32_t*>(t->host_pub + 1);
-      *t->host_inserted = 0u;
+      *t->host_inserted = 1u;   // an empty table is about to be filled
     }
     if (e != hipSuccess) rc = hip_fail(e, "krk_sparse_create allocations", __FILE__, __LINE__);
   }
