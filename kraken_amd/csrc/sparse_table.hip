@@ -21,7 +21,7 @@ namespace krk {
 
 constexpr int kBlock = 256;
 constexpr int64_t kTwoLaunchPull = 1 << 18;   // ids from which a pull runs as two launches
-constexpr int64_t kTwoLaunchWhileFilling = 1 << 15;   // the same while the pulls before it inserted rows
+constexpr int64_t kTwoLaunchWhileFilling = 1 << 13;   // the same while the pulls before it inserted rows
 constexpr int kMissingGrid = 512;             // workgroups (of 1024 lanes) of the launch that inserts missing ids
 // The positions whose id is missing are queued in kQueues lists, each with a counter on a line
 // of its own: workgroup b of the first launch appends to list b mod kQueues. One counter for the

@@ -91,7 +91,7 @@ def test_pooled_pull_device_arrays_and_edge_shapes(api, oracle):
 
 @pytest.mark.parametrize("dim", [16, 6])
 def test_pooled_pulls_while_a_table_is_being_filled(api, oracle, dim):
-    """A pooled pull of 32 768 positions or more that follows a pull which inserted rows looks its
+    """A pooled pull of 8192 positions or more that follows a pull which inserted rows looks its
     positions up without inserting, queues the missing ones and inserts them in a launch of their
     own (rows numbered once per workgroup). Steps whose id space keeps growing (every step brings
     new ids, repeated inside and across bags), then the same request twice: the pooled rows are

@@ -370,7 +370,7 @@ def test_large_pull_numbers_its_new_rows_once(api, oracle, dim):
 
 @pytest.mark.parametrize("dim", [8, 64])
 def test_pulls_while_a_table_is_being_filled(api, oracle, dim):
-    """A pull that inserted rows leaves a word behind in host memory, and the next pull of 32 768
+    """A pull that inserted rows leaves a word behind in host memory, and the next pull of 8192
     ids or more then runs as two launches (the second numbers new rows once per workgroup) instead
     of the fused kernel. Which of the two ran must not show: steps that bring half new ids, then
     the same ids twice (the first of them still takes the two launches, the second the fused
