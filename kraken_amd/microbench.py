@@ -152,6 +152,33 @@ def inserts():
           flush=True)
     out.free()
     t.close()
+    # a combined request over 26 tables keeps the fused kernel: its additions spread over 26 counters
+    dim, per = 16, 3792
+    tables = [api.SparseTable(dim, init, capacity_hint=1 << 16) for _ in range(26)]
+    for t in tables:
+        t.reserve(8 * per)
+    group = api.TableGroup(tables)
+    n = 26 * per
+    off = api.TableGroup._offsets([per] * 26)
+    out = api.DeviceArray((n, dim), np.float32)
+    cold = []
+    for i in range(5):
+        d = api.DeviceArray.from_host(splitmix64(np.arange(i * n, (i + 1) * n, dtype=np.uint64) + np.uint64(999)))
+        e0.record(group)
+        assert group.CombinePull(d, off, out=out, async_=True)[0] == 0
+        e1.record(group)
+        assert group.sync() == 0
+        cold.append(e0.elapsed_ms(e1) * 1e3)
+        if i < 4:
+            d.free()
+    warm = timed(group, lambda: group.CombinePull(d, off, out=out, async_=True), 5)
+    print("dim %3d n %8d over 26 tables, one combined pull | every id new %7.1f us (median of calls 2 to 5) | "
+          "resident %7.1f us" % (dim, n, float(np.median(cold[1:])), warm * 1e6), flush=True)
+    d.free()
+    out.free()
+    group.close()
+    for t in tables:
+        t.close()
 
 
 def raw():
