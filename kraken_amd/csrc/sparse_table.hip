@@ -22,6 +22,11 @@ namespace krk {
 constexpr int kBlock = 256;
 constexpr int64_t kTwoLaunchPull = 1 << 18;   // ids from which a pull runs as two launches
 constexpr int64_t kTwoLaunchWhileFilling = 1 << 13;   // the same while the pulls before it inserted rows
+// A wavefront tells the host that the table is being filled when that many of its sixteen (or
+// fewer) ids are new: two in one wavefront is rare when fewer than one id in three hundred is new,
+// the share from which the fused kernel's additions to the row counter cost more than a second
+// launch, and all but certain somewhere in a request when one in a hundred is.
+constexpr int kFillingIds = 2;
 constexpr int kMissingGrid = 512;             // workgroups (of 1024 lanes) of the launch that inserts missing ids
 // The positions whose id is missing are queued in kQueues lists, each with a counter on a line
 // of its own: workgroup b of the first launch appends to list b mod kQueues. One counter for the
@@ -134,7 +139,7 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
   if (__any(miss)) {
     const ProbeResult q = probe_insert(tv, id, miss, gl, group);
     if (miss) pr = q;
-    if (wave_lane() == 0) note_inserting(tv);
+    if (__popcll(__ballot(miss && gl == 0)) >= kFillingIds && wave_lane() == 0) note_inserting(tv);
   }
   if (!active) return;
   const uint32_t row = pr.row;
@@ -343,7 +348,8 @@ __global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, 
   const uint32_t count = __atomic_load_n(queue_counter(tv, parity, q), __ATOMIC_RELAXED);
   if (blockIdx.x < kQueues && threadIdx.x == 0) {
     *queue_counter(tv, parity ^ 1, q) = 0u;
-    if (count) note_inserting(tv);
+    // still being filled: this list's share of the request's missing ids is 0.4 % of it or more
+    if ((uint64_t)count * 256u >= (uint64_t)list_capacity) note_inserting(tv);
   }
   const uint32_t* list = todo + q * list_capacity;
   const uint32_t stride = (gridDim.x / kQueues) * kMissEntries;
@@ -487,7 +493,7 @@ __global__ __launch_bounds__(kBlock) void pooled_probe_kernel(TableView tv, Init
   const bool active = p < n;
   const uint64_t id = active ? ids[p] : 0;
   const ProbeResult pr = probe_insert(tv, id, active, gl, kBucket);
-  if (__any(active && pr.owner) && wave_lane() == 0) note_inserting(tv);
+  if (__popcll(__ballot(active && pr.owner && gl == 0)) >= kFillingIds && wave_lane() == 0) note_inserting(tv);
   if (!active) return;
   if (pr.fresh && pr.owner && pr.row != kEmptyRow) {
     float* rec = tv.recs + (int64_t)pr.row * tv.stride;
@@ -603,7 +609,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
     if (__any(miss)) {
       const ProbeResult q = probe_insert(tv, id, miss, gl4, kBucket);
       if (miss) pr = q;
-      if (lane == 0) note_inserting(tv);
+      if (__popcll(__ballot(miss && gl4 == 0)) >= kFillingIds && lane == 0) note_inserting(tv);
     }
     // where the id lives, for a push of the same ids that follows (kEmptyRow: the table is full)
     if (notes && active && gl4 == 0) notes[i] = pr.row;
