@@ -458,6 +458,13 @@ struct GroupCall {
   uint32_t block_start[kMaxGroupTables + 1];
   int64_t row_start[kMaxGroupTables + 1];
 };
+
+// What a combined pull carries besides when it queues its missing ids (the members' tables are
+// being filled): every member has its own 64 lists, counted by its own table's list counters.
+struct GroupFill {
+  uint32_t todo_start[kMaxGroupTables];   // first word of member t's lists in the work space
+  uint32_t parity_bits;                   // bit t: the set of member t's list counters in use
+};
 }  // namespace krk
 
 // Tables of one combined request (CombinePull/PushSparseTable): they share one stream, and a
@@ -474,6 +481,7 @@ struct krk_group : krk::ObjBase {
   // Row notes of one combined pull (see krk_sparse::notes): valid while noted_ids is not null
   // and every member's layout_version is what it was.
   krk::DeviceBuffer notes;
+  krk::DeviceBuffer todo;              // the lists of a combined pull that queues its missing ids
   const uint64_t* noted_ids = nullptr;
   std::vector<int64_t> noted_offsets;
   std::vector<uint64_t> noted_versions;

@@ -27,6 +27,10 @@ constexpr int64_t kTwoLaunchWhileFilling = 1 << 13;   // the same while the pull
 // the share from which the fused kernel's additions to the row counter cost more than a second
 // launch, and all but certain somewhere in a request when one in a hundred is.
 constexpr int kFillingIds = 2;
+// A combined request spreads its additions over its members' counters, and its two launches cost
+// 15 us more than its fused kernel where nothing is new: over 26 tables they pay from one new id
+// in five on (98.6k ids, one in ten new: 21 us fused, 27 us in two launches; all new: 64 and 34).
+constexpr int kFillingIdsCombined = 8;
 constexpr int kMissingGrid = 512;             // workgroups (of 1024 lanes) of the launch that inserts missing ids
 // The positions whose id is missing are queued in kQueues lists, each with a counter on a line
 // of its own: workgroup b of the first launch appends to list b mod kQueues. One counter for the
@@ -126,7 +130,8 @@ template <int VEC, bool MOSTLY_NEW = false>
 __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init,
                                           const uint64_t* __restrict__ ids, int64_t i, bool active,
                                           int gl, float* __restrict__ out, int dim, int elems,
-                                          int group, uint32_t* __restrict__ notes = nullptr) {
+                                          int group, uint32_t* __restrict__ notes = nullptr,
+                                          int filling_ids = kFillingIds) {
   const uint64_t id = active ? ids[i] : 0;
   // Most ids are resident: a search that never writes settles them, and only a wavefront that
   // holds a missing id goes through the claiming search as well.
@@ -139,7 +144,7 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
   if (__any(miss)) {
     const ProbeResult q = probe_insert(tv, id, miss, gl, group);
     if (miss) pr = q;
-    if (__popcll(__ballot(miss && gl == 0)) >= kFillingIds && wave_lane() == 0) note_inserting(tv);
+    if (__popcll(__ballot(miss && gl == 0)) >= filling_ids && wave_lane() == 0) note_inserting(tv);
   }
   if (!active) return;
   const uint32_t row = pr.row;
@@ -283,13 +288,14 @@ __global__ __launch_bounds__(kBlock) void pull_kernel(TableView tv, InitK init,
 // lists are empty and the second launch ends at once.
 // Two sets of list counters are used in turn; the second launch clears the other set for the
 // request after it (same stream, so that request's first kernel has not started).
+// bx: the workgroup's number among those of this table's request
 template <int VEC>
-__global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, const uint64_t* __restrict__ ids,
-                                                               int64_t n, float* __restrict__ out,
-                                                               uint32_t* __restrict__ todo, int parity, int dim,
-                                                               int elems, int group) {
+__device__ __forceinline__ void pull_resident_body(const TableView& tv, const uint64_t* __restrict__ ids,
+                                                   int64_t n, float* __restrict__ out,
+                                                   uint32_t* __restrict__ todo, int parity, int dim,
+                                                   int elems, int group, uint32_t bx) {
   const int per_block = kBlock / group;
-  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
+  const int64_t i = (int64_t)bx * per_block + threadIdx.x / group;
   const int gl = threadIdx.x & (group - 1);
   const bool active = i < n;
   const uint32_t row = probe_find(tv, active ? ids[i] : 0, active, gl, group);
@@ -299,7 +305,7 @@ __global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, con
   if (votes) {
     const int lane = wave_lane();
     const int first = __ffsll(votes) - 1;
-    const int q = blockIdx.x & (kQueues - 1);
+    const int q = bx & (kQueues - 1);
     uint32_t base = 0;
     if (lane == first) base = atomicAdd(queue_counter(tv, parity, q), (uint32_t)__popcll(votes));
     base = __shfl(base, first);
@@ -315,6 +321,14 @@ __global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, con
     vload<VEC>(rec + e * VEC, v);
     vstore_once<VEC>(dst + e * VEC, v);
   }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                               int64_t n, float* __restrict__ out,
+                                                               uint32_t* __restrict__ todo, int parity, int dim,
+                                                               int elems, int group) {
+  pull_resident_body<VEC>(tv, ids, n, out, todo, parity, dim, elems, group, blockIdx.x);
 }
 
 // The second launch: workgroups of 1024 lanes walk the lists, 256 entries at a time.
@@ -333,35 +347,26 @@ constexpr int kMissBlock = 1024;
 constexpr int kMissEntries = kMissBlock / kBucket;
 constexpr int kMissWaves = kMissBlock / kWave;
 
-template <int VEC, bool ROWS_ONLY = false>
-__global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, InitK init,
-                                                                  const uint64_t* __restrict__ ids,
-                                                                  float* __restrict__ out,
-                                                                  const uint32_t* __restrict__ todo, int parity,
-                                                                  int64_t list_capacity, int dim, int elems,
-                                                                  int group, uint32_t* __restrict__ rows_out = nullptr) {
+// Entries k_first, k_first + stride, ... of `count` queued positions, kMissEntries at a time (the
+// workgroups that share them are `stride` apart); position_of(k) names the k-th.
+template <int VEC, bool ROWS_ONLY, typename PositionOf>
+__device__ __forceinline__ void insert_queued(const TableView& tv, const InitK& init,
+                                              const uint64_t* __restrict__ ids, float* __restrict__ out,
+                                              PositionOf position_of, uint32_t count,
+                                              uint32_t k_first, uint32_t stride, int dim, int elems, int group,
+                                              uint32_t* __restrict__ rows_out) {
   __shared__ unsigned long long s_id[kMissEntries];
   __shared__ uint32_t s_pos[kMissEntries], s_row[kMissEntries], s_state[kMissEntries];
   __shared__ uint32_t s_wave[kMissWaves];
-  // workgroup b walks list b mod kQueues, together with the other gridDim.x / kQueues of that list
-  const int q = blockIdx.x & (kQueues - 1);
-  const uint32_t count = __atomic_load_n(queue_counter(tv, parity, q), __ATOMIC_RELAXED);
-  if (blockIdx.x < kQueues && threadIdx.x == 0) {
-    *queue_counter(tv, parity ^ 1, q) = 0u;
-    // still being filled: this list's share of the request's missing ids is 0.4 % of it or more
-    if ((uint64_t)count * 256u >= (uint64_t)list_capacity) note_inserting(tv);
-  }
-  const uint32_t* list = todo + q * list_capacity;
-  const uint32_t stride = (gridDim.x / kQueues) * kMissEntries;
   const int lane = wave_lane();
   const int wave = threadIdx.x / kWave;
   const int gl4 = threadIdx.x & (kBucket - 1);
   const int entry = threadIdx.x / kBucket;
   const int gl = threadIdx.x & (group - 1);
-  for (uint32_t k0 = (blockIdx.x / kQueues) * kMissEntries; k0 < count; k0 += stride) {
+  for (uint32_t k0 = k_first; k0 < count; k0 += stride) {
     const uint32_t k = k0 + (uint32_t)entry;
     const bool active = k < count;
-    const uint32_t pos = active ? list[k] : 0u;
+    const uint32_t pos = active ? position_of(k) : 0u;
     const uint64_t id = active ? ids[pos] : 0;
     bool won = false;
     Slot* slot = nullptr;
@@ -443,6 +448,27 @@ __global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, 
     }
     __syncthreads();                                   // the next trip writes the same LDS
   }
+}
+
+template <int VEC, bool ROWS_ONLY = false>
+__global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, InitK init,
+                                                                  const uint64_t* __restrict__ ids,
+                                                                  float* __restrict__ out,
+                                                                  const uint32_t* __restrict__ todo, int parity,
+                                                                  int64_t list_capacity, int dim, int elems,
+                                                                  int group, uint32_t* __restrict__ rows_out = nullptr) {
+  // workgroup b walks list b mod kQueues, together with the other gridDim.x / kQueues of that list
+  const int q = blockIdx.x & (kQueues - 1);
+  const uint32_t count = __atomic_load_n(queue_counter(tv, parity, q), __ATOMIC_RELAXED);
+  if (blockIdx.x < kQueues && threadIdx.x == 0) {
+    *queue_counter(tv, parity ^ 1, q) = 0u;
+    // still being filled: this list's share of the request's missing ids is 0.4 % of it or more
+    if ((uint64_t)count * 256u >= (uint64_t)list_capacity) note_inserting(tv);
+  }
+  const uint32_t* list = todo + q * list_capacity;
+  insert_queued<VEC, ROWS_ONLY>(tv, init, ids, out, [list](uint32_t k) { return list[k]; }, count,
+                                (blockIdx.x / kQueues) * kMissEntries, (gridDim.x / kQueues) * kMissEntries, dim,
+                                elems, group, rows_out);
 }
 
 // ---------------------------------------------------------------------------
@@ -592,7 +618,8 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
                                           const uint64_t* __restrict__ ids, int64_t first, int64_t end,
                                           float* __restrict__ out, int dim, int elems,
                                           uint32_t* __restrict__ todo, int parity,
-                                          uint32_t* __restrict__ notes = nullptr) {
+                                          uint32_t* __restrict__ notes = nullptr,
+                                          int filling_ids = kFillingIds) {
   const int lane = wave_lane();
   const int gl4 = lane & (kBucket - 1);
   const int64_t i = first + (lane >> 2);
@@ -609,7 +636,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
     if (__any(miss)) {
       const ProbeResult q = probe_insert(tv, id, miss, gl4, kBucket);
       if (miss) pr = q;
-      if (__popcll(__ballot(miss && gl4 == 0)) >= kFillingIds && lane == 0) note_inserting(tv);
+      if (__popcll(__ballot(miss && gl4 == 0)) >= filling_ids && lane == 0) note_inserting(tv);
     }
     // where the id lives, for a push of the same ids that follows (kEmptyRow: the table is full)
     if (notes && active && gl4 == 0) notes[i] = pr.row;
@@ -823,7 +850,7 @@ __global__ __launch_bounds__(kBlock) void group_pull_kernel(const TableDesc* __r
   const int64_t local = (int64_t)(blockIdx.x - call.block_start[t]) * per_block + threadIdx.x / group;
   const int64_t i = call.row_start[t] + local;
   pull_body<VEC>(tv, init, ids, i, i < call.row_start[t + 1], threadIdx.x & (group - 1), out, dim,
-                 elems, group, notes);
+                 elems, group, notes, kFillingIdsCombined);
 }
 
 // the same for rows 32 to 128 floats wide: a workgroup takes 64 positions of its table
@@ -841,7 +868,94 @@ __global__ __launch_bounds__(kBlock) void group_pull_wide_kernel(const TableDesc
                         kWideIds;
   const int64_t first = call.row_start[t] + local;
   if (first >= call.row_start[t + 1]) return;    // the whole wavefront
-  pull_wide<VEC, true, STEPS>(tv, init, ids, first, call.row_start[t + 1], out, dim, elems, nullptr, 0, notes);
+  pull_wide<VEC, true, STEPS>(tv, init, ids, first, call.row_start[t + 1], out, dim, elems, nullptr, 0, notes,
+                              kFillingIdsCombined);
+}
+
+// ---- combined pulls while the members' tables are being filled ---------------------------------
+// The two launches of a large pull, member by member: the first looks up and copies and queues
+// the positions whose id is missing in the member's own lists (positions count from the member's
+// first), the second gives every member kGroupMissPerTable workgroups of 1024 lanes that walk
+// four lists each. The fused kernels add to a member's row counter once per wavefront that
+// inserts: 98.6k new ids over 26 tables took 67 us that way against 9 us resident.
+constexpr int kGroupMissPerTable = 16;
+static_assert(kQueues % kGroupMissPerTable == 0, "every workgroup walks the same number of lists");
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void group_pull_resident_kernel(const TableDesc* __restrict__ descs,
+                                                                     GroupCall call, GroupFill fill,
+                                                                     const uint64_t* __restrict__ ids,
+                                                                     float* __restrict__ out,
+                                                                     uint32_t* __restrict__ todo, int dim,
+                                                                     int elems, int group) {
+  const uint32_t bx = blockIdx.x;
+  const int t = find_table(call, bx);
+  const int64_t a = call.row_start[t];
+  pull_resident_body<VEC>(descs[t].tv, ids + a, call.row_start[t + 1] - a, out + a * dim,
+                          todo + fill.todo_start[t], (int)((fill.parity_bits >> t) & 1u), dim, elems, group,
+                          bx - call.block_start[t]);
+}
+
+template <int VEC, int STEPS>
+__global__ __launch_bounds__(kBlock) void group_pull_resident_wide_kernel(const TableDesc* __restrict__ descs,
+                                                                          GroupCall call, GroupFill fill,
+                                                                          const uint64_t* __restrict__ ids,
+                                                                          float* __restrict__ out,
+                                                                          uint32_t* __restrict__ todo, int dim,
+                                                                          int elems) {
+  const uint32_t bx = blockIdx.x;
+  const int t = find_table(call, bx);
+  const int64_t a = call.row_start[t];
+  const int64_t n = call.row_start[t + 1] - a;
+  const int64_t first = ((int64_t)(bx - call.block_start[t]) * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds;
+  if (first >= n) return;                        // the whole wavefront
+  InitK none{};
+  pull_wide<VEC, false, STEPS>(descs[t].tv, none, ids + a, first, n, out + a * dim, dim, elems,
+                               todo + fill.todo_start[t], (int)((fill.parity_bits >> t) & 1u));
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kMissBlock) void group_pull_missing_kernel(const TableDesc* __restrict__ descs,
+                                                                        GroupCall call, GroupFill fill,
+                                                                        const uint64_t* __restrict__ ids,
+                                                                        float* __restrict__ out,
+                                                                        const uint32_t* __restrict__ todo,
+                                                                        int per_block, int dim, int elems,
+                                                                        int group) {
+  const int t = blockIdx.x / kGroupMissPerTable;
+  const int w = blockIdx.x % kGroupMissPerTable;
+  const int64_t a = call.row_start[t];
+  const int64_t n = call.row_start[t + 1] - a;
+  if (n <= 0) return;                              // a member without ids: its lists were not used
+  TableView tv = descs[t].tv;
+  tv.epoch = call.epoch[t];
+  const InitK init = descs[t].init;
+  const int parity = (int)((fill.parity_bits >> t) & 1u);
+  const int64_t capacity = queue_capacity(n, per_block);
+  const uint32_t* lists = todo + fill.todo_start[t];
+  // the workgroup's lists w, w + 16, ... as one: a member's lists are short (a sixty-fourth of
+  // its missing ids each), and a trip costs the same whether its 256 entries are all there or not
+  constexpr int kMine = kQueues / kGroupMissPerTable;
+  uint32_t upto[kMine];                              // entries in the workgroup's first j + 1 lists
+  uint32_t total = 0;
+#pragma unroll
+  for (int j = 0; j < kMine; ++j) {
+    const int q = w + j * kGroupMissPerTable;
+    total += __atomic_load_n(queue_counter(tv, parity, q), __ATOMIC_RELAXED);
+    upto[j] = total;
+    if (threadIdx.x == 0) *queue_counter(tv, parity ^ 1, q) = 0u;
+  }
+  // still being filled: the workgroup holds a sixteenth of the member's missing ids; a fifth of the
+  // member's ids or more are missing
+  if (threadIdx.x == 0 && (uint64_t)total * (5u * kGroupMissPerTable) >= (uint64_t)n) note_inserting(tv);
+  auto position_of = [&](uint32_t k) {
+    int j = 0;
+#pragma unroll
+    for (int i = 0; i + 1 < kMine; ++i) j += k >= upto[i] ? 1 : 0;
+    return lists[(int64_t)(w + j * kGroupMissPerTable) * capacity + (k - (j ? upto[j - 1] : 0u))];
+  };
+  insert_queued<VEC, false>(tv, init, ids + a, out + a * dim, position_of, total, 0u, kMissEntries, dim, elems,
+                            group, nullptr);
 }
 
 template <int OPT, int VEC>
@@ -2819,7 +2933,51 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
       notes = g->notes.as<uint32_t>();
     }
   }
-  if (wide && g->group == 8) {
+  // While the members' tables are being filled (see pull_enqueue) the request takes the two
+  // launches of a large pull, member by member.
+  bool filling = false;
+  for (krk_sparse* t : g->tables)
+    if (t->host_inserted && __atomic_exchange_n(t->host_inserted, 0u, __ATOMIC_RELAXED) != 0u) filling = true;
+  if (filling && !(flags & KRK_NOTE_ROWS) && total >= kTwoLaunchWhileFilling) {
+    GroupFill fill{};
+    const int per_block = wide ? (kBlock / kWave) * kWideIds : kBlock / g->group;
+    uint64_t words = 0;
+    for (size_t i = 0; i < g->tables.size(); ++i) {
+      const int64_t cnt = offsets[i + 1] - offsets[i];
+      fill.todo_start[i] = (uint32_t)words;
+      if (cnt <= 0) continue;
+      krk_sparse* t = g->tables[i];
+      words += (uint64_t)kQueues * (uint64_t)queue_capacity(cnt, per_block);
+      if (t->pull_parity) fill.parity_bits |= 1u << i;
+      t->pull_parity ^= 1;
+    }
+    KRK_TRY(g->todo.reserve((size_t)words * sizeof(uint32_t)));
+    uint32_t* todo = g->todo.as<uint32_t>();
+    const dim3 missing_grid((unsigned)call.n_tables * kGroupMissPerTable), missing_block(kMissBlock);
+    if (wide && g->group == 8) {
+      hipLaunchKernelGGL((group_pull_resident_wide_kernel<4, 2>), grid, block, 0, g->stream, g->d_descs, call, fill,
+                         d_ids, d_out, todo, (int)g->dim, g->elems);
+    } else if (wide && g->group == 16) {
+      hipLaunchKernelGGL((group_pull_resident_wide_kernel<4, 4>), grid, block, 0, g->stream, g->d_descs, call, fill,
+                         d_ids, d_out, todo, (int)g->dim, g->elems);
+    } else if (wide) {
+      hipLaunchKernelGGL((group_pull_resident_wide_kernel<4, 8>), grid, block, 0, g->stream, g->d_descs, call, fill,
+                         d_ids, d_out, todo, (int)g->dim, g->elems);
+    } else if (g->vec == 4) {
+      hipLaunchKernelGGL((group_pull_resident_kernel<4>), grid, block, 0, g->stream, g->d_descs, call, fill, d_ids,
+                         d_out, todo, (int)g->dim, g->elems, g->group);
+    } else {
+      hipLaunchKernelGGL((group_pull_resident_kernel<1>), grid, block, 0, g->stream, g->d_descs, call, fill, d_ids,
+                         d_out, todo, (int)g->dim, g->elems, g->group);
+    }
+    if (g->vec == 4) {
+      hipLaunchKernelGGL((group_pull_missing_kernel<4>), missing_grid, missing_block, 0, g->stream, g->d_descs, call,
+                         fill, d_ids, d_out, todo, per_block, (int)g->dim, g->elems, g->group);
+    } else {
+      hipLaunchKernelGGL((group_pull_missing_kernel<1>), missing_grid, missing_block, 0, g->stream, g->d_descs, call,
+                         fill, d_ids, d_out, todo, per_block, (int)g->dim, g->elems, g->group);
+    }
+  } else if (wide && g->group == 8) {
     hipLaunchKernelGGL((group_pull_wide_kernel<4, 2>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
                        (int)g->dim, g->elems, notes);
   } else if (wide && g->group == 16) {

@@ -5,7 +5,7 @@ way the reference does. Shape of the reference's own test: emitter_test.cc:75-87
 import numpy as np
 import pytest
 
-from util import OPTIM_CASES, assert_close, make_optims, zipf_ids
+from util import OPTIM_CASES, assert_close, make_optims, splitmix64, zipf_ids
 
 pytestmark = pytest.mark.gpu
 
@@ -82,6 +82,42 @@ def test_group_matches_oracle_loop(api, oracle, name, type_, conf, dim, n_tables
         if type_ == 1:
             assert np.array_equal(gsteps[og], rsteps[orr])
 
+
+@pytest.mark.parametrize("dim", [16, 6, 36, 64, 128])
+def test_group_pulls_while_the_tables_are_being_filled(api, oracle, dim):
+    """A combined pull of 8192 ids or more whose members' tables are being filled (new tables, or
+    a pull before it that met many new ids) looks up and copies in one launch, queues the missing
+    positions member by member and inserts them in a second one. Members of very different
+    sizes, one of them empty, ids that repeat inside a member, the ids 0 and all ones, new ids at
+    every step, then the same request twice (the second takes the fused kernel again): every
+    pulled row as the oracle's, every table holding each id once."""
+    rng = np.random.default_rng(dim)
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "17"})
+    counts = [9000, 0, 1, 17, 4000, 300, 2500]
+    tables = [api.SparseTable(dim, gi, capacity_hint=64) for _ in counts]
+    refs = [oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=17)) for _ in counts]
+    grp = api.TableGroup(tables)
+    per = None
+    for step in range(6):
+        if step < 4:
+            per = []
+            for c in counts:
+                ids = splitmix64(rng.integers(0, 6000 * (step + 1), size=c, dtype=np.uint64))
+                if c > 100:
+                    ids[:2] = np.array([0, 2**64 - 1], np.uint64)
+                    ids[2:40] = ids[50]                      # one id many times in a row
+                per.append(ids)
+        off = grp._offsets([p.size for p in per])
+        rc, got = grp.CombinePull(np.concatenate(per), off)
+        assert rc == 0
+        want = np.concatenate([r.pull(p)[1] for r, p in zip(refs, per) if p.size])
+        assert_close(got, want, "dim %d, step %d" % (dim, step), rtol=1e-6)
+        for t, r in zip(tables, refs):
+            assert len(t) == len(r)
+    for t, r in zip(tables, refs):
+        gid = t.export()[0]
+        assert np.array_equal(np.sort(gid), np.sort(r.export()[0]))
+    grp.close()
 
 def test_group_errors_and_async(api, oracle):
     gi = api.Initializer.create(0, {"value": "1"})
