@@ -349,7 +349,11 @@ constexpr int kMissWaves = kMissBlock / kWave;
 
 // Entries k_first, k_first + stride, ... of `count` queued positions, kMissEntries at a time (the
 // workgroups that share them are `stride` apart); position_of(k) names the k-th.
-template <int VEC, bool ROWS_ONLY, typename PositionOf>
+// MODE: what is done with an entry once its row is known.
+constexpr int kInsertAndCopy = 0;   // a pull: new rows are initialised, every entry's row goes to out
+constexpr int kInsertOnly = 1;      // ROWS_ONLY
+constexpr int kInsertGiven = 2;     // an import: the creator copies the row out[position] into the record
+template <int VEC, int MODE, typename PositionOf>
 __device__ __forceinline__ void insert_queued(const TableView& tv, const InitK& init,
                                               const uint64_t* __restrict__ ids, float* __restrict__ out,
                                               PositionOf position_of, uint32_t count,
@@ -413,7 +417,7 @@ __device__ __forceinline__ void insert_queued(const TableView& tv, const InitK& 
       s_pos[entry] = pos;
       s_row[entry] = pr.row;
       s_state[entry] = (active ? 1u : 0u) | (pr.owner ? 2u : 0u) | (pr.fresh ? 4u : 0u);
-      if (ROWS_ONLY && active) rows_out[pos] = pr.row;
+      if (MODE == kInsertOnly && active) rows_out[pos] = pr.row;
     }
     __syncthreads();
     for (int j = threadIdx.x / group; j < kMissEntries; j += kMissBlock / group) {
@@ -422,11 +426,16 @@ __device__ __forceinline__ void insert_queued(const TableView& tv, const InitK& 
       const uint32_t row = s_row[j];
       const uint64_t its_id = s_id[j];
       float* rec = row == kEmptyRow ? nullptr : tv.recs + (int64_t)row * tv.stride;
-      if constexpr (ROWS_ONLY) {
-        if ((state & 6u) == 6u) {                    // created here: the record's initial values
+      if constexpr (MODE != kInsertAndCopy) {
+        if ((state & 6u) == 6u) {                    // created here: the record's first values
+          const float* given = out + (int64_t)s_pos[j] * dim;
           for (int e = gl; e < elems; e += group) {
             float v[VEC];
-            init_vec<VEC, true>(init, its_id, (int64_t)e * VEC, v);
+            if constexpr (MODE == kInsertGiven) {
+              vload<VEC>(given + e * VEC, v);
+            } else {
+              init_vec<VEC, true>(init, its_id, (int64_t)e * VEC, v);
+            }
             vstore<VEC>(rec + e * VEC, v);
           }
         }
@@ -466,7 +475,7 @@ __global__ __launch_bounds__(kMissBlock) void pull_missing_kernel(TableView tv, 
     if ((uint64_t)count * 256u >= (uint64_t)list_capacity) note_inserting(tv);
   }
   const uint32_t* list = todo + q * list_capacity;
-  insert_queued<VEC, ROWS_ONLY>(tv, init, ids, out, [list](uint32_t k) { return list[k]; }, count,
+  insert_queued<VEC, ROWS_ONLY ? kInsertOnly : kInsertAndCopy>(tv, init, ids, out, [list](uint32_t k) { return list[k]; }, count,
                                 (blockIdx.x / kQueues) * kMissEntries, (gridDim.x / kQueues) * kMissEntries, dim,
                                 elems, group, rows_out);
 }
@@ -954,8 +963,8 @@ __global__ __launch_bounds__(kMissBlock) void group_pull_missing_kernel(const Ta
     for (int i = 0; i + 1 < kMine; ++i) j += k >= upto[i] ? 1 : 0;
     return lists[(int64_t)(w + j * kGroupMissPerTable) * capacity + (k - (j ? upto[j - 1] : 0u))];
   };
-  insert_queued<VEC, false>(tv, init, ids + a, out + a * dim, position_of, total, 0u, kMissEntries, dim, elems,
-                            group, nullptr);
+  insert_queued<VEC, kInsertAndCopy>(tv, init, ids + a, out + a * dim, position_of, total, 0u, kMissEntries, dim,
+                                     elems, group, nullptr);
 }
 
 template <int OPT, int VEC>
@@ -1014,27 +1023,17 @@ __global__ __launch_bounds__(kBlock) void lookup_kernel(TableView tv, const uint
   if (active && gl == 0) rows[i] = r == kEmptyRow ? -1 : (int32_t)r;
 }
 
-// import: like pull, but a new row takes its values from the caller
+// import: like pull, but a new row takes its values from the caller. Workgroups of 1024 lanes
+// take 256 ids each and number the rows they make with one addition to the row counter (a
+// checkpoint of 1e8 rows 32 floats wide is 12.5 million wavefronts of the table kernels' size).
 template <int VEC>
-__global__ __launch_bounds__(kBlock) void import_kernel(TableView tv, const uint64_t* __restrict__ ids,
-                                                        int64_t n, const float* __restrict__ vals,
-                                                        int dim, int elems, int group) {
-  const int per_block = kBlock / group;
-  const int64_t i = (int64_t)blockIdx.x * per_block + threadIdx.x / group;
-  const int gl = threadIdx.x & (group - 1);
-  const bool active = i < n;
-  const ProbeResult pr = probe_insert(tv, active ? ids[i] : 0, active, gl, group);
-  const uint32_t row = pr.row;
-  const bool owner = pr.owner;
-  if (active && owner) {
-    float* rec = tv.recs + (int64_t)row * tv.stride;
-    const float* src = vals + i * (int64_t)dim;
-    for (int e = gl; e < elems; e += group) {
-      float v[VEC];
-      vload<VEC>(src + e * VEC, v);
-      vstore<VEC>(rec + e * VEC, v);
-    }
-  }
+__global__ __launch_bounds__(kMissBlock) void import_kernel(TableView tv, const uint64_t* __restrict__ ids,
+                                                            int64_t n, const float* __restrict__ vals,
+                                                            int dim, int elems, int group) {
+  InitK none{};
+  insert_queued<VEC, kInsertGiven>(tv, none, ids, const_cast<float*>(vals), [](uint32_t k) { return k; },
+                                   (uint32_t)n, blockIdx.x * kMissEntries, gridDim.x * kMissEntries, dim, elems,
+                                   group, nullptr);
 }
 
 // {rows used, launch number} of up to 32 tables -> pinned host memory. Runs behind the launch
@@ -2289,8 +2288,7 @@ int32_t krk_sparse_import(krk_sparse* t, const uint64_t* ids, int64_t n, const f
   KRK_TRY(t->input(ids, (size_t)n, flags, 0, &d_ids));
   KRK_TRY(t->input(vals, (size_t)n * t->dim, flags, 1, &d_vals));
   KRK_TRY(sparse_next_epoch(t, n));
-  const int per_block = kBlock / t->group;
-  const dim3 grid(grid_for(n, per_block)), block(kBlock);
+  const dim3 grid(grid_for(n, kMissEntries)), block(kMissBlock);
   if (t->vec == 4) {
     hipLaunchKernelGGL((import_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_vals,
                        (int)t->dim, t->elems, t->group);
