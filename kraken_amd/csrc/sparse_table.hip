@@ -293,7 +293,8 @@ template <int VEC>
 __device__ __forceinline__ void pull_resident_body(const TableView& tv, const uint64_t* __restrict__ ids,
                                                    int64_t n, float* __restrict__ out,
                                                    uint32_t* __restrict__ todo, int parity, int dim,
-                                                   int elems, int group, uint32_t bx) {
+                                                   int elems, int group, uint32_t bx,
+                                                   uint32_t* __restrict__ notes) {
   const int per_block = kBlock / group;
   const int64_t i = (int64_t)bx * per_block + threadIdx.x / group;
   const int gl = threadIdx.x & (group - 1);
@@ -313,6 +314,8 @@ __device__ __forceinline__ void pull_resident_body(const TableView& tv, const ui
       todo[q * queue_capacity(n, per_block) + base + (uint32_t)__popcll(votes & ((1ull << lane) - 1ull))] =
           (uint32_t)i;
   }
+  // the note of a missing id is written by the launch that inserts it
+  if (notes && active && gl == 0 && row != kEmptyRow) notes[i] = row;
   if (!active || row == kEmptyRow) return;
   const float* rec = tv.recs + (int64_t)row * tv.stride;
   float* dst = out + i * (int64_t)dim;
@@ -327,8 +330,8 @@ template <int VEC>
 __global__ __launch_bounds__(kBlock) void pull_resident_kernel(TableView tv, const uint64_t* __restrict__ ids,
                                                                int64_t n, float* __restrict__ out,
                                                                uint32_t* __restrict__ todo, int parity, int dim,
-                                                               int elems, int group) {
-  pull_resident_body<VEC>(tv, ids, n, out, todo, parity, dim, elems, group, blockIdx.x);
+                                                               int elems, int group, uint32_t* __restrict__ notes) {
+  pull_resident_body<VEC>(tv, ids, n, out, todo, parity, dim, elems, group, blockIdx.x, notes);
 }
 
 // The second launch: workgroups of 1024 lanes walk the lists, 256 entries at a time.
@@ -417,7 +420,7 @@ __device__ __forceinline__ void insert_queued(const TableView& tv, const InitK& 
       s_pos[entry] = pos;
       s_row[entry] = pr.row;
       s_state[entry] = (active ? 1u : 0u) | (pr.owner ? 2u : 0u) | (pr.fresh ? 4u : 0u);
-      if (MODE == kInsertOnly && active) rows_out[pos] = pr.row;
+      if (rows_out && active) rows_out[pos] = pr.row;
     }
     __syncthreads();
     for (int j = threadIdx.x / group; j < kMissEntries; j += kMissBlock / group) {
@@ -666,6 +669,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
     }
     copy = active && f.found;
     pr.fresh = false;                              // nothing is created here: what was found is read
+    if (notes && copy && gl4 == 0) notes[i] = pr.row;   // a missing id's note: by the launch that inserts it
   }
   // the copy: lane group `sub` of the wavefront takes ids sub, sub + rows_per_step, ...
   constexpr int rows_per_step = kWideIds / STEPS;   // 8, 4 or 2
@@ -827,11 +831,12 @@ __global__ __launch_bounds__(kBlock) void pull_resident_wide_kernel(TableView tv
                                                                     const uint64_t* __restrict__ ids,
                                                                     int64_t n, float* __restrict__ out,
                                                                     uint32_t* __restrict__ todo, int parity,
-                                                                    int dim, int elems) {
+                                                                    int dim, int elems,
+                                                                    uint32_t* __restrict__ notes) {
   const int64_t first = ((int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds;
   if (first >= n) return;
   InitK none{};
-  pull_wide<VEC, false, STEPS>(tv, none, ids, first, n, out, dim, elems, todo, parity);
+  pull_wide<VEC, false, STEPS>(tv, none, ids, first, n, out, dim, elems, todo, parity, notes);
 }
 
 // ---- one launch over several tables of equal row width ------------------------
@@ -896,13 +901,14 @@ __global__ __launch_bounds__(kBlock) void group_pull_resident_kernel(const Table
                                                                      const uint64_t* __restrict__ ids,
                                                                      float* __restrict__ out,
                                                                      uint32_t* __restrict__ todo, int dim,
-                                                                     int elems, int group) {
+                                                                     int elems, int group,
+                                                                     uint32_t* __restrict__ notes) {
   const uint32_t bx = blockIdx.x;
   const int t = find_table(call, bx);
   const int64_t a = call.row_start[t];
   pull_resident_body<VEC>(descs[t].tv, ids + a, call.row_start[t + 1] - a, out + a * dim,
                           todo + fill.todo_start[t], (int)((fill.parity_bits >> t) & 1u), dim, elems, group,
-                          bx - call.block_start[t]);
+                          bx - call.block_start[t], notes ? notes + a : nullptr);
 }
 
 template <int VEC, int STEPS>
@@ -911,7 +917,7 @@ __global__ __launch_bounds__(kBlock) void group_pull_resident_wide_kernel(const 
                                                                           const uint64_t* __restrict__ ids,
                                                                           float* __restrict__ out,
                                                                           uint32_t* __restrict__ todo, int dim,
-                                                                          int elems) {
+                                                                          int elems, uint32_t* __restrict__ notes) {
   const uint32_t bx = blockIdx.x;
   const int t = find_table(call, bx);
   const int64_t a = call.row_start[t];
@@ -920,7 +926,8 @@ __global__ __launch_bounds__(kBlock) void group_pull_resident_wide_kernel(const 
   if (first >= n) return;                        // the whole wavefront
   InitK none{};
   pull_wide<VEC, false, STEPS>(descs[t].tv, none, ids + a, first, n, out + a * dim, dim, elems,
-                               todo + fill.todo_start[t], (int)((fill.parity_bits >> t) & 1u));
+                               todo + fill.todo_start[t], (int)((fill.parity_bits >> t) & 1u),
+                               notes ? notes + a : nullptr);
 }
 
 template <int VEC>
@@ -930,7 +937,7 @@ __global__ __launch_bounds__(kMissBlock) void group_pull_missing_kernel(const Ta
                                                                         float* __restrict__ out,
                                                                         const uint32_t* __restrict__ todo,
                                                                         int per_block, int dim, int elems,
-                                                                        int group) {
+                                                                        int group, uint32_t* __restrict__ notes) {
   const int t = blockIdx.x / kGroupMissPerTable;
   const int w = blockIdx.x % kGroupMissPerTable;
   const int64_t a = call.row_start[t];
@@ -964,7 +971,7 @@ __global__ __launch_bounds__(kMissBlock) void group_pull_missing_kernel(const Ta
     return lists[(int64_t)(w + j * kGroupMissPerTable) * capacity + (k - (j ? upto[j - 1] : 0u))];
   };
   insert_queued<VEC, kInsertAndCopy>(tv, init, ids + a, out + a * dim, position_of, total, 0u, kMissEntries, dim,
-                                     elems, group, nullptr);
+                                     elems, group, notes ? notes + a : nullptr);
 }
 
 template <int OPT, int VEC>
@@ -1943,9 +1950,9 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
   // wavefront that inserts, and those additions are served one after the other (98 600 new ids:
   // 137 us fused). Whether the table is being filled is what the pull before this one left
   // behind in host memory; it may lag by the requests that are still queued, and either choice
-  // gives the same rows. Row notes are kept by the fused kernels only.
+  // gives the same rows.
   const bool filling = t->host_inserted && __atomic_exchange_n(t->host_inserted, 0u, __ATOMIC_RELAXED) != 0u;
-  if (n >= kTwoLaunchPull || (filling && !notes && n >= kTwoLaunchWhileFilling)) {
+  if (n >= kTwoLaunchPull || (filling && n >= kTwoLaunchWhileFilling)) {
     KRK_TRY(t->scratch[5].reserve((size_t)kQueues * queue_capacity(n, per_block) * sizeof(uint32_t)));
     uint32_t* todo = t->scratch[5].as<uint32_t>();
     const int parity = t->pull_parity;
@@ -1955,24 +1962,24 @@ static int32_t pull_enqueue(krk_sparse* t, const uint64_t* d_ids, int64_t n, flo
     if (t->vec == 4) {
       if (wide && t->group == 8) {
         hipLaunchKernelGGL((pull_resident_wide_kernel<4, 2>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
-                           todo, parity, (int)t->dim, t->elems);
+                           todo, parity, (int)t->dim, t->elems, notes);
       } else if (wide && t->group == 16) {
         hipLaunchKernelGGL((pull_resident_wide_kernel<4, 4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
-                           todo, parity, (int)t->dim, t->elems);
+                           todo, parity, (int)t->dim, t->elems, notes);
       } else if (wide) {
         hipLaunchKernelGGL((pull_resident_wide_kernel<4, 8>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out,
-                           todo, parity, (int)t->dim, t->elems);
+                           todo, parity, (int)t->dim, t->elems, notes);
       } else {
         hipLaunchKernelGGL((pull_resident_kernel<4>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
-                           parity, (int)t->dim, t->elems, t->group);
+                           parity, (int)t->dim, t->elems, t->group, notes);
       }
       hipLaunchKernelGGL((pull_missing_kernel<4>), small, missing_block, 0, t->stream, t->view(), t->initk, d_ids,
-                         d_out, todo, parity, list_capacity, (int)t->dim, t->elems, t->group);
+                         d_out, todo, parity, list_capacity, (int)t->dim, t->elems, t->group, notes);
     } else {
       hipLaunchKernelGGL((pull_resident_kernel<1>), grid, block, 0, t->stream, t->view(), d_ids, n, d_out, todo,
-                         parity, (int)t->dim, t->elems, t->group);
+                         parity, (int)t->dim, t->elems, t->group, notes);
       hipLaunchKernelGGL((pull_missing_kernel<1>), small, missing_block, 0, t->stream, t->view(), t->initk, d_ids,
-                         d_out, todo, parity, list_capacity, (int)t->dim, t->elems, t->group);
+                         d_out, todo, parity, list_capacity, (int)t->dim, t->elems, t->group, notes);
     }
   } else if (t->vec == 4 && wide && t->group == 8) {
     hipLaunchKernelGGL((pull_wide_kernel<4, 2>), grid, block, 0, t->stream, t->view(), t->initk, d_ids, n, d_out,
@@ -2936,7 +2943,7 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
   bool filling = false;
   for (krk_sparse* t : g->tables)
     if (t->host_inserted && __atomic_exchange_n(t->host_inserted, 0u, __ATOMIC_RELAXED) != 0u) filling = true;
-  if (filling && !(flags & KRK_NOTE_ROWS) && total >= kTwoLaunchWhileFilling) {
+  if (filling && total >= kTwoLaunchWhileFilling) {
     GroupFill fill{};
     const int per_block = wide ? (kBlock / kWave) * kWideIds : kBlock / g->group;
     uint64_t words = 0;
@@ -2954,26 +2961,26 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
     const dim3 missing_grid((unsigned)call.n_tables * kGroupMissPerTable), missing_block(kMissBlock);
     if (wide && g->group == 8) {
       hipLaunchKernelGGL((group_pull_resident_wide_kernel<4, 2>), grid, block, 0, g->stream, g->d_descs, call, fill,
-                         d_ids, d_out, todo, (int)g->dim, g->elems);
+                         d_ids, d_out, todo, (int)g->dim, g->elems, notes);
     } else if (wide && g->group == 16) {
       hipLaunchKernelGGL((group_pull_resident_wide_kernel<4, 4>), grid, block, 0, g->stream, g->d_descs, call, fill,
-                         d_ids, d_out, todo, (int)g->dim, g->elems);
+                         d_ids, d_out, todo, (int)g->dim, g->elems, notes);
     } else if (wide) {
       hipLaunchKernelGGL((group_pull_resident_wide_kernel<4, 8>), grid, block, 0, g->stream, g->d_descs, call, fill,
-                         d_ids, d_out, todo, (int)g->dim, g->elems);
+                         d_ids, d_out, todo, (int)g->dim, g->elems, notes);
     } else if (g->vec == 4) {
       hipLaunchKernelGGL((group_pull_resident_kernel<4>), grid, block, 0, g->stream, g->d_descs, call, fill, d_ids,
-                         d_out, todo, (int)g->dim, g->elems, g->group);
+                         d_out, todo, (int)g->dim, g->elems, g->group, notes);
     } else {
       hipLaunchKernelGGL((group_pull_resident_kernel<1>), grid, block, 0, g->stream, g->d_descs, call, fill, d_ids,
-                         d_out, todo, (int)g->dim, g->elems, g->group);
+                         d_out, todo, (int)g->dim, g->elems, g->group, notes);
     }
     if (g->vec == 4) {
       hipLaunchKernelGGL((group_pull_missing_kernel<4>), missing_grid, missing_block, 0, g->stream, g->d_descs, call,
-                         fill, d_ids, d_out, todo, per_block, (int)g->dim, g->elems, g->group);
+                         fill, d_ids, d_out, todo, per_block, (int)g->dim, g->elems, g->group, notes);
     } else {
       hipLaunchKernelGGL((group_pull_missing_kernel<1>), missing_grid, missing_block, 0, g->stream, g->d_descs, call,
-                         fill, d_ids, d_out, todo, per_block, (int)g->dim, g->elems, g->group);
+                         fill, d_ids, d_out, todo, per_block, (int)g->dim, g->elems, g->group, notes);
     }
   } else if (wide && g->group == 8) {
     hipLaunchKernelGGL((group_pull_wide_kernel<4, 2>), grid, block, 0, g->stream, g->d_descs, call, d_ids, d_out,
