@@ -375,7 +375,7 @@ def test_pulls_while_a_table_is_being_filled(api, oracle, dim):
     of the fused kernel. Which of the two ran must not show: steps that bring half new ids, then
     the same ids twice (the first of them still takes the two launches, the second the fused
     kernel), then new ids again, every step against the oracle; a request that asks for row notes
-    keeps the fused kernel and the push that reuses them updates the same rows."""
+    gets them from either pair of kernels and the push that reuses them updates the same rows."""
     gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "29"})
     t = api.SparseTable(dim, gi, capacity_hint=64)
     r = oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=29))
