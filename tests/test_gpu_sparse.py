@@ -417,6 +417,39 @@ def test_pulls_while_a_table_is_being_filled(api, oracle, dim):
     for a in (d_ids, d_out, d_g):
         a.free()
 
+@pytest.mark.parametrize("dim", [16, 7, 128, 260])
+def test_import_of_rows_numbers_them_once_per_workgroup(api, oracle, dim):
+    """krk_sparse_import hands 256 ids to a workgroup that numbers its new rows with one addition
+    to the row counter. Request sizes on both sides of 256 and of a launch's workgroups, ids the
+    table already holds (they keep their values, as in the oracle), the ids 0 and all ones, and
+    a pull of everything afterwards."""
+    gi = api.Initializer.create(api.InitializerType.kNormal, {"stddev": "0.01", "seed": "31"})
+    t = api.SparseTable(dim, gi, capacity_hint=64)
+    r = oracle.SparseTable(dim, oracle.init(oracle.INIT_NORMAL, 0.0, 0.01, seed=31))
+    rng = np.random.default_rng(dim)
+    base = 0
+    held = []
+    for n in (1, 255, 256, 257, 1023, 5000, 70_000):
+        fresh = splitmix64(np.arange(base, base + n, dtype=np.uint64))
+        base += n
+        ids = fresh
+        if held:
+            ids = np.concatenate([fresh, rng.choice(np.concatenate(held), size=min(n, 300))])
+        if n == 5000:
+            ids = np.concatenate([ids, np.array([0, 2**64 - 1], np.uint64)])
+        ids = ids[rng.permutation(ids.size)]
+        vals = rng.standard_normal((ids.size, dim)).astype(np.float32)
+        t.load(ids, vals)
+        r.load(ids, vals)
+        held.append(fresh)
+        assert len(t) == len(r)
+    everything = np.concatenate(held + [np.array([0, 2**64 - 1], np.uint64)])
+    rc, got = t.Pull(everything)
+    _, want = r.pull(everything)
+    assert rc == 0 and np.array_equal(got, want)
+    gid = t.export()[0]
+    assert np.array_equal(np.sort(gid), np.sort(r.export()[0]))
+
 def test_wide_rows_group_pull_ragged_members(api, oracle):
     """A combined pull over tables of 64-float rows whose members bring 0, 1, 17 and 5000 ids."""
     dim = 64
