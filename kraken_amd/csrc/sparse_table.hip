@@ -144,7 +144,9 @@ __device__ __forceinline__ void pull_body(const TableView& tv, const InitK& init
   if (__any(miss)) {
     const ProbeResult q = probe_insert(tv, id, miss, gl, group);
     if (miss) pr = q;
-    if (__popcll(__ballot(miss && gl == 0)) >= filling_ids && wave_lane() == 0) note_inserting(tv);
+    // (a wavefront of a table whose lane groups are 64 lanes wide carries one id: any new id counts)
+    const int enough = filling_ids < kWave / group ? filling_ids : kWave / group;
+    if (__popcll(__ballot(miss && gl == 0)) >= enough && wave_lane() == 0) note_inserting(tv);
   }
   if (!active) return;
   const uint32_t row = pr.row;
