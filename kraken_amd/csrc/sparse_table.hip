@@ -23,10 +23,12 @@ constexpr int kBlock = 256;
 constexpr int64_t kTwoLaunchPull = 1 << 18;   // ids from which a pull runs as two launches
 constexpr int64_t kTwoLaunchWhileFilling = 1 << 13;   // the same while the pulls before it inserted rows
 // A wavefront tells the host that the table is being filled when that many of its sixteen (or
-// fewer) ids are new: two in one wavefront is rare when fewer than one id in three hundred is new,
-// the share from which the fused kernel's additions to the row counter cost more than a second
-// launch, and all but certain somewhere in a request when one in a hundred is.
-constexpr int kFillingIds = 2;
+// fewer) ids are new. From one new id in 250 on, the fused kernel's additions to the row counter
+// cost a request of 98 600 ids more than a second launch does (7 us more). Three new ids in one
+// wavefront: once in five such requests at that share, in every request from one new id in a
+// hundred on, and once in three hundred requests at one in a thousand (two in one wavefront
+// would send every other of those through the two launches for nothing).
+constexpr int kFillingIds = 3;
 // A combined request spreads its additions over its members' counters, and its two launches cost
 // 15 us more than its fused kernel where nothing is new: over 26 tables they pay from one new id
 // in five on (98.6k ids, one in ten new: 21 us fused, 27 us in two launches; all new: 64 and 34).
