@@ -668,7 +668,7 @@ __device__ __forceinline__ void pull_wide(const TableView& tv, const InitK& init
       if (lane == leader) base = atomicAdd(queue_counter(tv, parity, q), (uint32_t)__popcll(votes));
       base = __shfl(base, leader);
       if (queue)
-        todo[q * queue_capacity(end, (kBlock / kWave) * kWideIds) + base +
+        todo[q * queue_capacity(end, (int)(blockDim.x / kWave) * kWideIds) + base +
              (uint32_t)__popcll(votes & ((1ull << lane) - 1ull))] = (uint32_t)i;
     }
     copy = active && f.found;
@@ -882,7 +882,7 @@ __global__ __launch_bounds__(kBlock) void group_pull_wide_kernel(const TableDesc
   TableView tv = descs[t].tv;
   tv.epoch = call.epoch[t];
   const InitK init = descs[t].init;
-  const int64_t local = ((int64_t)(blockIdx.x - call.block_start[t]) * (kBlock / kWave) + threadIdx.x / kWave) *
+  const int64_t local = ((int64_t)(blockIdx.x - call.block_start[t]) * (blockDim.x / kWave) + threadIdx.x / kWave) *
                         kWideIds;
   const int64_t first = call.row_start[t] + local;
   if (first >= call.row_start[t + 1]) return;    // the whole wavefront
@@ -926,7 +926,7 @@ __global__ __launch_bounds__(kBlock) void group_pull_resident_wide_kernel(const 
   const int t = find_table(call, bx);
   const int64_t a = call.row_start[t];
   const int64_t n = call.row_start[t + 1] - a;
-  const int64_t first = ((int64_t)(bx - call.block_start[t]) * (kBlock / kWave) + threadIdx.x / kWave) * kWideIds;
+  const int64_t first = ((int64_t)(bx - call.block_start[t]) * (blockDim.x / kWave) + threadIdx.x / kWave) * kWideIds;
   if (first >= n) return;                        // the whole wavefront
   InitK none{};
   pull_wide<VEC, false, STEPS>(descs[t].tv, none, ids + a, first, n, out + a * dim, dim, elems,
@@ -1018,7 +1018,7 @@ __global__ __launch_bounds__(kBlock) void group_push_wide_kernel(const TableDesc
   pc.c1 = st1 >= 0 ? descs[t].col_off[st1] : -1;
   pc.c2 = st2 >= 0 ? descs[t].col_off[st2] : -1;
   pc.meta = use_meta ? descs[t].meta_off : -1;
-  const int64_t local = ((int64_t)(bx - call.block_start[t]) * (kBlock / kWave) + threadIdx.x / kWave) *
+  const int64_t local = ((int64_t)(bx - call.block_start[t]) * (blockDim.x / kWave) + threadIdx.x / kWave) *
                         kWideIds;
   const int64_t first = call.row_start[t] + local;
   if (first >= call.row_start[t + 1]) return;    // the whole wavefront
@@ -2903,6 +2903,12 @@ int32_t krk_group_sync(krk_group* g) {
   return group_finish(g, 0);
 }
 
+// Lanes of a workgroup of the combined kernels for wide rows. Rows of 64 floats take 128: their
+// launches are bound by what a compute unit moves, and the 6162 wavefronts of the benchmark's
+// request come to 6.02 workgroups of 256 lanes a unit, i.e. seven on some and six on the others
+// (a step at dim 64: 42.7 us with 256 lanes, 41.7 us with 128; rows of 16 and 32 floats lose with 128).
+static int group_wide_block(int group) { return group == 16 ? 128 : kBlock; }
+
 int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets, float* out,
                        uint32_t flags) {
   if (!g || !offsets) return KRK_E_ARGUMENT;
@@ -2912,7 +2918,7 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
   GroupCall call;
   int64_t total = 0;
   const bool wide = g->vec == 4 && pull_is_wide(g->group, g->elems);
-  KRK_TRY(group_plan(g, offsets, &call, &total, wide ? (kBlock / kWave) * kWideIds : 0));
+  KRK_TRY(group_plan(g, offsets, &call, &total, wide ? (group_wide_block(g->group) / kWave) * kWideIds : 0));
   if (total == 0) return group_finish(g, flags);
   if (!ids || !out) return KRK_E_ARGUMENT;
   if ((flags & KRK_DEVICE_PTRS) && g->vec == 4 && !aligned16(out)) return KRK_E_ARGUMENT;
@@ -2932,7 +2938,7 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
   float* d_out;
   KRK_TRY(g->input(ids, (size_t)total, flags, 0, &d_ids));
   KRK_TRY(g->output(out, (size_t)total * g->dim, flags, 1, &d_out));
-  const dim3 grid(call.block_start[call.n_tables]), block(kBlock);
+  const dim3 grid(call.block_start[call.n_tables]), block(wide ? group_wide_block(g->group) : kBlock);
   // KRK_NOTE_ROWS: the row of every position stays behind
   uint32_t* notes = nullptr;
   if (flags & KRK_NOTE_ROWS) {
@@ -2949,7 +2955,7 @@ int32_t krk_group_pull(krk_group* g, const uint64_t* ids, const int64_t* offsets
     if (t->host_inserted && __atomic_exchange_n(t->host_inserted, 0u, __ATOMIC_RELAXED) != 0u) filling = true;
   if (filling && total >= kTwoLaunchWhileFilling) {
     GroupFill fill{};
-    const int per_block = wide ? (kBlock / kWave) * kWideIds : kBlock / g->group;
+    const int per_block = wide ? (group_wide_block(g->group) / kWave) * kWideIds : kBlock / g->group;
     uint64_t words = 0;
     for (size_t i = 0; i < g->tables.size(); ++i) {
       const int64_t cnt = offsets[i + 1] - offsets[i];
@@ -3024,7 +3030,7 @@ template <int OPT, int VEC>
 static void launch_group_push_opt(krk_group* g, const GroupCall& call, const uint64_t* ids,
                                   const float* grads, float lr, const OptimK& k, const int32_t st[3],
                                   int use_meta, bool wide, const uint32_t* notes) {
-  const dim3 grid(call.block_start[call.n_tables]), block(kBlock);
+  const dim3 grid(call.block_start[call.n_tables]), block(wide ? group_wide_block(g->group) : kBlock);
   const int dim = (int)g->dim;
   if constexpr (VEC == 4) {
     if (wide) {
@@ -3042,7 +3048,7 @@ static void launch_group_push_opt(krk_group* g, const GroupCall& call, const uin
                      dim, g->elems, g->group, lr, k, st[0], st[1], st[2], use_meta, notes);
 }
 
-// wide: the request was laid out for group_push_wide_kernel (64 positions a workgroup)
+// wide: the request was laid out for group_push_wide_kernel (group_wide_block lanes a workgroup)
 template <int VEC>
 static void launch_group_push(krk_group* g, const krk_optim& o, const GroupCall& call,
                               const uint64_t* ids, const float* grads, float lr, bool wide,
@@ -3076,7 +3082,7 @@ int32_t krk_group_push(krk_group* g, const krk_optim* o, const uint64_t* ids, co
   GroupCall call;
   int64_t total = 0;
   const bool wide = push_is_wide(g->vec, g->group, g->elems);
-  KRK_TRY(group_plan(g, offsets, &call, &total, wide ? (kBlock / kWave) * kWideIds : 0));
+  KRK_TRY(group_plan(g, offsets, &call, &total, wide ? (group_wide_block(g->group) / kWave) * kWideIds : 0));
   if (total == 0) return group_finish(g, flags);
   if (!ids || !grads) return KRK_E_ARGUMENT;
   if ((flags & KRK_DEVICE_PTRS) && g->vec == 4 && !aligned16(grads)) return KRK_E_ARGUMENT;

@@ -47,7 +47,7 @@ def test_emitter_test_combined_shape(api, oracle):
 
 @pytest.mark.parametrize("name,type_,conf", [c for c in OPTIM_CASES if c[0] in (
     "sgd_mom", "adagrad", "adam", "rmsprop_all")], ids=lambda v: v if isinstance(v, str) else None)
-@pytest.mark.parametrize("dim,n_tables", [(16, 26), (30, 3), (128, 5)])
+@pytest.mark.parametrize("dim,n_tables", [(16, 26), (30, 3), (64, 7), (128, 5)])
 def test_group_matches_oracle_loop(api, oracle, name, type_, conf, dim, n_tables):
     """The Wide&Deep shape: n tables, one Zipf batch each, pull then push, several steps, with
     new ids arriving at every step (insert-on-pull inside the combined launch)."""
