@@ -180,9 +180,12 @@ __global__ __launch_bounds__(kBlock) void dedup_emit_kernel(DSlot* slots,
                                                             const uint32_t* __restrict__ slot_of,
                                                             const int32_t* __restrict__ rank,
                                                             const uint64_t* __restrict__ ids, int64_t n,
-                                                            uint64_t* __restrict__ uids) {
+                                                            uint64_t* __restrict__ uids,
+                                                            const int32_t* __restrict__ total,
+                                                            int32_t* __restrict__ host_total) {
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p >= n) return;
+  if (p == 0 && host_total) *host_total = *total;      // the count, where a blocking caller reads it
   DSlot* s = &slots[slot_of[p]];
   if (s->minpos == (uint32_t)p) {
     uids[rank[p]] = ids[p];
@@ -211,7 +214,8 @@ constexpr uint32_t kNoPos = 0xFFFFFFFFu;
 __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t* __restrict__ ids, int n,
                                                                   uint64_t* __restrict__ uids,
                                                                   long long* __restrict__ inv,
-                                                                  int32_t* __restrict__ total) {
+                                                                  int32_t* __restrict__ total,
+                                                                  int32_t* __restrict__ host_total) {
   __shared__ unsigned long long sid[kDedupSmall];
   __shared__ uint32_t tab[kDedupSmallSlots];           // position of the id's first occurrence, then its unique index
   __shared__ uint32_t wave_total[kDedupBlock / kWave];
@@ -278,7 +282,10 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
       ++rank;
     }
   }
-  if (t == 0) *total = (int32_t)all;
+  if (t == 0) {
+    *total = (int32_t)all;
+    if (host_total) *host_total = (int32_t)all;
+  }
   if (!inv) return;
   __syncthreads();
 #pragma unroll
@@ -1523,14 +1530,15 @@ static int32_t dedup_enqueue(const DedupWork& w, const uint64_t* d_ids, int64_t 
   hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, w.slots, w.slot_of, n, w.flag);
   KRK_HIP(hipGetLastError());
   KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
-  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids);
+  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids,
+                     w.d_total, (int32_t*)nullptr);
   if (d_inv) hipLaunchKernelGGL(dedup_inv_kernel, grid, block, 0, s, w.slots, w.slot_of, n, d_inv);
   KRK_HIP(hipGetLastError());
   return KRK_SUCCESS;
 }
 
-// Where a blocking dedup's count lands: page-locked host memory the last kernel's total is copied
-// into in stream order, so the host waits for the stream once and reads it (no blocking copy).
+// Where a blocking dedup's count lands: page-locked host memory that the kernel which knows the
+// total writes to, so the host waits for the stream once and reads it (no copy in the stream).
 static int32_t* g_dedup_count = nullptr;
 
 static int32_t dedup_count_buffer() {
@@ -1539,16 +1547,15 @@ static int32_t dedup_count_buffer() {
   return KRK_SUCCESS;
 }
 
-static int32_t dedup_read_count(const int32_t* d_total, hipStream_t s, int32_t* u) {
-  KRK_TRY(dedup_count_buffer());
-  KRK_HIP(hipMemcpyAsync(g_dedup_count, d_total, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+static int32_t dedup_read_count(hipStream_t s, int32_t* u) {
   KRK_HIP(hipStreamSynchronize(s));
-  *u = *g_dedup_count;
+  *u = *static_cast<volatile int32_t*>(g_dedup_count);
   return KRK_SUCCESS;
 }
 
 static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, uint64_t* d_uids,
                           long long* d_inv, hipStream_t s, int32_t* u) {
+  KRK_TRY(dedup_count_buffer());
   KRK_HIP(hipMemsetAsync(w.slots, 0xFF, (w.cap + 1) * sizeof(DSlot), s));
   const dim3 grid(grid_for(n, kBlock)), block(kBlock);
   hipLaunchKernelGGL(dedup_claim_kernel, dim3(grid_for(n, kDedupBlock)), dim3(kDedupBlock), 0, s, w.slots,
@@ -1556,10 +1563,11 @@ static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, 
   hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, w.slots, w.slot_of, n, w.flag);
   KRK_HIP(hipGetLastError());
   KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
-  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids);
+  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids,
+                     w.d_total, g_dedup_count);
   if (d_inv) hipLaunchKernelGGL(dedup_inv_kernel, grid, block, 0, s, w.slots, w.slot_of, n, d_inv);
   KRK_HIP(hipGetLastError());
-  return dedup_read_count(w.d_total, s, u);
+  return dedup_read_count(s, u);
 }
 
 int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, int64_t* n_unique,
@@ -1592,10 +1600,11 @@ int32_t krk_dedup(const uint64_t* ids, int64_t n, uint64_t* uids, int64_t* inv, 
   hipStream_t s = nullptr;
   int32_t u = 0;
   if (n <= kDedupSmall) {
+    KRK_TRY(dedup_count_buffer());
     hipLaunchKernelGGL(dedup_small_kernel, dim3(1), dim3(kDedupBlock), 0, s, d_ids, (int)n, d_uids,
-                       inv ? d_inv : nullptr, w.d_total);
+                       inv ? d_inv : nullptr, w.d_total, g_dedup_count);
     KRK_HIP(hipGetLastError());
-    KRK_TRY(dedup_read_count(w.d_total, s, &u));
+    KRK_TRY(dedup_read_count(s, &u));
   } else {
     KRK_TRY(dedup_core(w, d_ids, n, d_uids, inv ? d_inv : nullptr, s, &u));
   }
