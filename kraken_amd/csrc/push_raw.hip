@@ -205,19 +205,24 @@ __global__ __launch_bounds__(kBlock) void dedup_inv_kernel(const DSlot* __restri
 // sit in LDS; an open-addressing table of positions (a slot holds the smallest position of the
 // id that owns it, and the id itself is looked up through that position) replaces the index in
 // global memory; a lane owns eight consecutive positions, so one scan over the workgroup gives
-// every first occurrence its place in the unique list.
+// every first occurrence its place in the unique list. The unique ids are compacted in LDS (over
+// the ids, which nobody reads after the claims) and every position's slot is kept there too, so
+// that both results leave in position order, a wavefront's stores side by side: a lane writing
+// its own eight positions touched a 64-byte piece per store, 3.5 us more for 8192 ids.
 constexpr int kDedupSmall = 8192;
 constexpr int kDedupSmallSlots = 2 * kDedupSmall;
 constexpr int kDedupSmallOwn = kDedupSmall / kDedupBlock;
 constexpr uint32_t kNoPos = 0xFFFFFFFFu;
+static_assert(kDedupSmallSlots <= 65536, "a position's slot is kept in 16 bits");
 
 __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t* __restrict__ ids, int n,
                                                                   uint64_t* __restrict__ uids,
                                                                   long long* __restrict__ inv,
                                                                   int32_t* __restrict__ total,
                                                                   int32_t* __restrict__ host_total) {
-  __shared__ unsigned long long sid[kDedupSmall];
+  __shared__ unsigned long long sid[kDedupSmall];      // the ids by position, then the unique ids
   __shared__ uint32_t tab[kDedupSmallSlots];           // position of the id's first occurrence, then its unique index
+  __shared__ uint16_t slot_of[kDedupSmall];
   __shared__ uint32_t wave_total[kDedupBlock / kWave];
   const int t = threadIdx.x;
   // table size by request size: a small request clears and probes a small table
@@ -228,9 +233,12 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
   for (int i = t; i < n; i += kDedupBlock) sid[i] = ids[i];
   __syncthreads();
   uint32_t slot[kDedupSmallOwn];
+  unsigned long long mine_id[kDedupSmallOwn];
 #pragma unroll
   for (int i = 0; i < kDedupSmallOwn; ++i) {
     const int p = t * kDedupSmallOwn + i;
+    slot[i] = 0;
+    mine_id[i] = 0;
     if (p < n) {
       const unsigned long long id = sid[p];
       uint32_t h = (uint32_t)(mix64(id) >> 32) & mask;
@@ -247,9 +255,11 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
         h = (h + 1) & mask;
       }
       slot[i] = h;
+      mine_id[i] = id;
+      slot_of[p] = (uint16_t)h;
     }
   }
-  __syncthreads();
+  __syncthreads();                                     // the claims are over: nobody reads sid[] by position again
   uint32_t first = 0;                                  // bit i: my position i is its id's first
 #pragma unroll
   for (int i = 0; i < kDedupSmallOwn; ++i) {
@@ -276,8 +286,7 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
 #pragma unroll
   for (int i = 0; i < kDedupSmallOwn; ++i) {
     if (first & (1u << i)) {
-      const int p = t * kDedupSmallOwn + i;
-      uids[rank] = sid[p];
+      sid[rank] = mine_id[i];
       tab[slot[i]] = rank;                             // the table now answers with the unique index
       ++rank;
     }
@@ -286,13 +295,10 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
     *total = (int32_t)all;
     if (host_total) *host_total = (int32_t)all;
   }
-  if (!inv) return;
   __syncthreads();
-#pragma unroll
-  for (int i = 0; i < kDedupSmallOwn; ++i) {
-    const int p = t * kDedupSmallOwn + i;
-    if (p < n) inv[p] = (long long)tab[slot[i]];
-  }
+  for (int r = t; r < (int)all; r += kDedupBlock) uids[r] = sid[r];
+  if (!inv) return;
+  for (int p = t; p < n; p += kDedupBlock) inv[p] = (long long)tab[slot_of[p]];
 }
 
 // ---------------------------------------------------------------------------
