@@ -109,7 +109,8 @@ constexpr int kDedupLds = 2048;   // entries: at most half full
 
 __global__ __launch_bounds__(kDedupBlock) void dedup_claim_kernel(DSlot* slots, uint64_t mask,
                                                                   const uint64_t* __restrict__ ids, int64_t n,
-                                                                  uint32_t* __restrict__ slot_of) {
+                                                                  uint32_t* __restrict__ slot_of,
+                                                                  uint32_t first_block) {
   __shared__ unsigned long long lkey[kDedupLds + 1];   // the last entry belongs to the all-ones id
   __shared__ uint32_t lmin[kDedupLds + 1];
   __shared__ uint32_t lidx[kDedupLds + 1];
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_claim_kernel(DSlot* slots, 
     lmin[i] = 0xFFFFFFFFu;
   }
   __syncthreads();
-  const int64_t p = (int64_t)blockIdx.x * kDedupBlock + threadIdx.x;
+  const int64_t p = (int64_t)(blockIdx.x + first_block) * kDedupBlock + threadIdx.x;
   const bool active = p < n;
   const unsigned long long id = active ? ids[p] : 0ull;
   int entry = kDedupLds;
@@ -1525,14 +1526,33 @@ static int32_t dedup_layout(int64_t n, size_t extra_bytes, DedupWork* w) {
 // call waits for the device once.
 // The launches alone, nothing read back. The index is cleared by a fill kernel rather than a
 // memset node so that a caller may record these launches into a graph.
+// The claims of a request. Its first kDedupHead workgroups go ahead of the others in a launch of
+// their own: the ids that fill much of a skewed request are all among the first few thousand
+// positions, so every later workgroup finds their slots claimed and holding a smaller position,
+// with plain loads. Launched all at once, the few hundred workgroups that start together each see
+// such a slot empty and each send it a compare-and-swap and a minimum, and the memory serves the
+// atomics of one address one after the other.
+constexpr unsigned kDedupHead = 8;
+
+static void launch_dedup_claims(const DedupWork& w, const uint64_t* d_ids, int64_t n, hipStream_t s) {
+  const unsigned blocks = grid_for(n, kDedupBlock);
+  unsigned head = 0;
+  if (blocks >= 4 * kDedupHead) {
+    head = kDedupHead;
+    hipLaunchKernelGGL(dedup_claim_kernel, dim3(head), dim3(kDedupBlock), 0, s, w.slots, w.cap - 1, d_ids, n,
+                       w.slot_of, 0u);
+  }
+  hipLaunchKernelGGL(dedup_claim_kernel, dim3(blocks - head), dim3(kDedupBlock), 0, s, w.slots, w.cap - 1, d_ids,
+                     n, w.slot_of, head);
+}
+
 static int32_t dedup_enqueue(const DedupWork& w, const uint64_t* d_ids, int64_t n, uint64_t* d_uids,
                              long long* d_inv, hipStream_t s) {
   const int64_t words = (int64_t)(w.cap + 1) * (int64_t)(sizeof(DSlot) / 4);
   hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(words, kBlock)), dim3(kBlock), 0, s,
                      reinterpret_cast<uint32_t*>(w.slots), words, 0xFFFFFFFFu);
   const dim3 grid(grid_for(n, kBlock)), block(kBlock);
-  hipLaunchKernelGGL(dedup_claim_kernel, dim3(grid_for(n, kDedupBlock)), dim3(kDedupBlock), 0, s, w.slots,
-                     w.cap - 1, d_ids, n, w.slot_of);
+  launch_dedup_claims(w, d_ids, n, s);
   hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, w.slots, w.slot_of, n, w.flag);
   KRK_HIP(hipGetLastError());
   KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
@@ -1564,8 +1584,7 @@ static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, 
   KRK_TRY(dedup_count_buffer());
   KRK_HIP(hipMemsetAsync(w.slots, 0xFF, (w.cap + 1) * sizeof(DSlot), s));
   const dim3 grid(grid_for(n, kBlock)), block(kBlock);
-  hipLaunchKernelGGL(dedup_claim_kernel, dim3(grid_for(n, kDedupBlock)), dim3(kDedupBlock), 0, s, w.slots,
-                     w.cap - 1, d_ids, n, w.slot_of);
+  launch_dedup_claims(w, d_ids, n, s);
   hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, w.slots, w.slot_of, n, w.flag);
   KRK_HIP(hipGetLastError());
   KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
