@@ -256,7 +256,7 @@ def test_flagged_push_reads_the_notes_and_drops_stale_ones(api):
     t.close()
 
 
-@pytest.mark.parametrize("dim", [16, 32])
+@pytest.mark.parametrize("dim", [16, 32, 64])
 def test_group_push_of_unique_ids_with_notes_equals_without(api, dim):
     rng = np.random.default_rng(7 + dim)
     o = api.Optim.create(api.OptimType.kAdagrad)
