@@ -61,7 +61,11 @@ def test_dedup_empty(api):
     assert u.size == 0 and inv.size == 0
 
 
-@pytest.mark.parametrize("n,s,space", [(8192, 1.05, 10**6), (200_000, 1.3, 10**6), (1_000_000, 1.1, 10**7)])
+# 31 / 32 and 127 / 128 workgroups of 1024 positions: below, at and between the sizes from which
+# the first 8 or 32 workgroups claim their ids in a launch ahead of the others
+@pytest.mark.parametrize("n,s,space", [(8192, 1.05, 10**6), (31 * 1024 + 7, 1.2, 10**5), (32 * 1024, 1.2, 10**5),
+                                       (127 * 1024 + 1, 1.3, 10**6), (128 * 1024 + 1, 1.3, 10**6),
+                                       (200_000, 1.3, 10**6), (1_000_000, 1.1, 10**7)])
 def test_dedup_zipf_exact(api, oracle, n, s, space):
     rng = np.random.default_rng(n)
     ids = zipf_ids(rng, s, space, n)
