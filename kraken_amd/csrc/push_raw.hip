@@ -177,29 +177,28 @@ __global__ __launch_bounds__(kBlock) void dedup_flag_kernel(const DSlot* __restr
   flag[p] = slots[slot_of[p]].minpos == (uint32_t)p ? 1 : 0;
 }
 
+// Every position learns its id's index in the unique list from the rank of the id's first
+// position, and the first position also writes the id there and leaves the index in the slot
+// (one launch: a second one that read the index out of the slot had to wait for this one).
 __global__ __launch_bounds__(kBlock) void dedup_emit_kernel(DSlot* slots,
                                                             const uint32_t* __restrict__ slot_of,
                                                             const int32_t* __restrict__ rank,
                                                             const uint64_t* __restrict__ ids, int64_t n,
                                                             uint64_t* __restrict__ uids,
+                                                            long long* __restrict__ inv,
                                                             const int32_t* __restrict__ total,
                                                             int32_t* __restrict__ host_total) {
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p >= n) return;
   if (p == 0 && host_total) *host_total = *total;      // the count, where a blocking caller reads it
   DSlot* s = &slots[slot_of[p]];
-  if (s->minpos == (uint32_t)p) {
-    uids[rank[p]] = ids[p];
-    s->uidx = (uint32_t)rank[p];
+  const uint32_t first = s->minpos;
+  const int32_t r = rank[first];
+  if (inv) inv[p] = (long long)r;
+  if (first == (uint32_t)p) {
+    uids[r] = ids[p];
+    s->uidx = (uint32_t)r;
   }
-}
-
-__global__ __launch_bounds__(kBlock) void dedup_inv_kernel(const DSlot* __restrict__ slots,
-                                                           const uint32_t* __restrict__ slot_of,
-                                                           int64_t n, long long* __restrict__ inv) {
-  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (p >= n) return;
-  inv[p] = (long long)slots[slot_of[p]].uidx;
 }
 
 // Requests of at most kDedupSmall ids: the whole dedup in one launch of one workgroup. The ids
@@ -1557,9 +1556,8 @@ static int32_t dedup_enqueue(const DedupWork& w, const uint64_t* d_ids, int64_t 
   hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, w.slots, w.slot_of, n, w.flag);
   KRK_HIP(hipGetLastError());
   KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
-  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids,
+  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids, d_inv,
                      w.d_total, (int32_t*)nullptr);
-  if (d_inv) hipLaunchKernelGGL(dedup_inv_kernel, grid, block, 0, s, w.slots, w.slot_of, n, d_inv);
   KRK_HIP(hipGetLastError());
   return KRK_SUCCESS;
 }
@@ -1589,9 +1587,8 @@ static int32_t dedup_core(const DedupWork& w, const uint64_t* d_ids, int64_t n, 
   hipLaunchKernelGGL(dedup_flag_kernel, grid, block, 0, s, w.slots, w.slot_of, n, w.flag);
   KRK_HIP(hipGetLastError());
   KRK_TRY(exclusive_scan_i32(w.flag, w.rank, n, w.d_total, w.scan_tmp, s));
-  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids,
+  hipLaunchKernelGGL(dedup_emit_kernel, grid, block, 0, s, w.slots, w.slot_of, w.rank, d_ids, n, d_uids, d_inv,
                      w.d_total, g_dedup_count);
-  if (d_inv) hipLaunchKernelGGL(dedup_inv_kernel, grid, block, 0, s, w.slots, w.slot_of, n, d_inv);
   KRK_HIP(hipGetLastError());
   return dedup_read_count(s, u);
 }
