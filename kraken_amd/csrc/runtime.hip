@@ -169,17 +169,32 @@ __device__ inline int block_exclusive_scan(int v, int* lds, int& block_total) {
   return base + x - v;
 }
 
+// A lane's kScanItems consecutive values, as two 16-byte loads where the array allows it: one
+// 4-byte access per lane and trip touches a 32-byte piece of a line eight times over.
+static_assert(kScanItems == 8, "a lane's values are two 16-byte vectors");
+__device__ __forceinline__ void scan_load_items(const int32_t* in, int64_t base, int64_t n,
+                                                int (&v)[kScanItems]) {
+  if ((reinterpret_cast<uintptr_t>(in) & 15) == 0 && base + kScanItems <= n) {
+    const int4 a = *reinterpret_cast<const int4*>(in + base);
+    const int4 b = *reinterpret_cast<const int4*>(in + base + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) v[i] = base + i < n ? in[base + i] : 0;
+  }
+}
+
 __global__ __launch_bounds__(kScanThreads) void scan_block_sums(const int32_t* __restrict__ in,
                                                                 int64_t n,
                                                                 int32_t* __restrict__ sums) {
   __shared__ int lds[kScanThreads / 64];
   int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  int v[kScanItems];
+  scan_load_items(in, base, n, v);
   int s = 0;
 #pragma unroll
-  for (int i = 0; i < kScanItems; ++i) {
-    int64_t j = base + i;
-    if (j < n) s += in[j];
-  }
+  for (int i = 0; i < kScanItems; ++i) s += v[i];
   int tot;
   block_exclusive_scan(s, lds, tot);
   if (threadIdx.x == 0) sums[blockIdx.x] = tot;
@@ -200,26 +215,31 @@ __global__ __launch_bounds__(kScanThreads) void scan_of_sums(int32_t* __restrict
   if (threadIdx.x == 0 && total_out) *total_out = carry;
 }
 
-__global__ __launch_bounds__(kScanThreads) void scan_apply(const int32_t* __restrict__ in,
-                                                           int32_t* __restrict__ out, int64_t n,
+// in and out may be the same array: a lane reads its values before it writes them
+__global__ __launch_bounds__(kScanThreads) void scan_apply(const int32_t* in, int32_t* out, int64_t n,
                                                            const int32_t* __restrict__ sums) {
   __shared__ int lds[kScanThreads / 64];
   int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
   int v[kScanItems];
+  scan_load_items(in, base, n, v);
   int s = 0;
 #pragma unroll
-  for (int i = 0; i < kScanItems; ++i) {
-    int64_t j = base + i;
-    v[i] = j < n ? in[j] : 0;
-    s += v[i];
-  }
+  for (int i = 0; i < kScanItems; ++i) s += v[i];
   int tot;
   int ex = block_exclusive_scan(s, lds, tot) + sums[blockIdx.x];
+  int r[kScanItems];
 #pragma unroll
   for (int i = 0; i < kScanItems; ++i) {
-    int64_t j = base + i;
-    if (j < n) out[j] = ex;
+    r[i] = ex;
     ex += v[i];
+  }
+  if ((reinterpret_cast<uintptr_t>(out) & 15) == 0 && base + kScanItems <= n) {
+    *reinterpret_cast<int4*>(out + base) = make_int4(r[0], r[1], r[2], r[3]);
+    *reinterpret_cast<int4*>(out + base + 4) = make_int4(r[4], r[5], r[6], r[7]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i)
+      if (base + i < n) out[base + i] = r[i];
   }
 }
 
