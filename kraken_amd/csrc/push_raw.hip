@@ -214,13 +214,16 @@ constexpr int kDedupSmallSlots = 2 * kDedupSmall;
 constexpr int kDedupSmallOwn = kDedupSmall / kDedupBlock;
 constexpr uint32_t kNoPos = 0xFFFFFFFFu;
 static_assert(kDedupSmallSlots <= 65536, "a position's slot is kept in 16 bits");
+// Where id number p sits in LDS: one entry is left out after every eight, so that the lanes of a
+// wavefront, which own eight consecutive ids each, do not all meet in the same two banks.
+__device__ __forceinline__ int dedup_small_at(int p) { return p + (p >> 3); }
 
 __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t* __restrict__ ids, int n,
                                                                   uint64_t* __restrict__ uids,
                                                                   long long* __restrict__ inv,
                                                                   int32_t* __restrict__ total,
                                                                   int32_t* __restrict__ host_total) {
-  __shared__ unsigned long long sid[kDedupSmall];      // the ids by position, then the unique ids
+  __shared__ unsigned long long sid[kDedupSmall + kDedupSmall / 8];   // the ids by position, then the unique ids
   __shared__ uint32_t tab[kDedupSmallSlots];           // position of the id's first occurrence, then its unique index
   __shared__ uint16_t slot_of[kDedupSmall];
   __shared__ uint32_t wave_total[kDedupBlock / kWave];
@@ -230,7 +233,7 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
   while ((1 << bits) < 2 * n) ++bits;
   const uint32_t mask = (1u << bits) - 1u;
   for (int i = t; i <= (int)mask; i += kDedupBlock) tab[i] = kNoPos;
-  for (int i = t; i < n; i += kDedupBlock) sid[i] = ids[i];
+  for (int i = t; i < n; i += kDedupBlock) sid[dedup_small_at(i)] = ids[i];
   __syncthreads();
   uint32_t slot[kDedupSmallOwn];
   unsigned long long mine_id[kDedupSmallOwn];
@@ -240,7 +243,7 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
     slot[i] = 0;
     mine_id[i] = 0;
     if (p < n) {
-      const unsigned long long id = sid[p];
+      const unsigned long long id = sid[dedup_small_at(p)];
       uint32_t h = (uint32_t)(mix64(id) >> 32) & mask;
       for (;;) {
         uint32_t q = tab[h];
@@ -248,7 +251,7 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
           q = atomicCAS(&tab[h], kNoPos, (uint32_t)p);
           if (q == kNoPos) break;                      // the slot is this id's now
         }
-        if (sid[q] == id) {                            // whoever holds it, it is the same id
+        if (sid[dedup_small_at((int)q)] == id) {        // whoever holds it, it is the same id
           atomicMin(&tab[h], (uint32_t)p);
           break;
         }
@@ -286,7 +289,7 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
 #pragma unroll
   for (int i = 0; i < kDedupSmallOwn; ++i) {
     if (first & (1u << i)) {
-      sid[rank] = mine_id[i];
+      sid[dedup_small_at((int)rank)] = mine_id[i];
       tab[slot[i]] = rank;                             // the table now answers with the unique index
       ++rank;
     }
@@ -296,7 +299,7 @@ __global__ __launch_bounds__(kDedupBlock) void dedup_small_kernel(const uint64_t
     if (host_total) *host_total = (int32_t)all;
   }
   __syncthreads();
-  for (int r = t; r < (int)all; r += kDedupBlock) uids[r] = sid[r];
+  for (int r = t; r < (int)all; r += kDedupBlock) uids[r] = sid[dedup_small_at(r)];
   if (!inv) return;
   for (int p = t; p < n; p += kDedupBlock) inv[p] = (long long)tab[slot_of[p]];
 }
